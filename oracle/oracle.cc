@@ -1,0 +1,604 @@
+// CPU oracle for the quantized FULLY_CONNECTED path. TEST INFRASTRUCTURE ONLY:
+// see oracle.h. Compile with -ffp-contract=off and without fast-math.
+#include "oracle.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <limits>
+#include <vector>
+
+namespace {
+
+// ---- fixed-point helpers --------------------------------------------------
+
+// gemmlowp SaturatingRoundingDoublingHighMul (fixedpoint.h @16e8662c): the
+// high 32 bits of 2*a*b with round-to-nearest, ties away from zero, computed
+// with a truncating 64-bit division.
+inline int32_t Srdhm(int32_t a, int32_t b) {
+  if (a == b && a == std::numeric_limits<int32_t>::min()) {
+    return std::numeric_limits<int32_t>::max();
+  }
+  const int64_t ab = static_cast<int64_t>(a) * static_cast<int64_t>(b);
+  const int64_t nudge = ab >= 0 ? (1ll << 30) : (1 - (1ll << 30));
+  return static_cast<int32_t>((ab + nudge) / (1ll << 31));
+}
+
+// gemmlowp RoundingDivideByPOT: arithmetic shift right with round-to-nearest,
+// ties away from zero.
+inline int32_t RoundingDivideByPot(int32_t x, int exponent) {
+  const int32_t mask = static_cast<int32_t>((1ll << exponent) - 1);
+  const int32_t remainder = x & mask;
+  const int32_t threshold = (mask >> 1) + (x < 0 ? 1 : 0);
+  return (x >> exponent) + (remainder > threshold ? 1 : 0);
+}
+
+// common.cc:80-90. `x * (1 << left_shift)` wraps in the reference build (the
+// function is marked no-sanitize-integer-overflow); reproduce with unsigned.
+inline int32_t Mbqm(int32_t x, int32_t quantized_multiplier, int shift) {
+  const int left_shift = shift > 0 ? shift : 0;
+  const int right_shift = shift > 0 ? 0 : -shift;
+  const int32_t shifted = static_cast<int32_t>(static_cast<uint32_t>(x) << left_shift);
+  return RoundingDivideByPot(Srdhm(shifted, quantized_multiplier), right_shift);
+}
+
+// common.cc:33-47.
+inline int32_t MbqmSingleRounding(int32_t x, int32_t quantized_multiplier, int shift) {
+  const int64_t total_shift = 31 - shift;
+  const int64_t round = static_cast<int64_t>(1) << (total_shift - 1);
+  int64_t result = x * static_cast<int64_t>(quantized_multiplier) + round;
+  result = result >> total_shift;
+  return static_cast<int32_t>(result);
+}
+
+inline int32_t ClampI32(int32_t v, int32_t lo, int32_t hi) {
+  v = std::max(v, lo);
+  v = std::min(v, hi);
+  return v;
+}
+
+// kernel_util.cc:343-352: float division, round half away, then add.
+inline bool QuantizeForRange(float scale, int32_t zero_point, float f, int32_t* q) {
+  const float tmp = std::round(f / scale);
+  const bool fits = tmp >= static_cast<float>(std::numeric_limits<int32_t>::min()) &&
+                    tmp <= static_cast<float>(std::numeric_limits<int32_t>::max());
+  if (!fits) return false;
+  *q = zero_point + static_cast<int32_t>(tmp);
+  return true;
+}
+
+// ---- activation quantization ---------------------------------------------
+
+// neon_tensor_utils.cc:2347-2359.
+inline int32_t RoundToNearestVariant(float x, int variant) {
+  if (variant == ORC_QUANT_NEON_LEGACY) {
+    const float nudge = (x < 0.0f ? -1.0f : 0.0f) + 0.5f;
+    return static_cast<int32_t>(x + nudge);  // float add, then truncation
+  }
+  return static_cast<int32_t>(std::round(x));  // vcvta: nearest, ties away
+}
+
+// neon_tensor_utils.cc:2363-2399: min/max capped at zero; NaN handling aside,
+// the value equals min(0, min v) / max(0, max v).
+inline void MinMaxCappedAtZero(const float* values, int size, float* mn, float* mx) {
+  float rmin = 0.0f, rmax = 0.0f;
+  for (int i = 0; i < size; ++i) {
+    rmin = std::min(rmin, values[i]);
+    rmax = std::max(rmax, values[i]);
+  }
+  *mn = rmin;
+  *mx = rmax;
+}
+
+void AsymmetricQuantize(const float* values, int size, int8_t* quantized, float* scaling_factor,
+                        int32_t* offset, int variant) {
+  const double qmin = -128.0, qmax = 127.0;
+  double rmin, rmax, scale;
+  if (variant == ORC_QUANT_PORTABLE) {
+    // reference/portable_tensor_utils.cc:74-84: the range is widened to
+    // double before the subtraction.
+    const auto mm = std::minmax_element(values, values + size);
+    rmin = static_cast<double>(std::min(0.0f, *mm.first));
+    rmax = static_cast<double>(std::max(0.0f, *mm.second));
+    if (rmin == rmax) {
+      std::memset(quantized, 0, size);
+      *scaling_factor = 1;
+      *offset = 0;
+      return;
+    }
+    scale = (rmax - rmin) / (qmax - qmin);
+  } else {
+    // neon_tensor_utils.cc:2470-2486: rmin/rmax stay float, so the range
+    // subtraction is a float operation.
+    float fmin, fmax;
+    MinMaxCappedAtZero(values, size, &fmin, &fmax);
+    if (fmin == fmax) {
+      std::memset(quantized, 0, size);
+      *scaling_factor = 1;
+      *offset = 0;
+      return;
+    }
+    scale = (fmax - fmin) / (qmax - qmin);
+    rmin = fmin;
+    rmax = fmax;
+  }
+  const double zp_from_min = qmin - rmin / scale;
+  const double zp_from_max = qmax - rmax / scale;
+  const double err_from_min = std::abs(qmin) + std::abs(rmin / scale);
+  const double err_from_max = std::abs(qmax) + std::abs(rmax / scale);
+  const double zp_double = err_from_min < err_from_max ? zp_from_min : zp_from_max;
+  int8_t nudged;
+  if (zp_double <= qmin) {
+    nudged = -128;
+  } else if (zp_double >= qmax) {
+    nudged = 127;
+  } else {
+    nudged = static_cast<int8_t>(std::round(zp_double));
+  }
+  *scaling_factor = static_cast<float>(scale);
+  *offset = nudged;
+
+  if (variant == ORC_QUANT_PORTABLE) {
+    // reference/portable_tensor_utils.cc:112-118.
+    const float inv = 1.0f / *scaling_factor;
+    for (int i = 0; i < size; ++i) {
+      const float scaled = values[i] * inv;
+      const float shifted = static_cast<float>(*offset) + scaled;
+      const int32_t q = static_cast<int32_t>(std::round(shifted));
+      quantized[i] = static_cast<int8_t>(std::min(127, std::max(-128, q)));
+    }
+    return;
+  }
+  // neon_tensor_utils.cc:2509-2551: inverse through double, round first, add
+  // the zero point as an integer. The scalar tail (size % 8 elements) rounds
+  // with std::round whichever build it is.
+  const float inv = *scaling_factor == 0 ? 0.0f
+                                         : static_cast<float>(1.0 / static_cast<double>(*scaling_factor));
+  const int vector_end = size - (size % 8);
+  for (int i = 0; i < size; ++i) {
+    const float scaled = values[i] * inv;
+    int32_t q;
+    if (i < vector_end) {
+      q = RoundToNearestVariant(scaled, variant) + *offset;
+    } else {
+      q = static_cast<int32_t>(static_cast<float>(*offset) + std::round(inv * values[i]));
+    }
+    quantized[i] = static_cast<int8_t>(std::min(127, std::max(-128, q)));
+  }
+}
+
+void SymmetricQuantize(const float* values, int size, int8_t* quantized, float* scaling_factor,
+                       int variant) {
+  // reference/portable_tensor_utils.cc:41-71; neon_tensor_utils.cc:2401-2468.
+  const auto mm = std::minmax_element(values, values + size);
+  const float range = std::max(std::abs(*mm.first), std::abs(*mm.second));
+  if (range == 0) {
+    std::memset(quantized, 0, size);
+    *scaling_factor = 1;
+    return;
+  }
+  *scaling_factor = range / 127;
+  const float inv = 127 / range;
+  const int vector_end = (variant == ORC_QUANT_PORTABLE) ? 0 : size - (size % 8);
+  for (int i = 0; i < size; ++i) {
+    int32_t q;
+    if (i < vector_end) {
+      q = RoundToNearestVariant(values[i] * inv, variant);
+    } else {
+      q = static_cast<int32_t>(std::round(values[i] * inv));
+    }
+    quantized[i] = static_cast<int8_t>(std::min(127, std::max(-127, q)));
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+void orc_quantize_multiplier(double real_multiplier, int32_t* quantized_multiplier, int* shift) {
+  if (real_multiplier == 0.) {
+    *quantized_multiplier = 0;
+    *shift = 0;
+    return;
+  }
+  const double q = std::frexp(real_multiplier, shift);
+  int64_t q_fixed = static_cast<int64_t>(std::round(q * static_cast<double>(1ll << 31)));
+  if (q_fixed == (1ll << 31)) {
+    q_fixed /= 2;
+    ++*shift;
+  }
+  if (*shift < -31) {
+    *shift = 0;
+    q_fixed = 0;
+  }
+  *quantized_multiplier = static_cast<int32_t>(q_fixed);
+}
+
+int32_t orc_srdhm(int32_t a, int32_t b) { return Srdhm(a, b); }
+int32_t orc_rounding_divide_by_pot(int32_t x, int exponent) { return RoundingDivideByPot(x, exponent); }
+int32_t orc_mbqm(int32_t x, int32_t m, int shift) { return Mbqm(x, m, shift); }
+int32_t orc_mbqm_single_rounding(int32_t x, int32_t m, int shift) {
+  return MbqmSingleRounding(x, m, shift);
+}
+
+int orc_activation_range_int8(int activation, float out_scale, int32_t out_zero_point,
+                              int32_t* act_min, int32_t* act_max) {
+  const int32_t qmin = -128, qmax = 127;
+  int32_t q;
+  if (activation == ORC_ACT_RELU) {
+    if (!QuantizeForRange(out_scale, out_zero_point, 0.0f, &q)) return 1;
+    *act_min = std::max(qmin, q);
+    *act_max = qmax;
+  } else if (activation == ORC_ACT_RELU6) {
+    if (!QuantizeForRange(out_scale, out_zero_point, 0.0f, &q)) return 1;
+    *act_min = std::max(qmin, q);
+    if (!QuantizeForRange(out_scale, out_zero_point, 6.0f, &q)) return 1;
+    *act_max = std::min(qmax, q);
+  } else if (activation == ORC_ACT_RELU_N1_TO_1) {
+    if (!QuantizeForRange(out_scale, out_zero_point, -1.0f, &q)) return 1;
+    *act_min = std::max(qmin, q);
+    if (!QuantizeForRange(out_scale, out_zero_point, 1.0f, &q)) return 1;
+    *act_max = std::min(qmax, q);
+  } else {
+    *act_min = qmin;
+    *act_max = qmax;
+  }
+  return 0;
+}
+
+float orc_half_to_float(uint16_t h) {
+  const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
+  const uint32_t exp = (h >> 10) & 0x1Fu;
+  uint32_t man = h & 0x3FFu;
+  uint32_t bits;
+  if (exp == 0) {
+    if (man == 0) {
+      bits = sign;
+    } else {
+      // subnormal half: normalise into a float exponent
+      int e = -1;
+      do {
+        man <<= 1;
+        ++e;
+      } while ((man & 0x400u) == 0);
+      bits = sign | static_cast<uint32_t>(127 - 15 - e) << 23 | (man & 0x3FFu) << 13;
+    }
+  } else if (exp == 31) {
+    bits = sign | 0x7F800000u | man << 13;
+  } else {
+    bits = sign | (exp + (127 - 15)) << 23 | man << 13;
+  }
+  float f;
+  std::memcpy(&f, &bits, sizeof f);
+  return f;
+}
+
+void orc_unpack_int4(const int8_t* src, int num_elements, int8_t* dst) {
+  for (int i = 0; i < num_elements / 2; ++i) {
+    const int8_t byte = src[i];
+    dst[2 * i] = static_cast<int8_t>(static_cast<int8_t>(byte << 4) >> 4);
+    dst[2 * i + 1] = static_cast<int8_t>(byte >> 4);
+  }
+  if (num_elements % 2 != 0) {
+    const int8_t byte = src[num_elements / 2];
+    dst[num_elements - 1] = static_cast<int8_t>(static_cast<int8_t>(byte << 4) >> 4);
+  }
+}
+
+int orc_fc_prepare_per_channel(float input_scale, const float* filter_scales, int num_channels,
+                               float output_scale, int32_t* multipliers, int32_t* shifts) {
+  for (int i = 0; i < num_channels; ++i) {
+    const double filter_scale = static_cast<double>(filter_scales[i]);
+    const double effective = static_cast<double>(input_scale) * filter_scale /
+                             static_cast<double>(output_scale);
+    int shift;
+    orc_quantize_multiplier(effective, &multipliers[i], &shift);
+    shifts[i] = shift;
+  }
+  return 0;
+}
+
+int orc_fc_prepare_per_tensor(float input_scale, float filter_scale, int has_bias,
+                              float bias_scale, float output_scale, int32_t* multiplier,
+                              int32_t* shift) {
+  if (has_bias) {
+    // kernel_util.cc:296-322: product formed in double for the check.
+    const double product = static_cast<double>(input_scale) * static_cast<double>(filter_scale);
+    const double diff = std::abs(product - static_cast<double>(bias_scale));
+    if (!(diff / static_cast<double>(output_scale) <= 0.02)) return 1;
+  }
+  // kernel_util.cc:333-338: product formed in float, then widened.
+  const double product = static_cast<double>(input_scale * filter_scale);
+  if (!(product >= 0)) return 1;
+  const double real_multiplier = product / static_cast<double>(output_scale);
+  int s;
+  orc_quantize_multiplier(real_multiplier, multiplier, &s);
+  *shift = s;
+  return 0;
+}
+
+void orc_fc_int8_per_channel(const int8_t* input, const int8_t* filter, const int32_t* bias,
+                             const int32_t* multipliers, const int32_t* shifts, int8_t* output,
+                             int batches, int depth, int out_depth, int32_t input_offset,
+                             int32_t output_offset, int32_t act_min, int32_t act_max) {
+  for (int b = 0; b < batches; ++b) {
+    for (int c = 0; c < out_depth; ++c) {
+      int32_t acc = 0;
+      for (int d = 0; d < depth; ++d) {
+        acc += static_cast<int32_t>(filter[c * depth + d]) *
+               (static_cast<int32_t>(input[b * depth + d]) + input_offset);
+      }
+      if (bias) acc += bias[c];
+      int32_t v = Mbqm(acc, multipliers[c], shifts[c]) + output_offset;
+      output[c + out_depth * b] = static_cast<int8_t>(ClampI32(v, act_min, act_max));
+    }
+  }
+}
+
+void orc_fc_int8_per_channel_single_rounding(const int8_t* input, const int8_t* filter,
+                                             const int32_t* bias, const int32_t* multipliers,
+                                             const int32_t* shifts, int8_t* output, int batches,
+                                             int depth, int out_depth, int32_t input_offset,
+                                             int32_t output_offset, int32_t act_min,
+                                             int32_t act_max) {
+  for (int b = 0; b < batches; ++b) {
+    for (int c = 0; c < out_depth; ++c) {
+      int32_t acc = 0;
+      for (int d = 0; d < depth; ++d) {
+        acc += static_cast<int32_t>(filter[c * depth + d]) *
+               (static_cast<int32_t>(input[b * depth + d]) + input_offset);
+      }
+      if (bias) acc += bias[c];
+      int32_t v = MbqmSingleRounding(acc, multipliers[c], shifts[c]) + output_offset;
+      output[c + out_depth * b] = static_cast<int8_t>(ClampI32(v, act_min, act_max));
+    }
+  }
+}
+
+void orc_fc_int8_per_channel_float_scale(const int8_t* input, const int8_t* filter,
+                                         const int32_t* bias, const float* filter_scales,
+                                         float input_scale, float output_scale, int8_t* output,
+                                         int batches, int depth, int out_depth,
+                                         int32_t input_offset, int32_t output_offset,
+                                         int32_t act_min, int32_t act_max) {
+  for (int b = 0; b < batches; ++b) {
+    for (int c = 0; c < out_depth; ++c) {
+      int32_t acc = 0;
+      for (int d = 0; d < depth; ++d) {
+        acc += static_cast<int32_t>(filter[c * depth + d]) *
+               (static_cast<int32_t>(input[b * depth + d]) + input_offset);
+      }
+      if (bias) acc += bias[c];
+      const double effective = static_cast<double>(input_scale) *
+                               static_cast<double>(filter_scales[c]) /
+                               static_cast<double>(output_scale);
+      int32_t v = static_cast<int32_t>(std::round(static_cast<double>(acc) * effective));
+      v += output_offset;
+      output[c + out_depth * b] = static_cast<int8_t>(ClampI32(v, act_min, act_max));
+    }
+  }
+}
+
+void orc_fc_int8_per_tensor(const int8_t* input, const int8_t* filter, const int32_t* bias,
+                            int32_t multiplier, int shift, int8_t* output, int batches, int depth,
+                            int out_depth, int32_t input_offset, int32_t filter_offset,
+                            int32_t output_offset, int32_t act_min, int32_t act_max) {
+  for (int b = 0; b < batches; ++b) {
+    for (int c = 0; c < out_depth; ++c) {
+      int32_t acc = 0;
+      for (int d = 0; d < depth; ++d) {
+        acc += (static_cast<int32_t>(filter[c * depth + d]) + filter_offset) *
+               (static_cast<int32_t>(input[b * depth + d]) + input_offset);
+      }
+      if (bias) acc += bias[c];
+      int32_t v = Mbqm(acc, multiplier, shift) + output_offset;
+      output[c + out_depth * b] = static_cast<int8_t>(ClampI32(v, act_min, act_max));
+    }
+  }
+}
+
+void orc_fc_int8_per_tensor_float_scale(const int8_t* input, const int8_t* filter,
+                                        const int32_t* bias, float input_scale,
+                                        float filter_scale, float output_scale, int8_t* output,
+                                        int batches, int depth, int out_depth,
+                                        int32_t input_offset, int32_t filter_offset,
+                                        int32_t output_offset, int32_t act_min, int32_t act_max) {
+  const double effective = static_cast<double>(input_scale) * static_cast<double>(filter_scale) /
+                           static_cast<double>(output_scale);
+  for (int b = 0; b < batches; ++b) {
+    for (int c = 0; c < out_depth; ++c) {
+      int32_t acc = 0;
+      for (int d = 0; d < depth; ++d) {
+        acc += (static_cast<int32_t>(filter[c * depth + d]) + filter_offset) *
+               (static_cast<int32_t>(input[b * depth + d]) + input_offset);
+      }
+      if (bias) acc += bias[c];
+      int32_t v = static_cast<int32_t>(std::round(static_cast<double>(acc) * effective));
+      v += output_offset;
+      output[c + out_depth * b] = static_cast<int8_t>(ClampI32(v, act_min, act_max));
+    }
+  }
+}
+
+void orc_asymmetric_quantize_floats(const float* values, int size, int8_t* quantized,
+                                    float* scaling_factor, int32_t* offset, int variant) {
+  AsymmetricQuantize(values, size, quantized, scaling_factor, offset, variant);
+}
+
+void orc_symmetric_quantize_floats(const float* values, int size, int8_t* quantized,
+                                   float* scaling_factor, int variant) {
+  SymmetricQuantize(values, size, quantized, scaling_factor, variant);
+}
+
+void orc_batch_quantize_floats(const float* values, int n_batch, int n_data, int8_t* quantized,
+                               float* scaling_factors, int32_t* zero_points, int do_asymmetric,
+                               int variant) {
+  for (int b = 0; b < n_batch; ++b) {
+    const size_t off = static_cast<size_t>(b) * n_data;
+    if (do_asymmetric) {
+      AsymmetricQuantize(values + off, n_data, quantized + off, &scaling_factors[b],
+                         &zero_points[b], variant);
+    } else {
+      SymmetricQuantize(values + off, n_data, quantized + off, &scaling_factors[b], variant);
+      if (zero_points) zero_points[b] = 0;
+    }
+  }
+}
+
+void orc_matrix_batch_vector_multiply_accumulate(const int8_t* matrix, int m_rows, int m_cols,
+                                                 const int8_t* vectors,
+                                                 const float* scaling_factors, int n_batch,
+                                                 float* result, const float* per_channel_scale,
+                                                 const int32_t* input_offset, int32_t* row_sums,
+                                                 int compute_row_sums) {
+  if (input_offset == nullptr) {
+    // reference/portable_tensor_utils.cc:140-163.
+    for (int b = 0; b < n_batch; ++b) {
+      const int8_t* vec = vectors + static_cast<size_t>(b) * m_cols;
+      for (int r = 0; r < m_rows; ++r) {
+        const int8_t* row = matrix + static_cast<size_t>(r) * m_cols;
+        int32_t dot = 0;
+        for (int c = 0; c < m_cols; ++c) dot += row[c] * vec[c];
+        const float term = static_cast<float>(dot) * scaling_factors[b];
+        result[static_cast<size_t>(b) * m_rows + r] += term;
+      }
+    }
+    return;
+  }
+  if (compute_row_sums) {
+    for (int r = 0; r < m_rows; ++r) {
+      int32_t s = 0;
+      for (int c = 0; c < m_cols; ++c) s += matrix[static_cast<size_t>(r) * m_cols + c];
+      row_sums[r] = s;
+    }
+  }
+  for (int b = 0; b < n_batch; ++b) {
+    const int8_t* vec = vectors + static_cast<size_t>(b) * m_cols;
+    const float batch_scale = scaling_factors[b];
+    const int32_t batch_offset = input_offset[b];
+    for (int r = 0; r < m_rows; ++r) {
+      const int8_t* row = matrix + static_cast<size_t>(r) * m_cols;
+      float scale = batch_scale;
+      if (per_channel_scale) scale *= per_channel_scale[r];
+      int32_t dot = 0;
+      for (int c = 0; c < m_cols; ++c) dot += row[c] * vec[c];
+      dot -= row_sums[r] * batch_offset;
+      const float term = static_cast<float>(dot) * scale;
+      result[static_cast<size_t>(b) * m_rows + r] += term;
+    }
+  }
+}
+
+int orc_apply_activation(float* data, int size, int activation) {
+  switch (activation) {
+    case ORC_ACT_NONE:
+      return 0;
+    case ORC_ACT_RELU:
+      for (int i = 0; i < size; ++i) data[i] = std::max(0.0f, data[i]);
+      return 0;
+    case ORC_ACT_RELU_N1_TO_1:
+      for (int i = 0; i < size; ++i) data[i] = std::max(-1.0f, std::min(data[i], 1.0f));
+      return 0;
+    case ORC_ACT_RELU6:
+      for (int i = 0; i < size; ++i) data[i] = std::max(0.0f, std::min(data[i], 6.0f));
+      return 0;
+    case ORC_ACT_SIGN_BIT:
+      for (int i = 0; i < size; ++i) data[i] = std::signbit(data[i]) ? 1.0f : 0.0f;
+      return 0;
+    default:
+      return 1;
+  }
+}
+
+int orc_fc_hybrid(const float* input, int batches, int depth, const int8_t* filter, int out_depth,
+                  const float* per_channel_scales, float filter_scale, const float* bias,
+                  int asymmetric_quantize_inputs, int activation, int quant_variant,
+                  float* output, int8_t* q_out, float* sf_out, int32_t* zp_out) {
+  const size_t total_in = static_cast<size_t>(batches) * depth;
+  // fully_connected.cc:780-786.
+  for (int b = 0; b < batches; ++b) {
+    for (int n = 0; n < out_depth; ++n) {
+      output[static_cast<size_t>(b) * out_depth + n] = bias ? bias[n] : 0.0f;
+    }
+  }
+  // fully_connected.cc:789-795: all-zero input skips the product.
+  bool all_zero = true;
+  for (size_t i = 0; i < total_in; ++i) {
+    if (input[i] != 0.0f) {
+      all_zero = false;
+      break;
+    }
+  }
+  std::vector<int8_t> q(total_in);
+  std::vector<float> sf(batches);
+  std::vector<int32_t> zp(batches);
+  if (all_zero) {
+    if (q_out) std::memset(q_out, 0, total_in);
+    for (int b = 0; b < batches; ++b) {
+      if (sf_out) sf_out[b] = 1.0f;
+      if (zp_out) zp_out[b] = 0;
+    }
+    return orc_apply_activation(output, batches * out_depth, activation);
+  }
+  orc_batch_quantize_floats(input, batches, depth, q.data(), sf.data(), zp.data(),
+                            asymmetric_quantize_inputs, quant_variant);
+  if (q_out) std::memcpy(q_out, q.data(), total_in);
+  if (sf_out) std::memcpy(sf_out, sf.data(), batches * sizeof(float));
+  if (zp_out) std::memcpy(zp_out, zp.data(), batches * sizeof(int32_t));
+  if (!per_channel_scales) {
+    // fully_connected.cc:838-843.
+    for (int b = 0; b < batches; ++b) sf[b] *= filter_scale;
+  }
+  std::vector<int32_t> row_sums(out_depth);
+  orc_matrix_batch_vector_multiply_accumulate(filter, out_depth, depth, q.data(), sf.data(),
+                                              batches, output, per_channel_scales, zp.data(),
+                                              row_sums.data(), 1);
+  return orc_apply_activation(output, batches * out_depth, activation);
+}
+
+void orc_fc_blockwise_int4(const float* input, int batches, int depth,
+                           const uint8_t* packed_filter, int out_depth,
+                           const uint16_t* scales_f16, int blocksize, const float* bias,
+                           int quant_variant, float* output) {
+  const size_t num_blocks = static_cast<size_t>(depth) / blocksize;
+  const size_t k2 = (static_cast<size_t>(depth) + 1) & ~static_cast<size_t>(1);
+  std::vector<float> scales(static_cast<size_t>(out_depth) * num_blocks);
+  for (size_t i = 0; i < scales.size(); ++i) scales[i] = orc_half_to_float(scales_f16[i]);
+  std::vector<int8_t> q(static_cast<size_t>(batches) * depth);
+  std::vector<float> in_scales(batches);
+  std::vector<int32_t> in_zps(batches);
+  orc_batch_quantize_floats(input, batches, depth, q.data(), in_scales.data(), in_zps.data(),
+                            /*do_asymmetric=*/1, quant_variant);
+  for (int m = 0; m < batches; ++m) {
+    for (int n = 0; n < out_depth; ++n) {
+      float out = 0.0f;
+      float kfsum = 0.0f;
+      for (size_t bi = 0; bi < num_blocks; ++bi) {
+        int32_t ksum = 0;
+        int32_t acc = 0;
+        for (int ki = 0; ki < blocksize; ++ki) {
+          const size_t k = bi * blocksize + ki;
+          const size_t byte_index = (static_cast<size_t>(n) * k2 + k) / 2;
+          const uint8_t byte = packed_filter[byte_index];
+          const int nibble = (k % 2 == 0) ? (byte & 0xF) : (byte >> 4);
+          const int32_t w = (nibble ^ 0x8) - 8;
+          ksum += w;
+          acc += static_cast<int32_t>(q[static_cast<size_t>(m) * depth + k]) * w;
+        }
+        const float scale = scales[static_cast<size_t>(n) * num_blocks + bi];
+        const float term = static_cast<float>(acc) * scale;
+        out = out + term;
+        const float kterm = scale * static_cast<float>(ksum);
+        kfsum = kfsum + kterm;
+      }
+      const float zp_term = static_cast<float>(in_zps[m]) * kfsum;
+      out = out - zp_term;
+      out = out * in_scales[m];
+      if (bias) out = out + bias[n];
+      output[static_cast<size_t>(m) * out_depth + n] = out;
+    }
+  }
+}
+
+}  // extern "C"
