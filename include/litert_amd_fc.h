@@ -1,0 +1,186 @@
+/* litert_amd_fc.h — C ABI of the MI355X (gfx950) quantized FULLY_CONNECTED kernels.
+ *
+ * This is the thin layer between the TfLiteDelegate / LiteRT accelerator host
+ * code and the hand-written HIP kernels. Every entry point takes plain
+ * pointers and sizes. Unless a parameter says "host", data pointers are DEVICE
+ * pointers and `stream` is a hipStream_t passed as void* (NULL = the default
+ * stream). Calls are asynchronous with respect to the host: they enqueue work
+ * on `stream` and return. Every function returns 0 on success and a non-zero
+ * LrtFcStatus otherwise; lrtfc_last_error() then describes the failure for the
+ * calling thread.
+ *
+ * Tensor conventions are the reference's: input [batches, depth] row-major,
+ * filter [out_depth, depth] row-major, output [batches, out_depth] row-major
+ * (tflite/kernels/internal/reference/integer_ops/fully_connected.h:57-76).
+ */
+#ifndef LITERT_AMD_FC_H_
+#define LITERT_AMD_FC_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LRTFC_ABI_VERSION 1
+
+typedef enum LrtFcStatus {
+  LRTFC_OK = 0,
+  LRTFC_INVALID_ARGUMENT = 1, /* shape, alignment or NULL-pointer contract broken */
+  LRTFC_NO_DEVICE = 2,        /* no gfx950 device visible to HIP */
+  LRTFC_HIP_ERROR = 3,        /* a HIP runtime call failed */
+  LRTFC_UNSUPPORTED = 4,      /* valid request this build does not implement */
+} LrtFcStatus;
+
+/* Fused activation, numbered as TfLiteFusedActivation
+ * (tflite/converter/core/c/builtin_op_data.h:79-87). */
+typedef enum LrtFcActivation {
+  LRTFC_ACT_NONE = 0,
+  LRTFC_ACT_RELU = 1,
+  LRTFC_ACT_RELU_N1_TO_1 = 2,
+  LRTFC_ACT_RELU6 = 3,
+} LrtFcActivation;
+
+/* Which build of the reference's activation quantizer to reproduce bit for bit
+ * (dispatch: tflite/kernels/internal/optimized/sse_tensor_utils.h:286-305). */
+typedef enum LrtFcQuantVariant {
+  LRTFC_QUANT_PORTABLE = 0,    /* reference/portable_tensor_utils.cc:41-119 (default) */
+  LRTFC_QUANT_NEON_V8 = 1,     /* optimized/neon_tensor_utils.cc:2412-2552, ARMv8 rounding */
+  LRTFC_QUANT_NEON_LEGACY = 2, /* same file, RoundToNearest fallback :2351-2357 */
+} LrtFcQuantVariant;
+
+/* ---- library ------------------------------------------------------------ */
+
+int lrtfc_abi_version(void);
+/* Message for the last failing call on this thread ("" when none). */
+const char* lrtfc_last_error(void);
+/* Selects `device_ordinal` and checks that it is a gfx950 part. Must succeed
+ * before any entry point that touches device memory is used. */
+int lrtfc_init(int device_ordinal);
+
+/* ---- Prepare-time math (host only, no device access) --------------------- */
+
+/* Replaces tflite::QuantizeMultiplier,
+ * tflite/kernels/internal/quantization_util.cc:53-104. */
+int lrtfc_quantize_multiplier(double real_multiplier, int32_t* quantized_multiplier, int* shift);
+
+/* Replaces the per-channel loop of fully_connected::PrepareImpl,
+ * tflite/kernels/fully_connected.cc:552-564. Host arrays of `num_channels`. */
+int lrtfc_prepare_per_channel(float input_scale, const float* filter_scales, int num_channels,
+                              float output_scale, int32_t* multipliers, int32_t* shifts);
+
+/* Replaces the per-tensor branch, tflite/kernels/fully_connected.cc:566-573 with
+ * GetQuantizedConvolutionMultipler, tflite/kernels/kernel_util.cc:291-341
+ * (bias-scale sanity check included: fails with LRTFC_INVALID_ARGUMENT as the
+ * reference fails Prepare). */
+int lrtfc_prepare_per_tensor(float input_scale, float filter_scale, int has_bias,
+                             float bias_scale, float output_scale, int32_t* multiplier,
+                             int32_t* shift);
+
+/* Replaces CalculateActivationRangeQuantized for an int8 output,
+ * tflite/kernels/kernel_util.cc:354-412. */
+int lrtfc_activation_range_int8(int activation, float output_scale, int32_t output_zero_point,
+                                int32_t* act_min, int32_t* act_max);
+
+/* ---- weight preparation on the device (once per constant filter) --------- */
+
+/* row_sums[n] = sum_k filter[n,k]. Replaces PortableReductionSumVector as used
+ * for the hybrid path's compute_row_sums step
+ * (tflite/kernels/internal/reference/portable_tensor_utils.cc:179-184); the
+ * full-integer kernels use the same sums to fold input_offset. */
+int lrtfc_row_sums_int8(const int8_t* filter, int out_depth, int depth, int32_t* row_sums,
+                        void* stream);
+
+/* Replaces tensor_utils::UnpackPackedIntToInt8 (bit_width 4, signed),
+ * tflite/kernels/internal/portable_tensor_utils.cc:96-127: low nibble first. */
+int lrtfc_unpack_int4(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
+                      void* stream);
+
+/* kfsum[n] = sum over blocks, in block order and float32, of
+ * scale[n,b] * float(sum_k filter[n, b*blocksize + k]): the weight-only part of
+ * EvalBlockwise4Bit's zero-point correction
+ * (tflite/kernels/fully_connected.cc:1056-1077), hoisted out of the per-call loop. */
+int lrtfc_blockwise_int4_kfsum(const uint8_t* packed_filter, const uint16_t* scales_f16,
+                               int out_depth, int depth, int blocksize, float* kfsum,
+                               void* stream);
+
+/* ---- Eval --------------------------------------------------------------- */
+
+/* Full-integer int8 FULLY_CONNECTED with MultiplyByQuantizedMultiplier
+ * requantization (double rounding, tflite/kernels/internal/common.cc:80-90).
+ * Replaces FullyConnectedPerChannelInt8 / FullyConnectedInt8
+ * (tflite/kernels/fully_connected.cc:1383-1421, 1254-1284) and the kernels they
+ * call (reference/integer_ops/fully_connected.h:35-77, 136-180).
+ *   per_channel != 0: multipliers/shifts are arrays of out_depth, filter_offset
+ *                     must be 0 (weights symmetric).
+ *   per_channel == 0: multipliers/shifts point at one value each.
+ *   bias may be NULL. filter_row_sums (from lrtfc_row_sums_int8) is required
+ *   when input_offset != 0. Any batches >= 1: small batches run the bandwidth-
+ *   bound GEMV kernel, large ones the int8 MFMA GEMM. */
+int lrtfc_fc_int8(const int8_t* input, const int8_t* filter, const int32_t* bias,
+                  const int32_t* multipliers, const int32_t* shifts, int per_channel,
+                  const int32_t* filter_row_sums, int8_t* output, int batches, int depth,
+                  int out_depth, int32_t input_offset, int32_t filter_offset,
+                  int32_t output_offset, int32_t act_min, int32_t act_max, void* stream);
+
+/* Per-row activation quantization. Replaces tensor_utils::BatchQuantizeFloats,
+ * tflite/kernels/internal/portable_tensor_utils.h:158-176. zero_points may be
+ * NULL when do_asymmetric == 0. */
+int lrtfc_batch_quantize_floats(const float* values, int n_batch, int n_data, int8_t* quantized,
+                                float* scaling_factors, int32_t* zero_points, int do_asymmetric,
+                                int variant, void* stream);
+
+/* Hybrid product on already-quantized activations. Replaces
+ * MatrixBatchVectorMultiplyAccumulate (per-channel / offset form,
+ * tflite/kernels/internal/reference/portable_tensor_utils.cc:165-206) together
+ * with the bias initialisation and ApplyActivationToVector of EvalHybridDense
+ * (tflite/kernels/fully_connected.cc:780-786, 854-856).
+ *   per_channel_scales NULL: per-tensor, filter_scale is folded into the batch
+ *   scaling factor as the reference does (:838-843). bias may be NULL.
+ *   zero_points NULL means symmetric activations (all zero). */
+int lrtfc_fc_hybrid_int8(const int8_t* quantized_input, const float* scaling_factors,
+                         const int32_t* zero_points, const int8_t* filter,
+                         const float* per_channel_scales, float filter_scale,
+                         const int32_t* filter_row_sums, const float* bias, float* output,
+                         int batches, int depth, int out_depth, int activation, void* stream);
+
+/* Bytes of device scratch lrtfc_fc_hybrid / lrtfc_fc_blockwise_int4 need for
+ * (batches, depth): quantized activations, scaling factors and zero points. */
+size_t lrtfc_activation_workspace_bytes(int batches, int depth);
+
+/* EvalHybridDense end to end (tflite/kernels/fully_connected.cc:763-858):
+ * quantizes `input` per row into `workspace`, then runs lrtfc_fc_hybrid_int8.
+ * The reference's all-zero-input early exit (:789-795) needs no special case:
+ * an all-zero row quantizes to zeros and contributes nothing. */
+int lrtfc_fc_hybrid(const float* input, const int8_t* filter, const float* per_channel_scales,
+                    float filter_scale, const int32_t* filter_row_sums, const float* bias,
+                    float* output, int batches, int depth, int out_depth,
+                    int asymmetric_quantize_inputs, int activation, int quant_variant,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* Blockwise-int4 hybrid FULLY_CONNECTED. Replaces EvalBlockwise4Bit,
+ * tflite/kernels/fully_connected.cc:1014-1086: asymmetric per-row activation
+ * quantization, per-block int32 sums, float32 accumulation over blocks in block
+ * order, zero-point correction, input scale, bias; the fused activation is
+ * ignored as in the reference. packed_filter: out_depth rows of depth/2 bytes,
+ * low nibble = even k (depth even). scales_f16: [out_depth, depth/blocksize]
+ * IEEE binary16. kfsum from lrtfc_blockwise_int4_kfsum. bias may be NULL. */
+int lrtfc_fc_blockwise_int4(const float* input, const uint8_t* packed_filter,
+                            const uint16_t* scales_f16, const float* kfsum, const float* bias,
+                            float* output, int batches, int depth, int out_depth, int blocksize,
+                            int quant_variant, void* workspace, size_t workspace_bytes,
+                            void* stream);
+
+/* Same product on already-quantized activations (workspace layout not needed). */
+int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
+                                      const float* scaling_factors, const int32_t* zero_points,
+                                      const uint8_t* packed_filter, const uint16_t* scales_f16,
+                                      const float* kfsum, const float* bias, float* output,
+                                      int batches, int depth, int out_depth, int blocksize,
+                                      void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LITERT_AMD_FC_H_ */

@@ -1,0 +1,78 @@
+"""ctypes binding of the C-ABI kernel library (include/litert_amd_fc.h).
+
+The library is loaded from litert_amd/lib/liblitert_amd_fc.so, which
+`python -m litert_amd.build` (or __graft_entry__.build()) produces. There is no
+fallback: if the library is missing, or no gfx950 device is visible, the calls
+raise.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "liblitert_amd_fc.so")
+
+OK, INVALID_ARGUMENT, NO_DEVICE, HIP_ERROR, UNSUPPORTED = range(5)
+ACT_NONE, ACT_RELU, ACT_RELU_N1_TO_1, ACT_RELU6 = range(4)
+QUANT_PORTABLE, QUANT_NEON_V8, QUANT_NEON_LEGACY = range(3)
+
+# Every symbol include/litert_amd_fc.h declares: (name, restype, argtypes).
+_vp, _i, _i32, _i64, _f, _d, _sz = (C.c_void_p, C.c_int, C.c_int32, C.c_int64, C.c_float,
+                                    C.c_double, C.c_size_t)
+_pi32, _pint, _pf = C.POINTER(C.c_int32), C.POINTER(C.c_int), C.POINTER(C.c_float)
+SYMBOLS = [
+    ("lrtfc_abi_version", _i, []),
+    ("lrtfc_last_error", C.c_char_p, []),
+    ("lrtfc_init", _i, [_i]),
+    ("lrtfc_quantize_multiplier", _i, [_d, _pi32, _pint]),
+    ("lrtfc_prepare_per_channel", _i, [_f, _pf, _i, _f, _pi32, _pi32]),
+    ("lrtfc_prepare_per_tensor", _i, [_f, _f, _i, _f, _f, _pi32, _pi32]),
+    ("lrtfc_activation_range_int8", _i, [_i, _f, _i32, _pi32, _pi32]),
+    ("lrtfc_row_sums_int8", _i, [_vp, _i, _i, _vp, _vp]),
+    ("lrtfc_unpack_int4", _i, [_vp, _i64, _vp, _vp]),
+    ("lrtfc_blockwise_int4_kfsum", _i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    ("lrtfc_fc_int8", _i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i32, _i32, _i32,
+                           _i32, _i32, _vp]),
+    ("lrtfc_batch_quantize_floats", _i, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp]),
+    ("lrtfc_fc_hybrid_int8", _i, [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i,
+                                  _vp]),
+    ("lrtfc_activation_workspace_bytes", _sz, [_i, _i]),
+    ("lrtfc_fc_hybrid", _i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz,
+                             _vp]),
+    ("lrtfc_fc_blockwise_int4", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz,
+                                     _vp]),
+    ("lrtfc_fc_blockwise_int4_quantized", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
+                                               _i, _vp]),
+]
+
+_LIB = None
+
+
+class LrtFcError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("litert_amd_fc status %d: %s" % (status, message))
+        self.status = status
+
+
+def load():
+    """Loads the shared library and binds every declared symbol (no device needed)."""
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                LIB_PATH + " is missing: run `python -m litert_amd.build` (hipcc, gfx950) first")
+        lib = C.CDLL(LIB_PATH)
+        for name, restype, argtypes in SYMBOLS:
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _LIB = lib
+    return _LIB
+
+
+def check(status):
+    if status != OK:
+        raise LrtFcError(status, load().lrtfc_last_error().decode())
+
+
+def init(device=0):
+    check(load().lrtfc_init(device))

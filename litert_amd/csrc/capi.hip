@@ -1,0 +1,432 @@
+// C-ABI layer of the gfx950 FULLY_CONNECTED kernels: argument checking, the
+// Prepare-time host math, and dispatch to the kernel launchers.
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <limits>
+
+#include "kernels.h"
+
+namespace {
+
+thread_local char g_last_error[512] = "";
+
+int Fail(int status, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof g_last_error, fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+int FromHip(hipError_t err, const char* what) {
+  if (err == hipSuccess) return LRTFC_OK;
+  if (err == hipErrorNotSupported) return Fail(LRTFC_UNSUPPORTED, "%s: not supported", what);
+  return Fail(LRTFC_HIP_ERROR, "%s: %s", what, hipGetErrorString(err));
+}
+
+hipStream_t AsStream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+bool g_initialised = false;
+
+int RequireInit() {
+  if (g_initialised) return LRTFC_OK;
+  return Fail(LRTFC_NO_DEVICE, "lrtfc_init() has not succeeded: no gfx950 device selected");
+}
+
+#define LRTFC_REQUIRE(cond, ...) \
+  do {                           \
+    if (!(cond)) return Fail(LRTFC_INVALID_ARGUMENT, __VA_ARGS__); \
+  } while (0)
+
+// Batches from this size on go to the MFMA GEMM when its tiling fits.
+constexpr int kGemmMinBatches = 128;
+
+// Workspace layout for the hybrid paths: quantized activations, then scaling
+// factors, then zero points, each 256-byte aligned.
+size_t AlignUp(size_t v, size_t a) { return (v + a - 1) / a * a; }
+struct Workspace {
+  int8_t* q;
+  float* sf;
+  int32_t* zp;
+};
+size_t WorkspaceBytes(int batches, int depth) {
+  return AlignUp(static_cast<size_t>(batches) * depth, 256) +
+         2 * AlignUp(static_cast<size_t>(batches) * 4, 256);
+}
+Workspace SplitWorkspace(void* base, int batches, int depth) {
+  char* p = static_cast<char*>(base);
+  Workspace w;
+  w.q = reinterpret_cast<int8_t*>(p);
+  p += AlignUp(static_cast<size_t>(batches) * depth, 256);
+  w.sf = reinterpret_cast<float*>(p);
+  p += AlignUp(static_cast<size_t>(batches) * 4, 256);
+  w.zp = reinterpret_cast<int32_t*>(p);
+  return w;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lrtfc_abi_version(void) { return LRTFC_ABI_VERSION; }
+
+const char* lrtfc_last_error(void) { return g_last_error; }
+
+int lrtfc_init(int device_ordinal) {
+  int count = 0;
+  hipError_t err = hipGetDeviceCount(&count);
+  if (err != hipSuccess || count == 0) {
+    g_initialised = false;
+    return Fail(LRTFC_NO_DEVICE, "no HIP device visible (%s)",
+                err == hipSuccess ? "device count is 0" : hipGetErrorString(err));
+  }
+  if (device_ordinal < 0 || device_ordinal >= count) {
+    return Fail(LRTFC_INVALID_ARGUMENT, "device %d out of range (%d visible)", device_ordinal,
+                count);
+  }
+  hipDeviceProp_t prop;
+  err = hipGetDeviceProperties(&prop, device_ordinal);
+  if (err != hipSuccess) return FromHip(err, "hipGetDeviceProperties");
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    g_initialised = false;
+    return Fail(LRTFC_NO_DEVICE, "device %d is %s; this library is built for gfx950 only",
+                device_ordinal, prop.gcnArchName);
+  }
+  err = hipSetDevice(device_ordinal);
+  if (err != hipSuccess) return FromHip(err, "hipSetDevice");
+  g_initialised = true;
+  return LRTFC_OK;
+}
+
+// ---- Prepare-time math -------------------------------------------------------
+
+int lrtfc_quantize_multiplier(double real_multiplier, int32_t* quantized_multiplier, int* shift) {
+  LRTFC_REQUIRE(quantized_multiplier && shift, "null output pointer");
+  if (real_multiplier == 0.) {
+    *quantized_multiplier = 0;
+    *shift = 0;
+    return LRTFC_OK;
+  }
+  const double q = std::frexp(real_multiplier, shift);
+  int64_t q_fixed = static_cast<int64_t>(std::round(q * 2147483648.0));
+  LRTFC_REQUIRE(q_fixed <= (1ll << 31), "multiplier significand out of range");
+  if (q_fixed == (1ll << 31)) {
+    q_fixed /= 2;
+    ++*shift;
+  }
+  if (*shift < -31) {  // would shift every bit out: flush to zero
+    *shift = 0;
+    q_fixed = 0;
+  }
+  *quantized_multiplier = static_cast<int32_t>(q_fixed);
+  return LRTFC_OK;
+}
+
+int lrtfc_prepare_per_channel(float input_scale, const float* filter_scales, int num_channels,
+                              float output_scale, int32_t* multipliers, int32_t* shifts) {
+  LRTFC_REQUIRE(filter_scales && multipliers && shifts, "null pointer");
+  LRTFC_REQUIRE(num_channels >= 0, "negative channel count");
+  for (int i = 0; i < num_channels; ++i) {
+    const double effective = static_cast<double>(input_scale) *
+                             static_cast<double>(filter_scales[i]) /
+                             static_cast<double>(output_scale);
+    int s = 0;
+    const int rc = lrtfc_quantize_multiplier(effective, &multipliers[i], &s);
+    if (rc != LRTFC_OK) return rc;
+    shifts[i] = s;
+  }
+  return LRTFC_OK;
+}
+
+int lrtfc_prepare_per_tensor(float input_scale, float filter_scale, int has_bias,
+                             float bias_scale, float output_scale, int32_t* multiplier,
+                             int32_t* shift) {
+  LRTFC_REQUIRE(multiplier && shift, "null output pointer");
+  if (has_bias) {
+    const double product = static_cast<double>(input_scale) * static_cast<double>(filter_scale);
+    const double diff = std::abs(product - static_cast<double>(bias_scale));
+    LRTFC_REQUIRE(diff / static_cast<double>(output_scale) <= 0.02,
+                  "bias scale differs from input_scale * filter_scale by more than 0.02 output "
+                  "quanta");
+  }
+  // The product is formed in float before widening, as the reference does.
+  const double product = static_cast<double>(input_scale * filter_scale);
+  LRTFC_REQUIRE(product >= 0, "negative input_scale * filter_scale");
+  int s = 0;
+  const int rc =
+      lrtfc_quantize_multiplier(product / static_cast<double>(output_scale), multiplier, &s);
+  *shift = s;
+  return rc;
+}
+
+int lrtfc_activation_range_int8(int activation, float output_scale, int32_t output_zero_point,
+                                int32_t* act_min, int32_t* act_max) {
+  LRTFC_REQUIRE(act_min && act_max, "null output pointer");
+  const int32_t qmin = -128, qmax = 127;
+  auto quantize = [&](float f, int32_t* q) {
+    const float rounded = std::round(f / output_scale);
+    if (!(rounded >= static_cast<float>(std::numeric_limits<int32_t>::min()) &&
+          rounded <= static_cast<float>(std::numeric_limits<int32_t>::max()))) {
+      return false;
+    }
+    *q = output_zero_point + static_cast<int32_t>(rounded);
+    return true;
+  };
+  int32_t lo = qmin, hi = qmax, q = 0;
+  bool ok = true;
+  switch (activation) {
+    case LRTFC_ACT_RELU:
+      ok = quantize(0.0f, &q);
+      lo = std::max(qmin, q);
+      break;
+    case LRTFC_ACT_RELU6:
+      ok = quantize(0.0f, &q);
+      lo = std::max(qmin, q);
+      ok = ok && quantize(6.0f, &q);
+      hi = std::min(qmax, q);
+      break;
+    case LRTFC_ACT_RELU_N1_TO_1:
+      ok = quantize(-1.0f, &q);
+      lo = std::max(qmin, q);
+      ok = ok && quantize(1.0f, &q);
+      hi = std::min(qmax, q);
+      break;
+    default:
+      break;
+  }
+  LRTFC_REQUIRE(ok, "activation bound does not fit int32 at this output scale");
+  *act_min = lo;
+  *act_max = hi;
+  return LRTFC_OK;
+}
+
+// ---- weight preparation ------------------------------------------------------
+
+int lrtfc_row_sums_int8(const int8_t* filter, int out_depth, int depth, int32_t* row_sums,
+                        void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(out_depth >= 0 && depth >= 0, "negative dimension");
+  if (out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(filter && row_sums, "null pointer");
+  return FromHip(lrtfc::LaunchRowSumsInt8(filter, out_depth, depth, row_sums, AsStream(stream)),
+                 "row sums");
+}
+
+int lrtfc_unpack_int4(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
+                      void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(num_elements >= 0, "negative element count");
+  if (num_elements == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(packed && unpacked, "null pointer");
+  LRTFC_REQUIRE((num_elements + 1) / 2 <= 0x7fffffffll * 256, "tensor too large");
+  return FromHip(lrtfc::LaunchUnpackInt4(packed, num_elements, unpacked, AsStream(stream)),
+                 "int4 unpack");
+}
+
+int lrtfc_blockwise_int4_kfsum(const uint8_t* packed_filter, const uint16_t* scales_f16,
+                               int out_depth, int depth, int blocksize, float* kfsum,
+                               void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(out_depth >= 0 && depth >= 0, "negative dimension");
+  LRTFC_REQUIRE(blocksize > 0 && depth % blocksize == 0, "blocksize %d does not divide depth %d",
+                blocksize, depth);
+  if (out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(packed_filter && scales_f16 && kfsum, "null pointer");
+  return FromHip(lrtfc::LaunchBlockwiseInt4Kfsum(packed_filter, scales_f16, out_depth, depth,
+                                                 blocksize, kfsum, AsStream(stream)),
+                 "blockwise kfsum");
+}
+
+// ---- Eval --------------------------------------------------------------------
+
+int lrtfc_fc_int8(const int8_t* input, const int8_t* filter, const int32_t* bias,
+                  const int32_t* multipliers, const int32_t* shifts, int per_channel,
+                  const int32_t* filter_row_sums, int8_t* output, int batches, int depth,
+                  int out_depth, int32_t input_offset, int32_t filter_offset,
+                  int32_t output_offset, int32_t act_min, int32_t act_max, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth >= 0 && out_depth >= 0, "negative dimension");
+  // Empty output: nothing to do (tflite/kernels/fully_connected.cc:1966-1968).
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(output, "null output");
+  if (depth == 0) {
+    // filter.dims[1] == 0 zero-fills the output (fully_connected.cc:1970-1973).
+    return FromHip(lrtfc::LaunchZeroFill(output, static_cast<size_t>(batches) * out_depth,
+                                         AsStream(stream)),
+                   "zero fill");
+  }
+  LRTFC_REQUIRE(input && filter && multipliers && shifts, "null pointer");
+  LRTFC_REQUIRE(act_min <= act_max, "activation range is empty");
+  LRTFC_REQUIRE(!(per_channel && filter_offset != 0),
+                "per-channel filters are symmetric: filter_offset must be 0");
+  LRTFC_REQUIRE(input_offset == 0 || filter_row_sums,
+                "filter_row_sums is required when input_offset != 0");
+  lrtfc::FcInt8Args a{};
+  a.input = input;
+  a.filter = filter;
+  a.batches = batches;
+  a.depth = depth;
+  a.out_depth = out_depth;
+  a.filter_row_sums = filter_row_sums;
+  a.bias_i32 = bias;
+  a.multipliers = multipliers;
+  a.shifts = shifts;
+  a.per_channel = per_channel;
+  a.input_offset = input_offset;
+  a.filter_offset = filter_offset;
+  a.output_offset = output_offset;
+  a.act_min = act_min;
+  a.act_max = act_max;
+  a.output_i8 = output;
+  if (batches >= kGemmMinBatches && lrtfc::FcInt8GemmMfmaSupports(a)) {
+    return FromHip(lrtfc::LaunchFcInt8GemmMfma(a, AsStream(stream)), "int8 MFMA GEMM");
+  }
+  return FromHip(
+      lrtfc::LaunchFcInt8Gemv(a, lrtfc::Int8Epilogue::kRequantize, AsStream(stream)),
+      "int8 GEMV");
+}
+
+int lrtfc_batch_quantize_floats(const float* values, int n_batch, int n_data, int8_t* quantized,
+                                float* scaling_factors, int32_t* zero_points, int do_asymmetric,
+                                int variant, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(n_batch >= 0 && n_data >= 0, "negative dimension");
+  if (n_batch == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(values && quantized && scaling_factors, "null pointer");
+  LRTFC_REQUIRE(!do_asymmetric || zero_points, "zero_points is required for asymmetric mode");
+  LRTFC_REQUIRE(variant >= 0 && variant <= LRTFC_QUANT_NEON_LEGACY, "unknown quantizer variant");
+  LRTFC_REQUIRE(n_data > 0, "empty rows cannot be quantized");
+  return FromHip(lrtfc::LaunchBatchQuantize(values, n_batch, n_data, quantized, scaling_factors,
+                                            zero_points, do_asymmetric, variant,
+                                            AsStream(stream)),
+                 "batch quantize");
+}
+
+int lrtfc_fc_hybrid_int8(const int8_t* quantized_input, const float* scaling_factors,
+                         const int32_t* zero_points, const int8_t* filter,
+                         const float* per_channel_scales, float filter_scale,
+                         const int32_t* filter_row_sums, const float* bias, float* output,
+                         int batches, int depth, int out_depth, int activation, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth >= 0 && out_depth >= 0, "negative dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(output, "null output");
+  LRTFC_REQUIRE(depth > 0, "depth 0 is handled by the caller (zero fill)");
+  LRTFC_REQUIRE(quantized_input && scaling_factors && filter, "null pointer");
+  LRTFC_REQUIRE(!zero_points || filter_row_sums,
+                "filter_row_sums is required with activation zero points");
+  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  lrtfc::FcInt8Args a{};
+  a.input = quantized_input;
+  a.filter = filter;
+  a.batches = batches;
+  a.depth = depth;
+  a.out_depth = out_depth;
+  a.filter_row_sums = filter_row_sums;
+  a.scaling_factors = scaling_factors;
+  a.zero_points = zero_points;
+  a.per_channel_scales = per_channel_scales;
+  a.filter_scale = filter_scale;
+  a.bias_f32 = bias;
+  a.activation = activation;
+  a.output_f32 = output;
+  return FromHip(lrtfc::LaunchFcInt8Gemv(a, lrtfc::Int8Epilogue::kHybrid, AsStream(stream)),
+                 "hybrid GEMV");
+}
+
+size_t lrtfc_activation_workspace_bytes(int batches, int depth) {
+  if (batches <= 0 || depth <= 0) return 0;
+  return WorkspaceBytes(batches, depth);
+}
+
+int lrtfc_fc_hybrid(const float* input, const int8_t* filter, const float* per_channel_scales,
+                    float filter_scale, const int32_t* filter_row_sums, const float* bias,
+                    float* output, int batches, int depth, int out_depth,
+                    int asymmetric_quantize_inputs, int activation, int quant_variant,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth >= 0 && out_depth >= 0, "negative dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(output, "null output");
+  if (depth == 0) {
+    return FromHip(lrtfc::LaunchZeroFill(output, sizeof(float) * batches * out_depth,
+                                         AsStream(stream)),
+                   "zero fill");
+  }
+  LRTFC_REQUIRE(input && workspace, "null pointer");
+  LRTFC_REQUIRE(workspace_bytes >= WorkspaceBytes(batches, depth),
+                "workspace too small: %zu < %zu bytes", workspace_bytes,
+                WorkspaceBytes(batches, depth));
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
+                "workspace must be 256-byte aligned");
+  const Workspace w = SplitWorkspace(workspace, batches, depth);
+  int rc = lrtfc_batch_quantize_floats(input, batches, depth, w.q, w.sf, w.zp,
+                                       asymmetric_quantize_inputs, quant_variant, stream);
+  if (rc != LRTFC_OK) return rc;
+  // Symmetric quantization still writes zero points of 0, so the offset form of the
+  // product applies to both modes, as in EvalHybridDense.
+  return lrtfc_fc_hybrid_int8(w.q, w.sf, w.zp, filter, per_channel_scales, filter_scale,
+                              filter_row_sums, bias, output, batches, depth, out_depth, activation,
+                              stream);
+}
+
+int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
+                                      const float* scaling_factors, const int32_t* zero_points,
+                                      const uint8_t* packed_filter, const uint16_t* scales_f16,
+                                      const float* kfsum, const float* bias, float* output,
+                                      int batches, int depth, int out_depth, int blocksize,
+                                      void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth >= 0 && out_depth >= 0, "negative dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(output, "null output");
+  LRTFC_REQUIRE(depth > 0 && depth % 2 == 0, "depth %d must be positive and even", depth);
+  LRTFC_REQUIRE(blocksize > 0 && depth % blocksize == 0, "blocksize %d does not divide depth %d",
+                blocksize, depth);
+  LRTFC_REQUIRE(quantized_input && scaling_factors && zero_points && packed_filter &&
+                    scales_f16 && kfsum,
+                "null pointer");
+  lrtfc::FcInt4Args a{};
+  a.input = quantized_input;
+  a.scaling_factors = scaling_factors;
+  a.zero_points = zero_points;
+  a.packed_filter = packed_filter;
+  a.scales_f16 = scales_f16;
+  a.kfsum = kfsum;
+  a.bias = bias;
+  a.output = output;
+  a.batches = batches;
+  a.depth = depth;
+  a.out_depth = out_depth;
+  a.blocksize = blocksize;
+  return FromHip(lrtfc::LaunchFcBlockwiseInt4(a, AsStream(stream)), "blockwise int4 GEMV");
+}
+
+int lrtfc_fc_blockwise_int4(const float* input, const uint8_t* packed_filter,
+                            const uint16_t* scales_f16, const float* kfsum, const float* bias,
+                            float* output, int batches, int depth, int out_depth, int blocksize,
+                            int quant_variant, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth >= 0 && out_depth >= 0, "negative dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(input && workspace, "null pointer");
+  LRTFC_REQUIRE(depth > 0, "depth must be positive");
+  LRTFC_REQUIRE(workspace_bytes >= WorkspaceBytes(batches, depth),
+                "workspace too small: %zu < %zu bytes", workspace_bytes,
+                WorkspaceBytes(batches, depth));
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
+                "workspace must be 256-byte aligned");
+  const Workspace w = SplitWorkspace(workspace, batches, depth);
+  // EvalBlockwise4Bit always quantizes asymmetrically (fully_connected.cc:1044-1047).
+  int rc = lrtfc_batch_quantize_floats(input, batches, depth, w.q, w.sf, w.zp,
+                                       /*do_asymmetric=*/1, quant_variant, stream);
+  if (rc != LRTFC_OK) return rc;
+  return lrtfc_fc_blockwise_int4_quantized(w.q, w.sf, w.zp, packed_filter, scales_f16, kfsum, bias,
+                                           output, batches, depth, out_depth, blocksize, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,110 @@
+// Device-side helpers shared by the gfx950 FULLY_CONNECTED kernels.
+#ifndef LITERT_AMD_CSRC_DEVICE_UTILS_H_
+#define LITERT_AMD_CSRC_DEVICE_UTILS_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lrtfc {
+
+constexpr int kWaveSize = 64;
+
+// 128-bit register quad: the unit of every weight load (global_load_dwordx4).
+using i32x4 = int __attribute__((ext_vector_type(4)));
+using i32x2 = int __attribute__((ext_vector_type(2)));
+
+// ---- integer requantization -------------------------------------------------
+
+// SaturatingRoundingDoublingHighMul (gemmlowp fixedpoint, as used by
+// tflite/kernels/internal/common.cc:83-89): (ab + nudge) / 2^31 with a truncating
+// division, nudge = 2^30 for ab >= 0 and 1 - 2^30 otherwise. For either sign that
+// quotient equals floor((ab + 2^30) / 2^31), which needs no sign test: one 64-bit
+// multiply-add and an arithmetic shift.
+__device__ __forceinline__ int32_t Srdhm(int32_t a, int32_t b) {
+  if (a == b && a == INT32_MIN) return INT32_MAX;
+  const int64_t t = static_cast<int64_t>(a) * static_cast<int64_t>(b) + (1ll << 30);
+  return static_cast<int32_t>(t >> 31);
+}
+
+// RoundingDivideByPOT: shift right, nearest, ties away from zero.
+__device__ __forceinline__ int32_t RoundingDivideByPot(int32_t x, int exponent) {
+  const int32_t mask = static_cast<int32_t>((1ll << exponent) - 1);
+  const int32_t remainder = x & mask;
+  const int32_t threshold = (mask >> 1) + (x < 0 ? 1 : 0);
+  return (x >> exponent) + (remainder > threshold ? 1 : 0);
+}
+
+// MultiplyByQuantizedMultiplier, double-rounding build
+// (tflite/kernels/internal/common.cc:80-90). The left shift wraps as the
+// reference's int32 multiply does.
+__device__ __forceinline__ int32_t Mbqm(int32_t x, int32_t quantized_multiplier, int shift) {
+  const int left_shift = shift > 0 ? shift : 0;
+  const int right_shift = shift > 0 ? 0 : -shift;
+  const int32_t shifted = static_cast<int32_t>(static_cast<uint32_t>(x) << left_shift);
+  return RoundingDivideByPot(Srdhm(shifted, quantized_multiplier), right_shift);
+}
+
+__device__ __forceinline__ int32_t ClampI32(int32_t v, int32_t lo, int32_t hi) {
+  return min(max(v, lo), hi);
+}
+
+// ---- float helpers (explicitly rounded: no FMA contraction) -----------------
+
+__device__ __forceinline__ float ApplyFloatActivation(float v, int activation) {
+  // tflite/kernels/internal/portable_tensor_utils.cc:41-62: max/min forms.
+  switch (activation) {
+    case 1:
+      return fmaxf(0.0f, v);
+    case 2:
+      return fmaxf(-1.0f, fminf(v, 1.0f));
+    case 3:
+      return fmaxf(0.0f, fminf(v, 6.0f));
+    default:
+      return v;
+  }
+}
+
+// IEEE binary16 -> binary32, exact for every finite pattern, subnormals included.
+__device__ __forceinline__ float HalfBitsToFloat(uint16_t h) {
+  const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
+  const uint32_t exp = (h >> 10) & 0x1Fu;
+  const uint32_t man = h & 0x3FFu;
+  if (exp == 0) {
+    // subnormal or zero: man * 2^-24, exact in float
+    const float mag = static_cast<float>(man) * 5.9604644775390625e-08f;
+    return __uint_as_float(__float_as_uint(mag) | sign);
+  }
+  if (exp == 31) return __uint_as_float(sign | 0x7F800000u | (man << 13));
+  return __uint_as_float(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+// ---- wave64 reductions --------------------------------------------------------
+
+// Sum over the 64 lanes of a wavefront; every lane receives the total. Integer
+// addition is associative, so the order of the butterfly cannot change results.
+__device__ __forceinline__ int32_t WaveSumI32(int32_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWaveSize);
+  return v;
+}
+
+__device__ __forceinline__ float WaveMinF32(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, kWaveSize));
+  return v;
+}
+
+__device__ __forceinline__ float WaveMaxF32(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWaveSize));
+  return v;
+}
+
+// 4-way int8 dot product with int32 accumulate (v_dot4_i32_i8).
+__device__ __forceinline__ int32_t Dot4(int32_t a, int32_t b, int32_t acc) {
+  return __builtin_amdgcn_sdot4(a, b, acc, false);
+}
+
+}  // namespace lrtfc
+
+#endif  // LITERT_AMD_CSRC_DEVICE_UTILS_H_

@@ -1,0 +1,75 @@
+// Internal launcher interface between the C-ABI layer (capi.hip) and the kernel
+// translation units. All pointers are device pointers.
+#ifndef LITERT_AMD_CSRC_KERNELS_H_
+#define LITERT_AMD_CSRC_KERNELS_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/litert_amd_fc.h"
+#include "device_utils.h"
+
+namespace lrtfc {
+
+// Arguments of the int8-weight kernels (full-integer and hybrid epilogues).
+struct FcInt8Args {
+  const int8_t* input;   // [batches, depth] int8 (quantized activations)
+  const int8_t* filter;  // [out_depth, depth]
+  int batches, depth, out_depth;
+  const int32_t* filter_row_sums;  // [out_depth] or nullptr
+  // full-integer epilogue
+  const int32_t* bias_i32;
+  const int32_t* multipliers;
+  const int32_t* shifts;
+  int per_channel;
+  int32_t input_offset, filter_offset, output_offset, act_min, act_max;
+  int8_t* output_i8;
+  // hybrid epilogue
+  const float* scaling_factors;     // [batches]
+  const int32_t* zero_points;       // [batches] or nullptr
+  const float* per_channel_scales;  // [out_depth] or nullptr
+  float filter_scale;
+  const float* bias_f32;
+  int activation;
+  float* output_f32;
+};
+
+enum class Int8Epilogue { kRequantize, kHybrid };
+
+hipError_t LaunchBatchQuantize(const float* values, int n_batch, int n_data, int8_t* quantized,
+                               float* scaling_factors, int32_t* zero_points, int do_asymmetric,
+                               int variant, hipStream_t stream);
+
+hipError_t LaunchZeroFill(void* dst, size_t bytes, hipStream_t stream);
+hipError_t LaunchRowSumsInt8(const int8_t* filter, int out_depth, int depth, int32_t* row_sums,
+                             hipStream_t stream);
+hipError_t LaunchUnpackInt4(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
+                            hipStream_t stream);
+
+// Small-batch path: bandwidth-bound GEMV (any shape; fast path needs depth % 16 == 0).
+hipError_t LaunchFcInt8Gemv(const FcInt8Args& a, Int8Epilogue epilogue, hipStream_t stream);
+// Large-batch full-integer path: int8 MFMA GEMM. Returns hipErrorNotSupported when
+// the shape does not meet its tiling constraints (caller falls back to the GEMV).
+hipError_t LaunchFcInt8GemmMfma(const FcInt8Args& a, hipStream_t stream);
+bool FcInt8GemmMfmaSupports(const FcInt8Args& a);
+
+struct FcInt4Args {
+  const int8_t* input;           // [batches, depth] quantized activations
+  const float* scaling_factors;  // [batches]
+  const int32_t* zero_points;    // [batches]
+  const uint8_t* packed_filter;  // [out_depth, depth / 2]
+  const uint16_t* scales_f16;    // [out_depth, depth / blocksize]
+  const float* kfsum;            // [out_depth]
+  const float* bias;
+  float* output;
+  int batches, depth, out_depth, blocksize;
+};
+
+hipError_t LaunchBlockwiseInt4Kfsum(const uint8_t* packed_filter, const uint16_t* scales_f16,
+                                    int out_depth, int depth, int blocksize, float* kfsum,
+                                    hipStream_t stream);
+hipError_t LaunchFcBlockwiseInt4(const FcInt4Args& a, hipStream_t stream);
+
+}  // namespace lrtfc
+
+#endif  // LITERT_AMD_CSRC_KERNELS_H_

@@ -1,0 +1,233 @@
+"""Host-side mirror of the reference's quantized FULLY_CONNECTED op for Python callers.
+
+Each class follows the builtin op's two phases (tflite/kernels/fully_connected.cc):
+the constructor is `Prepare` (validates the tensor / quantization-parameter
+combination, derives multipliers and activation bounds, uploads and pre-reduces the
+constant filter) and `__call__` is `Eval` (launches the HIP kernels through the C
+ABI on torch's current stream). Tensors handed to `__call__` are torch CUDA tensors;
+torch is used only for device memory and streams.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import capi
+
+_ACT = {"none": capi.ACT_NONE, "relu": capi.ACT_RELU, "relu_n1_to_1": capi.ACT_RELU_N1_TO_1,
+        "relu6": capi.ACT_RELU6}
+
+
+def _act(a):
+    return _ACT[a] if isinstance(a, str) else int(a)
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _dev(a, dtype):
+    if a is None:
+        return None
+    if isinstance(a, torch.Tensor):
+        return a.to(device="cuda", dtype=dtype).contiguous()
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device="cuda", dtype=dtype).contiguous()
+
+
+def _ensure_init():
+    capi.init(torch.cuda.current_device())
+
+
+def quantize_multiplier(m):
+    q, s = C.c_int32(), C.c_int()
+    capi.check(capi.load().lrtfc_quantize_multiplier(float(m), C.byref(q), C.byref(s)))
+    return q.value, s.value
+
+
+def activation_range_int8(activation, out_scale, out_zp):
+    lo, hi = C.c_int32(), C.c_int32()
+    capi.check(capi.load().lrtfc_activation_range_int8(_act(activation), out_scale, out_zp,
+                                                       C.byref(lo), C.byref(hi)))
+    return lo.value, hi.value
+
+
+def prepare_per_channel(in_scale, filter_scales, out_scale):
+    fs = np.ascontiguousarray(filter_scales, dtype=np.float32)
+    mult = np.empty(fs.size, np.int32)
+    shift = np.empty(fs.size, np.int32)
+    capi.check(capi.load().lrtfc_prepare_per_channel(
+        in_scale, fs.ctypes.data_as(C.POINTER(C.c_float)), fs.size, out_scale,
+        mult.ctypes.data_as(C.POINTER(C.c_int32)), shift.ctypes.data_as(C.POINTER(C.c_int32))))
+    return mult, shift
+
+
+def prepare_per_tensor(in_scale, filter_scale, out_scale, bias_scale=None):
+    m, s = C.c_int32(), C.c_int32()
+    capi.check(capi.load().lrtfc_prepare_per_tensor(
+        in_scale, filter_scale, bias_scale is not None,
+        0.0 if bias_scale is None else bias_scale, out_scale, C.byref(m), C.byref(s)))
+    return m.value, s.value
+
+
+def batch_quantize_floats(x, asymmetric=True, variant=capi.QUANT_PORTABLE):
+    """tensor_utils::BatchQuantizeFloats on the GPU: returns (q int8 [B,K], scale [B], zp [B])."""
+    _ensure_init()
+    x = x.contiguous()
+    B, K = x.shape
+    q = torch.empty((B, K), dtype=torch.int8, device=x.device)
+    sf = torch.empty(B, dtype=torch.float32, device=x.device)
+    zp = torch.zeros(B, dtype=torch.int32, device=x.device)
+    capi.check(capi.load().lrtfc_batch_quantize_floats(_ptr(x), B, K, _ptr(q), _ptr(sf), _ptr(zp),
+                                                       int(asymmetric), variant, _stream()))
+    return q, sf, zp
+
+
+class FullyConnectedInt8:
+    """Full-integer int8 FC: Prepare = fully_connected.cc:526-581, Eval = :1383-1421 / :1254-1284.
+
+    filter: int8 [N,K], or packed int4 (pass int4=True: [N, ceil(K/2)] bytes, unpacked once here
+    as fully_connected.cc:1670-1677 does on every call). filter_scales of size N > 1 selects
+    the per-channel form, otherwise per-tensor (filter_zero_point then applies).
+    """
+
+    def __init__(self, filter, bias, input_scale, input_zero_point, filter_scales,
+                 output_scale, output_zero_point, activation="none", filter_zero_point=0,
+                 bias_scale=None, int4=False, depth=None):
+        _ensure_init()
+        lib = capi.load()
+        fs = np.atleast_1d(np.asarray(filter_scales, dtype=np.float32))
+        self.per_channel = fs.size > 1
+        if int4:
+            packed = _dev(filter, torch.uint8)
+            n = packed.shape[0]
+            if depth is None:
+                raise ValueError("depth is required for packed int4 filters")
+            self.filter = torch.empty((n, depth), dtype=torch.int8, device="cuda")
+            capi.check(lib.lrtfc_unpack_int4(_ptr(packed), n * depth, _ptr(self.filter), _stream()))
+        else:
+            self.filter = _dev(filter, torch.int8)
+        self.out_depth, self.depth = self.filter.shape
+        if self.per_channel:
+            if fs.size != self.out_depth:
+                raise ValueError("per-channel scales must have one entry per output channel")
+            if filter_zero_point != 0:
+                raise ValueError("per-channel filters are symmetric")
+            mult, shift = prepare_per_channel(input_scale, fs, output_scale)
+        else:
+            m, s = prepare_per_tensor(input_scale, float(fs[0]), output_scale,
+                                      bias_scale if bias is not None else None)
+            mult, shift = np.array([m], np.int32), np.array([s], np.int32)
+        self.multipliers = _dev(mult, torch.int32)
+        self.shifts = _dev(shift, torch.int32)
+        self.bias = _dev(bias, torch.int32)
+        self.input_offset = -int(input_zero_point)
+        self.filter_offset = -int(filter_zero_point)
+        self.output_offset = int(output_zero_point)
+        self.act_min, self.act_max = activation_range_int8(activation, output_scale,
+                                                           output_zero_point)
+        self.row_sums = torch.empty(self.out_depth, dtype=torch.int32, device="cuda")
+        capi.check(lib.lrtfc_row_sums_int8(_ptr(self.filter), self.out_depth, self.depth,
+                                           _ptr(self.row_sums), _stream()))
+
+    def __call__(self, x, out=None):
+        x = x.contiguous()
+        batches = x.numel() // self.depth if self.depth else 0
+        if out is None:
+            out = torch.empty((batches, self.out_depth), dtype=torch.int8, device=x.device)
+        capi.check(capi.load().lrtfc_fc_int8(
+            _ptr(x), _ptr(self.filter), _ptr(self.bias), _ptr(self.multipliers), _ptr(self.shifts),
+            int(self.per_channel), _ptr(self.row_sums), _ptr(out), batches, self.depth,
+            self.out_depth, self.input_offset, self.filter_offset, self.output_offset,
+            self.act_min, self.act_max, _stream()))
+        return out
+
+
+class FullyConnectedHybrid:
+    """Hybrid FC (float activations, int8 filter): EvalHybridDense, fully_connected.cc:763-858."""
+
+    def __init__(self, filter, per_channel_scales=None, filter_scale=1.0, bias=None,
+                 asymmetric_quantize_inputs=True, activation="none",
+                 quant_variant=capi.QUANT_PORTABLE):
+        _ensure_init()
+        self.filter = _dev(filter, torch.int8)
+        self.out_depth, self.depth = self.filter.shape
+        self.pcs = _dev(per_channel_scales, torch.float32)
+        self.filter_scale = float(filter_scale)
+        self.bias = _dev(bias, torch.float32)
+        self.asymmetric = bool(asymmetric_quantize_inputs)
+        self.activation = _act(activation)
+        self.variant = quant_variant
+        self.row_sums = torch.empty(self.out_depth, dtype=torch.int32, device="cuda")
+        capi.check(capi.load().lrtfc_row_sums_int8(_ptr(self.filter), self.out_depth, self.depth,
+                                                   _ptr(self.row_sums), _stream()))
+        self._ws = None
+
+    def _workspace(self, batches):
+        need = capi.load().lrtfc_activation_workspace_bytes(batches, self.depth)
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        return self._ws
+
+    def __call__(self, x, out=None):
+        x = x.contiguous()
+        batches = x.numel() // self.depth
+        if out is None:
+            out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
+        ws = self._workspace(batches)
+        capi.check(capi.load().lrtfc_fc_hybrid(
+            _ptr(x), _ptr(self.filter), _ptr(self.pcs), self.filter_scale, _ptr(self.row_sums),
+            _ptr(self.bias), _ptr(out), batches, self.depth, self.out_depth, int(self.asymmetric),
+            self.activation, self.variant, _ptr(ws), ws.numel(), _stream()))
+        return out
+
+
+class FullyConnectedBlockwiseInt4:
+    """Blockwise-int4 hybrid FC: EvalBlockwise4Bit, fully_connected.cc:1014-1086.
+
+    packed_filter: uint8 [N, K/2], low nibble = even k; scales_f16: [N, K/blocksize] as
+    float16 (or its uint16 bit patterns).
+    """
+
+    def __init__(self, packed_filter, scales_f16, depth, blocksize=32, bias=None,
+                 quant_variant=capi.QUANT_PORTABLE):
+        _ensure_init()
+        self.filter = _dev(packed_filter, torch.uint8)
+        self.out_depth = self.filter.shape[0]
+        self.depth = int(depth)
+        self.blocksize = int(blocksize)
+        if isinstance(scales_f16, np.ndarray) and scales_f16.dtype == np.float16:
+            scales_f16 = scales_f16.view(np.uint16)
+        if isinstance(scales_f16, torch.Tensor) and scales_f16.dtype == torch.float16:
+            scales_f16 = scales_f16.view(torch.int16)
+        if isinstance(scales_f16, np.ndarray):
+            scales_f16 = scales_f16.view(np.int16)
+        self.scales = _dev(scales_f16, torch.int16)
+        self.bias = _dev(bias, torch.float32)
+        self.variant = quant_variant
+        self.kfsum = torch.empty(self.out_depth, dtype=torch.float32, device="cuda")
+        capi.check(capi.load().lrtfc_blockwise_int4_kfsum(
+            _ptr(self.filter), _ptr(self.scales), self.out_depth, self.depth, self.blocksize,
+            _ptr(self.kfsum), _stream()))
+        self._ws = None
+
+    def _workspace(self, batches):
+        need = capi.load().lrtfc_activation_workspace_bytes(batches, self.depth)
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        return self._ws
+
+    def __call__(self, x, out=None):
+        x = x.contiguous()
+        batches = x.numel() // self.depth
+        if out is None:
+            out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
+        ws = self._workspace(batches)
+        capi.check(capi.load().lrtfc_fc_blockwise_int4(
+            _ptr(x), _ptr(self.filter), _ptr(self.scales), _ptr(self.kfsum), _ptr(self.bias),
+            _ptr(out), batches, self.depth, self.out_depth, self.blocksize, self.variant,
+            _ptr(ws), ws.numel(), _stream()))
+        return out

@@ -14,8 +14,8 @@ namespace {
 // ---- fixed-point helpers --------------------------------------------------
 
 // gemmlowp SaturatingRoundingDoublingHighMul (fixedpoint.h @16e8662c): the
-// high 32 bits of 2*a*b with round-to-nearest, ties away from zero, computed
-// with a truncating 64-bit division.
+// high 32 bits of 2*a*b, rounded to nearest through a sign-dependent nudge and a
+// truncating 64-bit division (exact halves end up rounded toward +infinity).
 inline int32_t Srdhm(int32_t a, int32_t b) {
   if (a == b && a == std::numeric_limits<int32_t>::min()) {
     return std::numeric_limits<int32_t>::max();

@@ -1,0 +1,62 @@
+"""CPU-side checks of the product's C ABI: the library loads, exports every symbol the
+header declares, does the Prepare-time host math like the oracle, and refuses to
+compute without a gfx950 device instead of falling back."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import oracle
+from litert_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "litert_amd_fc.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lrtfc_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = capi.load()
+    declared = _header_symbols()
+    assert len(declared) >= 17
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert sorted(n for n, _, _ in capi.SYMBOLS) == declared
+    assert lib.lrtfc_abi_version() == 1
+
+
+def test_host_prepare_math_matches_oracle():
+    lib = capi.load()
+    rng = np.random.default_rng(1)
+    for m in np.concatenate([np.exp(rng.uniform(np.log(1e-11), np.log(50), 3000)), [0.0, 0.5, 1.0]]):
+        q, s = C.c_int32(), C.c_int()
+        assert lib.lrtfc_quantize_multiplier(float(m), C.byref(q), C.byref(s)) == 0
+        assert (q.value, s.value) == oracle.quantize_multiplier(float(m))
+    from litert_amd import fully_connected as fc
+    ws = np.exp(rng.uniform(np.log(1e-3), np.log(1e-2), 257)).astype(np.float32)
+    m1, s1 = fc.prepare_per_channel(0.02, ws, 0.05)
+    m2, s2 = oracle.fc_prepare_per_channel(0.02, ws, 0.05)
+    assert np.array_equal(m1, m2) and np.array_equal(s1, s2)
+    assert fc.prepare_per_tensor(0.5, 0.5, 1.0, 0.25) == oracle.fc_prepare_per_tensor(0.5, 0.5, 1.0, 0.25)
+    with pytest.raises(capi.LrtFcError):
+        fc.prepare_per_tensor(0.5, 0.5, 1.0, 0.5)  # bias scale off by 0.25 output quanta
+    for act in range(4):
+        for scale, zp in ((0.05, 5), (1.0, -1), (0.4, 3), (0.01, -128)):
+            assert fc.activation_range_int8(act, scale, zp) == oracle.activation_range_int8(act, scale, zp)
+
+
+def test_no_device_is_an_error_not_a_fallback():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    lib = capi.load()
+    assert lib.lrtfc_init(0) == capi.NO_DEVICE
+    assert b"HIP device" in lib.lrtfc_last_error()
+    # compute entry points refuse to run before a successful init
+    rc = lib.lrtfc_row_sums_int8(None, 4, 16, None, None)
+    assert rc == capi.NO_DEVICE

@@ -1,0 +1,360 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle on the same seeded
+inputs. Bars: bit-exact for full-integer int8 outputs and for quantized activations
+(values, scales and zero points); float outputs of the hybrid and blockwise paths are
+held to rtol 1e-5 with atol 1e-5 * max|ref| (the reference's comparator form,
+litert/ats/inference_fixture.h:262-286) and are in fact expected bit-identical, which
+is asserted where the kernel replays the reference's operation order.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from litert_amd import workloads as wl
+from tests import kat_harness as kh
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def fc():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a gfx950 device; none visible")
+    from litert_amd import fully_connected
+    fully_connected._ensure_init()
+    return fully_connected
+
+
+def _cuda(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _close(got, want, rtol=1e-5):
+    atol = rtol * float(np.abs(want).max())
+    return np.all(np.abs(got - want) <= atol + rtol * np.abs(want))
+
+
+def _bits_equal(a, b):
+    return np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+# ---- full-integer int8 -------------------------------------------------------------
+
+def _run_int8(fc, c, activation="none", bias=True):
+    op = fc.FullyConnectedInt8(c["w"], c["bias"] if bias else None, float(c["in_scale"]),
+                               c["in_zp"], c["w_scale"], float(c["out_scale"]), c["out_zp"],
+                               activation=activation)
+    y = op(_cuda(c["x"])).cpu().numpy()
+    mult, shift = oracle.fc_prepare_per_channel(float(c["in_scale"]), c["w_scale"],
+                                                float(c["out_scale"]))
+    lo, hi = oracle.activation_range_int8(fc._act(activation), float(c["out_scale"]), c["out_zp"])
+    want = oracle.fc_int8_per_channel(c["x"], c["w"], c["bias"] if bias else None, mult, shift,
+                                      -c["in_zp"], c["out_zp"], lo, hi)
+    return y, want
+
+
+def test_int8_config1_bit_exact(fc):
+    """Config 1: [1,2048] x [2048,2048], per-channel, bias, no activation."""
+    y, want = _run_int8(fc, wl.int8_fc())
+    assert np.array_equal(y, want)
+    assert len(np.unique(y)) > 100  # the case exercises the whole int8 range, not a clamp
+
+
+@pytest.mark.parametrize("B,K,N", [(1, 16, 1), (2, 48, 5), (3, 1040, 17), (4, 2048, 256),
+                                   (5, 512, 67), (8, 4096, 512), (9, 256, 33), (16, 128, 40),
+                                   (1, 16384, 64), (2, 10, 3), (3, 33, 7), (1, 100, 9)])
+@pytest.mark.parametrize("activation", ["none", "relu6"])
+def test_int8_gemv_shapes_bit_exact(fc, B, K, N, activation):
+    """Ragged shapes: depth off the 16-byte grid takes the generic kernel, batches that are
+    not a power of two split into tiles, rows that do not fill a pass are clamped."""
+    c = wl.int8_fc(B, K, N, seed=100 + B + K + N)
+    y, want = _run_int8(fc, c, activation, bias=(N % 2 == 1))
+    assert np.array_equal(y, want)
+
+
+def test_int8_per_tensor_with_filter_zero_point(fc):
+    rng = np.random.default_rng(5)
+    for B, K, N in ((2, 10, 3), (3, 64, 9), (8, 256, 40)):
+        x = rng.integers(-128, 128, (B, K)).astype(np.int8)
+        w = rng.integers(-128, 128, (N, K)).astype(np.int8)
+        bias = rng.integers(-1000, 1000, N).astype(np.int32)
+        op = fc.FullyConnectedInt8(w, bias, 0.5, -1, [0.5], 1.0, -1, activation="relu",
+                                   filter_zero_point=-1, bias_scale=0.25)
+        y = op(_cuda(x)).cpu().numpy()
+        m, s = oracle.fc_prepare_per_tensor(0.5, 0.5, 1.0, 0.25)
+        lo, hi = oracle.activation_range_int8(oracle.ACT_RELU, 1.0, -1)
+        want = oracle.fc_int8_per_tensor(x, w, bias, m, s, 1, 1, -1, lo, hi)
+        assert np.array_equal(y, want)
+
+
+def test_int8_reference_kats_through_hip(fc):
+    """tflite/kernels/fully_connected_test.cc:816-840, :863-888, :1463-1487, :1530-1562."""
+    W10 = [1, 2, 3, 4, 5, 6, 7, 8, 9, 10]
+    X2 = [1, 2, 3, 4, 5, 6, 7, 8, -9, -10, 1, 2, 3, 4, 5, 6, 7, -8, 9, -10]
+
+    def per_tensor(in_range, out_range, units, x, bias):
+        in_s, in_zp = kh.quantization_params(*in_range)
+        out_s, out_zp = kh.quantization_params(*out_range)
+        w_s, w_zp = kh.quantization_params(-63.5, 64)
+        wq = kh.quantize(W10 * units, w_s, w_zp).reshape(units, 10)
+        xq = kh.quantize(x, in_s, in_zp).reshape(-1, 10)
+        bs = np.float32(in_s * w_s)
+        op = fc.FullyConnectedInt8(wq, kh.quantize_bias(bias, bs), float(in_s), in_zp, [float(w_s)],
+                                   float(out_s), out_zp, filter_zero_point=w_zp,
+                                   bias_scale=float(bs))
+        return op(_cuda(xq)).cpu().numpy().ravel().tolist()
+
+    assert per_tensor((-63.5, 64), (-127, 128), 3, X2, [1, 2, 3]) == [23, 24, 25, 57, 58, 59]
+    assert per_tensor((-63.5, 64), (-127, 128), 4, X2[10:], [1, 2, 3, 4]) == [57, 58, 59, 60]
+    assert per_tensor((-127, 128), (-63.5, 64), 3, X2, [1, 2, 3]) == [47, 49, 51, 115, 117, 119]
+
+    in_s, in_zp = kh.quantization_params(-63.5, 64)
+    out_s, out_zp = kh.quantization_params(-127, 128)
+    scales = np.array([0.2, 0.25, 0.5], np.float32)
+    w = np.array(W10 * 3, np.float32).reshape(3, 10)
+    wq = np.clip(kh._round_half_away(w * (np.float32(1) / scales)[:, None]), -127, 127).astype(np.int8)
+    bq = kh._round_half_away(np.array([1, 2, 3], np.float32) / (scales * in_s)).astype(np.int32)
+    op = fc.FullyConnectedInt8(wq, bq, float(in_s), in_zp, scales, float(out_s), out_zp)
+    y = op(_cuda(kh.quantize(X2, in_s, in_zp).reshape(2, 10))).cpu().numpy().ravel().tolist()
+    assert y == [23, 24, 25, 57, 58, 59]
+
+
+def test_int8_int4_weights_kat(fc):
+    """fully_connected_test.cc:950-976: packed int4 per-channel weights, unpacked on the GPU."""
+    in_s, in_zp = kh.quantization_params(-63.5, 64)
+    out_s, out_zp = kh.quantization_params(-127, 128)
+    w4 = np.array([1, 2, 3, 4, 5, 6, 7, 6, 5, 4] * 3, np.int8).reshape(3, 10)
+    X2 = [1, 2, 3, 4, 5, 6, 7, 8, -9, -10, 1, 2, 3, 4, 5, 6, 7, -8, 9, -10]
+    bq = kh._round_half_away(np.array([1, 2, 3], np.float32) / np.float32(in_s)).astype(np.int32)
+    op = fc.FullyConnectedInt8(wl.pack_int4(w4), bq, float(in_s), in_zp, [1.0, 1.0, 1.0],
+                               float(out_s), out_zp, activation="relu", int4=True, depth=10)
+    y = op(_cuda(kh.quantize(X2, in_s, in_zp).reshape(2, 10))).cpu().numpy().ravel().tolist()
+    assert y == [103, 104, 105, 97, 98, 99]
+
+
+@pytest.mark.parametrize("activation", ["none", "relu6"])
+def test_int8_prefill_gemm_bit_exact(fc, activation):
+    """Config 4 shape class on the MFMA path, at a size the scalar oracle finishes in seconds."""
+    c = wl.prefill_int8_fc(256, 512, 512, seed=77)
+    y, want = _run_int8(fc, c, activation)
+    assert np.array_equal(y, want)
+    c = wl.int8_fc(128, 256, 256, in_zp=-3, out_zp=5, seed=78)  # non-zero input offset on the GEMM
+    y, want = _run_int8(fc, c, activation)
+    assert np.array_equal(y, want)
+
+
+def test_int8_prefill_full_size_properties(fc):
+    """Config 4 at full size (2048 x 4096 x 4096), RELU6 on and off, checked through
+    size-independent properties: a random sample of outputs against an int64 numpy
+    evaluation of the definition, agreement with the GEMV kernel on a slice of rows, and
+    clamp(no-activation output) == RELU6 output."""
+    c = wl.prefill_int8_fc()
+    x = _cuda(c["x"])
+    outs = {}
+    for activation in ("none", "relu6"):
+        op = fc.FullyConnectedInt8(c["w"], c["bias"], float(c["in_scale"]), c["in_zp"],
+                                   c["w_scale"], float(c["out_scale"]), c["out_zp"],
+                                   activation=activation)
+        outs[activation] = op(x).cpu().numpy()
+        if activation == "none":
+            y_gemv = op(x[:8]).cpu().numpy()  # 8 rows take the GEMV kernel
+            assert np.array_equal(outs["none"][:8], y_gemv)
+    lo, hi = oracle.activation_range_int8(oracle.ACT_RELU6, 0.05, 0)
+    assert np.array_equal(np.clip(outs["none"], lo, hi), outs["relu6"])
+    mult, shift = oracle.fc_prepare_per_channel(0.03, c["w_scale"], 0.05)
+    rng = np.random.default_rng(9)
+    ms, ns = rng.integers(0, 2048, 4000), rng.integers(0, 4096, 4000)
+    acc = np.einsum("ik,ik->i", c["x"][ms].astype(np.int64), c["w"][ns].astype(np.int64)) + c["bias"][ns]
+    want = np.array([oracle.mbqm(int(a), int(mult[n]), int(shift[n])) for a, n in zip(acc, ns)])
+    assert np.array_equal(outs["none"][ms, ns], np.clip(want, -128, 127).astype(np.int8))
+
+
+# ---- activation quantization ---------------------------------------------------------
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("asym", [True, False])
+def test_batch_quantize_floats_bit_exact(fc, variant, asym):
+    rng = np.random.default_rng(41)
+    for B, K in ((1, 4096), (4, 2048), (8, 4096), (3, 1001), (2, 7), (5, 16384), (1, 9)):
+        x = rng.standard_normal((B, K)).astype(np.float32)
+        if B > 1:
+            x[1] = 0.0                      # all-zero row: scale 1, zero point 0
+        if B > 2:
+            x[2] = np.abs(x[2]) * 1e-4      # rmin clamps to zero
+        q, sf, zp = fc.batch_quantize_floats(_cuda(x), asym, variant)
+        wq, wsf, wzp = oracle.batch_quantize_floats(x, asym, variant)
+        assert np.array_equal(q.cpu().numpy(), wq)
+        assert _bits_equal(sf.cpu().numpy(), wsf)
+        assert np.array_equal(zp.cpu().numpy(), wzp)
+
+
+def test_batch_quantize_reference_kats_through_hip(fc):
+    """tflite/kernels/internal/tensor_utils_test.cc:220-345."""
+    a = np.array([[-640, -635.0, -630, 10.0, 2.0, -5.0, -10.0, 0.0, 1000.0]], np.float32)
+    small = np.array([[-1e-5, 3e-5, -7e-6, -9e-5, 1e-6, 4e-5, 9e-6, 2e-4, 0]], np.float32)
+    q, _, _ = fc.batch_quantize_floats(_cuda(a), False)
+    assert q.cpu().numpy()[0].tolist() == [-81, -81, -80, 1, 0, -1, -1, 0, 127]
+    q, _, _ = fc.batch_quantize_floats(_cuda(small), False)
+    assert q.cpu().numpy()[0].tolist() == [-6, 19, -4, -57, 1, 25, 6, 127, 0]
+    q, _, zp = fc.batch_quantize_floats(_cuda(a), True)
+    assert q.cpu().numpy()[0].tolist() == [-128, -127, -126, -26, -28, -29, -30, -28, 127]
+    q, sf, zp = fc.batch_quantize_floats(_cuda(np.full((1, 9), 2000, np.float32)), True)
+    assert q.cpu().numpy()[0].tolist() == [127] * 9
+    q, _, _ = fc.batch_quantize_floats(_cuda(small), True)
+    assert q.cpu().numpy()[0].tolist() == [-58, -23, -55, -128, -48, -14, -41, 127, -49]
+    q, sf, zp = fc.batch_quantize_floats(_cuda(np.zeros((1, 9), np.float32)), True)
+    assert q.cpu().numpy()[0].tolist() == [0] * 9 and sf.item() == 1 and zp.item() == 0
+
+
+# ---- hybrid ----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("B", [1, 4, 8])
+def test_hybrid_config2_shape(fc, B):
+    """Config 2 at its real depth with a reduced number of output channels (the scalar
+    oracle needs ~60 ms per 1000 channels per batch row)."""
+    c = wl.hybrid_fc(B, 4096, 2048)
+    op = fc.FullyConnectedHybrid(c["w"], c["pcs"])
+    y = op(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"])
+    assert _close(y, want)
+    assert _bits_equal(y, want)
+
+
+@pytest.mark.parametrize("B,K,N", [(1, 64, 5), (3, 1040, 33), (2, 100, 7), (6, 512, 130)])
+@pytest.mark.parametrize("asym", [True, False])
+@pytest.mark.parametrize("per_channel", [True, False])
+@pytest.mark.parametrize("activation", ["none", "relu", "relu_n1_to_1", "relu6"])
+def test_hybrid_variants(fc, B, K, N, asym, per_channel, activation):
+    c = wl.hybrid_fc(B, K, N, seed=7 + B + K)
+    bias = np.random.default_rng(3).standard_normal(N).astype(np.float32)
+    pcs = c["pcs"] if per_channel else None
+    op = fc.FullyConnectedHybrid(c["w"], pcs, filter_scale=0.005, bias=bias,
+                                 asymmetric_quantize_inputs=asym, activation=activation)
+    y = op(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_hybrid(c["x"], c["w"], pcs, 0.005, bias, asym, fc._act(activation))
+    assert _close(y, want)
+    assert _bits_equal(y, want)
+
+
+def test_hybrid_dot_reference_kats_through_hip(fc):
+    """tflite/kernels/internal/tensor_utils_test.cc:1214-1231 (per-channel + offsets), exact."""
+    from tests.test_oracle_kat import _mv_data
+    from litert_amd import capi
+    import ctypes as C
+    for (rows, cols, batch), idx_want in (
+            ((4, 16, 1), {0: 620, 1: 3160, 2: 2540, 3: 7000}),
+            ((4, 32, 2), dict(enumerate([5208, 26288, 4245, 23312, 9138, 70756, 18708, 60916]))),
+            ((32, 512, 5), {0: 207783, 13: 411552, 39: 835936, 50: 440368, 100: 875192,
+                            123: 1775536, 150: 1050930})):
+        m, v, sf, _, pcs, offs = _mv_data(rows, cols, batch, per_channel=True)
+        dm, dv = _cuda(m), _cuda(v)
+        dsf, dpcs, doffs = _cuda(sf[:batch].copy()), _cuda(pcs), _cuda(offs)
+        rs = torch.empty(rows, dtype=torch.int32, device="cuda")
+        out = torch.empty((batch, rows), dtype=torch.float32, device="cuda")
+        lib = capi.load()
+        p = lambda t: C.c_void_p(t.data_ptr())
+        capi.check(lib.lrtfc_row_sums_int8(p(dm), rows, cols, p(rs), None))
+        capi.check(lib.lrtfc_fc_hybrid_int8(p(dv), p(dsf), p(doffs), p(dm), p(dpcs), 1.0, p(rs),
+                                            None, p(out), batch, cols, rows, 0, None))
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().ravel()
+        for i, w in idx_want.items():
+            assert got[i] == w
+
+
+def test_hybrid_full_size_properties(fc):
+    """Config 2 at full size (14336 x 4096, B = 8): row sums against numpy, a sample of
+    output channels against the oracle, and batch-row independence (row b of a B=8 call
+    equals the B=1 call on that row)."""
+    c = wl.hybrid_fc(8)
+    op = fc.FullyConnectedHybrid(c["w"], c["pcs"])
+    x = _cuda(c["x"])
+    y8 = op(x).cpu().numpy()
+    assert np.array_equal(op.row_sums.cpu().numpy(), c["w"].astype(np.int32).sum(1))
+    y1 = op(x[3:4]).cpu().numpy()
+    assert _bits_equal(y8[3:4], y1)
+    pick = np.random.default_rng(2).choice(14336, 256, replace=False)
+    want = oracle.fc_hybrid(c["x"], c["w"][pick], c["pcs"][pick])
+    assert _bits_equal(np.ascontiguousarray(y8[:, pick]), want)
+
+
+# ---- blockwise int4 -------------------------------------------------------------------------
+
+def _run_int4(fc, c, bias=None):
+    N = c["w"].shape[0]
+    op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], c["w"].shape[1], c["blocksize"],
+                                        bias)
+    y = op(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_blockwise_int4(c["x"], c["packed"], N, c["scales"].view(np.uint16),
+                                    c["blocksize"], bias)
+    return y, want
+
+
+@pytest.mark.parametrize("B,K,N", [(1, 4096, 1024), (4, 2048, 512), (1, 2048, 256), (4, 16384, 64),
+                                   (1, 16384, 130), (2, 32, 4), (3, 96, 9), (8, 1024, 77),
+                                   (5, 4096, 40), (1, 8192, 31)])
+def test_blockwise_int4_shapes(fc, B, K, N):
+    """Config 3 / config 5 depths (2048, 4096, 16384) and ragged sizes, blocksize 32, with the
+    full signed nibble range including -8."""
+    c = wl.blockwise_int4_fc(B, K, N, seed=11 + B + K + N, lo=-8, hi=7)
+    bias = np.random.default_rng(4).standard_normal(N).astype(np.float32) if N % 2 else None
+    y, want = _run_int4(fc, c, bias)
+    assert _close(y, want)
+    assert _bits_equal(y, want)
+
+
+@pytest.mark.parametrize("B,K,N,bs", [(2, 128, 6, 64), (1, 64, 5, 16), (3, 256, 4, 128), (2, 96, 8, 8)])
+def test_blockwise_int4_other_block_sizes(fc, B, K, N, bs):
+    c = wl.blockwise_int4_fc(B, K, N, blocksize=bs, seed=5 + bs, lo=-8, hi=7)
+    y, want = _run_int4(fc, c)
+    assert _close(y, want)
+    assert _bits_equal(y, want)
+
+
+def test_blockwise_int4_subnormal_and_large_scales(fc):
+    c = wl.blockwise_int4_fc(2, 256, 16, seed=3)
+    s = c["scales"].view(np.uint16).copy()
+    s[0, :] = [0x0001, 0x03FF, 0x0400, 0x7BFF, 0x8001, 0x0000, 0x3C00, 0xBC00]  # subnormals, max, -0...
+    c["scales"] = s.view(np.float16)
+    y, want = _run_int4(fc, c)
+    assert _bits_equal(y, want)
+
+
+def test_blockwise_int4_config3_full_size_properties(fc):
+    """Config 3 at full size (14336 x 4096): a sample of output channels against the oracle
+    and batch-row independence between B=4 and B=1 calls."""
+    c = wl.blockwise_int4_fc(4)
+    op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], 4096, 32)
+    x = _cuda(c["x"])
+    y4 = op(x).cpu().numpy()
+    y1 = op(x[2:3]).cpu().numpy()
+    assert _bits_equal(y4[2:3], y1)
+    pick = np.random.default_rng(6).choice(14336, 192, replace=False)
+    want = oracle.fc_blockwise_int4(c["x"], c["packed"][pick], pick.size,
+                                    c["scales"][pick].view(np.uint16), 32)
+    assert _bits_equal(np.ascontiguousarray(y4[:, pick]), want)
+
+
+# ---- edge cases of the op contract ------------------------------------------------------------
+
+def test_empty_and_zero_depth(fc):
+    """NumElements(output) == 0 is a no-op and depth 0 zero-fills
+    (tflite/kernels/fully_connected.cc:1966-1973)."""
+    import ctypes as C
+    from litert_amd import capi
+    lib = capi.load()
+    out = torch.full((2, 3), 7, dtype=torch.int8, device="cuda")
+    one = torch.ones(1, dtype=torch.int32, device="cuda")
+    p = lambda t: C.c_void_p(t.data_ptr())
+    capi.check(lib.lrtfc_fc_int8(None, None, None, p(one), p(one), 0, None, p(out), 0, 16, 3, 0, 0,
+                                 0, -128, 127, None))
+    torch.cuda.synchronize()
+    assert out.eq(7).all()
+    capi.check(lib.lrtfc_fc_int8(None, None, None, p(one), p(one), 0, None, p(out), 2, 0, 3, 0, 0,
+                                 0, -128, 127, None))
+    torch.cuda.synchronize()
+    assert out.eq(0).all()
+    rc = lib.lrtfc_fc_int8(p(out), p(out), None, p(one), p(one), 0, None, p(out), 2, 16, 3, 5, 0, 0,
+                           -128, 127, None)
+    assert rc == capi.INVALID_ARGUMENT and b"filter_row_sums" in lib.lrtfc_last_error()

@@ -72,10 +72,8 @@ def test_mbqm_kat_max_operands():
 def _srdhm_exact(a, b):
     if a == b == INT32_MIN:
         return INT32_MAX
-    v = Fraction(a * b, 2 ** 31)
-    # nearest, ties away from zero
-    n = int(abs(v) + Fraction(1, 2))
-    return n if v >= 0 else -n
+    # nearest; the nudge 1 - 2^30 for negative products sends exact halves upward
+    return (Fraction(a * b, 2 ** 31) + Fraction(1, 2)).__floor__()
 
 
 def _rdbp_exact(x, e):
@@ -85,9 +83,10 @@ def _rdbp_exact(x, e):
 
 
 def test_mbqm_against_exact_rationals():
-    """Each of the two roundings is round-to-nearest, ties away from zero, of the
-    exact quotient: checked with Python big rationals, which share no code with the
-    C implementation (a wrong nudge sign, threshold or shift fails here)."""
+    """The doubling high multiply is floor(ab / 2^31 + 1/2) and the power-of-two
+    division is round-to-nearest, ties away from zero: checked with Python big
+    rationals, which share no code with the C implementation (a wrong nudge sign,
+    threshold or shift fails here)."""
     rng = np.random.default_rng(11)
     L = oracle.lib()
     xs = rng.integers(INT32_MIN, INT32_MAX, 4000, endpoint=True)
@@ -106,6 +105,10 @@ def test_mbqm_against_exact_rationals():
             if INT32_MIN <= x <= INT32_MAX:
                 assert L.orc_rounding_divide_by_pot(x, e) == _rdbp_exact(x, e)
     assert L.orc_srdhm(INT32_MIN, INT32_MIN) == INT32_MAX
+    # exact halves of the high multiply: a * b = (2j + 1) * 2^30
+    for j in (-7, -2, -1, 0, 1, 5):
+        for a, b in (((2 * j + 1), 1 << 30), ((2 * j + 1) << 10, 1 << 20), (-(2 * j + 1), -(1 << 30))):
+            assert L.orc_srdhm(a, b) == _srdhm_exact(a, b) == j + 1
     # accumulator-sized inputs with a left shift (multiplier > 1)
     for x in rng.integers(-(1 << 27), 1 << 27, 2000).tolist():
         for s in (1, 2, 3):
