@@ -1,0 +1,328 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X quantized FULLY_CONNECTED hot path (one GPU).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-extras] [--skip-cpu]
+
+A step is one pass of the headline workload: the hybrid dynamic-range FC of
+14336 x 4096 (float32 activations quantized per row inside the op, int8 per-channel
+weights) at decode batch sizes B = 1, 4 and 8, one op each. Every op is what the
+delegate launches for the node: the activation-quantization kernel followed by the GEMV
+kernel. Inputs are resident in HBM before the timed region. Steps rotate over several
+copies of the weights so that they are served from HBM rather than from the 256 MB
+Infinity Cache ("cold"); the cache-hot rate is reported beside it.
+
+Launches are replayed from HIP graphs, so the GPU runs kernels back to back and the
+host's launch cost (which exceeds these kernels' few microseconds) stays out of the
+measurement. Kernel durations for the roofline figures come from HIP events around
+graph replays of that kernel alone.
+
+The one JSON line printed at the end carries the headline value, the roofline of the
+dominant kernel, the CPU baseline (the oracle port, one host core, bounded sample) and,
+under "also", the other configurations of the benchmark contract.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "FC GEMV µs & HBM GB/s (% peak), int8 GEMM TOPS (% MFMA peak), 1 GPU"
+HBM_PEAK_GBPS = 8000.0
+INT8_MFMA_PEAK_TOPS = 5000.0
+N_OUT, K_IN = 14336, 4096
+BATCHES = (1, 4, 8)
+WEIGHT_COPIES = 6  # 6 x 58.7 MB > 256 MB Infinity Cache
+
+
+def hybrid_bytes(b, n=N_OUT, k=K_IN):
+    """Algorithmic bytes of one hybrid FC op: W + per-channel scales + row sums + x + y."""
+    return n * k + 4 * n + 4 * n + 4 * k * b + 4 * n * b
+
+
+def int4_bytes(b, n, k, bs=32):
+    return n * k // 2 + 2 * n * (k // bs) + 4 * k * b + 4 * n * b
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--skip-extras", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the op shards "
+              "by output channel with no collective; see DESIGN.md). Run with --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from litert_amd import capi
+    from litert_amd import fully_connected as fc
+    from litert_amd import workloads as wl
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a gfx950 GPU", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    fc._ensure_init()
+    lib = capi.load()
+    p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+    stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def timed_replays(graphs, reps):
+        """Average milliseconds per replay, graphs[i % len] replayed reps times."""
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(reps):
+            graphs[i % len(graphs)].replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    def capture(fn):
+        fn()  # warm: sets function attributes, touches lazily loaded code objects
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g
+
+    # ---- headline workload: config 2 -------------------------------------------------
+    c = wl.hybrid_fc(max(BATCHES))
+    ops = []
+    for i in range(WEIGHT_COPIES):
+        ops.append(fc.FullyConnectedHybrid(np.roll(c["w"], i, axis=0) if i else c["w"],
+                                           np.roll(c["pcs"], i) if i else c["pcs"]))
+    x_all = torch.from_numpy(c["x"]).cuda()
+    xs = {b: x_all[:b].contiguous() for b in BATCHES}
+    outs = {b: torch.empty((b, N_OUT), dtype=torch.float32, device="cuda") for b in BATCHES}
+    for op in ops:
+        op._workspace(max(BATCHES))
+
+    def step_fn(op):
+        def run():
+            for b in BATCHES:
+                op(xs[b], out=outs[b])
+        return run
+
+    # One graph holds one step on each weight copy (6 steps, 36 kernels), so that the
+    # GPU, not the host's replay call, sets the pace; K % 6 leftover steps replay
+    # single-step graphs.
+    step_graphs = [capture(step_fn(op)) for op in ops]
+    round_fns = [step_fn(op) for op in ops]
+    round_graph = capture(lambda: [f() for f in round_fns])
+    hot_graph = capture(lambda: [round_fns[0]() for _ in ops])
+    for i in range(args.warmup):
+        step_graphs[i % len(ops)].replay()
+    torch.cuda.synchronize()
+    # exactly K timed steps, bracketed by synchronize on both sides
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps // len(ops)):
+        round_graph.replay()
+    for i in range(args.steps % len(ops)):
+        step_graphs[i].replay()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_cold = e0.elapsed_time(e1) / args.steps
+    ms_hot = timed_replays([hot_graph], max(args.steps // len(ops), 1)) / len(ops)
+    step_bytes = sum(hybrid_bytes(b) for b in BATCHES)
+    value = step_bytes / (ms_cold * 1e-3) / 1e9
+
+    # ---- per-kernel durations for the roofline -----------------------------------------
+    qbuf = {b: fc.batch_quantize_floats(xs[b]) for b in BATCHES}
+
+    def gemv_only(op, b):
+        q, sf, zp = qbuf[b]
+        def run():
+            capi.check(lib.lrtfc_fc_hybrid_int8(p(q), p(sf), p(zp), p(op.filter), p(op.pcs), 1.0,
+                                                p(op.row_sums), None, p(outs[b]), b, K_IN, N_OUT,
+                                                0, stream()))
+        return run
+
+    def quant_only(b):
+        q, sf, zp = qbuf[b]
+        def run():
+            capi.check(lib.lrtfc_batch_quantize_floats(p(xs[b]), b, K_IN, p(q), p(sf), p(zp), 1, 0,
+                                                       stream()))
+        return run
+
+    ROUNDS = 4  # launches per graph = ROUNDS x weight copies
+
+    def many(fns):
+        """Graph of ROUNDS passes over fns; returns (graph, launches per replay)."""
+        return capture(lambda: [f() for _ in range(ROUNDS) for f in fns]), ROUNDS * len(fns)
+
+    def per_launch_us(fns, replays=25):
+        g, n = many(fns)
+        return timed_replays([g], replays) * 1e3 / n
+
+    per_b = {}
+    for b in BATCHES:
+        cold_us = per_launch_us([gemv_only(op, b) for op in ops])
+        hot_us = per_launch_us([gemv_only(ops[0], b)] * len(ops))
+        quant_us = per_launch_us([quant_only(b)] * len(ops))
+        op_us = per_launch_us([(lambda o: lambda: o(xs[b], out=outs[b]))(op) for op in ops])
+        per_b[b] = dict(gemv_us_cold=round(cold_us, 3), gemv_us_hot=round(hot_us, 3),
+                        quantize_us=round(quant_us, 3), op_us_cold=round(op_us, 3),
+                        gemv_gbps_cold=round(hybrid_bytes(b) / cold_us / 1e3, 1),
+                        gemv_gbps_hot=round(hybrid_bytes(b) / hot_us / 1e3, 1),
+                        op_gbps_cold=round(hybrid_bytes(b) / op_us / 1e3, 1),
+                        frac_of_hbm_peak_cold=round(hybrid_bytes(b) / cold_us / 1e3 / HBM_PEAK_GBPS, 4))
+    b_dom = 1
+    achieved = hybrid_bytes(b_dom) / per_b[b_dom]["gemv_us_cold"] / 1e3
+    roofline = dict(bound="hbm", kernel="FcInt8GemvKernel<R=4,BT=1,hybrid> (config 2, B=1, cold)",
+                    achieved=round(achieved, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
+                    frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=None,
+                    algorithmic_bytes_per_launch=hybrid_bytes(b_dom),
+                    avg_launch_us=per_b[b_dom]["gemv_us_cold"])
+
+    also = {"config2_hybrid_per_batch": per_b,
+            "config2_step_ms_hot": round(ms_hot, 5),
+            "config2_step_gbps_hot": round(step_bytes / (ms_hot * 1e-3) / 1e9, 1)}
+
+    if not args.skip_extras:
+        also.update(extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_launch_us))
+
+    cpu_baseline = None
+    if not args.skip_cpu:
+        cpu_baseline = cpu_baseline_leg(c)
+
+    line = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_cold, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: hybrid f32 x int8 per-channel FULLY_CONNECTED "
+                               "14336x4096, one op each at B=1,4,8 per step (quantize kernel + "
+                               "GEMV kernel), weights rotated over %d copies (HBM-cold)"
+                               % WEIGHT_COPIES,
+                   "algorithmic_bytes_per_step": step_bytes,
+                   "host_wall_ms_per_step": round(wall_ms_per_step, 5)},
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "also": also,
+    }
+    print(json.dumps(line))
+
+
+def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_launch_us):
+    """Configs 1, 3, 4 and 5 of the benchmark contract (reported under "also")."""
+    out = {}
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    # config 1: int8 GEMV 2048 -> 2048, B = 1 (4 MiB of weights: launch-latency dominated)
+    c1 = wl.int8_fc()
+    op1 = fc.FullyConnectedInt8(c1["w"], c1["bias"], float(c1["in_scale"]), c1["in_zp"],
+                                c1["w_scale"], float(c1["out_scale"]), c1["out_zp"])
+    x1 = dev(c1["x"])
+    y1 = torch.empty((1, 2048), dtype=torch.int8, device="cuda")
+    us = per_launch_us([lambda: op1(x1, out=y1)] * 6)
+    b1 = 2048 * 2048 + 2048 + 3 * 4 * 2048 + 2048
+    out["config1_int8_gemv_2048x2048_B1"] = dict(us=round(us, 3), gbps=round(b1 / us / 1e3, 1),
+                                                 frac_of_hbm_peak=round(b1 / us / 1e3 / HBM_PEAK_GBPS, 4),
+                                                 note="weights fit in cache: hot figure")
+
+    # config 3: blockwise int4 GEMV 14336 x 4096, B = 1
+    c3 = wl.blockwise_int4_fc(1)
+    ops3 = [fc.FullyConnectedBlockwiseInt4(np.roll(c3["packed"], i, axis=0), np.roll(c3["scales"], i, axis=0),
+                                           4096, 32) for i in range(8)]
+    x3 = dev(c3["x"])
+    y3 = torch.empty((1, 14336), dtype=torch.float32, device="cuda")
+    q3 = fc.batch_quantize_floats(x3)
+
+    def int4_kernel_only(op):
+        def run():
+            capi.check(lib.lrtfc_fc_blockwise_int4_quantized(
+                p(q3[0]), p(q3[1]), p(q3[2]), p(op.filter), p(op.scales), p(op.kfsum), None, p(y3),
+                1, 4096, 14336, 32, stream()))
+        return run
+
+    k_cold = per_launch_us([int4_kernel_only(op) for op in ops3])
+    k_hot = per_launch_us([int4_kernel_only(ops3[0])] * len(ops3))
+    o_cold = per_launch_us([(lambda o: lambda: o(x3, out=y3))(op) for op in ops3])
+    b3 = int4_bytes(1, 14336, 4096)
+    out["config3_int4_gemv_14336x4096_B1"] = dict(
+        kernel_us_cold=round(k_cold, 3), kernel_us_hot=round(k_hot, 3), op_us_cold=round(o_cold, 3),
+        kernel_gbps_cold=round(b3 / k_cold / 1e3, 1), kernel_gbps_hot=round(b3 / k_hot / 1e3, 1),
+        op_gbps_cold=round(b3 / o_cold / 1e3, 1),
+        frac_of_hbm_peak_cold=round(b3 / k_cold / 1e3 / HBM_PEAK_GBPS, 4), algorithmic_bytes=b3)
+    del ops3
+
+    # config 4: prefill int8 GEMM 2048 x 4096 x 4096, RELU6 off / on
+    c4 = wl.prefill_int8_fc()
+    x4 = dev(c4["x"])
+    y4 = torch.empty((2048, 4096), dtype=torch.int8, device="cuda")
+    ops_per_call = 2.0 * 2048 * 4096 * 4096
+    for act in ("none", "relu6"):
+        op4 = fc.FullyConnectedInt8(c4["w"], c4["bias"], float(c4["in_scale"]), c4["in_zp"],
+                                    c4["w_scale"], float(c4["out_scale"]), c4["out_zp"],
+                                    activation=act)
+        us = per_launch_us([lambda: op4(x4, out=y4)] * 4)
+        tops = ops_per_call / us / 1e6
+        out["config4_int8_gemm_2048x4096x4096_" + act] = dict(
+            us=round(us, 2), tops=round(tops, 1),
+            frac_of_int8_mfma_peak=round(tops / INT8_MFMA_PEAK_TOPS, 4))
+
+    # config 5: FC chain of a Gemma-2B-shaped 18-layer decoder, blockwise int4, B = 1 and 4.
+    # Each node gets its own seeded N(0,1) input (FC-only chain: outputs are discarded).
+    g = torch.Generator(device="cuda").manual_seed(5)
+    nodes = []
+    for layer in range(wl.GEMMA2B_LAYERS):
+        for name, k, n in wl.GEMMA2B_LAYER_FCS:
+            packed = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda", generator=g)
+            scales = (torch.rand((n, k // 32), device="cuda", generator=g) * 1.5e-2 + 5e-3).half()
+            nodes.append(fc.FullyConnectedBlockwiseInt4(packed, scales, k, 32))
+    chain_bytes = sum(int4_bytes(0, op.out_depth, op.depth) for op in nodes)
+    for b in (1, 4):
+        xin = {k: torch.randn((b, k), device="cuda", generator=g) for k in (2048, 16384)}
+        yout = {n: torch.empty((b, n), dtype=torch.float32, device="cuda") for n in (256, 2048, 16384)}
+
+        def chain():
+            for op in nodes:
+                op(xin[op.depth], out=yout[op.out_depth])
+
+        gc = capture(chain)
+        us = timed_replays([gc], 30) * 1e3
+        out["config5_gemma2b_fc_chain_B%d" % b] = dict(
+            us_per_token=round(us, 1), fc_nodes=len(nodes), weight_bytes=chain_bytes,
+            gbps=round(chain_bytes / us / 1e3, 1),
+            frac_of_hbm_peak=round(chain_bytes / us / 1e3 / HBM_PEAK_GBPS, 4))
+        del gc
+    return out
+
+
+def cpu_baseline_leg(c):
+    """The oracle's restatement of EvalHybridDense (portable reference kernels, scalar, one
+    thread) on the host, on a bounded sample: B = 1, full 14336 x 4096 filter, repeated for
+    about 10 seconds. Reported in the headline unit (algorithmic GB/s of the op)."""
+    import oracle
+    x = c["x"][:1]
+    row_sums = c["w"].astype(np.int32).sum(1).astype(np.int32)  # cached after the first Eval
+    oracle.fc_hybrid(x, c["w"][:256], c["pcs"][:256])  # load + warm
+    reps, t_total = 0, 0.0
+    while t_total < 10.0 and reps < 200:
+        t0 = time.perf_counter()
+        oracle.fc_hybrid(x, c["w"], c["pcs"], row_sums=row_sums)
+        t_total += time.perf_counter() - t0
+        reps += 1
+    sec = t_total / reps
+    return {"value": round(hybrid_bytes(1) / sec / 1e9, 3), "unit": "GB/s", "cores": 1,
+            "kind": "port", "us_per_op": round(sec * 1e6, 1),
+            "sample": "config 2 at B=1 only (14336x4096 hybrid FC, quantize + int8 dot with cached "
+                      "row sums), %d repetitions, oracle built with g++ -O2 "
+                      "-ffp-contract=off" % reps}
+
+
+if __name__ == "__main__":
+    main()

@@ -81,6 +81,7 @@ def lib():
         L.orc_apply_activation.argtypes = [_f32p, C.c_int, C.c_int]
         L.orc_fc_hybrid.argtypes = [_f32p, C.c_int, C.c_int, _i8p, C.c_int, _f32p, C.c_float,
                                     _f32p, C.c_int, C.c_int, C.c_int, _f32p, _i8p, _f32p, _i32p]
+        L.orc_fc_hybrid_cached.argtypes = L.orc_fc_hybrid.argtypes + [_i32p, C.c_int]
         L.orc_fc_blockwise_int4.argtypes = [_f32p, C.c_int, C.c_int, _u8p, C.c_int, _u16p,
                                             C.c_int, _f32p, C.c_int, _f32p]
         _LIB = L
@@ -260,7 +261,9 @@ def matrix_batch_vector_multiply_accumulate(matrix, vectors, scaling_factors, re
 
 
 def fc_hybrid(x, w, per_channel_scales=None, filter_scale=1.0, bias=None, asymmetric=True,
-              activation=ACT_NONE, variant=QUANT_PORTABLE, return_quant=False):
+              activation=ACT_NONE, variant=QUANT_PORTABLE, return_quant=False, row_sums=None):
+    """row_sums: an int32 [N] array already filled by an earlier call (the op's cached
+    persistent temporary); None recomputes them."""
     x = _c(x, np.float32)
     w = _c(w, np.int8)
     N, K = w.shape
@@ -271,9 +274,13 @@ def fc_hybrid(x, w, per_channel_scales=None, filter_scale=1.0, bias=None, asymme
     q = np.empty((B, K), dtype=np.int8)
     sf = np.empty(B, dtype=np.float32)
     zp = np.empty(B, dtype=np.int32)
-    rc = lib().orc_fc_hybrid(_p(x, _f32p), B, K, _p(w, _i8p), N, _p(pcs, _f32p), filter_scale,
-                             _p(bias, _f32p), int(asymmetric), activation, variant, _p(y, _f32p),
-                             _p(q, _i8p), _p(sf, _f32p), _p(zp, _i32p))
+    compute = row_sums is None
+    if compute:
+        row_sums = np.empty(N, dtype=np.int32)
+    rc = lib().orc_fc_hybrid_cached(_p(x, _f32p), B, K, _p(w, _i8p), N, _p(pcs, _f32p),
+                                    filter_scale, _p(bias, _f32p), int(asymmetric), activation,
+                                    variant, _p(y, _f32p), _p(q, _i8p), _p(sf, _f32p),
+                                    _p(zp, _i32p), _p(row_sums, _i32p), int(compute))
     if rc:
         raise ValueError("activation not restated in the oracle")
     return (y, q, sf, zp) if return_quant else y

@@ -511,10 +511,11 @@ int orc_apply_activation(float* data, int size, int activation) {
   }
 }
 
-int orc_fc_hybrid(const float* input, int batches, int depth, const int8_t* filter, int out_depth,
-                  const float* per_channel_scales, float filter_scale, const float* bias,
-                  int asymmetric_quantize_inputs, int activation, int quant_variant,
-                  float* output, int8_t* q_out, float* sf_out, int32_t* zp_out) {
+int orc_fc_hybrid_cached(const float* input, int batches, int depth, const int8_t* filter,
+                         int out_depth, const float* per_channel_scales, float filter_scale,
+                         const float* bias, int asymmetric_quantize_inputs, int activation,
+                         int quant_variant, float* output, int8_t* q_out, float* sf_out,
+                         int32_t* zp_out, int32_t* row_sums, int compute_row_sums) {
   const size_t total_in = static_cast<size_t>(batches) * depth;
   // fully_connected.cc:780-786.
   for (int b = 0; b < batches; ++b) {
@@ -550,11 +551,20 @@ int orc_fc_hybrid(const float* input, int batches, int depth, const int8_t* filt
     // fully_connected.cc:838-843.
     for (int b = 0; b < batches; ++b) sf[b] *= filter_scale;
   }
-  std::vector<int32_t> row_sums(out_depth);
   orc_matrix_batch_vector_multiply_accumulate(filter, out_depth, depth, q.data(), sf.data(),
                                               batches, output, per_channel_scales, zp.data(),
-                                              row_sums.data(), 1);
+                                              row_sums, compute_row_sums);
   return orc_apply_activation(output, batches * out_depth, activation);
+}
+
+int orc_fc_hybrid(const float* input, int batches, int depth, const int8_t* filter, int out_depth,
+                  const float* per_channel_scales, float filter_scale, const float* bias,
+                  int asymmetric_quantize_inputs, int activation, int quant_variant,
+                  float* output, int8_t* q_out, float* sf_out, int32_t* zp_out) {
+  std::vector<int32_t> row_sums(out_depth);
+  return orc_fc_hybrid_cached(input, batches, depth, filter, out_depth, per_channel_scales,
+                              filter_scale, bias, asymmetric_quantize_inputs, activation,
+                              quant_variant, output, q_out, sf_out, zp_out, row_sums.data(), 1);
 }
 
 void orc_fc_blockwise_int4(const float* input, int batches, int depth,

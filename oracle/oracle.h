@@ -163,6 +163,15 @@ int orc_fc_hybrid(const float* input, int batches, int depth, const int8_t* filt
                   int asymmetric_quantize_inputs, int activation, int quant_variant,
                   float* output, int8_t* q_out, float* sf_out, int32_t* zp_out);
 
+/* Same, with the row sums kept by the caller as the op keeps them in a persistent
+ * temporary (fully_connected.cc:700-708): computed when compute_row_sums != 0,
+ * reused otherwise. This is the form the CPU-baseline timing uses. */
+int orc_fc_hybrid_cached(const float* input, int batches, int depth, const int8_t* filter,
+                         int out_depth, const float* per_channel_scales, float filter_scale,
+                         const float* bias, int asymmetric_quantize_inputs, int activation,
+                         int quant_variant, float* output, int8_t* q_out, float* sf_out,
+                         int32_t* zp_out, int32_t* row_sums, int compute_row_sums);
+
 /* ---- blockwise int4 weights -------------------------------------------- */
 
 /* tflite/kernels/fully_connected.cc:1014-1086 (EvalBlockwise4Bit), float ops
