@@ -1,0 +1,641 @@
+// TfLiteDelegate plugin that claims quantized FULLY_CONNECTED nodes and runs them on
+// an MI355X through the C ABI of include/litert_amd_fc.h.
+//
+// Boundary (reference tree): the plugin is loaded by TfLiteExternalDelegateCreate
+// (tflite/delegates/external/external_delegate.cc:39-60, 215-223) through
+// tflite_plugin_create_delegate / tflite_plugin_destroy_delegate
+// (external_delegate_interface.h:65-74). Delegate::Prepare inspects the execution
+// plan and hands the nodes it supports to ReplaceNodeSubsetsWithDelegateKernels
+// (tflite/core/c/common.h:982-986); the runtime then drives the kernel registration's
+// init / prepare / invoke / free for each partition (tflite/core/subgraph.cc:523-637,
+// 1691-1775). Nodes the predicate below declines stay on the CPU kernels.
+//
+// Device residency: constant tensors (filter, bias, scales) are uploaded and
+// pre-reduced once in `prepare`; activations cross PCIe once in and once out per
+// partition invoke, and tensors produced and consumed inside one partition never
+// leave HBM.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "litert_amd_fc.h"
+#include "tflite_abi.h"
+
+namespace {
+
+constexpr int kMaxFcVersion = 14;  // tflite/core/kernels/register.cc:84-86
+
+struct Options {
+  int device = 0;
+  int quant_variant = LRTFC_QUANT_PORTABLE;
+  bool claim_int8 = true;
+  bool claim_hybrid = true;
+  bool claim_int4_blockwise = true;
+};
+
+struct DelegateState {
+  Options options;
+  TfLiteDelegate delegate;
+};
+
+enum class FcKind { kNone, kInt8, kHybrid, kInt4Blockwise };
+
+int64_t NumElements(const TfLiteIntArray* dims) {
+  int64_t n = 1;
+  for (int i = 0; i < dims->size; ++i) n *= dims->data[i];
+  return n;
+}
+
+bool IsConstant(const TfLiteTensor& t) {
+  // tflite/kernels/kernel_util.h:191-193
+  return t.allocation_type == kTfLiteMmapRo && t.data.raw != nullptr;
+}
+
+const TfLiteTensor* OptionalInput(const TfLiteContext* ctx, const TfLiteNode* node, int i) {
+  if (i >= node->inputs->size) return nullptr;
+  const int idx = node->inputs->data[i];
+  if (idx == kTfLiteOptionalTensor) return nullptr;
+  return &ctx->tensors[idx];
+}
+
+bool ClippingActivation(TfLiteFusedActivation a) {
+  return a == kTfLiteActNone || a == kTfLiteActRelu || a == kTfLiteActReluN1To1 ||
+         a == kTfLiteActRelu6;
+}
+
+// The node-claim predicate: the same tensor / quantization-parameter / fused-activation
+// combinations the builtin kernel accepts for these three paths
+// (tflite/kernels/fully_connected.cc:254-308, 440-761), nothing else.
+FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
+                const TfLiteRegistration* registration, const Options& opt,
+                std::string* why_not) {
+  auto no = [&](const char* reason) {
+    if (why_not) *why_not = reason;
+    return FcKind::kNone;
+  };
+  if (registration->builtin_code != kTfLiteBuiltinFullyConnected) return no("not FULLY_CONNECTED");
+  if (registration->version > kMaxFcVersion) return no("op version newer than 14");
+  if (!node->builtin_data) return no("no builtin data");
+  const auto* params = static_cast<const TfLiteFullyConnectedParams*>(node->builtin_data);
+  if (params->weights_format != kTfLiteFullyConnectedWeightsFormatDefault) {
+    return no("shuffled weights format");
+  }
+  if (node->inputs->size != 2 && node->inputs->size != 3) return no("needs 2 or 3 inputs");
+  if (node->outputs->size != 1) return no("needs exactly one output");
+  const TfLiteTensor& input = ctx->tensors[node->inputs->data[0]];
+  const TfLiteTensor& filter = ctx->tensors[node->inputs->data[1]];
+  const TfLiteTensor* bias = OptionalInput(ctx, node, 2);
+  const TfLiteTensor& output = ctx->tensors[node->outputs->data[0]];
+  if (!filter.dims || filter.dims->size != 2) return no("filter is not rank 2");
+  if (!IsConstant(filter)) return no("filter is not a constant tensor");
+  if (filter.sparsity != nullptr) return no("sparse filter");
+  if (bias && !IsConstant(*bias)) return no("bias is not a constant tensor");
+  if (!input.dims || input.dims->size < 1) return no("input has no shape");
+  const int out_depth = filter.dims->data[0];
+  const int depth = filter.dims->data[1];
+  if (bias && NumElements(bias->dims) != out_depth) return no("bias size != output channels");
+
+  if (input.type == kTfLiteInt8 && output.type == kTfLiteInt8 &&
+      (filter.type == kTfLiteInt8 || filter.type == kTfLiteInt4)) {
+    if (!opt.claim_int8) return no("int8 path disabled by option");
+    if (!ClippingActivation(params->activation)) return no("activation not a clamp");
+    if (bias && bias->type != kTfLiteInt32) return no("bias is not int32");
+    if (input.quantization.type != kTfLiteAffineQuantization ||
+        filter.quantization.type != kTfLiteAffineQuantization) {
+      return no("input/filter lack affine quantization");
+    }
+    const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
+    if (!fq || !fq->scale || fq->scale->size < 1) return no("filter has no scales");
+    if (fq->scale->size > 1) {
+      if (fq->quantized_dimension != 0) return no("quantized_dimension != 0");
+      if (fq->scale->size != out_depth) return no("scale count != output channels");
+    }
+    if (fq->zero_point) {
+      const bool per_channel = fq->scale->size > 1;
+      for (int i = 0; i < fq->zero_point->size; ++i) {
+        if ((per_channel || filter.type == kTfLiteInt4) && fq->zero_point->data[i] != 0) {
+          return no("non-zero filter zero point");
+        }
+      }
+    }
+    if (output.params.scale <= 0.0f || input.params.scale <= 0.0f) return no("missing scales");
+    return FcKind::kInt8;
+  }
+
+  if (input.type == kTfLiteFloat32 && output.type == kTfLiteFloat32) {
+    if (bias && bias->type != kTfLiteFloat32) return no("bias is not float32");
+    if (filter.type == kTfLiteInt8) {
+      if (!opt.claim_hybrid) return no("hybrid path disabled by option");
+      // The hybrid path accepts every fused activation; tanh/sigmoid/signbit go through
+      // Eigen in the reference and are left to the CPU.
+      if (!ClippingActivation(params->activation)) return no("activation not a clamp");
+      if (filter.quantization.type != kTfLiteAffineQuantization) return no("filter not affine");
+      const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
+      if (!fq || !fq->scale || fq->scale->size < 1) return no("filter has no scales");
+      if (fq->scale->size > 1 && (fq->quantized_dimension != 0 || fq->scale->size != out_depth)) {
+        return no("per-channel scales do not match output channels");
+      }
+      if (depth == 0) return no("empty depth");
+      return FcKind::kHybrid;
+    }
+    if (filter.type == kTfLiteInt4 && filter.quantization.type == kTfLiteBlockwiseQuantization) {
+      if (!opt.claim_int4_blockwise) return no("int4 blockwise path disabled by option");
+      // Gate of the builtin's 4-bit path (fully_connected.cc:609-633): even depth,
+      // at least 4 output channels and 32 of depth.
+      if (depth % 2 != 0 || out_depth < 4 || depth < 32) return no("shape outside 4-bit gate");
+      const auto* bq = static_cast<const TfLiteBlockwiseQuantization*>(filter.quantization.params);
+      if (!bq || bq->blocksize <= 0 || depth % bq->blocksize != 0) return no("bad blocksize");
+      if (bq->scale < 0 || static_cast<size_t>(bq->scale) >= ctx->tensors_size) {
+        return no("scale tensor index out of range");
+      }
+      const TfLiteTensor& scales = ctx->tensors[bq->scale];
+      if (scales.type != kTfLiteFloat16 || !IsConstant(scales)) return no("scales not const fp16");
+      if (NumElements(scales.dims) != static_cast<int64_t>(out_depth) * (depth / bq->blocksize)) {
+        return no("scale count != channels x blocks");
+      }
+      return FcKind::kInt4Blockwise;
+    }
+    return no("float activations with this filter type are left to the CPU kernels");
+  }
+  return no("tensor type combination not handled");
+}
+
+// ---- device memory ---------------------------------------------------------------
+
+class DeviceBuffer {
+ public:
+  DeviceBuffer() = default;
+  DeviceBuffer(const DeviceBuffer&) = delete;
+  DeviceBuffer& operator=(const DeviceBuffer&) = delete;
+  DeviceBuffer(DeviceBuffer&& o) noexcept : ptr_(o.ptr_), bytes_(o.bytes_) {
+    o.ptr_ = nullptr;
+    o.bytes_ = 0;
+  }
+  ~DeviceBuffer() { Release(); }
+  void Release() {
+    if (ptr_) (void)hipFree(ptr_);
+    ptr_ = nullptr;
+    bytes_ = 0;
+  }
+  hipError_t Ensure(size_t bytes) {
+    if (bytes <= bytes_) return hipSuccess;
+    Release();
+    hipError_t err = hipMalloc(&ptr_, bytes);
+    if (err == hipSuccess) bytes_ = bytes;
+    return err;
+  }
+  hipError_t Upload(const void* host, size_t bytes, hipStream_t stream) {
+    hipError_t err = Ensure(bytes);
+    if (err != hipSuccess || bytes == 0) return err;
+    return hipMemcpyAsync(ptr_, host, bytes, hipMemcpyHostToDevice, stream);
+  }
+  template <typename T>
+  T* as() const {
+    return static_cast<T*>(ptr_);
+  }
+  void* get() const { return ptr_; }
+  size_t bytes() const { return bytes_; }
+
+ private:
+  void* ptr_ = nullptr;
+  size_t bytes_ = 0;
+};
+
+struct FcNode {
+  int node_index = -1;
+  FcKind kind = FcKind::kNone;
+  int input = -1, filter = -1, bias = -1, output = -1, scales = -1;
+  TfLiteFullyConnectedParams params{};
+  int batches = 0, depth = 0, out_depth = 0, blocksize = 0;
+  bool per_channel = false;
+  float filter_scale = 1.0f;
+  int32_t input_offset = 0, filter_offset = 0, output_offset = 0, act_min = 0, act_max = 0;
+  const void* uploaded_filter = nullptr;  // host pointer the device copy was made from
+  DeviceBuffer filter_dev, bias_dev, mult_dev, shift_dev, row_sums_dev, pcs_dev, scales_dev,
+      kfsum_dev;
+};
+
+struct PartitionKernel {
+  DelegateState* state = nullptr;
+  std::vector<FcNode> nodes;
+  std::map<int, DeviceBuffer> activations;  // tensor index -> device copy
+  std::vector<int> uploads;                 // activation tensors read from the host each invoke
+  std::vector<int> downloads;               // tensors written back to the host each invoke
+  DeviceBuffer workspace;
+  hipStream_t stream = nullptr;
+  ~PartitionKernel() {
+    if (stream) (void)hipStreamDestroy(stream);
+  }
+};
+
+#define RETURN_IF_HIP(ctx, expr)                                                          \
+  do {                                                                                    \
+    const hipError_t e__ = (expr);                                                        \
+    if (e__ != hipSuccess) {                                                              \
+      (ctx)->ReportError((ctx), "litert_amd delegate: %s failed: %s", #expr,             \
+                         hipGetErrorString(e__));                                         \
+      return kTfLiteError;                                                                \
+    }                                                                                     \
+  } while (0)
+
+#define RETURN_IF_FC(ctx, expr)                                                           \
+  do {                                                                                    \
+    const int rc__ = (expr);                                                              \
+    if (rc__ != LRTFC_OK) {                                                               \
+      (ctx)->ReportError((ctx), "litert_amd delegate: %s", lrtfc_last_error());          \
+      return kTfLiteError;                                                                \
+    }                                                                                     \
+  } while (0)
+
+// ---- kernel registration callbacks -----------------------------------------------------
+
+void* KernelInit(TfLiteContext* ctx, const char* buffer, size_t /*length*/) {
+  const auto* params = reinterpret_cast<const TfLiteDelegateParams*>(buffer);
+  if (!params || !params->delegate || !params->nodes_to_replace) return reinterpret_cast<void*>(-1);
+  auto* state = static_cast<DelegateState*>(params->delegate->data_);
+  auto kernel = std::make_unique<PartitionKernel>();
+  kernel->state = state;
+  if (hipSetDevice(state->options.device) != hipSuccess ||
+      hipStreamCreate(&kernel->stream) != hipSuccess) {
+    ctx->ReportError(ctx, "litert_amd delegate: cannot create a HIP stream on device %d",
+                     state->options.device);
+    return reinterpret_cast<void*>(-1);  // TfLiteKernelInitFailed(), tflite/core/c/common.cc:867
+  }
+  std::map<int, bool> produced;
+  for (int i = 0; i < params->nodes_to_replace->size; ++i) {
+    const int node_index = params->nodes_to_replace->data[i];
+    TfLiteNode* node = nullptr;
+    TfLiteRegistration* reg = nullptr;
+    if (ctx->GetNodeAndRegistration(ctx, node_index, &node, &reg) != kTfLiteOk) {
+      return reinterpret_cast<void*>(-1);
+    }
+    std::string why;
+    const FcKind kind = Classify(ctx, node, reg, state->options, &why);
+    if (kind == FcKind::kNone) {
+      ctx->ReportError(ctx, "litert_amd delegate: node %d handed to the kernel is unsupported: %s",
+                       node_index, why.c_str());
+      return reinterpret_cast<void*>(-1);
+    }
+    FcNode n;
+    n.node_index = node_index;
+    n.kind = kind;
+    n.input = node->inputs->data[0];
+    n.filter = node->inputs->data[1];
+    n.bias = (node->inputs->size == 3) ? node->inputs->data[2] : kTfLiteOptionalTensor;
+    n.output = node->outputs->data[0];
+    n.params = *static_cast<const TfLiteFullyConnectedParams*>(node->builtin_data);
+    if (!produced.count(n.input)) {
+      bool listed = false;
+      for (int t : kernel->uploads) listed = listed || (t == n.input);
+      if (!listed) kernel->uploads.push_back(n.input);
+    }
+    produced[n.output] = true;
+    kernel->nodes.push_back(std::move(n));
+  }
+  // Every tensor the runtime lists as an output of the partition goes back to the host.
+  for (int i = 0; i < params->output_tensors->size; ++i) {
+    kernel->downloads.push_back(params->output_tensors->data[i]);
+  }
+  return kernel.release();
+}
+
+void KernelFree(TfLiteContext* /*ctx*/, void* buffer) {
+  if (buffer && buffer != reinterpret_cast<void*>(-1)) delete static_cast<PartitionKernel*>(buffer);
+}
+
+TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
+  const TfLiteTensor& input = ctx->tensors[n->input];
+  const TfLiteTensor& filter = ctx->tensors[n->filter];
+  const TfLiteTensor* bias = n->bias == kTfLiteOptionalTensor ? nullptr : &ctx->tensors[n->bias];
+  const TfLiteTensor& output = ctx->tensors[n->output];
+  n->out_depth = filter.dims->data[0];
+  n->depth = filter.dims->data[1];
+  const int64_t in_elems = NumElements(input.dims);
+  n->batches = n->depth > 0 ? static_cast<int>(in_elems / n->depth) : 0;
+  if (n->depth > 0 && static_cast<int64_t>(n->batches) * n->depth != in_elems) {
+    ctx->ReportError(ctx, "litert_amd delegate: node %d input size %lld is not a multiple of depth %d",
+                     n->node_index, static_cast<long long>(in_elems), n->depth);
+    return kTfLiteError;
+  }
+  if (n->depth > 0 && NumElements(output.dims) != static_cast<int64_t>(n->batches) * n->out_depth) {
+    ctx->ReportError(ctx, "litert_amd delegate: node %d output shape does not hold %d x %d values",
+                     n->node_index, n->batches, n->out_depth);
+    return kTfLiteError;
+  }
+  hipStream_t s = k->stream;
+  const bool reupload = n->uploaded_filter != filter.data.raw;
+  const size_t weights = static_cast<size_t>(n->out_depth) * n->depth;
+
+  if (n->kind == FcKind::kInt8) {
+    const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
+    n->per_channel = fq->scale->size > 1;
+    n->input_offset = -input.params.zero_point;
+    n->filter_offset = n->per_channel ? 0 : -filter.params.zero_point;
+    n->output_offset = output.params.zero_point;
+    std::vector<int32_t> mult(n->per_channel ? n->out_depth : 1), shift(mult.size());
+    if (n->per_channel) {
+      RETURN_IF_FC(ctx, lrtfc_prepare_per_channel(input.params.scale, fq->scale->data,
+                                                  n->out_depth, output.params.scale, mult.data(),
+                                                  shift.data()));
+    } else {
+      // GetQuantizedConvolutionMultipler reads the per-tensor params.scale fields.
+      RETURN_IF_FC(ctx, lrtfc_prepare_per_tensor(input.params.scale, filter.params.scale,
+                                                 bias != nullptr, bias ? bias->params.scale : 0.0f,
+                                                 output.params.scale, &mult[0], &shift[0]));
+    }
+    RETURN_IF_FC(ctx, lrtfc_activation_range_int8(n->params.activation, output.params.scale,
+                                                  output.params.zero_point, &n->act_min,
+                                                  &n->act_max));
+    RETURN_IF_HIP(ctx, n->mult_dev.Upload(mult.data(), mult.size() * 4, s));
+    RETURN_IF_HIP(ctx, n->shift_dev.Upload(shift.data(), shift.size() * 4, s));
+    RETURN_IF_HIP(ctx, hipStreamSynchronize(s));  // mult/shift are stack-owned
+    if (reupload && weights > 0) {
+      if (filter.type == kTfLiteInt4) {
+        // Unpacked once here; the builtin unpacks on every Eval (fully_connected.cc:1670-1677).
+        DeviceBuffer packed;
+        RETURN_IF_HIP(ctx, packed.Upload(filter.data.raw, (weights + 1) / 2, s));
+        RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
+        RETURN_IF_FC(ctx, lrtfc_unpack_int4(packed.as<uint8_t>(), static_cast<int64_t>(weights),
+                                            n->filter_dev.as<int8_t>(), s));
+        RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+      } else {
+        RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
+      }
+      RETURN_IF_HIP(ctx, n->row_sums_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
+      RETURN_IF_FC(ctx, lrtfc_row_sums_int8(n->filter_dev.as<int8_t>(), n->out_depth, n->depth,
+                                            n->row_sums_dev.as<int32_t>(), s));
+    }
+    if (bias) RETURN_IF_HIP(ctx, n->bias_dev.Upload(bias->data.raw, static_cast<size_t>(n->out_depth) * 4, s));
+  } else if (n->kind == FcKind::kHybrid) {
+    const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
+    n->per_channel = fq->scale->size > 1;  // VerifyPerChannelQuantization, fully_connected.cc:827
+    n->filter_scale = filter.params.scale;
+    if (reupload) {
+      RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
+      RETURN_IF_HIP(ctx, n->row_sums_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
+      RETURN_IF_FC(ctx, lrtfc_row_sums_int8(n->filter_dev.as<int8_t>(), n->out_depth, n->depth,
+                                            n->row_sums_dev.as<int32_t>(), s));
+    }
+    if (n->per_channel) {
+      RETURN_IF_HIP(ctx, n->pcs_dev.Upload(fq->scale->data, static_cast<size_t>(n->out_depth) * 4, s));
+    }
+    if (bias) RETURN_IF_HIP(ctx, n->bias_dev.Upload(bias->data.raw, static_cast<size_t>(n->out_depth) * 4, s));
+  } else {  // blockwise int4
+    const auto* bq = static_cast<const TfLiteBlockwiseQuantization*>(filter.quantization.params);
+    n->blocksize = bq->blocksize;
+    n->scales = bq->scale;
+    const TfLiteTensor& scales = ctx->tensors[bq->scale];
+    if (reupload) {
+      RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights / 2, s));
+      RETURN_IF_HIP(ctx, n->scales_dev.Upload(scales.data.raw,
+                                              static_cast<size_t>(NumElements(scales.dims)) * 2, s));
+      RETURN_IF_HIP(ctx, n->kfsum_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
+      RETURN_IF_FC(ctx, lrtfc_blockwise_int4_kfsum(n->filter_dev.as<uint8_t>(),
+                                                   n->scales_dev.as<uint16_t>(), n->out_depth,
+                                                   n->depth, n->blocksize,
+                                                   n->kfsum_dev.as<float>(), s));
+    }
+    if (bias) RETURN_IF_HIP(ctx, n->bias_dev.Upload(bias->data.raw, static_cast<size_t>(n->out_depth) * 4, s));
+  }
+  n->uploaded_filter = filter.data.raw;
+
+  // Device homes for this node's activations.
+  RETURN_IF_HIP(ctx, k->activations[n->input].Ensure(input.bytes));
+  RETURN_IF_HIP(ctx, k->activations[n->output].Ensure(output.bytes));
+  if (n->kind != FcKind::kInt8) {
+    RETURN_IF_HIP(ctx, k->workspace.Ensure(lrtfc_activation_workspace_bytes(n->batches, n->depth)));
+  }
+  return kTfLiteOk;
+}
+
+TfLiteStatus KernelPrepare(TfLiteContext* ctx, TfLiteNode* node) {
+  auto* k = static_cast<PartitionKernel*>(node->user_data);
+  RETURN_IF_HIP(ctx, hipSetDevice(k->state->options.device));
+  for (FcNode& n : k->nodes) {
+    const TfLiteStatus st = PrepareNode(ctx, k, &n);
+    if (st != kTfLiteOk) return st;
+  }
+  RETURN_IF_HIP(ctx, hipStreamSynchronize(k->stream));
+  return kTfLiteOk;
+}
+
+TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
+  auto* k = static_cast<PartitionKernel*>(node->user_data);
+  RETURN_IF_HIP(ctx, hipSetDevice(k->state->options.device));
+  hipStream_t s = k->stream;
+  // Tensor data pointers may move between invokes: read them from the context each time.
+  for (int t : k->uploads) {
+    const TfLiteTensor& tensor = ctx->tensors[t];
+    if (tensor.bytes == 0) continue;
+    RETURN_IF_HIP(ctx, hipMemcpyAsync(k->activations[t].get(), tensor.data.raw, tensor.bytes,
+                                      hipMemcpyHostToDevice, s));
+  }
+  for (FcNode& n : k->nodes) {
+    const TfLiteTensor& output = ctx->tensors[n.output];
+    if (NumElements(output.dims) == 0) continue;  // fully_connected.cc:1966-1968
+    void* out_dev = k->activations[n.output].get();
+    if (n.depth == 0) {                           // fully_connected.cc:1970-1973
+      RETURN_IF_HIP(ctx, hipMemsetAsync(out_dev, 0, output.bytes, s));
+      continue;
+    }
+    const void* in_dev = k->activations[n.input].get();
+    const bool has_bias = n.bias != kTfLiteOptionalTensor;
+    switch (n.kind) {
+      case FcKind::kInt8:
+        RETURN_IF_FC(ctx, lrtfc_fc_int8(static_cast<const int8_t*>(in_dev),
+                                        n.filter_dev.as<int8_t>(),
+                                        has_bias ? n.bias_dev.as<int32_t>() : nullptr,
+                                        n.mult_dev.as<int32_t>(), n.shift_dev.as<int32_t>(),
+                                        n.per_channel, n.row_sums_dev.as<int32_t>(),
+                                        static_cast<int8_t*>(out_dev), n.batches, n.depth,
+                                        n.out_depth, n.input_offset, n.filter_offset,
+                                        n.output_offset, n.act_min, n.act_max, s));
+        break;
+      case FcKind::kHybrid:
+        RETURN_IF_FC(ctx, lrtfc_fc_hybrid(static_cast<const float*>(in_dev),
+                                          n.filter_dev.as<int8_t>(),
+                                          n.per_channel ? n.pcs_dev.as<float>() : nullptr,
+                                          n.filter_scale, n.row_sums_dev.as<int32_t>(),
+                                          has_bias ? n.bias_dev.as<float>() : nullptr,
+                                          static_cast<float*>(out_dev), n.batches, n.depth,
+                                          n.out_depth, n.params.asymmetric_quantize_inputs,
+                                          n.params.activation, k->state->options.quant_variant,
+                                          k->workspace.get(), k->workspace.bytes(), s));
+        break;
+      case FcKind::kInt4Blockwise:
+        RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4(static_cast<const float*>(in_dev),
+                                                  n.filter_dev.as<uint8_t>(),
+                                                  n.scales_dev.as<uint16_t>(),
+                                                  n.kfsum_dev.as<float>(),
+                                                  has_bias ? n.bias_dev.as<float>() : nullptr,
+                                                  static_cast<float*>(out_dev), n.batches, n.depth,
+                                                  n.out_depth, n.blocksize,
+                                                  k->state->options.quant_variant,
+                                                  k->workspace.get(), k->workspace.bytes(), s));
+        break;
+      default:
+        return kTfLiteError;
+    }
+  }
+  for (int t : k->downloads) {
+    TfLiteTensor& tensor = ctx->tensors[t];
+    if (tensor.bytes == 0) continue;
+    auto it = k->activations.find(t);
+    if (it == k->activations.end()) continue;
+    RETURN_IF_HIP(ctx, hipMemcpyAsync(tensor.data.raw, it->second.get(), tensor.bytes,
+                                      hipMemcpyDeviceToHost, s));
+  }
+  // The runtime reads the outputs as soon as invoke returns.
+  RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+  return kTfLiteOk;
+}
+
+TfLiteRegistration KernelRegistration() {
+  TfLiteRegistration r{};
+  r.init = KernelInit;
+  r.free = KernelFree;
+  r.prepare = KernelPrepare;
+  r.invoke = KernelInvoke;
+  r.profiling_string = nullptr;
+  r.builtin_code = kTfLiteBuiltinDelegate;
+  r.custom_name = "LiteRtAmdFullyConnected";
+  r.version = 1;
+  return r;
+}
+
+// ---- TfLiteDelegate::Prepare -----------------------------------------------------------
+
+TfLiteStatus DelegatePrepare(TfLiteContext* ctx, TfLiteDelegate* delegate) {
+  auto* state = static_cast<DelegateState*>(delegate->data_);
+  TfLiteIntArray* plan = nullptr;
+  if (ctx->GetExecutionPlan(ctx, &plan) != kTfLiteOk || !plan) {
+    ctx->ReportError(ctx, "litert_amd delegate: GetExecutionPlan failed");
+    return kTfLiteDelegateError;
+  }
+  // The plan array belongs to the runtime and dies with the next call: copy what we keep.
+  std::vector<int> claimed;
+  for (int i = 0; i < plan->size; ++i) {
+    const int node_index = plan->data[i];
+    TfLiteNode* node = nullptr;
+    TfLiteRegistration* reg = nullptr;
+    if (ctx->GetNodeAndRegistration(ctx, node_index, &node, &reg) != kTfLiteOk) {
+      return kTfLiteDelegateError;
+    }
+    if (Classify(ctx, node, reg, state->options, nullptr) != FcKind::kNone) {
+      claimed.push_back(node_index);
+    }
+  }
+  auto* nodes = static_cast<TfLiteIntArray*>(
+      std::malloc(sizeof(TfLiteIntArray) + sizeof(int) * claimed.size()));
+  if (!nodes) return kTfLiteDelegateError;
+  nodes->size = static_cast<int>(claimed.size());
+  for (size_t i = 0; i < claimed.size(); ++i) nodes->data[i] = claimed[i];
+  // The node list stays ours (common.h:982-986); an empty list is a valid no-op.
+  const TfLiteStatus st =
+      ctx->ReplaceNodeSubsetsWithDelegateKernels(ctx, KernelRegistration(), nodes, delegate);
+  std::free(nodes);
+  return st;
+}
+
+bool ParseOptions(const char* const* keys, const char* const* values, size_t n, Options* opt,
+                  std::string* error) {
+  for (size_t i = 0; i < n; ++i) {
+    const std::string key = keys[i] ? keys[i] : "";
+    const std::string val = values[i] ? values[i] : "";
+    if (key == "device") {
+      opt->device = std::atoi(val.c_str());
+    } else if (key == "quant_variant") {
+      if (val == "portable") {
+        opt->quant_variant = LRTFC_QUANT_PORTABLE;
+      } else if (val == "neon_v8") {
+        opt->quant_variant = LRTFC_QUANT_NEON_V8;
+      } else if (val == "neon_legacy") {
+        opt->quant_variant = LRTFC_QUANT_NEON_LEGACY;
+      } else {
+        *error = "quant_variant must be portable, neon_v8 or neon_legacy, got '" + val + "'";
+        return false;
+      }
+    } else if (key == "claim") {
+      opt->claim_int8 = opt->claim_hybrid = opt->claim_int4_blockwise = false;
+      size_t pos = 0;
+      while (pos <= val.size()) {
+        const size_t comma = val.find(',', pos);
+        const std::string item = val.substr(pos, comma == std::string::npos ? comma : comma - pos);
+        if (item == "int8") {
+          opt->claim_int8 = true;
+        } else if (item == "hybrid") {
+          opt->claim_hybrid = true;
+        } else if (item == "int4_blockwise") {
+          opt->claim_int4_blockwise = true;
+        } else if (!item.empty()) {
+          *error = "claim accepts int8, hybrid, int4_blockwise; got '" + item + "'";
+          return false;
+        }
+        if (comma == std::string::npos) break;
+        pos = comma + 1;
+      }
+    } else {
+      *error = "unknown option '" + key + "'";
+      return false;
+    }
+  }
+  return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+TfLiteDelegate* tflite_plugin_create_delegate(const char* const* options_keys,
+                                              const char* const* options_values,
+                                              size_t num_options,
+                                              void (*report_error)(const char*)) {
+  auto fail = [&](const std::string& msg) -> TfLiteDelegate* {
+    if (report_error) report_error(("litert_amd delegate: " + msg).c_str());
+    return nullptr;
+  };
+  auto state = std::make_unique<DelegateState>();
+  std::string error;
+  if (!ParseOptions(options_keys, options_values, num_options, &state->options, &error)) {
+    return fail(error);
+  }
+  // No GPU, no delegate: the caller keeps its CPU kernels. Nothing here falls back silently.
+  if (lrtfc_init(state->options.device) != LRTFC_OK) return fail(lrtfc_last_error());
+  state->delegate = TfLiteDelegate{};
+  state->delegate.data_ = state.get();
+  state->delegate.Prepare = DelegatePrepare;
+  state->delegate.CopyFromBufferHandle = nullptr;
+  state->delegate.CopyToBufferHandle = nullptr;
+  state->delegate.FreeBufferHandle = nullptr;
+  state->delegate.flags = kTfLiteDelegateFlagsNone;  // static shapes; re-prepared after a resize
+  state->delegate.opaque_delegate_builder = nullptr;
+  return &state.release()->delegate;
+}
+
+void tflite_plugin_destroy_delegate(TfLiteDelegate* delegate) {
+  if (!delegate) return;
+  delete static_cast<DelegateState*>(delegate->data_);
+}
+
+// Test and tooling hook: the claim predicate on its own (no device needed). Returns
+// 0 = declined, 1 = int8, 2 = hybrid, 3 = int4 blockwise; `reason` (may be NULL)
+// receives why a node was declined.
+int litert_amd_classify_node(const TfLiteContext* ctx, const TfLiteNode* node,
+                             const TfLiteRegistration* registration, char* reason,
+                             size_t reason_size) {
+  std::string why;
+  const FcKind kind = Classify(ctx, node, registration, Options{}, &why);
+  if (reason && reason_size) {
+    std::snprintf(reason, reason_size, "%s", why.c_str());
+  }
+  return static_cast<int>(kind);
+}
+
+}  // extern "C"

@@ -1,0 +1,112 @@
+"""Host-side behaviour of the delegate plugin that needs no GPU: exported entry points,
+option handling, the node-claim predicate (same accept/decline decisions as the builtin
+kernel's type and shape checks), and loud failure when no gfx950 device exists."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from tests import fake_host as fhm
+from tests.fake_host import FakeHost, FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, INT16
+
+
+def test_plugin_exports_entry_points():
+    lib = C.CDLL(fhm.DELEGATE_LIB)
+    for name in ("tflite_plugin_create_delegate", "tflite_plugin_destroy_delegate",
+                 "litert_amd_classify_node"):
+        assert hasattr(lib, name)
+
+
+def _int8_node(h, B=2, K=32, N=8, per_channel=True, filter_type=INT8, in_type=INT8, out_type=INT8,
+               const_filter=True, w_zp=0, bias=True, **kw):
+    x = h.tensor(in_type, (B, K), scale=0.02, zero_point=-3)
+    h.affine(x, [0.02], [-3])
+    wbytes = N * K if filter_type != INT4 else N * K // 2
+    w = h.tensor(filter_type, (N, K), data=np.zeros(wbytes, np.int8), const=const_filter)
+    if per_channel:
+        h.affine(w, np.full(N, 0.005), np.full(N, w_zp))
+    else:
+        h.affine(w, [0.005], [w_zp])
+    b = h.tensor(INT32, (N,), data=np.zeros(N, np.int32), const=True) if bias else None
+    y = h.tensor(out_type, (B, N), scale=0.05, zero_point=5)
+    h.affine(y, [0.05], [5])
+    return h.fc(x, w, b, y, **kw)
+
+
+def test_claim_predicate_int8():
+    with FakeHost() as h:
+        assert h.classify(_int8_node(h))[0] == "int8"
+        assert h.classify(_int8_node(h, per_channel=False, w_zp=-1))[0] == "int8"
+        assert h.classify(_int8_node(h, filter_type=INT4))[0] == "int8"
+        assert h.classify(_int8_node(h, bias=False))[0] == "int8"
+        assert h.classify(_int8_node(h, bias=False, optional_bias_slot=True))[0] == "int8"
+        for act in (0, 1, 2, 3):
+            assert h.classify(_int8_node(h, activation=act))[0] == "int8"
+        # declined: left to the CPU kernels
+        assert h.classify(_int8_node(h, in_type=UINT8, out_type=UINT8, filter_type=UINT8)) == (
+            None, "tensor type combination not handled")
+        assert h.classify(_int8_node(h, in_type=INT16, out_type=INT16))[0] is None
+        assert h.classify(_int8_node(h, const_filter=False)) == (None, "filter is not a constant tensor")
+        assert h.classify(_int8_node(h, weights_format=1)) == (None, "shuffled weights format")
+        assert h.classify(_int8_node(h, w_zp=3)) == (None, "non-zero filter zero point")
+        assert h.classify(_int8_node(h, per_channel=False, filter_type=INT4, w_zp=1))[0] is None
+        assert h.classify(_int8_node(h, activation=4)) == (None, "activation not a clamp")
+        assert h.classify(_int8_node(h, version=15)) == (None, "op version newer than 14")
+        a, b = h.tensor(FLOAT32, (2, 4)), h.tensor(FLOAT32, (2, 4))
+        assert h.classify(h.other(0, a, b)) == (None, "not FULLY_CONNECTED")
+
+
+def _float_node(h, B=2, K=64, N=8, filter_type=INT8, blockwise=False, bs=32, per_channel=True,
+                scale_type=FLOAT16, **kw):
+    x = h.tensor(FLOAT32, (B, K))
+    if blockwise:
+        w = h.tensor(INT4, (N, K), data=np.zeros(N * K // 2, np.uint8), const=True)
+        s = h.tensor(scale_type, (N, K // bs), data=np.ones((N, K // bs), np.float16 if scale_type == FLOAT16 else np.float32), const=True)
+        h.blockwise(w, s, bs)
+    else:
+        nbytes = N * K if filter_type == INT8 else N * K // 2
+        w = h.tensor(filter_type, (N, K), data=np.zeros(nbytes, np.int8), const=True)
+        h.affine(w, np.full(N if per_channel else 1, 0.004))
+    y = h.tensor(FLOAT32, (B, N))
+    return h.fc(x, w, None, y, **kw)
+
+
+def test_claim_predicate_float_activations():
+    with FakeHost() as h:
+        assert h.classify(_float_node(h))[0] == "hybrid"
+        assert h.classify(_float_node(h, per_channel=False, asymmetric=False))[0] == "hybrid"
+        assert h.classify(_float_node(h, activation=3))[0] == "hybrid"
+        assert h.classify(_float_node(h, activation=6)) == (None, "activation not a clamp")
+        assert h.classify(_float_node(h, blockwise=True))[0] == "int4_blockwise"
+        assert h.classify(_float_node(h, blockwise=True, K=128, bs=64))[0] == "int4_blockwise"
+        # the builtin's 4-bit gate: N >= 4, K >= 32, K even, blocksize | K
+        assert h.classify(_float_node(h, blockwise=True, N=2)) == (None, "shape outside 4-bit gate")
+        assert h.classify(_float_node(h, blockwise=True, K=16, bs=16)) == (None, "shape outside 4-bit gate")
+        assert h.classify(_float_node(h, blockwise=True, K=96, bs=64)) == (None, "bad blocksize")
+        assert h.classify(_float_node(h, blockwise=True, scale_type=FLOAT32)) == (None, "scales not const fp16")
+        # per-channel int4 hybrid (EvalHybridDense4Bit) is a different algorithm: declined
+        assert h.classify(_float_node(h, filter_type=INT4))[0] is None
+
+
+def test_bad_options_are_rejected_before_touching_the_device():
+    with FakeHost() as h:
+        assert h.load_delegate({"no_such_option": "1"}) == 1
+        assert "unknown option 'no_such_option'" in h.errors()
+    with FakeHost() as h:
+        assert h.load_delegate({"quant_variant": "fast"}) == 1
+        assert "quant_variant must be" in h.errors()
+    with FakeHost() as h:
+        assert h.load_delegate({"claim": "int8,float"}) == 1
+        assert "claim accepts" in h.errors()
+
+
+def test_no_gpu_means_no_delegate():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    with FakeHost() as h:
+        _int8_node(h)
+        assert h.load_delegate() == 1  # create_delegate returned NULL
+        assert "HIP device" in h.errors()
+        # the graph is untouched: every node still belongs to the CPU
+        assert [kind for kind, _, _ in h.plan()] == ["cpu"]

@@ -1,0 +1,239 @@
+"""The delegate plugin end to end on the GPU, driven by the fake TFLite host exactly as
+the interpreter drives an external delegate: Prepare -> ReplaceNodeSubsetsWithDelegateKernels
+-> init -> prepare -> invoke. Outputs are compared with the CPU oracle on the same
+seeded inputs: bit-exact for int8, bit-identical floats for the hybrid and blockwise paths."""
+import numpy as np
+import pytest
+
+import oracle
+from litert_amd import workloads as wl
+from tests.fake_host import (FakeHost, FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, OK,
+                             DELEGATE_ERROR)
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(autouse=True)
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a gfx950 device; none visible")
+
+
+def _add_int8_fc(h, c, x=None, activation=0, bias=True, out_scale=None, out_zp=None):
+    B, K = c["x"].shape
+    N = c["w"].shape[0]
+    if x is None:
+        x = h.tensor(INT8, (B, K), data=c["x"])
+        h.affine(x, [c["in_scale"]], [c["in_zp"]])
+    w = h.tensor(INT8, (N, K), data=c["w"], const=True)
+    h.affine(w, c["w_scale"])
+    b = h.tensor(INT32, (N,), data=c["bias"], const=True) if bias else None
+    y = h.tensor(INT8, (B, N))
+    h.affine(y, [c["out_scale"] if out_scale is None else out_scale],
+             [c["out_zp"] if out_zp is None else out_zp])
+    return h.fc(x, w, b, y, activation=activation), x, y
+
+
+def _oracle_int8(c, x, activation=0, bias=True, in_scale=None, in_zp=None):
+    in_scale = float(c["in_scale"]) if in_scale is None else in_scale
+    in_zp = c["in_zp"] if in_zp is None else in_zp
+    mult, shift = oracle.fc_prepare_per_channel(in_scale, c["w_scale"], float(c["out_scale"]))
+    lo, hi = oracle.activation_range_int8(activation, float(c["out_scale"]), c["out_zp"])
+    return oracle.fc_int8_per_channel(x, c["w"], c["bias"] if bias else None, mult, shift, -in_zp,
+                                      c["out_zp"], lo, hi)
+
+
+def test_int8_node_config1_through_delegate():
+    c = wl.int8_fc()
+    with FakeHost() as h:
+        node, x, y = _add_int8_fc(h, c)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK, h.errors()
+        assert h.plan()[0][:2] == ("delegate", [node])
+        assert h.allocate_tensors() == OK, h.errors()
+        assert h.invoke() == OK, h.errors()
+        assert np.array_equal(h.read(y), _oracle_int8(c, c["x"]))
+        # the arena may hand out new addresses between invokes
+        h.write(x, np.roll(c["x"], 7, axis=1))
+        h.move(x)
+        h.move(y)
+        assert h.invoke() == OK, h.errors()
+        assert np.array_equal(h.read(y), _oracle_int8(c, np.roll(c["x"], 7, axis=1)))
+
+
+@pytest.mark.parametrize("B", [1, 4])
+def test_hybrid_node_through_delegate(B):
+    c = wl.hybrid_fc(B, 4096, 1024)
+    bias = np.random.default_rng(1).standard_normal(1024).astype(np.float32)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (B, 4096), data=c["x"])
+        w = h.tensor(INT8, (1024, 4096), data=c["w"], const=True)
+        h.affine(w, c["pcs"])
+        b = h.tensor(FLOAT32, (1024,), data=bias, const=True)
+        y = h.tensor(FLOAT32, (B, 1024))
+        h.fc(x, w, b, y, activation=1, asymmetric=True)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.invoke() == OK, h.errors()
+        want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"], 1.0, bias, True, oracle.ACT_RELU)
+        assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+
+
+def test_blockwise_int4_node_through_delegate():
+    c = wl.blockwise_int4_fc(2, 2048, 512, lo=-8, hi=7)
+    bias = np.random.default_rng(2).standard_normal(512).astype(np.float32)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (2, 2048), data=c["x"])
+        w = h.tensor(INT4, (512, 2048), data=c["packed"], const=True)
+        s = h.tensor(FLOAT16, (512, 64), data=c["scales"], const=True)
+        h.blockwise(w, s, 32)
+        b = h.tensor(FLOAT32, (512,), data=bias, const=True)
+        y = h.tensor(FLOAT32, (2, 512))
+        h.fc(x, w, b, y, activation=1)  # the reference ignores the fused activation on this path
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.invoke() == OK, h.errors()
+        want = oracle.fc_blockwise_int4(c["x"], c["packed"], 512, c["scales"].view(np.uint16), 32, bias)
+        assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+        assert (want < 0).any()  # so an applied RELU would have shown
+
+
+def test_chain_stays_on_device_and_splits_around_cpu_nodes():
+    """FC -> FC -> (other op) -> FC: the first two share one partition (their link never
+    goes back to the host), the third sits in its own after the CPU node."""
+    c1 = wl.int8_fc(3, 256, 128, seed=1)
+    c2 = wl.int8_fc(3, 128, 64, in_scale=float(c1["out_scale"]), in_zp=c1["out_zp"], seed=2)
+    c3 = wl.int8_fc(3, 64, 32, in_scale=float(c2["out_scale"]), in_zp=c2["out_zp"], seed=3)
+    with FakeHost() as h:
+        n1, x, y1 = _add_int8_fc(h, c1, activation=3)
+        n2, _, y2 = _add_int8_fc(h, c2, x=y1)
+        mid = h.tensor(INT8, (3, 64))
+        h.affine(mid, [c2["out_scale"]], [c2["out_zp"]])
+        other = h.other(0, y2, mid)  # builtin ADD: not ours
+        n3, _, y3 = _add_int8_fc(h, c3, x=mid, bias=False)
+        ran_on_cpu = []
+
+        def cpu(node):
+            ran_on_cpu.append(node)
+            h.write(mid, h.read(y2))  # identity stand-in for the foreign op
+            return 0
+        from tests.fake_host import CPU_CB
+        cb = CPU_CB(cpu)
+        h.L.fh_set_cpu_callback(h.h, cb)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK, h.errors()
+        plan = h.plan()
+        assert [(k, r) for k, r, _ in plan] == [("delegate", [n1, n2]), ("cpu", [other]), ("delegate", [n3])]
+        ins, outs = h.node_io(plan[0][2])
+        assert outs == [y2] and x in ins and y1 not in ins and y1 not in outs
+        assert h.L.fh_tensor_has_delegate(h.h, y2) and not h.L.fh_tensor_has_delegate(h.h, y1)
+        assert h.allocate_tensors() == OK and h.invoke() == OK, h.errors()
+        w1 = _oracle_int8(c1, c1["x"], activation=3)
+        w2 = _oracle_int8(c2, w1)
+        w3 = _oracle_int8(c3, w2, bias=False)
+        assert ran_on_cpu == [other]
+        assert np.array_equal(h.read(y2), w2) and np.array_equal(h.read(y3), w3)
+
+
+def test_shared_input_and_unclaimed_node_fall_back_to_cpu():
+    """q/k/v-style fan-out from one input, plus a uint8 FC the delegate must leave alone."""
+    c = wl.hybrid_fc(2, 512, 96, seed=9)
+    rng = np.random.default_rng(3)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (2, 512), data=c["x"])
+        outs = []
+        for i in range(3):
+            w = h.tensor(INT8, (32, 512), data=c["w"][32 * i:32 * i + 32], const=True)
+            h.affine(w, c["pcs"][32 * i:32 * i + 32])
+            y = h.tensor(FLOAT32, (2, 32))
+            h.fc(x, w, None, y, asymmetric=(i != 1))
+            outs.append(y)
+        xu = h.tensor(UINT8, (2, 16), data=rng.integers(0, 255, (2, 16)).astype(np.uint8))
+        wu = h.tensor(UINT8, (4, 16), data=rng.integers(0, 255, (4, 16)).astype(np.uint8), const=True)
+        h.affine(wu, [0.01], [128])
+        yu = h.tensor(UINT8, (2, 4))
+        nu = h.fc(xu, wu, None, yu)
+        ran = []
+        from tests.fake_host import CPU_CB
+        cb = CPU_CB(lambda n: (ran.append(n), 0)[1])
+        h.L.fh_set_cpu_callback(h.h, cb)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert [k for k, _, _ in h.plan()] == ["delegate", "cpu"]
+        assert h.invoke() == OK, h.errors()
+        assert ran == [nu]
+        for i, y in enumerate(outs):
+            want = oracle.fc_hybrid(c["x"], c["w"][32 * i:32 * i + 32], c["pcs"][32 * i:32 * i + 32],
+                                    asymmetric=(i != 1))
+            assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+
+
+def test_claim_option_and_quant_variant_option():
+    c = wl.int8_fc(2, 64, 16, seed=4)
+    ch = wl.hybrid_fc(1, 72, 8, seed=5)  # 72 = 8 * 9: no ragged tail, ties still differ by variant
+    ch["x"][0, :4] = [-125.0, 130.0, 2.5, 0.0]  # scale 1, zero point -3, one exact tie
+    ch["x"][0, 4:] = np.clip(ch["x"][0, 4:], -100, 100)
+    with FakeHost() as h:
+        n_int8, _, _ = _add_int8_fc(h, c)
+        x = h.tensor(FLOAT32, (1, 72), data=ch["x"])
+        w = h.tensor(INT8, (8, 72), data=ch["w"], const=True)
+        h.affine(w, ch["pcs"])
+        y = h.tensor(FLOAT32, (1, 8))
+        n_h = h.fc(x, w, None, y)
+        ran = h.use_oracle_for_cpu_nodes()
+        assert h.load_delegate({"claim": "hybrid", "quant_variant": "neon_v8"}) == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert [(k, r) for k, r, _ in h.plan()] == [("cpu", [n_int8]), ("delegate", [n_h])]
+        assert h.invoke() == OK, h.errors()
+        assert ran == [n_int8]
+        want_v8 = oracle.fc_hybrid(ch["x"], ch["w"], ch["pcs"], variant=oracle.QUANT_NEON_V8)
+        want_p = oracle.fc_hybrid(ch["x"], ch["w"], ch["pcs"], variant=oracle.QUANT_PORTABLE)
+        got = h.read(y)
+        assert np.array_equal(got.view(np.uint32), want_v8.view(np.uint32))
+        assert not np.array_equal(want_v8, want_p)  # the option is observable
+
+
+def test_resize_then_reprepare():
+    c = wl.hybrid_fc(4, 256, 64, seed=6)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (1, 256), data=c["x"][:1])
+        w = h.tensor(INT8, (64, 256), data=c["w"], const=True)
+        h.affine(w, c["pcs"])
+        y = h.tensor(FLOAT32, (1, 64))
+        h.fc(x, w, None, y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.invoke() == OK
+        assert np.array_equal(h.read(y), oracle.fc_hybrid(c["x"][:1], c["w"], c["pcs"]))
+        h.resize(x, (4, 256))
+        h.resize(y, (4, 64))
+        h.write(x, c["x"])
+        assert h.allocate_tensors() == OK, h.errors()  # prepare runs again after a resize
+        assert h.invoke() == OK, h.errors()
+        assert np.array_equal(h.read(y), oracle.fc_hybrid(c["x"], c["w"], c["pcs"]))
+
+
+def test_prepare_failure_is_reported_not_hidden():
+    """An output tensor whose shape cannot hold batches x channels makes the delegate
+    kernel's prepare fail with a message, like a builtin kernel's Prepare would."""
+    c = wl.hybrid_fc(2, 64, 8, seed=7)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (2, 64), data=c["x"])
+        w = h.tensor(INT8, (8, 64), data=c["w"], const=True)
+        h.affine(w, c["pcs"])
+        y = h.tensor(FLOAT32, (2, 7))
+        h.fc(x, w, None, y)
+        assert h.load_delegate() == 0
+        assert h.modify_graph_with_delegate() == OK
+        assert h.allocate_tensors() != OK
+        assert "output shape does not hold" in h.errors()
+
+
+def test_empty_graph_and_nothing_to_claim():
+    with FakeHost() as h:
+        a, b = h.tensor(FLOAT32, (1, 4)), h.tensor(FLOAT32, (1, 4))
+        h.other(0, a, b)
+        assert h.load_delegate() == 0
+        assert h.modify_graph_with_delegate() == OK
+        assert [k for k, _, _ in h.plan()] == ["cpu"]
