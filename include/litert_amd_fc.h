@@ -105,6 +105,16 @@ int lrtfc_blockwise_int4_kfsum(const uint8_t* packed_filter, const uint16_t* sca
                                int out_depth, int depth, int blocksize, float* kfsum,
                                void* stream);
 
+/* Re-tiles a row-major int8 filter [out_depth, depth] for the matrix-core GEMV: tiles of
+ * 16 output channels x 64 depth (1 KiB each, zero-padded at the edges), the 16 bytes of
+ * lane L inside a tile being channel L % 16, depth 16 * (L / 16) .. +16; tiles of one
+ * channel group are consecutive along the depth. This plays the part of the reference's
+ * prepacked-LHS cache (tflite/kernels/cpu_backend_gemm_params.h:33-42: constant weights
+ * are packed once and reused). `packed` must hold lrtfc_packed_int8_filter_bytes(). */
+size_t lrtfc_packed_int8_filter_bytes(int out_depth, int depth);
+int lrtfc_pack_int8_filter(const int8_t* filter, int out_depth, int depth, int8_t* packed,
+                           void* stream);
+
 /* ---- Eval --------------------------------------------------------------- */
 
 /* Full-integer int8 FULLY_CONNECTED with MultiplyByQuantizedMultiplier
@@ -123,6 +133,17 @@ int lrtfc_fc_int8(const int8_t* input, const int8_t* filter, const int32_t* bias
                   const int32_t* filter_row_sums, int8_t* output, int batches, int depth,
                   int out_depth, int32_t input_offset, int32_t filter_offset,
                   int32_t output_offset, int32_t act_min, int32_t act_max, void* stream);
+
+/* lrtfc_fc_int8 for decode batches on a filter packed by lrtfc_pack_int8_filter: one
+ * kernel on the int8 matrix cores whose cost does not grow with the batch up to 16 rows
+ * (larger batches run in tiles of 16). Same arithmetic contract as lrtfc_fc_int8 with
+ * filter_offset == 0; filter_row_sums (of the unpacked filter) is required when
+ * input_offset != 0. */
+int lrtfc_fc_int8_packed(const int8_t* input, const int8_t* packed_filter, const int32_t* bias,
+                         const int32_t* multipliers, const int32_t* shifts, int per_channel,
+                         const int32_t* filter_row_sums, int8_t* output, int batches, int depth,
+                         int out_depth, int32_t input_offset, int32_t output_offset,
+                         int32_t act_min, int32_t act_max, void* stream);
 
 /* Per-row activation quantization. Replaces tensor_utils::BatchQuantizeFloats,
  * tflite/kernels/internal/portable_tensor_utils.h:158-176. zero_points may be
@@ -158,6 +179,16 @@ int lrtfc_fc_hybrid(const float* input, const int8_t* filter, const float* per_c
                     float* output, int batches, int depth, int out_depth,
                     int asymmetric_quantize_inputs, int activation, int quant_variant,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* EvalHybridDense as ONE kernel on a packed filter: each workgroup quantizes the float
+ * rows itself (BatchQuantizeFloats semantics, same three variants) while its weight loads
+ * are in flight, so no workspace and no separate quantization launch are needed. Results
+ * are bit-identical to lrtfc_fc_hybrid. */
+int lrtfc_fc_hybrid_packed(const float* input, const int8_t* packed_filter,
+                           const float* per_channel_scales, float filter_scale,
+                           const int32_t* filter_row_sums, const float* bias, float* output,
+                           int batches, int depth, int out_depth, int asymmetric_quantize_inputs,
+                           int activation, int quant_variant, void* stream);
 
 /* Blockwise-int4 hybrid FULLY_CONNECTED. Replaces EvalBlockwise4Bit,
  * tflite/kernels/fully_connected.cc:1014-1086: asymmetric per-row activation

@@ -13,7 +13,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
-LIB = os.path.join(HERE, "lib")
+LIB = os.environ.get("LITERT_AMD_LIB_DIR", os.path.join(HERE, "lib"))
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 # -ffp-contract=off: several float steps reproduce the reference's unfused
@@ -21,9 +21,10 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall",
           "-Wno-unused-function", "-I" + os.path.join(ROOT, "include")]
+COMMON += os.environ.get("LITERT_AMD_EXTRA_HIPCC_FLAGS", "").split()
 
-FC_SOURCES = ["capi.hip", "quantize.hip", "fc_int8_gemv.hip", "fc_int8_gemm_mfma.hip",
-              "fc_int4_blockwise.hip"]
+FC_SOURCES = ["capi.hip", "quantize.hip", "fc_int8_gemv.hip", "fc_int8_packed_gemv.hip",
+              "fc_int8_gemm_mfma.hip", "fc_int4_blockwise.hip"]
 
 
 def _run(cmd):

@@ -288,6 +288,91 @@ int lrtfc_fc_int8(const int8_t* input, const int8_t* filter, const int32_t* bias
       "int8 GEMV");
 }
 
+size_t lrtfc_packed_int8_filter_bytes(int out_depth, int depth) {
+  if (out_depth <= 0 || depth <= 0) return 0;
+  return lrtfc::PackedInt8FilterBytes(out_depth, depth);
+}
+
+int lrtfc_pack_int8_filter(const int8_t* filter, int out_depth, int depth, int8_t* packed,
+                           void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(out_depth >= 0 && depth >= 0, "negative dimension");
+  if (out_depth == 0 || depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(filter && packed, "null pointer");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(packed) & 15) == 0, "packed must be 16-byte aligned");
+  return FromHip(lrtfc::LaunchPackInt8Filter(filter, out_depth, depth, packed, AsStream(stream)),
+                 "pack int8 filter");
+}
+
+int lrtfc_fc_int8_packed(const int8_t* input, const int8_t* packed_filter, const int32_t* bias,
+                         const int32_t* multipliers, const int32_t* shifts, int per_channel,
+                         const int32_t* filter_row_sums, int8_t* output, int batches, int depth,
+                         int out_depth, int32_t input_offset, int32_t output_offset,
+                         int32_t act_min, int32_t act_max, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(input && packed_filter && multipliers && shifts && output, "null pointer");
+  LRTFC_REQUIRE(act_min <= act_max, "activation range is empty");
+  LRTFC_REQUIRE(input_offset == 0 || filter_row_sums,
+                "filter_row_sums is required when input_offset != 0");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(packed_filter) & 15) == 0,
+                "packed filter must be 16-byte aligned");
+  lrtfc::FcInt8Args a{};
+  a.input = input;
+  a.filter = packed_filter;
+  a.batches = batches;
+  a.depth = depth;
+  a.out_depth = out_depth;
+  a.filter_row_sums = filter_row_sums;
+  a.bias_i32 = bias;
+  a.multipliers = multipliers;
+  a.shifts = shifts;
+  a.per_channel = per_channel;
+  a.input_offset = input_offset;
+  a.output_offset = output_offset;
+  a.act_min = act_min;
+  a.act_max = act_max;
+  a.output_i8 = output;
+  return FromHip(lrtfc::LaunchFcInt8PackedGemv(a, lrtfc::Int8Epilogue::kRequantize, nullptr, 0, 0,
+                                               AsStream(stream)),
+                 "packed int8 GEMV");
+}
+
+int lrtfc_fc_hybrid_packed(const float* input, const int8_t* packed_filter,
+                           const float* per_channel_scales, float filter_scale,
+                           const int32_t* filter_row_sums, const float* bias, float* output,
+                           int batches, int depth, int out_depth, int asymmetric_quantize_inputs,
+                           int activation, int quant_variant, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(input && packed_filter && output, "null pointer");
+  LRTFC_REQUIRE(!asymmetric_quantize_inputs || filter_row_sums,
+                "filter_row_sums is required for asymmetric activation quantization");
+  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  LRTFC_REQUIRE(quant_variant >= 0 && quant_variant <= LRTFC_QUANT_NEON_LEGACY,
+                "unknown quantizer variant");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(packed_filter) & 15) == 0,
+                "packed filter must be 16-byte aligned");
+  lrtfc::FcInt8Args a{};
+  a.filter = packed_filter;
+  a.batches = batches;
+  a.depth = depth;
+  a.out_depth = out_depth;
+  a.filter_row_sums = filter_row_sums;
+  a.per_channel_scales = per_channel_scales;
+  a.filter_scale = filter_scale;
+  a.bias_f32 = bias;
+  a.activation = activation;
+  a.output_f32 = output;
+  return FromHip(lrtfc::LaunchFcInt8PackedGemv(a, lrtfc::Int8Epilogue::kHybrid, input,
+                                               asymmetric_quantize_inputs, quant_variant,
+                                               AsStream(stream)),
+                 "packed hybrid GEMV");
+}
+
 int lrtfc_batch_quantize_floats(const float* values, int n_batch, int n_data, int8_t* quantized,
                                 float* scaling_factors, int32_t* zero_points, int do_asymmetric,
                                 int variant, void* stream) {

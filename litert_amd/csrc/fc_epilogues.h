@@ -1,0 +1,58 @@
+// Output epilogues shared by the int8-weight kernels. Integer accumulators are exact, so
+// these few lines are where bit-exactness with the reference is decided.
+#ifndef LITERT_AMD_CSRC_FC_EPILOGUES_H_
+#define LITERT_AMD_CSRC_FC_EPILOGUES_H_
+
+#include "kernels.h"
+
+namespace lrtfc {
+
+// Requantization of one accumulator: reference/integer_ops/fully_connected.h:65-74.
+// `acc` already holds every additive term (dot product, offset corrections, bias).
+__device__ __forceinline__ int8_t RequantizeCore(int32_t acc, int32_t multiplier, int shift,
+                                                 int32_t output_offset, int32_t act_min,
+                                                 int32_t act_max) {
+  const int32_t v = Mbqm(acc, multiplier, shift) + output_offset;
+  return static_cast<int8_t>(ClampI32(v, act_min, act_max));
+}
+
+// Hybrid output value: reference/portable_tensor_utils.cc:186-203 after the bias
+// initialisation of fully_connected.cc:780-786, then ApplyActivationToVector.
+// channel_scale is the per-channel scale, or the per-tensor filter scale.
+__device__ __forceinline__ float HybridCore(int32_t dot, float batch_scale, float channel_scale,
+                                            int32_t batch_zero_point, int32_t row_sum, float base,
+                                            int activation) {
+  const float scale = __fmul_rn(batch_scale, channel_scale);
+  dot -= row_sum * batch_zero_point;
+  const float out = __fadd_rn(base, __fmul_rn(static_cast<float>(dot), scale));
+  return ApplyFloatActivation(out, activation);
+}
+
+// Pointer forms used by the row-major kernels.
+__device__ __forceinline__ void StoreRequantized(const FcInt8Args& a, int b, int n, int32_t dot,
+                                                 int32_t xsum) {
+  // sum (w + fo)(x + io) = dot + io * sum(w) + fo * sum(x) + depth * fo * io
+  int32_t acc = dot;
+  if (a.input_offset != 0) acc += a.input_offset * a.filter_row_sums[n];
+  if (a.filter_offset != 0) {
+    acc += a.filter_offset * xsum + a.depth * a.filter_offset * a.input_offset;
+  }
+  if (a.bias_i32) acc += a.bias_i32[n];
+  const int32_t m = a.per_channel ? a.multipliers[n] : a.multipliers[0];
+  const int s = a.per_channel ? a.shifts[n] : a.shifts[0];
+  a.output_i8[static_cast<size_t>(b) * a.out_depth + n] =
+      RequantizeCore(acc, m, s, a.output_offset, a.act_min, a.act_max);
+}
+
+__device__ __forceinline__ void StoreHybrid(const FcInt8Args& a, int b, int n, int32_t dot,
+                                            float batch_scale, int32_t batch_zero_point) {
+  const float channel_scale = a.per_channel_scales ? a.per_channel_scales[n] : a.filter_scale;
+  const int32_t row_sum = batch_zero_point != 0 ? a.filter_row_sums[n] : 0;
+  const float base = a.bias_f32 ? a.bias_f32[n] : 0.0f;
+  a.output_f32[static_cast<size_t>(b) * a.out_depth + n] =
+      HybridCore(dot, batch_scale, channel_scale, batch_zero_point, row_sum, base, a.activation);
+}
+
+}  // namespace lrtfc
+
+#endif  // LITERT_AMD_CSRC_FC_EPILOGUES_H_

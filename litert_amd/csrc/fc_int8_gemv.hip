@@ -8,6 +8,7 @@
 // the depth, so a wave64 butterfly finishes each dot product. Integer sums are
 // exact, so any summation order gives the reference's accumulator; only the
 // epilogues below have an order that matters.
+#include "fc_epilogues.h"
 #include "kernels.h"
 
 namespace lrtfc {
@@ -15,39 +16,6 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWavesPerBlock = kThreads / kWaveSize;
-
-// Requantizing epilogue: reference/integer_ops/fully_connected.h:65-74 / :166-175.
-__device__ __forceinline__ void StoreRequantized(const FcInt8Args& a, int b, int n, int32_t dot,
-                                                 int32_t xsum) {
-  // sum (w + fo)(x + io) = dot + io * sum(w) + fo * sum(x) + depth * fo * io
-  int32_t acc = dot;
-  if (a.input_offset != 0) acc += a.input_offset * a.filter_row_sums[n];
-  if (a.filter_offset != 0) {
-    acc += a.filter_offset * xsum + a.depth * a.filter_offset * a.input_offset;
-  }
-  if (a.bias_i32) acc += a.bias_i32[n];
-  const int32_t m = a.per_channel ? a.multipliers[n] : a.multipliers[0];
-  const int s = a.per_channel ? a.shifts[n] : a.shifts[0];
-  int32_t v = Mbqm(acc, m, s) + a.output_offset;
-  v = ClampI32(v, a.act_min, a.act_max);
-  a.output_i8[static_cast<size_t>(b) * a.out_depth + n] = static_cast<int8_t>(v);
-}
-
-// Hybrid epilogue: reference/portable_tensor_utils.cc:186-203 after the bias
-// initialisation of fully_connected.cc:780-786, then ApplyActivationToVector.
-__device__ __forceinline__ void StoreHybrid(const FcInt8Args& a, int b, int n, int32_t dot) {
-  float scale = a.scaling_factors[b];
-  if (a.per_channel_scales) {
-    scale = __fmul_rn(scale, a.per_channel_scales[n]);
-  } else {
-    scale = __fmul_rn(scale, a.filter_scale);
-  }
-  if (a.zero_points) dot -= a.filter_row_sums[n] * a.zero_points[b];
-  const float base = a.bias_f32 ? a.bias_f32[n] : 0.0f;
-  float out = __fadd_rn(base, __fmul_rn(static_cast<float>(dot), scale));
-  out = ApplyFloatActivation(out, a.activation);
-  a.output_f32[static_cast<size_t>(b) * a.out_depth + n] = out;
-}
 
 template <int R, int BT, Int8Epilogue EPI, bool FILTER_OFFSET>
 __global__ __launch_bounds__(kThreads) void FcInt8GemvKernel(FcInt8Args a, int batch0) {
@@ -144,7 +112,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8GemvKernel(FcInt8Args a, int b
         if (EPI == Int8Epilogue::kRequantize) {
           StoreRequantized(a, b, n, mine, mine_xsum);
         } else {
-          StoreHybrid(a, b, n, mine);
+          StoreHybrid(a, b, n, mine, a.scaling_factors[b], a.zero_points ? a.zero_points[b] : 0);
         }
       }
     }
@@ -169,7 +137,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8GenericKernel(FcInt8Args a) {
   if (EPI == Int8Epilogue::kRequantize) {
     StoreRequantized(a, b, n, dot, xsum);
   } else {
-    StoreHybrid(a, b, n, dot);
+    StoreHybrid(a, b, n, dot, a.scaling_factors[b], a.zero_points ? a.zero_points[b] : 0);
   }
 }
 

@@ -1,0 +1,539 @@
+// Decode-regime FULLY_CONNECTED with int8 weights, batches 1..16, on pre-packed
+// weights and the gfx950 matrix cores.
+//
+// Why matrix cores for a GEMV: with sdot4 every extra batch row costs a full set of
+// VALU dot products and a cross-lane reduction, and the kernel turns ALU-bound at
+// batch 8. v_mfma_i32_16x16x64_i8 multiplies a 16-row x 64-deep weight tile by up to 16
+// activation columns in 16 cycles, far above the HBM rate, for any batch 1..16, and
+// its accumulator layout needs no cross-lane reduction at all.
+//
+// HBM layout ("tile16x64", built once per constant filter by PackInt8FilterKernel):
+// the filter is cut into tiles of 16 output channels x 64 depth = 1 KiB; inside a tile
+// lane L's 16 bytes are channel (L % 16), depth 16 * (L / 16) .. +16, which is the MFMA
+// A-operand register layout. Tiles of one 16-channel group are contiguous along the
+// depth, so a wavefront's load instruction reads 1 KiB of consecutive bytes and a
+// wavefront's whole share is one contiguous run.
+//
+// Each wavefront owns one 16-channel group over the whole depth and streams its
+// contiguous run through a ring of 16 outstanding 1 KiB loads, refilling a slot as soon
+// as the matrix core has consumed it; four wavefronts (four groups) form a workgroup and
+// share the staged activation rows. Short filters, which would leave most CUs without a
+// wavefront, split the depth over 2 or 4 wavefronts of the workgroup instead and add
+// their int32 partial tiles through LDS (exact: integer adds). The activation rows are
+// requested before the first weight load and staged in LDS while the ring fills. In the
+// hybrid form the staging step *is* the BatchQuantizeFloats of the op: the workgroup
+// reduces min/max of each float row, derives scale and zero point, and writes the
+// quantized row straight to LDS, so the op is a single kernel.
+#include "fc_epilogues.h"
+#include "kernels.h"
+#include "quantize_device.h"
+
+namespace lrtfc {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWaveSize;
+constexpr int kTileRows = 16;
+constexpr int kSlabDepth = 64;
+constexpr int kQPad = 16;         // bytes of padding per staged activation row (bank spread)
+
+__global__ __launch_bounds__(kThreads) void PackInt8FilterKernel(const int8_t* __restrict__ src,
+                                                                 int out_depth, int depth,
+                                                                 int slabs, int64_t chunks,
+                                                                 int8_t* __restrict__ dst) {
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (c >= chunks) return;
+  const int lane = static_cast<int>(c & 63);
+  const int64_t tile_slab = c >> 6;
+  const int slab = static_cast<int>(tile_slab % slabs);
+  const int tile = static_cast<int>(tile_slab / slabs);
+  const int row = tile * kTileRows + (lane & 15);
+  const int k0 = slab * kSlabDepth + (lane >> 4) * 16;
+  int8_t out[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    const int k = k0 + t;
+    out[t] = (row < out_depth && k < depth) ? src[static_cast<size_t>(row) * depth + k] : 0;
+  }
+  *reinterpret_cast<i32x4*>(dst + c * 16) = *reinterpret_cast<const i32x4*>(out);
+}
+
+struct PackedArgs {
+  FcInt8Args a;            // a.filter is the packed filter; a.input the int8 rows (unfused)
+  const float* input_f32;  // fused form: float rows to quantize in the prologue
+  int asymmetric;
+  int slabs;               // padded depth / 64
+};
+
+// LDS map (dynamic): [bt rows x (slabs * 64 + kQPad)] int8 activations, then the
+// cross-wave partial tiles, then per-row quantization state.
+struct Shared {
+  int8_t* q;
+  i32x4* partial;  // [kWaves][64]
+  float* sf;       // [16]
+  float* inv;      // [16]
+  int32_t* zp;     // [16]
+  int32_t* zero;   // [16]
+  float* mm;       // [16][kWaves][2]
+};
+
+__device__ __forceinline__ Shared CarveShared(int8_t* base, int bt, int qstride) {
+  Shared s;
+  s.q = base;
+  size_t off = (static_cast<size_t>(bt) * qstride + 15) & ~static_cast<size_t>(15);
+  s.partial = reinterpret_cast<i32x4*>(base + off);
+  off += kWaves * 64 * sizeof(i32x4);
+  s.sf = reinterpret_cast<float*>(base + off);
+  off += 16 * 4;
+  s.inv = reinterpret_cast<float*>(base + off);
+  off += 16 * 4;
+  s.zp = reinterpret_cast<int32_t*>(base + off);
+  off += 16 * 4;
+  s.zero = reinterpret_cast<int32_t*>(base + off);
+  off += 16 * 4;
+  s.mm = reinterpret_cast<float*>(base + off);
+  return s;
+}
+
+size_t SharedBytes(int bt, int qstride) {
+  return ((static_cast<size_t>(bt) * qstride + 15) & ~static_cast<size_t>(15)) +
+         kWaves * 64 * sizeof(i32x4) + 4 * 16 * 4 + 16 * kWaves * 2 * 4;
+}
+
+constexpr int kRing = 16;  // weight tiles in flight per wavefront
+
+// REG_ROWS: how many float rows the fused prologue may keep in registers (1, 2 or 4); a
+// smaller value frees registers. ksplit: wavefronts sharing one channel group (1, 2, 4).
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS>
+__global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p, int batch0,
+                                                                   int bt, int ksplit) {
+  extern __shared__ __align__(16) int8_t smem[];
+  const FcInt8Args& a = p.a;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWaveSize - 1);
+  const int wave = tid / kWaveSize;
+  const int col = lane & 15;     // batch column of this lane in the MFMA tiles
+  const int kgroup = lane >> 4;  // which 16 of a tile's 64 depth positions this lane holds
+  const int slabs = p.slabs;
+  const int depth = a.depth;
+  const int qstride = slabs * kSlabDepth + kQPad;
+  const Shared sh = CarveShared(smem, bt, qstride);
+  const int tiles = (a.out_depth + kTileRows - 1) / kTileRows;
+  const int tiles_per_wg = kWaves / ksplit;
+  const int tile = blockIdx.x * tiles_per_wg + wave / ksplit;  // may run past the last group
+  const int part = wave % ksplit;
+  const int per_part = (slabs + ksplit - 1) / ksplit;
+  const int s0 = part * per_part;
+  const int s1 = min(slabs, s0 + per_part);
+  const i32x4* wbase = reinterpret_cast<const i32x4*>(a.filter) +
+                       (static_cast<size_t>(min(tile, tiles - 1)) * slabs) * 64 + lane;
+
+  // Vector memory returns in issue order, so whatever the prologue needs must be requested
+  // BEFORE the weight loads: then waiting for it leaves the weight loads in flight. Small
+  // activation tiles are therefore fetched into registers first (kXRegs float4 per row per
+  // thread for up to REG_ROWS rows, or kQRegs 16-byte chunks of int8), without branches;
+  // larger ones are staged completely before the weights are requested.
+  constexpr int kXRegs = 4, kQRegs = 4;
+  const int padded = slabs * kSlabDepth;
+  const int vector_end = depth - (depth % 8);
+  float4 xr[REG_ROWS][kXRegs];
+  i32x4 qr[kQRegs];
+  bool in_regs = false;
+  if (FUSED) {
+    const bool vec_ok = (depth % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.input_f32) & 15) == 0);
+    in_regs = vec_ok && bt <= REG_ROWS && depth <= kXRegs * kThreads * 4;
+    if (in_regs) {
+#pragma unroll
+      for (int b = 0; b < REG_ROWS; ++b) {
+#pragma unroll
+        for (int j = 0; j < kXRegs; ++j) {
+          const int i = (j * kThreads + tid) * 4;
+          // Raw, clamped load; nothing may consume it before the weight loads are out.
+          xr[b][j] = *reinterpret_cast<const float4*>(
+              p.input_f32 + static_cast<size_t>(batch0 + min(b, bt - 1)) * depth +
+              min(i, depth - 4));
+        }
+      }
+    } else {
+      // Slow form: the min/max pass reads memory before any weight load.
+      for (int b = 0; b < bt; ++b) {
+        const float* x = p.input_f32 + static_cast<size_t>(batch0 + b) * depth;
+        float mn = 0.0f, mx = 0.0f;
+        if (vec_ok) {
+          for (int i = tid * 4; i < depth; i += kThreads * 4) {
+            const float4 t = *reinterpret_cast<const float4*>(x + i);
+            mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
+            mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
+          }
+        } else {
+          for (int i = tid; i < depth; i += kThreads) {
+            mn = fminf(mn, x[i]);
+            mx = fmaxf(mx, x[i]);
+          }
+        }
+        mn = WaveMinF32(mn);
+        mx = WaveMaxF32(mx);
+        if (lane == 0) {
+          sh.mm[(b * kWaves + wave) * 2] = mn;
+          sh.mm[(b * kWaves + wave) * 2 + 1] = mx;
+        }
+      }
+    }
+  } else {
+    const bool vec_ok = (depth % 16 == 0) && ((reinterpret_cast<uintptr_t>(a.input) & 15) == 0);
+    in_regs = vec_ok && bt * (padded / 16) <= kQRegs * kThreads;
+#ifdef LRT_EXP_NOQ
+    in_regs = false;
+    if (false) {
+#else
+    if (in_regs) {
+#endif
+      const int chunks_per_row = padded / 16;
+#pragma unroll
+      for (int j = 0; j < kQRegs; ++j) {
+        const int c = j * kThreads + tid;
+        const int b = c / chunks_per_row;
+        const int i = (c - b * chunks_per_row) * 16;
+        qr[j] = *reinterpret_cast<const i32x4*>(
+            a.input + static_cast<size_t>(batch0 + min(b, bt - 1)) * depth + min(i, depth - 16));
+      }
+#ifdef LRT_EXP_NOQ
+    } else if (false) {
+#else
+    } else {
+#endif
+      for (int b = 0; b < bt; ++b) {
+        const int8_t* x = a.input + static_cast<size_t>(batch0 + b) * depth;
+        int8_t* qrow = sh.q + b * qstride;
+        if (vec_ok) {
+          for (int i = tid * 16; i < padded; i += kThreads * 16) {
+            i32x4 v = {0, 0, 0, 0};
+            if (i < depth) v = *reinterpret_cast<const i32x4*>(x + i);
+            *reinterpret_cast<i32x4*>(qrow + i) = v;
+          }
+        } else {
+          for (int i = tid; i < padded; i += kThreads) qrow[i] = i < depth ? x[i] : 0;
+        }
+      }
+    }
+  }
+
+  // 1. Fill the ring (branch-free; a share shorter than the ring re-reads its last tile).
+  i32x4 ring[kRing];
+#pragma unroll
+  for (int u = 0; u < kRing; ++u) {
+    ring[u] = __builtin_nontemporal_load(wbase + static_cast<size_t>(min(s0 + u, slabs - 1)) * 64);
+  }
+
+  // Per-channel epilogue parameters of this lane's four channels: requested right behind
+  // the first ring of weights (they return in order, long before the last tile is consumed)
+  // so that no latency is left for the epilogue to wait for.
+  // Loaded raw: combining them here would wait for memory before the weights are requested.
+  int32_t ep_i0[4], ep_i1[4], ep_i2[4], ep_i3[4];  // requantize: multiplier, shift, bias, row sum
+  float ep_f0[4], ep_f1[4];                         // hybrid: channel scale, bias (+ ep_i0 row sum)
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = min(min(tile, tiles - 1) * kTileRows + 4 * kgroup + i, a.out_depth - 1);
+#ifdef LRT_EXP_NOPARAM
+    ep_i0[i] = 1 << 30; ep_i1[i] = -5; ep_i2[i] = n; ep_i3[i] = 1; ep_f0[i] = 1.f; ep_f1[i] = 0.f;
+    continue;
+#endif
+    if (EPI == Int8Epilogue::kRequantize) {
+      ep_i0[i] = a.per_channel ? a.multipliers[n] : a.multipliers[0];
+      ep_i1[i] = a.per_channel ? a.shifts[n] : a.shifts[0];
+      ep_i2[i] = a.bias_i32 ? a.bias_i32[n] : 0;
+      ep_i3[i] = a.input_offset != 0 ? a.filter_row_sums[n] : 0;
+    } else {
+      ep_i0[i] = a.filter_row_sums ? a.filter_row_sums[n] : 0;
+      ep_f0[i] = a.per_channel_scales ? a.per_channel_scales[n] : a.filter_scale;
+      ep_f1[i] = a.bias_f32 ? a.bias_f32[n] : 0.0f;
+    }
+  }
+
+  // 2. Activation rows into LDS, zero-padded to the slab grid. In the fused form this is
+  // the op's BatchQuantizeFloats.
+  if (FUSED) {
+    if (in_regs) {
+#pragma unroll
+      for (int b = 0; b < REG_ROWS; ++b) {
+        if (b < bt) {
+          float mn = 0.0f, mx = 0.0f;
+#pragma unroll
+          for (int j = 0; j < kXRegs; ++j) {
+            // lanes past the row hold a clamped duplicate of real elements: harmless for min/max
+            const float4 t = xr[b][j];
+            mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
+            mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
+          }
+          mn = WaveMinF32(mn);
+          mx = WaveMaxF32(mx);
+          if (lane == 0) {
+            sh.mm[(b * kWaves + wave) * 2] = mn;
+            sh.mm[(b * kWaves + wave) * 2 + 1] = mx;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (tid < bt) {  // one lane per row derives that row's scale and zero point
+      float mn = sh.mm[tid * kWaves * 2], mx = sh.mm[tid * kWaves * 2 + 1];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) {
+        mn = fminf(mn, sh.mm[(tid * kWaves + w) * 2]);
+        mx = fmaxf(mx, sh.mm[(tid * kWaves + w) * 2 + 1]);
+      }
+      const RowQuantParams qp =
+          p.asymmetric ? AsymmetricRowParams<VARIANT>(mn, mx) : SymmetricRowParams(mn, mx);
+      sh.sf[tid] = qp.scale;
+      sh.inv[tid] = qp.inv;
+      sh.zp[tid] = qp.zero_point;
+      sh.zero[tid] = qp.all_zero ? 1 : 0;
+    }
+    __syncthreads();
+    if (in_regs) {
+#pragma unroll
+      for (int b = 0; b < REG_ROWS; ++b) {
+        if (b < bt) {
+          RowQuantParams qp;
+          qp.scale = sh.sf[b];
+          qp.inv = sh.inv[b];
+          qp.zero_point = sh.zp[b];
+          qp.all_zero = sh.zero[b] != 0;
+          int8_t* qrow = sh.q + b * qstride;
+#pragma unroll
+          for (int j = 0; j < kXRegs; ++j) {
+            const int i = (j * kThreads + tid) * 4;
+            if (i < padded) {
+              int32_t packed = 0;
+              if (i < depth) {
+                const float4 t = xr[b][j];
+                const bool tail = i >= vector_end;
+                packed = PackBytes(QuantizeElement<VARIANT>(t.x, qp, p.asymmetric, tail),
+                                   QuantizeElement<VARIANT>(t.y, qp, p.asymmetric, tail),
+                                   QuantizeElement<VARIANT>(t.z, qp, p.asymmetric, tail),
+                                   QuantizeElement<VARIANT>(t.w, qp, p.asymmetric, tail));
+              }
+              *reinterpret_cast<int32_t*>(qrow + i) = packed;
+            }
+          }
+        }
+      }
+    } else {
+      const bool vec_ok =
+          (depth % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.input_f32) & 15) == 0);
+      for (int b = 0; b < bt; ++b) {
+        const float* x = p.input_f32 + static_cast<size_t>(batch0 + b) * depth;
+        RowQuantParams qp;
+        qp.scale = sh.sf[b];
+        qp.inv = sh.inv[b];
+        qp.zero_point = sh.zp[b];
+        qp.all_zero = sh.zero[b] != 0;
+        int8_t* qrow = sh.q + b * qstride;
+        if (vec_ok) {
+          for (int i = tid * 4; i < padded; i += kThreads * 4) {
+            int32_t packed = 0;
+            if (i < depth) {
+              const float4 t = *reinterpret_cast<const float4*>(x + i);
+              const bool tail = i >= vector_end;
+              packed = PackBytes(QuantizeElement<VARIANT>(t.x, qp, p.asymmetric, tail),
+                                 QuantizeElement<VARIANT>(t.y, qp, p.asymmetric, tail),
+                                 QuantizeElement<VARIANT>(t.z, qp, p.asymmetric, tail),
+                                 QuantizeElement<VARIANT>(t.w, qp, p.asymmetric, tail));
+            }
+            *reinterpret_cast<int32_t*>(qrow + i) = packed;
+          }
+        } else {
+          for (int i = tid; i < padded; i += kThreads) {
+            qrow[i] = i < depth ? static_cast<int8_t>(QuantizeElement<VARIANT>(
+                                      x[i], qp, p.asymmetric, i >= vector_end))
+                                : 0;
+          }
+        }
+      }
+    }
+  } else if (in_regs) {
+    const int chunks_per_row = padded / 16;
+#pragma unroll
+    for (int j = 0; j < kQRegs; ++j) {
+      const int c = j * kThreads + tid;
+      const int b = c / chunks_per_row;
+      const int i = (c - b * chunks_per_row) * 16;
+      if (b < bt) {
+        *reinterpret_cast<i32x4*>(sh.q + b * qstride + i) = i < depth ? qr[j] : i32x4{0, 0, 0, 0};
+      }
+    }
+  }
+  __syncthreads();
+
+  // 3. Matrix-core loop. B operand: lane L supplies batch column (L % 16), the same 16
+  // depth positions as its weight bytes. Columns past the tile read row 0; their
+  // results are never stored. Four accumulators break the MFMA dependency chain.
+  const int8_t* qbase = sh.q + (col < bt ? col : 0) * qstride + kgroup * 16;
+  i32x4 acc4[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc4[i] = i32x4{0, 0, 0, 0};
+  int base = s0;
+  for (; base + kRing < s1; base += kRing) {  // full rounds: consume a slot, refill it
+#pragma unroll
+    for (int g = 0; g < kRing; g += 4) {
+      i32x4 bq[4];  // four activation operands per LDS wait
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        bq[u] = *reinterpret_cast<const i32x4*>(qbase + (base + g + u) * kSlabDepth);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+#ifdef LRT_EXP_NOMFMA
+        acc4[u] ^= ring[g + u] ^ bq[u];
+#else
+        acc4[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ring[g + u], bq[u], acc4[u], 0, 0, 0);
+#endif
+        ring[g + u] = __builtin_nontemporal_load(
+            wbase + static_cast<size_t>(min(base + kRing + g + u, slabs - 1)) * 64);
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kRing; ++u) {  // last round
+    if (base + u < s1) {
+      const i32x4 bq = *reinterpret_cast<const i32x4*>(qbase + (base + u) * kSlabDepth);
+      acc4[u & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ring[u], bq, acc4[u & 3], 0, 0, 0);
+    }
+  }
+  i32x4 acc = (acc4[0] + acc4[1]) + (acc4[2] + acc4[3]);
+
+  // 4. Depth shares of one channel group meet in LDS.
+  if (ksplit > 1) {
+    sh.partial[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (part != 0) return;
+    for (int w = 1; w < ksplit; ++w) acc += sh.partial[(wave + w) * 64 + lane];
+  }
+
+  // 5. Epilogue. Accumulator register i holds channel 4 * (L / 16) + i, column L % 16.
+#ifdef LRT_EXP_NOSTORE
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) != 0x12345678) return;
+#endif
+  if (col >= bt || tile >= tiles) return;
+  const int b = batch0 + col;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = tile * kTileRows + 4 * kgroup + i;
+    if (n >= a.out_depth) continue;
+    if (EPI == Int8Epilogue::kRequantize) {
+      a.output_i8[static_cast<size_t>(b) * a.out_depth + n] =
+          RequantizeCore(acc[i] + ep_i2[i] + a.input_offset * ep_i3[i], ep_i0[i], ep_i1[i],
+                         a.output_offset, a.act_min, a.act_max);
+    } else {
+      const float batch_scale = FUSED ? sh.sf[col] : a.scaling_factors[b];
+      const int32_t batch_zp = FUSED ? sh.zp[col] : (a.zero_points ? a.zero_points[b] : 0);
+      a.output_f32[static_cast<size_t>(b) * a.out_depth + n] = HybridCore(
+          acc[i], batch_scale, ep_f0[i], batch_zp, ep_i0[i], ep_f1[i], a.activation);
+    }
+  }
+}
+
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS>
+hipError_t LaunchSized(const PackedArgs& p, int batch0, int bt, hipStream_t stream) {
+  const int qstride = p.slabs * kSlabDepth + kQPad;
+  const size_t lds = SharedBytes(bt, qstride);
+  auto kernel = FcInt8PackedGemvKernel<EPI, FUSED, VARIANT, REG_ROWS>;
+  if (lds > 48 * 1024) {
+    static size_t granted = 0;
+    if (lds > granted) {
+      hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(lds));
+      if (err != hipSuccess) return err;
+      granted = lds;
+    }
+  }
+  const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
+  // One wavefront per channel group when that already gives the chip ~2 wavefronts per
+  // SIMD-pair; otherwise split the depth so that short filters still spread out.
+  int ksplit = 1;
+  while (ksplit < kWaves && tiles * ksplit < 512 && p.slabs / (ksplit * 2) >= 4) ksplit *= 2;
+  const int tiles_per_wg = kWaves / ksplit;
+  const int grid = (tiles + tiles_per_wg - 1) / tiles_per_wg;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, p, batch0, bt, ksplit);
+  return hipGetLastError();
+}
+
+template <Int8Epilogue EPI, bool FUSED, int VARIANT>
+hipError_t LaunchOne(const PackedArgs& p, int batch0, int bt, hipStream_t stream) {
+  if (!FUSED || bt <= 1) return LaunchSized<EPI, FUSED, VARIANT, 1>(p, batch0, bt, stream);
+  if (bt <= 2) return LaunchSized<EPI, FUSED, VARIANT, 2>(p, batch0, bt, stream);
+  return LaunchSized<EPI, FUSED, VARIANT, 4>(p, batch0, bt, stream);
+}
+
+template <Int8Epilogue EPI, bool FUSED>
+hipError_t LaunchVariant(const PackedArgs& p, int variant, int batch0, int bt,
+                         hipStream_t stream) {
+  if (!FUSED) return LaunchOne<EPI, false, LRTFC_QUANT_PORTABLE>(p, batch0, bt, stream);
+  switch (variant) {
+    case LRTFC_QUANT_NEON_V8:
+      return LaunchOne<EPI, FUSED, LRTFC_QUANT_NEON_V8>(p, batch0, bt, stream);
+    case LRTFC_QUANT_NEON_LEGACY:
+      return LaunchOne<EPI, FUSED, LRTFC_QUANT_NEON_LEGACY>(p, batch0, bt, stream);
+    default:
+      return LaunchOne<EPI, FUSED, LRTFC_QUANT_PORTABLE>(p, batch0, bt, stream);
+  }
+}
+
+}  // namespace
+
+size_t PackedInt8FilterBytes(int out_depth, int depth) {
+  const size_t tiles = (static_cast<size_t>(out_depth) + kTileRows - 1) / kTileRows;
+  const size_t slabs = (static_cast<size_t>(depth) + kSlabDepth - 1) / kSlabDepth;
+  return tiles * slabs * 1024;
+}
+
+hipError_t LaunchPackInt8Filter(const int8_t* filter, int out_depth, int depth, int8_t* packed,
+                                hipStream_t stream) {
+  if (out_depth == 0 || depth == 0) return hipSuccess;
+  const int slabs = (depth + kSlabDepth - 1) / kSlabDepth;
+  const int64_t chunks = static_cast<int64_t>(PackedInt8FilterBytes(out_depth, depth) / 16);
+  const unsigned grid = static_cast<unsigned>((chunks + kThreads - 1) / kThreads);
+  hipLaunchKernelGGL(PackInt8FilterKernel, dim3(grid), dim3(kThreads), 0, stream, filter,
+                     out_depth, depth, slabs, chunks, packed);
+  return hipGetLastError();
+}
+
+bool FcInt8PackedGemvSupports(const FcInt8Args& a) {
+  // The per-tensor form with a non-zero filter zero point needs sum(x), which this
+  // kernel does not carry; the row-major GEMV handles it.
+  const size_t qstride = (static_cast<size_t>(a.depth) + kSlabDepth - 1) / kSlabDepth * kSlabDepth +
+                         kQPad;
+  return a.filter_offset == 0 && a.depth > 0 && SharedBytes(1, static_cast<int>(qstride)) <= 150 * 1024;
+}
+
+hipError_t LaunchFcInt8PackedGemv(const FcInt8Args& a, Int8Epilogue epilogue,
+                                  const float* input_f32, int asymmetric, int variant,
+                                  hipStream_t stream) {
+  if (a.batches == 0 || a.out_depth == 0) return hipSuccess;
+  if (!FcInt8PackedGemvSupports(a)) return hipErrorNotSupported;
+  PackedArgs p;
+  p.a = a;
+  p.input_f32 = input_f32;
+  p.asymmetric = asymmetric;
+  p.slabs = (a.depth + kSlabDepth - 1) / kSlabDepth;
+  const int qstride = p.slabs * kSlabDepth + kQPad;
+  int batch0 = 0;
+  while (batch0 < a.batches) {
+    int bt = min(16, a.batches - batch0);
+    while (bt > 1 && SharedBytes(bt, qstride) > 150 * 1024) --bt;
+    hipError_t err;
+    if (epilogue == Int8Epilogue::kRequantize) {
+      err = LaunchVariant<Int8Epilogue::kRequantize, false>(p, variant, batch0, bt, stream);
+    } else if (input_f32) {
+      err = LaunchVariant<Int8Epilogue::kHybrid, true>(p, variant, batch0, bt, stream);
+    } else {
+      err = LaunchVariant<Int8Epilogue::kHybrid, false>(p, variant, batch0, bt, stream);
+    }
+    if (err != hipSuccess) return err;
+    batch0 += bt;
+  }
+  return hipSuccess;
+}
+
+}  // namespace lrtfc

@@ -53,6 +53,16 @@ hipError_t LaunchFcInt8Gemv(const FcInt8Args& a, Int8Epilogue epilogue, hipStrea
 hipError_t LaunchFcInt8GemmMfma(const FcInt8Args& a, hipStream_t stream);
 bool FcInt8GemmMfmaSupports(const FcInt8Args& a);
 
+// Matrix-core GEMV on a filter re-tiled by LaunchPackInt8Filter (a.filter = packed).
+// input_f32 != nullptr selects the fused form that quantizes the float rows in-kernel.
+size_t PackedInt8FilterBytes(int out_depth, int depth);
+hipError_t LaunchPackInt8Filter(const int8_t* filter, int out_depth, int depth, int8_t* packed,
+                                hipStream_t stream);
+bool FcInt8PackedGemvSupports(const FcInt8Args& a);
+hipError_t LaunchFcInt8PackedGemv(const FcInt8Args& a, Int8Epilogue epilogue,
+                                  const float* input_f32, int asymmetric, int variant,
+                                  hipStream_t stream);
+
 struct FcInt4Args {
   const int8_t* input;           // [batches, depth] quantized activations
   const float* scaling_factors;  // [batches]

@@ -3,6 +3,7 @@
 // row, a min/max pass, the scale / zero-point derivation in double precision
 // exactly as the CPU kernels do it, then the elementwise pass.
 #include "kernels.h"
+#include "quantize_device.h"
 
 namespace lrtfc {
 namespace {
@@ -35,44 +36,6 @@ __device__ __forceinline__ RowRange BlockMinMax(float mn, float mx) {
   return r;
 }
 
-// The rounding used inside the NEON loops
-// (tflite/kernels/internal/optimized/neon_tensor_utils.cc:2347-2359).
-template <int VARIANT>
-__device__ __forceinline__ int32_t RoundToNearest(float x) {
-  if (VARIANT == LRTFC_QUANT_NEON_LEGACY) {
-    const float nudge = __fadd_rn(x < 0.0f ? -1.0f : 0.0f, 0.5f);
-    return static_cast<int32_t>(__fadd_rn(x, nudge));  // truncation
-  }
-  return static_cast<int32_t>(roundf(x));
-}
-
-template <int VARIANT>
-__device__ __forceinline__ int8_t QuantizeAsym(float v, float inv, int32_t zp, bool in_tail) {
-  int32_t q;
-  if (VARIANT == LRTFC_QUANT_PORTABLE) {
-    // reference/portable_tensor_utils.cc:112-118: float multiply, float add,
-    // then round half away. An FMA here would change results.
-    q = static_cast<int32_t>(roundf(__fadd_rn(static_cast<float>(zp), __fmul_rn(v, inv))));
-  } else if (in_tail) {
-    // neon_tensor_utils.cc:2546-2551, scalar postamble.
-    q = static_cast<int32_t>(__fadd_rn(static_cast<float>(zp), roundf(__fmul_rn(inv, v))));
-  } else {
-    q = RoundToNearest<VARIANT>(__fmul_rn(v, inv)) + zp;
-  }
-  return static_cast<int8_t>(min(127, max(-128, q)));
-}
-
-template <int VARIANT>
-__device__ __forceinline__ int8_t QuantizeSym(float v, float inv, bool in_tail) {
-  int32_t q;
-  if (VARIANT == LRTFC_QUANT_PORTABLE || in_tail) {
-    q = static_cast<int32_t>(roundf(__fmul_rn(v, inv)));
-  } else {
-    q = RoundToNearest<VARIANT>(__fmul_rn(v, inv));
-  }
-  return static_cast<int8_t>(min(127, max(-127, q)));
-}
-
 template <int VARIANT>
 __global__ __launch_bounds__(kThreads) void BatchQuantizeKernel(
     const float* __restrict__ values, int n_data, int8_t* __restrict__ quantized,
@@ -102,56 +65,12 @@ __global__ __launch_bounds__(kThreads) void BatchQuantizeKernel(
   const RowRange range = BlockMinMax(mn, mx);
 
   // Scale and zero point, every thread redundantly (a few dozen flops).
-  float sf;
-  float inv;
-  int32_t zp = 0;
-  bool all_zero = false;
-  if (do_asymmetric) {
-    if (range.mn == range.mx) {
-      all_zero = true;  // both are 0: memset, scale 1, offset 0
-      sf = 1.0f;
-      inv = 1.0f;
-    } else {
-      const double qmin = -128.0, qmax = 127.0;
-      const double rmin = static_cast<double>(range.mn);
-      const double rmax = static_cast<double>(range.mx);
-      // Portable widens to double before subtracting
-      // (reference/portable_tensor_utils.cc:81-87); the NEON build subtracts in
-      // float (neon_tensor_utils.cc:2486).
-      const double span = (VARIANT == LRTFC_QUANT_PORTABLE)
-                              ? (rmax - rmin)
-                              : static_cast<double>(__fsub_rn(range.mx, range.mn));
-      const double scale = span / (qmax - qmin);
-      const double zp_from_min = qmin - rmin / scale;
-      const double zp_from_max = qmax - rmax / scale;
-      const double err_from_min = fabs(qmin) + fabs(rmin / scale);
-      const double err_from_max = fabs(qmax) + fabs(rmax / scale);
-      const double zp_double = err_from_min < err_from_max ? zp_from_min : zp_from_max;
-      if (zp_double <= qmin) {
-        zp = -128;
-      } else if (zp_double >= qmax) {
-        zp = 127;
-      } else {
-        zp = static_cast<int8_t>(round(zp_double));
-      }
-      sf = static_cast<float>(scale);
-      if (VARIANT == LRTFC_QUANT_PORTABLE) {
-        inv = __fdiv_rn(1.0f, sf);
-      } else {
-        inv = sf == 0.0f ? 0.0f : static_cast<float>(1.0 / static_cast<double>(sf));
-      }
-    }
-  } else {
-    const float absmax = fmaxf(fabsf(range.mn), fabsf(range.mx));
-    if (absmax == 0.0f) {
-      all_zero = true;
-      sf = 1.0f;
-      inv = 1.0f;
-    } else {
-      sf = __fdiv_rn(absmax, 127.0f);
-      inv = __fdiv_rn(127.0f, absmax);
-    }
-  }
+  const RowQuantParams qp = do_asymmetric ? AsymmetricRowParams<VARIANT>(range.mn, range.mx)
+                                          : SymmetricRowParams(range.mn, range.mx);
+  const float sf = qp.scale;
+  const float inv = qp.inv;
+  const int32_t zp = qp.zero_point;
+  const bool all_zero = qp.all_zero;
   if (threadIdx.x == 0) {
     scaling_factors[row] = sf;
     if (zero_points) zero_points[row] = zp;
@@ -171,15 +90,15 @@ __global__ __launch_bounds__(kThreads) void BatchQuantizeKernel(
         const float4 t = v4[i];
         const bool tail = 4 * i >= vector_end;
         if (do_asymmetric) {
-          o.x = QuantizeAsym<VARIANT>(t.x, inv, zp, tail);
-          o.y = QuantizeAsym<VARIANT>(t.y, inv, zp, tail);
-          o.z = QuantizeAsym<VARIANT>(t.z, inv, zp, tail);
-          o.w = QuantizeAsym<VARIANT>(t.w, inv, zp, tail);
+          o.x = static_cast<char>(QuantizeAsym<VARIANT>(t.x, inv, zp, tail));
+          o.y = static_cast<char>(QuantizeAsym<VARIANT>(t.y, inv, zp, tail));
+          o.z = static_cast<char>(QuantizeAsym<VARIANT>(t.z, inv, zp, tail));
+          o.w = static_cast<char>(QuantizeAsym<VARIANT>(t.w, inv, zp, tail));
         } else {
-          o.x = QuantizeSym<VARIANT>(t.x, inv, tail);
-          o.y = QuantizeSym<VARIANT>(t.y, inv, tail);
-          o.z = QuantizeSym<VARIANT>(t.z, inv, tail);
-          o.w = QuantizeSym<VARIANT>(t.w, inv, tail);
+          o.x = static_cast<char>(QuantizeSym<VARIANT>(t.x, inv, tail));
+          o.y = static_cast<char>(QuantizeSym<VARIANT>(t.y, inv, tail));
+          o.z = static_cast<char>(QuantizeSym<VARIANT>(t.z, inv, tail));
+          o.w = static_cast<char>(QuantizeSym<VARIANT>(t.w, inv, tail));
         }
       }
       q4[i] = o;
@@ -189,8 +108,8 @@ __global__ __launch_bounds__(kThreads) void BatchQuantizeKernel(
       int8_t o = 0;
       if (!all_zero) {
         const bool tail = i >= vector_end;
-        o = do_asymmetric ? QuantizeAsym<VARIANT>(v[i], inv, zp, tail)
-                          : QuantizeSym<VARIANT>(v[i], inv, tail);
+        o = static_cast<int8_t>(do_asymmetric ? QuantizeAsym<VARIANT>(v[i], inv, zp, tail)
+                                              : QuantizeSym<VARIANT>(v[i], inv, tail));
       }
       q[i] = o;
     }

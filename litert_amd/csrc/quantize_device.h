@@ -1,0 +1,131 @@
+// Device-side pieces of the per-row activation quantizer, shared by the standalone
+// BatchQuantizeFloats kernel and by the GEMV kernels that quantize their input rows in
+// their own prologue. Semantics: tflite/kernels/internal/reference/portable_tensor_utils.cc
+// :41-119 (portable, normative) and optimized/neon_tensor_utils.cc:2347-2552 (the two
+// NEON-flavoured variants).
+#ifndef LITERT_AMD_CSRC_QUANTIZE_DEVICE_H_
+#define LITERT_AMD_CSRC_QUANTIZE_DEVICE_H_
+
+#include "device_utils.h"
+#include "../../include/litert_amd_fc.h"
+
+namespace lrtfc {
+
+struct RowQuantParams {
+  float scale;     // scaling factor stored for the row
+  float inv;       // multiplier applied to each element
+  int32_t zero_point;
+  bool all_zero;   // the row quantizes to zeros with scale 1 / zero point 0
+};
+
+// mn = min(0, min v), mx = max(0, max v) of the row.
+template <int VARIANT>
+__device__ __forceinline__ RowQuantParams AsymmetricRowParams(float mn, float mx) {
+  RowQuantParams p;
+  p.zero_point = 0;
+  p.all_zero = false;
+  if (mn == mx) {  // both 0
+    p.all_zero = true;
+    p.scale = 1.0f;
+    p.inv = 1.0f;
+    return p;
+  }
+  const double qmin = -128.0, qmax = 127.0;
+  const double rmin = static_cast<double>(mn);
+  const double rmax = static_cast<double>(mx);
+  // Portable widens to double before subtracting (portable_tensor_utils.cc:81-87); the
+  // NEON build subtracts in float (neon_tensor_utils.cc:2486).
+  const double span = (VARIANT == LRTFC_QUANT_PORTABLE)
+                          ? (rmax - rmin)
+                          : static_cast<double>(__fsub_rn(mx, mn));
+  const double scale = span / (qmax - qmin);
+  const double zp_from_min = qmin - rmin / scale;
+  const double zp_from_max = qmax - rmax / scale;
+  const double err_from_min = fabs(qmin) + fabs(rmin / scale);
+  const double err_from_max = fabs(qmax) + fabs(rmax / scale);
+  const double zp_double = err_from_min < err_from_max ? zp_from_min : zp_from_max;
+  if (zp_double <= qmin) {
+    p.zero_point = -128;
+  } else if (zp_double >= qmax) {
+    p.zero_point = 127;
+  } else {
+    p.zero_point = static_cast<int8_t>(round(zp_double));
+  }
+  p.scale = static_cast<float>(scale);
+  if (VARIANT == LRTFC_QUANT_PORTABLE) {
+    p.inv = __fdiv_rn(1.0f, p.scale);
+  } else {
+    p.inv = p.scale == 0.0f ? 0.0f : static_cast<float>(1.0 / static_cast<double>(p.scale));
+  }
+  return p;
+}
+
+__device__ __forceinline__ RowQuantParams SymmetricRowParams(float mn, float mx) {
+  RowQuantParams p;
+  p.zero_point = 0;
+  const float absmax = fmaxf(fabsf(mn), fabsf(mx));
+  p.all_zero = absmax == 0.0f;
+  if (p.all_zero) {
+    p.scale = 1.0f;
+    p.inv = 1.0f;
+  } else {
+    p.scale = __fdiv_rn(absmax, 127.0f);
+    p.inv = __fdiv_rn(127.0f, absmax);
+  }
+  return p;
+}
+
+// The rounding used inside the NEON loops (neon_tensor_utils.cc:2347-2359).
+template <int VARIANT>
+__device__ __forceinline__ int32_t RoundToNearest(float x) {
+  if (VARIANT == LRTFC_QUANT_NEON_LEGACY) {
+    const float nudge = __fadd_rn(x < 0.0f ? -1.0f : 0.0f, 0.5f);
+    return static_cast<int32_t>(__fadd_rn(x, nudge));  // truncation
+  }
+  return static_cast<int32_t>(roundf(x));
+}
+
+// in_tail: the element belongs to the last n % 8 of the row, which the NEON builds
+// finish with a scalar expression that rounds differently.
+template <int VARIANT>
+__device__ __forceinline__ int32_t QuantizeAsym(float v, float inv, int32_t zp, bool in_tail) {
+  int32_t q;
+  if (VARIANT == LRTFC_QUANT_PORTABLE) {
+    // portable_tensor_utils.cc:112-118: float multiply, float add, then round half
+    // away. An FMA here would change results.
+    q = static_cast<int32_t>(roundf(__fadd_rn(static_cast<float>(zp), __fmul_rn(v, inv))));
+  } else if (in_tail) {
+    q = static_cast<int32_t>(__fadd_rn(static_cast<float>(zp), roundf(__fmul_rn(inv, v))));
+  } else {
+    q = RoundToNearest<VARIANT>(__fmul_rn(v, inv)) + zp;
+  }
+  return min(127, max(-128, q));
+}
+
+template <int VARIANT>
+__device__ __forceinline__ int32_t QuantizeSym(float v, float inv, bool in_tail) {
+  int32_t q;
+  if (VARIANT == LRTFC_QUANT_PORTABLE || in_tail) {
+    q = static_cast<int32_t>(roundf(__fmul_rn(v, inv)));
+  } else {
+    q = RoundToNearest<VARIANT>(__fmul_rn(v, inv));
+  }
+  return min(127, max(-127, q));
+}
+
+template <int VARIANT>
+__device__ __forceinline__ int32_t QuantizeElement(float v, const RowQuantParams& p,
+                                                   bool asymmetric, bool in_tail) {
+  if (p.all_zero) return 0;
+  return asymmetric ? QuantizeAsym<VARIANT>(v, p.inv, p.zero_point, in_tail)
+                    : QuantizeSym<VARIANT>(v, p.inv, in_tail);
+}
+
+// Four quantized values packed little-endian into one dword.
+__device__ __forceinline__ int32_t PackBytes(int32_t a, int32_t b, int32_t c, int32_t d) {
+  return (a & 0xFF) | ((b & 0xFF) << 8) | ((c & 0xFF) << 16) | (static_cast<uint32_t>(d) << 24);
+}
+
+}  // namespace lrtfc
+
+#endif  // LITERT_AMD_CSRC_QUANTIZE_DEVICE_H_

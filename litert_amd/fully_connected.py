@@ -42,6 +42,15 @@ def _ensure_init():
     capi.init(torch.cuda.current_device())
 
 
+def _pack_int8(filter_dev):
+    """Re-tiles a row-major int8 [N, K] device tensor for the matrix-core GEMV."""
+    n, k = filter_dev.shape
+    lib = capi.load()
+    packed = torch.empty(lib.lrtfc_packed_int8_filter_bytes(n, k), dtype=torch.int8, device="cuda")
+    capi.check(lib.lrtfc_pack_int8_filter(_ptr(filter_dev), n, k, _ptr(packed), _stream()))
+    return packed
+
+
 def quantize_multiplier(m):
     q, s = C.c_int32(), C.c_int()
     capi.check(capi.load().lrtfc_quantize_multiplier(float(m), C.byref(q), C.byref(s)))
@@ -96,18 +105,18 @@ class FullyConnectedInt8:
 
     def __init__(self, filter, bias, input_scale, input_zero_point, filter_scales,
                  output_scale, output_zero_point, activation="none", filter_zero_point=0,
-                 bias_scale=None, int4=False, depth=None):
+                 bias_scale=None, int4=False, depth=None, packed=True):
         _ensure_init()
         lib = capi.load()
         fs = np.atleast_1d(np.asarray(filter_scales, dtype=np.float32))
         self.per_channel = fs.size > 1
         if int4:
-            packed = _dev(filter, torch.uint8)
-            n = packed.shape[0]
+            nibbles = _dev(filter, torch.uint8)
+            n = nibbles.shape[0]
             if depth is None:
                 raise ValueError("depth is required for packed int4 filters")
             self.filter = torch.empty((n, depth), dtype=torch.int8, device="cuda")
-            capi.check(lib.lrtfc_unpack_int4(_ptr(packed), n * depth, _ptr(self.filter), _stream()))
+            capi.check(lib.lrtfc_unpack_int4(_ptr(nibbles), n * depth, _ptr(self.filter), _stream()))
         else:
             self.filter = _dev(filter, torch.int8)
         self.out_depth, self.depth = self.filter.shape
@@ -132,12 +141,26 @@ class FullyConnectedInt8:
         self.row_sums = torch.empty(self.out_depth, dtype=torch.int32, device="cuda")
         capi.check(lib.lrtfc_row_sums_int8(_ptr(self.filter), self.out_depth, self.depth,
                                            _ptr(self.row_sums), _stream()))
+        # Decode batches run on a re-tiled copy of the filter (matrix-core GEMV); prefill
+        # batches use the row-major filter (MFMA GEMM).
+        self.packed_filter = None
+        if packed and self.filter_offset == 0 and self.depth > 0:
+            self.packed_filter = _pack_int8(self.filter)
+
+    GEMM_MIN_BATCHES = 128
 
     def __call__(self, x, out=None):
         x = x.contiguous()
         batches = x.numel() // self.depth if self.depth else 0
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.int8, device=x.device)
+        if self.packed_filter is not None and batches < self.GEMM_MIN_BATCHES:
+            capi.check(capi.load().lrtfc_fc_int8_packed(
+                _ptr(x), _ptr(self.packed_filter), _ptr(self.bias), _ptr(self.multipliers),
+                _ptr(self.shifts), int(self.per_channel), _ptr(self.row_sums), _ptr(out), batches,
+                self.depth, self.out_depth, self.input_offset, self.output_offset, self.act_min,
+                self.act_max, _stream()))
+            return out
         capi.check(capi.load().lrtfc_fc_int8(
             _ptr(x), _ptr(self.filter), _ptr(self.bias), _ptr(self.multipliers), _ptr(self.shifts),
             int(self.per_channel), _ptr(self.row_sums), _ptr(out), batches, self.depth,
@@ -151,7 +174,7 @@ class FullyConnectedHybrid:
 
     def __init__(self, filter, per_channel_scales=None, filter_scale=1.0, bias=None,
                  asymmetric_quantize_inputs=True, activation="none",
-                 quant_variant=capi.QUANT_PORTABLE):
+                 quant_variant=capi.QUANT_PORTABLE, packed=True):
         _ensure_init()
         self.filter = _dev(filter, torch.int8)
         self.out_depth, self.depth = self.filter.shape
@@ -165,6 +188,9 @@ class FullyConnectedHybrid:
         capi.check(capi.load().lrtfc_row_sums_int8(_ptr(self.filter), self.out_depth, self.depth,
                                                    _ptr(self.row_sums), _stream()))
         self._ws = None
+        # packed: one fused kernel (quantize in the prologue, matrix-core GEMV);
+        # otherwise the two-kernel form on the row-major filter.
+        self.packed_filter = _pack_int8(self.filter) if packed else None
 
     def _workspace(self, batches):
         need = capi.load().lrtfc_activation_workspace_bytes(batches, self.depth)
@@ -177,6 +203,12 @@ class FullyConnectedHybrid:
         batches = x.numel() // self.depth
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
+        if self.packed_filter is not None:
+            capi.check(capi.load().lrtfc_fc_hybrid_packed(
+                _ptr(x), _ptr(self.packed_filter), _ptr(self.pcs), self.filter_scale,
+                _ptr(self.row_sums), _ptr(self.bias), _ptr(out), batches, self.depth,
+                self.out_depth, int(self.asymmetric), self.activation, self.variant, _stream()))
+            return out
         ws = self._workspace(batches)
         capi.check(capi.load().lrtfc_fc_hybrid(
             _ptr(x), _ptr(self.filter), _ptr(self.pcs), self.filter_scale, _ptr(self.row_sums),

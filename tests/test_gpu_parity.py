@@ -41,10 +41,10 @@ def _bits_equal(a, b):
 
 # ---- full-integer int8 -------------------------------------------------------------
 
-def _run_int8(fc, c, activation="none", bias=True):
+def _run_int8(fc, c, activation="none", bias=True, packed=True):
     op = fc.FullyConnectedInt8(c["w"], c["bias"] if bias else None, float(c["in_scale"]),
                                c["in_zp"], c["w_scale"], float(c["out_scale"]), c["out_zp"],
-                               activation=activation)
+                               activation=activation, packed=packed)
     y = op(_cuda(c["x"])).cpu().numpy()
     mult, shift = oracle.fc_prepare_per_channel(float(c["in_scale"]), c["w_scale"],
                                                 float(c["out_scale"]))
@@ -54,22 +54,26 @@ def _run_int8(fc, c, activation="none", bias=True):
     return y, want
 
 
-def test_int8_config1_bit_exact(fc):
-    """Config 1: [1,2048] x [2048,2048], per-channel, bias, no activation."""
-    y, want = _run_int8(fc, wl.int8_fc())
+@pytest.mark.parametrize("packed", [True, False])
+def test_int8_config1_bit_exact(fc, packed):
+    """Config 1: [1,2048] x [2048,2048], per-channel, bias, no activation; on the re-tiled
+    filter (matrix-core GEMV) and on the row-major one (dot4 GEMV)."""
+    y, want = _run_int8(fc, wl.int8_fc(), packed=packed)
     assert np.array_equal(y, want)
     assert len(np.unique(y)) > 100  # the case exercises the whole int8 range, not a clamp
 
 
 @pytest.mark.parametrize("B,K,N", [(1, 16, 1), (2, 48, 5), (3, 1040, 17), (4, 2048, 256),
                                    (5, 512, 67), (8, 4096, 512), (9, 256, 33), (16, 128, 40),
-                                   (1, 16384, 64), (2, 10, 3), (3, 33, 7), (1, 100, 9)])
+                                   (1, 16384, 64), (2, 10, 3), (3, 33, 7), (1, 100, 9),
+                                   (17, 320, 19), (40, 64, 16), (1, 20000, 5)])
 @pytest.mark.parametrize("activation", ["none", "relu6"])
-def test_int8_gemv_shapes_bit_exact(fc, B, K, N, activation):
+@pytest.mark.parametrize("packed", [True, False])
+def test_int8_gemv_shapes_bit_exact(fc, B, K, N, activation, packed):
     """Ragged shapes: depth off the 16-byte grid takes the generic kernel, batches that are
     not a power of two split into tiles, rows that do not fill a pass are clamped."""
     c = wl.int8_fc(B, K, N, seed=100 + B + K + N)
-    y, want = _run_int8(fc, c, activation, bias=(N % 2 == 1))
+    y, want = _run_int8(fc, c, activation, bias=(N % 2 == 1), packed=packed)
     assert np.array_equal(y, want)
 
 
@@ -210,27 +214,32 @@ def test_batch_quantize_reference_kats_through_hip(fc):
 # ---- hybrid ----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("B", [1, 4, 8])
-def test_hybrid_config2_shape(fc, B):
+@pytest.mark.parametrize("packed", [True, False])
+def test_hybrid_config2_shape(fc, B, packed):
     """Config 2 at its real depth with a reduced number of output channels (the scalar
-    oracle needs ~60 ms per 1000 channels per batch row)."""
+    oracle needs ~60 ms per 1000 channels per batch row); the fused single-kernel form on
+    the re-tiled filter and the two-kernel form on the row-major one."""
     c = wl.hybrid_fc(B, 4096, 2048)
-    op = fc.FullyConnectedHybrid(c["w"], c["pcs"])
+    op = fc.FullyConnectedHybrid(c["w"], c["pcs"], packed=packed)
     y = op(_cuda(c["x"])).cpu().numpy()
     want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"])
     assert _close(y, want)
     assert _bits_equal(y, want)
 
 
-@pytest.mark.parametrize("B,K,N", [(1, 64, 5), (3, 1040, 33), (2, 100, 7), (6, 512, 130)])
+@pytest.mark.parametrize("B,K,N", [(1, 64, 5), (3, 1040, 33), (2, 100, 7), (6, 512, 130),
+                                   (19, 257, 21)])
 @pytest.mark.parametrize("asym", [True, False])
 @pytest.mark.parametrize("per_channel", [True, False])
 @pytest.mark.parametrize("activation", ["none", "relu", "relu_n1_to_1", "relu6"])
-def test_hybrid_variants(fc, B, K, N, asym, per_channel, activation):
+@pytest.mark.parametrize("packed", [True, False])
+def test_hybrid_variants(fc, B, K, N, asym, per_channel, activation, packed):
     c = wl.hybrid_fc(B, K, N, seed=7 + B + K)
     bias = np.random.default_rng(3).standard_normal(N).astype(np.float32)
     pcs = c["pcs"] if per_channel else None
     op = fc.FullyConnectedHybrid(c["w"], pcs, filter_scale=0.005, bias=bias,
-                                 asymmetric_quantize_inputs=asym, activation=activation)
+                                 asymmetric_quantize_inputs=asym, activation=activation,
+                                 packed=packed)
     y = op(_cuda(c["x"])).cpu().numpy()
     want = oracle.fc_hybrid(c["x"], c["w"], pcs, 0.005, bias, asym, fc._act(activation))
     assert _close(y, want)
@@ -261,6 +270,18 @@ def test_hybrid_dot_reference_kats_through_hip(fc):
         got = out.cpu().numpy().ravel()
         for i, w in idx_want.items():
             assert got[i] == w
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+def test_hybrid_fused_quantizer_variants(fc, variant):
+    """The in-kernel quantizer of the fused form reproduces the NEON-flavoured variants too,
+    including the scalar tail of a row whose length is not a multiple of 8."""
+    c = wl.hybrid_fc(3, 1004, 40, seed=21)
+    c["x"][0, :4] = [-125.0, 130.0, 2.5, -2.5]
+    op = fc.FullyConnectedHybrid(c["w"], c["pcs"], quant_variant=variant)
+    y = op(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"], variant=variant)
+    assert _bits_equal(y, want)
 
 
 def test_hybrid_full_size_properties(fc):
