@@ -203,6 +203,32 @@ int lrtfc_fc_blockwise_int4(const float* input, const uint8_t* packed_filter,
                             int quant_variant, void* workspace, size_t workspace_bytes,
                             void* stream);
 
+/* Re-tiles a blockwise-int4 filter (block size 32) and its fp16 scales for the streaming
+ * kernel: tiles of 8 output channels x 64 blocks, nine consecutive 1 KiB planes each (eight
+ * of nibbles stored as w + 8, one of scales), tiles of a channel group consecutive along
+ * the depth. `packed` must hold lrtfc_packed_int4_blockwise_bytes(). Like the int8
+ * re-tiling this stands where the reference prepacks constant weights once
+ * (tflite/kernels/fully_connected.cc:1130-1150 does so for its own 4-bit kernels). */
+size_t lrtfc_packed_int4_blockwise_bytes(int out_depth, int depth);
+int lrtfc_pack_int4_blockwise(const uint8_t* packed_filter, const uint16_t* scales_f16,
+                              int out_depth, int depth, int blocksize, uint8_t* retiled,
+                              void* stream);
+
+/* lrtfc_fc_blockwise_int4 as ONE kernel on a re-tiled filter: the activation rows are
+ * quantized in the kernel's prologue (no workspace). Bit-identical results. */
+int lrtfc_fc_blockwise_int4_packed(const float* input, const uint8_t* retiled_filter,
+                                   const float* kfsum, const float* bias, float* output,
+                                   int batches, int depth, int out_depth, int quant_variant,
+                                   void* stream);
+
+/* The same on already-quantized activations. */
+int lrtfc_fc_blockwise_int4_packed_quantized(const int8_t* quantized_input,
+                                             const float* scaling_factors,
+                                             const int32_t* zero_points,
+                                             const uint8_t* retiled_filter, const float* kfsum,
+                                             const float* bias, float* output, int batches,
+                                             int depth, int out_depth, void* stream);
+
 /* Same product on already-quantized activations (workspace layout not needed). */
 int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
                                       const float* scaling_factors, const int32_t* zero_points,

@@ -46,6 +46,11 @@ SYMBOLS = [
                              _vp]),
     ("lrtfc_fc_blockwise_int4", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz,
                                      _vp]),
+    ("lrtfc_packed_int4_blockwise_bytes", _sz, [_i, _i]),
+    ("lrtfc_pack_int4_blockwise", _i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    ("lrtfc_fc_blockwise_int4_packed", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    ("lrtfc_fc_blockwise_int4_packed_quantized", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i,
+                                                      _i, _vp]),
     ("lrtfc_fc_blockwise_int4_quantized", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
                                                _i, _vp]),
 ]

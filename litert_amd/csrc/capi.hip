@@ -490,6 +490,76 @@ int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
   return FromHip(lrtfc::LaunchFcBlockwiseInt4(a, AsStream(stream)), "blockwise int4 GEMV");
 }
 
+size_t lrtfc_packed_int4_blockwise_bytes(int out_depth, int depth) {
+  if (out_depth <= 0 || depth <= 0) return 0;
+  return lrtfc::PackedInt4BlockwiseBytes(out_depth, depth);
+}
+
+int lrtfc_pack_int4_blockwise(const uint8_t* packed_filter, const uint16_t* scales_f16,
+                              int out_depth, int depth, int blocksize, uint8_t* retiled,
+                              void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(out_depth >= 0 && depth >= 0, "negative dimension");
+  if (out_depth == 0 || depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(lrtfc::FcInt4PackedSupports(depth, blocksize),
+                "the re-tiled form needs blocksize 32 dividing the depth (got blocksize %d, "
+                "depth %d)", blocksize, depth);
+  LRTFC_REQUIRE(packed_filter && scales_f16 && retiled, "null pointer");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(retiled) & 15) == 0, "retiled must be 16-byte aligned");
+  return FromHip(lrtfc::LaunchPackInt4Blockwise(packed_filter, scales_f16, out_depth, depth,
+                                                retiled, AsStream(stream)),
+                 "pack int4 blockwise filter");
+}
+
+namespace {
+int FcInt4PackedCommon(const float* input_f32, const int8_t* q, const float* sf, const int32_t* zp,
+                       const uint8_t* retiled, const float* kfsum, const float* bias,
+                       float* output, int batches, int depth, int out_depth, int variant,
+                       void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(lrtfc::FcInt4PackedSupports(depth, 32), "depth %d is not a multiple of 32", depth);
+  LRTFC_REQUIRE(retiled && kfsum && output, "null pointer");
+  LRTFC_REQUIRE(input_f32 || (q && sf && zp), "null input");
+  LRTFC_REQUIRE(variant >= 0 && variant <= LRTFC_QUANT_NEON_LEGACY, "unknown quantizer variant");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(retiled) & 15) == 0,
+                "retiled filter must be 16-byte aligned");
+  lrtfc::FcInt4Args a{};
+  a.input = q;
+  a.scaling_factors = sf;
+  a.zero_points = zp;
+  a.kfsum = kfsum;
+  a.bias = bias;
+  a.output = output;
+  a.batches = batches;
+  a.depth = depth;
+  a.out_depth = out_depth;
+  a.blocksize = 32;
+  return FromHip(lrtfc::LaunchFcInt4Packed(a, retiled, input_f32, variant, AsStream(stream)),
+                 "re-tiled blockwise int4 GEMV");
+}
+}  // namespace
+
+int lrtfc_fc_blockwise_int4_packed(const float* input, const uint8_t* retiled_filter,
+                                   const float* kfsum, const float* bias, float* output,
+                                   int batches, int depth, int out_depth, int quant_variant,
+                                   void* stream) {
+  if (batches > 0 && out_depth > 0 && !input) return Fail(LRTFC_INVALID_ARGUMENT, "null input");
+  return FcInt4PackedCommon(input, nullptr, nullptr, nullptr, retiled_filter, kfsum, bias, output,
+                            batches, depth, out_depth, quant_variant, stream);
+}
+
+int lrtfc_fc_blockwise_int4_packed_quantized(const int8_t* quantized_input,
+                                             const float* scaling_factors,
+                                             const int32_t* zero_points,
+                                             const uint8_t* retiled_filter, const float* kfsum,
+                                             const float* bias, float* output, int batches,
+                                             int depth, int out_depth, void* stream) {
+  return FcInt4PackedCommon(nullptr, quantized_input, scaling_factors, zero_points, retiled_filter,
+                            kfsum, bias, output, batches, depth, out_depth, 0, stream);
+}
+
 int lrtfc_fc_blockwise_int4(const float* input, const uint8_t* packed_filter,
                             const uint16_t* scales_f16, const float* kfsum, const float* bias,
                             float* output, int batches, int depth, int out_depth, int blocksize,

@@ -2,6 +2,7 @@
 #ifndef LITERT_AMD_CSRC_DEVICE_UTILS_H_
 #define LITERT_AMD_CSRC_DEVICE_UTILS_H_
 
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -76,6 +77,12 @@ __device__ __forceinline__ float HalfBitsToFloat(uint16_t h) {
   }
   if (exp == 31) return __uint_as_float(sign | 0x7F800000u | (man << 13));
   return __uint_as_float(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+// The same conversion through the hardware's half-to-float instruction, which handles
+// subnormals, infinities and NaNs as IEEE 754 prescribes (the conversion is exact).
+__device__ __forceinline__ float HalfBitsToFloatFast(uint16_t h) {
+  return __half2float(__ushort_as_half(h));
 }
 
 // ---- wave64 reductions --------------------------------------------------------

@@ -1,0 +1,570 @@
+// Blockwise-int4 FULLY_CONNECTED (EvalBlockwise4Bit, tflite/kernels/fully_connected.cc
+// :1014-1086) on a re-tiled filter, block size 32: the streaming form used for decode.
+//
+// HBM layout ("tile8x64b", built once per constant filter by PackInt4BlockwiseKernel):
+// the filter is cut into tiles of 8 output channels x 64 quantization blocks (2048
+// depth). A tile is nine consecutive 1 KiB planes: plane j < 8 holds, for lane L, the 16
+// bytes (32 nibbles) of channel j, block L; plane 8 holds, for lane L, the eight fp16
+// scales of block L for the tile's channels. Nibbles are stored as (w + 8), i.e. XOR 8,
+// so that they are small positive bytes for dot4; tiles of one channel group are
+// consecutive along the depth. Every load instruction of a wavefront therefore reads
+// 1 KiB of consecutive bytes, weights and scales alike, and one lane finishes a block's
+// int32 sum alone (8 dot4): sum(w * q) = dot4(w + 8, q) - 8 * sum(q).
+//
+// A wavefront owns 8 channels over the whole depth. All loads of its first two tiles go
+// out first (a ring that is refilled tile by tile for deeper filters); the activation
+// rows are quantized (BatchQuantizeFloats, always asymmetric on this path) and staged in
+// LDS, de-interleaved into even-k / odd-k bytes to line up with low / high nibbles,
+// while the ring fills. The reference then adds float(block_sum) * scale over the blocks
+// of a row in block order in float32; that order is kept: the products of a tile are
+// parked in LDS and 8 x batch lanes walk them in order, tile after tile, each walk
+// overlapping the wait for the next tile's bytes.
+#include "kernels.h"
+#include "quantize_device.h"
+
+namespace lrtfc {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWaveSize;
+constexpr int kBlock = 32;       // weights per quantization block
+constexpr int kTileRows = 8;
+constexpr int kTileBlocks = 64;
+constexpr int kPlanes = kTileRows + 1;
+constexpr int kTileBytes = kPlanes * 1024;
+constexpr int kTileVecs = kPlanes * 64;  // i32x4 per tile
+constexpr int kRingTiles = 2;
+constexpr int kPStride = kTileBlocks + 4;  // floats per (row, batch) line of parked products
+
+__global__ __launch_bounds__(kThreads) void PackInt4BlockwiseKernel(
+    const uint8_t* __restrict__ filter, const uint16_t* __restrict__ scales, int out_depth,
+    int depth, int chunks, int64_t total_vecs, uint8_t* __restrict__ dst) {
+  const int64_t v = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (v >= total_vecs) return;
+  const int lane = static_cast<int>(v & 63);
+  const int64_t plane_index = v >> 6;
+  const int plane = static_cast<int>(plane_index % kPlanes);
+  const int64_t tile = plane_index / kPlanes;
+  const int chunk = static_cast<int>(tile % chunks);
+  const int group = static_cast<int>(tile / chunks);
+  const int nblk = depth / kBlock;
+  const int blk = chunk * kTileBlocks + lane;
+  const size_t row_bytes = static_cast<size_t>(depth) / 2;
+  uint8_t out[16];
+  if (plane < kTileRows) {
+    const int row = group * kTileRows + plane;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      uint8_t byte = 0;  // weight 0, weight 0
+      if (row < out_depth && blk < nblk) byte = filter[row * row_bytes + blk * 16 + t];
+      out[t] = byte ^ 0x88;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < kTileRows; ++j) {
+      const int row = group * kTileRows + j;
+      uint16_t s = 0;
+      if (row < out_depth && blk < nblk) s = scales[static_cast<size_t>(row) * nblk + blk];
+      out[2 * j] = static_cast<uint8_t>(s & 0xFF);
+      out[2 * j + 1] = static_cast<uint8_t>(s >> 8);
+    }
+  }
+  *reinterpret_cast<i32x4*>(dst + v * 16) = *reinterpret_cast<const i32x4*>(out);
+}
+
+struct Int4PackedArgs {
+  const uint8_t* packed;       // tile8x64b
+  const float* input_f32;      // fused form
+  const int8_t* input_q;       // unfused form: quantized rows + their scales / zero points
+  const float* scaling_factors;
+  const int32_t* zero_points;
+  const float* kfsum;
+  const float* bias;
+  float* output;
+  int batches, depth, out_depth, chunks;
+};
+
+// Even-k bytes and odd-k bytes of eight consecutive int8 (lo = k0..k0+3, hi = k0+4..k0+7).
+__device__ __forceinline__ void Deinterleave(uint32_t lo, uint32_t hi, int32_t* even,
+                                             int32_t* odd) {
+  *even = static_cast<int32_t>((lo & 0xFFu) | ((lo >> 8) & 0xFF00u) | ((hi & 0xFFu) << 16) |
+                               ((hi << 8) & 0xFF000000u));
+  *odd = static_cast<int32_t>(((lo >> 8) & 0xFFu) | ((lo >> 16) & 0xFF00u) |
+                              ((hi << 8) & 0xFF0000u) | (hi & 0xFF000000u));
+}
+
+// LDS map: [BT][padded depth] de-interleaved activations; per wavefront [8 * BT][kPStride]
+// parked products; per-row quantization state.
+template <int BT>
+struct Int4Shared {
+  int32_t* q;   // dwords: per row padded_depth / 4
+  float* p;     // [kWaves][8 * BT][kPStride]
+  float* sf;    // [BT]
+  float* inv;   // [BT]
+  int32_t* zp;  // [BT]
+  int32_t* zero;
+  float* mm;    // [BT][kWaves][2]
+  __device__ Int4Shared(int8_t* base, int padded) {
+    q = reinterpret_cast<int32_t*>(base);
+    size_t off = static_cast<size_t>(BT) * padded;
+    p = reinterpret_cast<float*>(base + off);
+    off += static_cast<size_t>(kWaves) * 8 * BT * kPStride * 4;
+    sf = reinterpret_cast<float*>(base + off);
+    inv = sf + 8;
+    zp = reinterpret_cast<int32_t*>(inv + 8);
+    zero = zp + 8;
+    mm = reinterpret_cast<float*>(zero + 8);
+  }
+  static size_t Bytes(int padded) {
+    return static_cast<size_t>(BT) * padded + static_cast<size_t>(kWaves) * 8 * BT * kPStride * 4 +
+           4 * 8 * 4 + 8 * kWaves * 2 * 4;
+  }
+};
+
+// GPT: groups of 8 depth positions each thread keeps in registers between the two passes of
+// the prologue; the register form covers depth <= GPT * 256 * 8.
+template <int BT, bool FUSED, int VARIANT, int GPT>
+__global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a, int batch0,
+                                                               int bt) {
+  extern __shared__ __align__(16) int8_t smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWaveSize - 1);
+  const int wave = tid / kWaveSize;
+  const int depth = a.depth;
+  const int chunks = a.chunks;
+  const int padded = chunks * kTileBlocks * kBlock;  // depth padded to whole tiles
+  const int groups = (a.out_depth + kTileRows - 1) / kTileRows;
+  const int group = blockIdx.x * kWaves + wave;  // may run past the last group
+  const i32x4* tbase = reinterpret_cast<const i32x4*>(a.packed) +
+                       static_cast<size_t>(min(group, groups - 1)) * chunks * kTileVecs + lane;
+  Int4Shared<BT> sh(smem, padded);
+
+  // Activation loads first (raw, branch-free): whatever the prologue waits for must be
+  // requested before the weight ring, because vector memory returns in issue order.
+  // Each thread owns groups of 8 consecutive depth positions: g = tid + 256 * j.
+  constexpr int kGroupsPerThread = GPT;
+  float4 xr[BT][kGroupsPerThread][2];
+  i32x2 qr[BT][kGroupsPerThread];
+  const int groups8 = depth / 8;
+  bool in_regs;
+  if (FUSED) {
+    in_regs = ((reinterpret_cast<uintptr_t>(a.input_f32) & 15) == 0) &&
+              groups8 <= kGroupsPerThread * kThreads;
+    if (in_regs) {
+#pragma unroll
+      for (int b = 0; b < BT; ++b) {
+        const float* x = a.input_f32 + static_cast<size_t>(batch0 + min(b, bt - 1)) * depth;
+#pragma unroll
+        for (int j = 0; j < kGroupsPerThread; ++j) {
+          const int g = min(j * kThreads + tid, groups8 - 1);
+          xr[b][j][0] = *reinterpret_cast<const float4*>(x + g * 8);
+          xr[b][j][1] = *reinterpret_cast<const float4*>(x + g * 8 + 4);
+        }
+      }
+    } else {
+      for (int b = 0; b < bt; ++b) {  // slow form: min/max from memory before the ring
+        const float* x = a.input_f32 + static_cast<size_t>(batch0 + b) * depth;
+        float mn = 0.0f, mx = 0.0f;
+        for (int i = tid; i < depth; i += kThreads) {
+          mn = fminf(mn, x[i]);
+          mx = fmaxf(mx, x[i]);
+        }
+        mn = WaveMinF32(mn);
+        mx = WaveMaxF32(mx);
+        if (lane == 0) {
+          sh.mm[(b * kWaves + wave) * 2] = mn;
+          sh.mm[(b * kWaves + wave) * 2 + 1] = mx;
+        }
+      }
+    }
+  } else {
+    in_regs = ((reinterpret_cast<uintptr_t>(a.input_q) & 7) == 0) &&
+              groups8 <= kGroupsPerThread * kThreads;
+    if (in_regs) {
+#pragma unroll
+      for (int b = 0; b < BT; ++b) {
+        const int8_t* x = a.input_q + static_cast<size_t>(batch0 + min(b, bt - 1)) * depth;
+#pragma unroll
+        for (int j = 0; j < kGroupsPerThread; ++j) {
+          const int g = min(j * kThreads + tid, groups8 - 1);
+          qr[b][j] = *reinterpret_cast<const i32x2*>(x + g * 8);
+        }
+      }
+    } else {
+      for (int b = 0; b < bt; ++b) {
+        const int8_t* x = a.input_q + static_cast<size_t>(batch0 + b) * depth;
+        for (int g = tid; g < padded / 8; g += kThreads) {
+          uint32_t lo = 0, hi = 0;
+          if (g < groups8) {
+            for (int t = 0; t < 4; ++t) {
+              lo |= static_cast<uint32_t>(static_cast<uint8_t>(x[g * 8 + t])) << (8 * t);
+              hi |= static_cast<uint32_t>(static_cast<uint8_t>(x[g * 8 + 4 + t])) << (8 * t);
+            }
+          }
+          int32_t even, odd;
+          Deinterleave(lo, hi, &even, &odd);
+          sh.q[b * (padded / 4) + 2 * g] = even;
+          sh.q[b * (padded / 4) + 2 * g + 1] = odd;
+        }
+      }
+    }
+  }
+
+  // The ring: two tiles (18 KiB) per wavefront in flight.
+  i32x4 ring[kRingTiles][kPlanes];
+#pragma unroll
+  for (int t = 0; t < kRingTiles; ++t) {
+    const int c = min(t, chunks - 1);
+#pragma unroll
+    for (int j = 0; j < kPlanes; ++j) {
+      ring[t][j] = __builtin_nontemporal_load(tbase + static_cast<size_t>(c) * kTileVecs + j * 64);
+    }
+  }
+  // Per-channel epilogue inputs of the chain lanes (lane = row * BT + batch).
+  const int chain_row = lane / BT;
+  const int chain_b = lane - chain_row * BT;
+  const bool chain_lane = lane < kTileRows * BT;
+  const int chain_n = min(min(group, groups - 1) * kTileRows + min(chain_row, kTileRows - 1),
+                          a.out_depth - 1);
+  const float kfsum_n = a.kfsum[chain_n];
+  const float bias_n = a.bias ? a.bias[chain_n] : 0.0f;
+
+  // Activation rows into LDS.
+  if (FUSED) {
+    if (in_regs) {
+#pragma unroll
+      for (int b = 0; b < BT; ++b) {
+        float mn = 0.0f, mx = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kGroupsPerThread; ++j) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const float4 t = xr[b][j][h];  // clamped duplicates past the row are harmless here
+            mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
+            mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
+          }
+        }
+        mn = WaveMinF32(mn);
+        mx = WaveMaxF32(mx);
+        if (lane == 0) {
+          sh.mm[(b * kWaves + wave) * 2] = mn;
+          sh.mm[(b * kWaves + wave) * 2 + 1] = mx;
+        }
+      }
+    }
+    __syncthreads();
+    if (tid < bt) {
+      float mn = sh.mm[tid * kWaves * 2], mx = sh.mm[tid * kWaves * 2 + 1];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) {
+        mn = fminf(mn, sh.mm[(tid * kWaves + w) * 2]);
+        mx = fmaxf(mx, sh.mm[(tid * kWaves + w) * 2 + 1]);
+      }
+      const RowQuantParams qp = AsymmetricRowParams<VARIANT>(mn, mx);
+      sh.sf[tid] = qp.scale;
+      sh.inv[tid] = ElementwiseInv(qp);
+      sh.zp[tid] = qp.zero_point;
+      sh.zero[tid] = qp.all_zero ? 1 : 0;
+    }
+    __syncthreads();
+    const int vector_end = depth - (depth % 8);
+    if (in_regs) {
+#pragma unroll
+      for (int b = 0; b < BT; ++b) {
+        if (b < bt) {
+          RowQuantParams qp;
+          qp.scale = sh.sf[b];
+          qp.inv = sh.inv[b];
+          qp.zero_point = sh.zp[b];
+          qp.all_zero = sh.zero[b] != 0;
+#pragma unroll
+          for (int j = 0; j < kGroupsPerThread; ++j) {
+            const int g = j * kThreads + tid;
+            if (g < padded / 8) {
+              int32_t even = 0, odd = 0;
+              if (g < groups8) {
+                const float4 lo = xr[b][j][0], hi = xr[b][j][1];
+                const bool tail = g * 8 >= vector_end;
+                even = PackBytes(QuantizeElement<VARIANT>(lo.x, qp, true, tail),
+                                 QuantizeElement<VARIANT>(lo.z, qp, true, tail),
+                                 QuantizeElement<VARIANT>(hi.x, qp, true, tail),
+                                 QuantizeElement<VARIANT>(hi.z, qp, true, tail));
+                odd = PackBytes(QuantizeElement<VARIANT>(lo.y, qp, true, tail),
+                                QuantizeElement<VARIANT>(lo.w, qp, true, tail),
+                                QuantizeElement<VARIANT>(hi.y, qp, true, tail),
+                                QuantizeElement<VARIANT>(hi.w, qp, true, tail));
+              }
+              *reinterpret_cast<i32x2*>(sh.q + b * (padded / 4) + 2 * g) = i32x2{even, odd};
+            }
+          }
+        }
+      }
+    } else {
+      for (int b = 0; b < bt; ++b) {
+        const float* x = a.input_f32 + static_cast<size_t>(batch0 + b) * depth;
+        RowQuantParams qp;
+        qp.scale = sh.sf[b];
+        qp.inv = sh.inv[b];
+        qp.zero_point = sh.zp[b];
+        qp.all_zero = sh.zero[b] != 0;
+        for (int g = tid; g < padded / 8; g += kThreads) {
+          int32_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+          if (g < groups8) {
+            for (int t = 0; t < 8; ++t) {
+              v[t] = QuantizeElement<VARIANT>(x[g * 8 + t], qp, true, g * 8 + t >= vector_end);
+            }
+          }
+          sh.q[b * (padded / 4) + 2 * g] = PackBytes(v[0], v[2], v[4], v[6]);
+          sh.q[b * (padded / 4) + 2 * g + 1] = PackBytes(v[1], v[3], v[5], v[7]);
+        }
+      }
+    }
+  } else if (in_regs) {
+#pragma unroll
+    for (int b = 0; b < BT; ++b) {
+      if (b < bt) {
+#pragma unroll
+        for (int j = 0; j < kGroupsPerThread; ++j) {
+          const int g = j * kThreads + tid;
+          if (g < padded / 8) {
+            int32_t even = 0, odd = 0;
+            if (g < groups8) {
+              Deinterleave(static_cast<uint32_t>(qr[b][j].x), static_cast<uint32_t>(qr[b][j].y),
+                           &even, &odd);
+            }
+            *reinterpret_cast<i32x2*>(sh.q + b * (padded / 4) + 2 * g) = i32x2{even, odd};
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  float row_scale = 0.0f;
+  float row_zp = 0.0f;
+  if (chain_lane && chain_b < bt) {
+    row_scale = FUSED ? sh.sf[chain_b] : a.scaling_factors[batch0 + chain_b];
+    row_zp = static_cast<float>(FUSED ? sh.zp[chain_b] : a.zero_points[batch0 + chain_b]);
+  }
+
+  // Tile loop. Lane L owns block L of the tile for each of the 8 channels.
+  float* pw = sh.p + static_cast<size_t>(wave) * 8 * BT * kPStride;
+  float out = 0.0f;
+  const int nblk = depth / kBlock;
+  for (int c = 0; c < chunks; ++c) {
+    const int slot = c % kRingTiles;
+    // This block's activations (8 dwords per batch row) and 8 * sum(q).
+    i32x4 qe[BT], qo[BT];
+    int32_t qsum8[BT];
+    const int blk = c * kTileBlocks + lane;
+#pragma unroll
+    for (int b = 0; b < BT; ++b) {
+      const i32x4* qp = reinterpret_cast<const i32x4*>(sh.q + b * (padded / 4) + blk * 8);
+      qe[b] = qp[0];
+      qo[b] = qp[1];
+      int32_t s = 0;
+      s = Dot4(qe[b].x, 0x01010101, s);
+      s = Dot4(qe[b].y, 0x01010101, s);
+      s = Dot4(qe[b].z, 0x01010101, s);
+      s = Dot4(qe[b].w, 0x01010101, s);
+      s = Dot4(qo[b].x, 0x01010101, s);
+      s = Dot4(qo[b].y, 0x01010101, s);
+      s = Dot4(qo[b].z, 0x01010101, s);
+      s = Dot4(qo[b].w, 0x01010101, s);
+      qsum8[b] = 8 * s;
+    }
+#pragma unroll
+    for (int t = 0; t < kRingTiles; ++t) {
+      if (t == slot) {  // static ring indexing
+        const i32x4 sc = ring[t][kTileRows];
+#pragma unroll
+        for (int j = 0; j < kTileRows; ++j) {
+          const uint32_t pair = static_cast<uint32_t>(sc[j >> 1]);
+          const float scale = HalfBitsToFloatFast(static_cast<uint16_t>((j & 1) ? (pair >> 16) : (pair & 0xFFFF)));
+          const i32x4 wv = ring[t][j];
+          uint32_t lo[4], hi[4];
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            lo[d] = static_cast<uint32_t>(wv[d]) & 0x0F0F0F0Fu;
+            hi[d] = (static_cast<uint32_t>(wv[d]) >> 4) & 0x0F0F0F0Fu;
+          }
+#pragma unroll
+          for (int b = 0; b < BT; ++b) {
+            int32_t acc = -qsum8[b];
+            acc = Dot4(lo[0], qe[b].x, acc);
+            acc = Dot4(hi[0], qe[b].y, acc);
+            acc = Dot4(lo[1], qe[b].z, acc);
+            acc = Dot4(hi[1], qe[b].w, acc);
+            acc = Dot4(lo[2], qo[b].x, acc);
+            acc = Dot4(hi[2], qo[b].y, acc);
+            acc = Dot4(lo[3], qo[b].z, acc);
+            acc = Dot4(hi[3], qo[b].w, acc);
+            pw[(j * BT + b) * kPStride + lane] = __fmul_rn(static_cast<float>(acc), scale);
+          }
+        }
+        // Refill the slot with the tile two ahead.
+        if (c + kRingTiles < chunks) {
+#pragma unroll
+          for (int j = 0; j < kPlanes; ++j) {
+            ring[t][j] = __builtin_nontemporal_load(
+                tbase + static_cast<size_t>(c + kRingTiles) * kTileVecs + j * 64);
+          }
+        }
+      }
+    }
+    // Ordered float32 accumulation over this tile's blocks (same wavefront wrote them).
+    if (chain_lane) {
+      const int count = min(kTileBlocks, nblk - c * kTileBlocks);
+      const float* line = pw + lane * kPStride;
+      if (count == kTileBlocks) {
+        // Whole tile: fetch the 64 products with back-to-back LDS reads, then add in order.
+        float4 v[kTileBlocks / 4];
+#pragma unroll
+        for (int j = 0; j < kTileBlocks / 4; ++j) v[j] = reinterpret_cast<const float4*>(line)[j];
+#pragma unroll
+        for (int j = 0; j < kTileBlocks / 4; ++j) {
+          out = __fadd_rn(out, v[j].x);
+          out = __fadd_rn(out, v[j].y);
+          out = __fadd_rn(out, v[j].z);
+          out = __fadd_rn(out, v[j].w);
+        }
+      } else {
+        for (int j = 0; j < count; ++j) out = __fadd_rn(out, line[j]);
+      }
+    }
+  }
+
+  // fully_connected.cc:1078-1082.
+  if (chain_lane && chain_b < bt && group < groups) {
+    const int n = group * kTileRows + chain_row;
+    if (n < a.out_depth) {
+      out = __fsub_rn(out, __fmul_rn(row_zp, kfsum_n));
+      out = __fmul_rn(out, row_scale);
+      if (a.bias) out = __fadd_rn(out, bias_n);
+      a.output[static_cast<size_t>(batch0 + chain_b) * a.out_depth + n] = out;
+    }
+  }
+}
+
+template <int BT, bool FUSED, int VARIANT, int GPT>
+hipError_t LaunchOne(const Int4PackedArgs& a, int batch0, int bt, hipStream_t stream) {
+  const int padded = a.chunks * kTileBlocks * kBlock;
+  const size_t lds = Int4Shared<BT>::Bytes(padded);
+  auto kernel = FcInt4PackedKernel<BT, FUSED, VARIANT, GPT>;
+  if (lds > 48 * 1024) {
+    static size_t granted = 0;
+    if (lds > granted) {
+      hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(lds));
+      if (err != hipSuccess) return err;
+      granted = lds;
+    }
+  }
+  const int groups = (a.out_depth + kTileRows - 1) / kTileRows;
+  const int grid = (groups + kWaves - 1) / kWaves;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, batch0, bt);
+  return hipGetLastError();
+}
+
+template <int BT, bool FUSED, int GPT>
+hipError_t LaunchVariant(const Int4PackedArgs& a, int variant, int batch0, int bt,
+                         hipStream_t stream) {
+  if constexpr (!FUSED) {
+    return LaunchOne<BT, false, LRTFC_QUANT_PORTABLE, GPT>(a, batch0, bt, stream);
+  } else {
+    switch (variant) {
+    case LRTFC_QUANT_NEON_V8:
+      return LaunchOne<BT, FUSED, LRTFC_QUANT_NEON_V8, GPT>(a, batch0, bt, stream);
+    case LRTFC_QUANT_NEON_LEGACY:
+      return LaunchOne<BT, FUSED, LRTFC_QUANT_NEON_LEGACY, GPT>(a, batch0, bt, stream);
+    default:
+      return LaunchOne<BT, FUSED, LRTFC_QUANT_PORTABLE, GPT>(a, batch0, bt, stream);
+  }
+  }
+}
+
+// Depth up to 4096 keeps two groups per thread; up to 16384, eight. A fused launch holds
+// the float rows (16 registers per group and row), so its deep form stops at two rows.
+constexpr int kShallowDepth = 2 * kThreads * 8;
+constexpr int kDeepDepth = 8 * kThreads * 8;
+
+template <bool FUSED>
+int MaxBatchTile(int depth) {
+  return (FUSED && depth > kShallowDepth && depth <= kDeepDepth) ? 2 : 4;
+}
+
+template <bool FUSED>
+hipError_t LaunchTile(const Int4PackedArgs& a, int variant, int batch0, int bt,
+                      hipStream_t stream) {
+  if (a.depth > kShallowDepth && a.depth <= kDeepDepth) {
+    if (bt <= 1) return LaunchVariant<1, FUSED, 8>(a, variant, batch0, bt, stream);
+    if (bt <= 2) return LaunchVariant<2, FUSED, 8>(a, variant, batch0, bt, stream);
+    if (!FUSED) return LaunchVariant<4, false, 8>(a, variant, batch0, bt, stream);
+    return hipErrorInvalidValue;  // MaxBatchTile keeps fused deep launches at two rows
+  }
+  if (bt <= 1) return LaunchVariant<1, FUSED, 2>(a, variant, batch0, bt, stream);
+  if (bt <= 2) return LaunchVariant<2, FUSED, 2>(a, variant, batch0, bt, stream);
+  return LaunchVariant<4, FUSED, 2>(a, variant, batch0, bt, stream);
+}
+
+}  // namespace
+
+size_t PackedInt4BlockwiseBytes(int out_depth, int depth) {
+  const size_t groups = (static_cast<size_t>(out_depth) + kTileRows - 1) / kTileRows;
+  const size_t chunks = (static_cast<size_t>(depth) / kBlock + kTileBlocks - 1) / kTileBlocks;
+  return groups * chunks * kTileBytes;
+}
+
+hipError_t LaunchPackInt4Blockwise(const uint8_t* filter, const uint16_t* scales, int out_depth,
+                                   int depth, uint8_t* packed, hipStream_t stream) {
+  if (out_depth == 0 || depth == 0) return hipSuccess;
+  const int chunks = (depth / kBlock + kTileBlocks - 1) / kTileBlocks;
+  const int64_t total_vecs = static_cast<int64_t>(PackedInt4BlockwiseBytes(out_depth, depth) / 16);
+  const unsigned grid = static_cast<unsigned>((total_vecs + kThreads - 1) / kThreads);
+  hipLaunchKernelGGL(PackInt4BlockwiseKernel, dim3(grid), dim3(kThreads), 0, stream, filter,
+                     scales, out_depth, depth, chunks, total_vecs, packed);
+  return hipGetLastError();
+}
+
+bool FcInt4PackedSupports(int depth, int blocksize) {
+  if (blocksize != kBlock || depth <= 0 || depth % kBlock != 0) return false;
+  const int chunks = (depth / kBlock + kTileBlocks - 1) / kTileBlocks;
+  return Int4Shared<1>::Bytes(chunks * kTileBlocks * kBlock) <= 150 * 1024;
+}
+
+hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const float* input_f32,
+                              int variant, hipStream_t stream) {
+  if (q.batches == 0 || q.out_depth == 0) return hipSuccess;
+  if (!FcInt4PackedSupports(q.depth, q.blocksize)) return hipErrorNotSupported;
+  Int4PackedArgs a;
+  a.packed = packed;
+  a.input_f32 = input_f32;
+  a.input_q = q.input;
+  a.scaling_factors = q.scaling_factors;
+  a.zero_points = q.zero_points;
+  a.kfsum = q.kfsum;
+  a.bias = q.bias;
+  a.output = q.output;
+  a.batches = q.batches;
+  a.depth = q.depth;
+  a.out_depth = q.out_depth;
+  a.chunks = (q.depth / kBlock + kTileBlocks - 1) / kTileBlocks;
+  const int padded = a.chunks * kTileBlocks * kBlock;
+  int batch0 = 0;
+  while (batch0 < q.batches) {
+    int bt = min(input_f32 ? MaxBatchTile<true>(q.depth) : MaxBatchTile<false>(q.depth),
+                 q.batches - batch0);
+    while (bt > 1 && (bt > 2 ? Int4Shared<4>::Bytes(padded) : Int4Shared<2>::Bytes(padded)) >
+                         150 * 1024) {
+      bt = bt > 2 ? 2 : 1;
+    }
+    const hipError_t err = input_f32 ? LaunchTile<true>(a, variant, batch0, bt, stream)
+                                     : LaunchTile<false>(a, variant, batch0, bt, stream);
+    if (err != hipSuccess) return err;
+    batch0 += bt;
+  }
+  return hipSuccess;
+}
+
+}  // namespace lrtfc

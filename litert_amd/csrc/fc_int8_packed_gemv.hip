@@ -182,12 +182,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
   } else {
     const bool vec_ok = (depth % 16 == 0) && ((reinterpret_cast<uintptr_t>(a.input) & 15) == 0);
     in_regs = vec_ok && bt * (padded / 16) <= kQRegs * kThreads;
-#ifdef LRT_EXP_NOQ
-    in_regs = false;
-    if (false) {
-#else
     if (in_regs) {
-#endif
       const int chunks_per_row = padded / 16;
 #pragma unroll
       for (int j = 0; j < kQRegs; ++j) {
@@ -197,11 +192,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
         qr[j] = *reinterpret_cast<const i32x4*>(
             a.input + static_cast<size_t>(batch0 + min(b, bt - 1)) * depth + min(i, depth - 16));
       }
-#ifdef LRT_EXP_NOQ
-    } else if (false) {
-#else
     } else {
-#endif
       for (int b = 0; b < bt; ++b) {
         const int8_t* x = a.input + static_cast<size_t>(batch0 + b) * depth;
         int8_t* qrow = sh.q + b * qstride;
@@ -234,10 +225,6 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int n = min(min(tile, tiles - 1) * kTileRows + 4 * kgroup + i, a.out_depth - 1);
-#ifdef LRT_EXP_NOPARAM
-    ep_i0[i] = 1 << 30; ep_i1[i] = -5; ep_i2[i] = n; ep_i3[i] = 1; ep_f0[i] = 1.f; ep_f1[i] = 0.f;
-    continue;
-#endif
     if (EPI == Int8Epilogue::kRequantize) {
       ep_i0[i] = a.per_channel ? a.multipliers[n] : a.multipliers[0];
       ep_i1[i] = a.per_channel ? a.shifts[n] : a.shifts[0];
@@ -285,7 +272,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
       const RowQuantParams qp =
           p.asymmetric ? AsymmetricRowParams<VARIANT>(mn, mx) : SymmetricRowParams(mn, mx);
       sh.sf[tid] = qp.scale;
-      sh.inv[tid] = qp.inv;
+      sh.inv[tid] = ElementwiseInv(qp);
       sh.zp[tid] = qp.zero_point;
       sh.zero[tid] = qp.all_zero ? 1 : 0;
     }
@@ -383,11 +370,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-#ifdef LRT_EXP_NOMFMA
-        acc4[u] ^= ring[g + u] ^ bq[u];
-#else
         acc4[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ring[g + u], bq[u], acc4[u], 0, 0, 0);
-#endif
         ring[g + u] = __builtin_nontemporal_load(
             wbase + static_cast<size_t>(min(base + kRing + g + u, slabs - 1)) * 64);
       }
@@ -411,9 +394,6 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
   }
 
   // 5. Epilogue. Accumulator register i holds channel 4 * (L / 16) + i, column L % 16.
-#ifdef LRT_EXP_NOSTORE
-  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) != 0x12345678) return;
-#endif
   if (col >= bt || tile >= tiles) return;
   const int b = batch0 + col;
 #pragma unroll

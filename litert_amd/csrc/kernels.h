@@ -80,6 +80,16 @@ hipError_t LaunchBlockwiseInt4Kfsum(const uint8_t* packed_filter, const uint16_t
                                     hipStream_t stream);
 hipError_t LaunchFcBlockwiseInt4(const FcInt4Args& a, hipStream_t stream);
 
+// Streaming kernel on a filter re-tiled by LaunchPackInt4Blockwise (block size 32).
+// input_f32 != nullptr quantizes the rows in-kernel; otherwise q.input/scaling_factors/
+// zero_points are used.
+size_t PackedInt4BlockwiseBytes(int out_depth, int depth);
+hipError_t LaunchPackInt4Blockwise(const uint8_t* filter, const uint16_t* scales, int out_depth,
+                                   int depth, uint8_t* packed, hipStream_t stream);
+bool FcInt4PackedSupports(int depth, int blocksize);
+hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const float* input_f32,
+                              int variant, hipStream_t stream);
+
 }  // namespace lrtfc
 
 #endif  // LITERT_AMD_CSRC_KERNELS_H_

@@ -75,6 +75,15 @@ __device__ __forceinline__ RowQuantParams SymmetricRowParams(float mn, float mx)
   return p;
 }
 
+// std::round (nearest, ties away from zero) in five VALU operations. trunc, the
+// subtraction and the +-1 step are all exact in float, so this is bit-identical to roundf.
+__device__ __forceinline__ float RoundHalfAway(float x) {
+  const float t = truncf(x);
+  const float frac = x - t;
+  const float step = copysignf(1.0f, x);
+  return fabsf(frac) >= 0.5f ? t + step : t;
+}
+
 // The rounding used inside the NEON loops (neon_tensor_utils.cc:2347-2359).
 template <int VARIANT>
 __device__ __forceinline__ int32_t RoundToNearest(float x) {
@@ -82,7 +91,7 @@ __device__ __forceinline__ int32_t RoundToNearest(float x) {
     const float nudge = __fadd_rn(x < 0.0f ? -1.0f : 0.0f, 0.5f);
     return static_cast<int32_t>(__fadd_rn(x, nudge));  // truncation
   }
-  return static_cast<int32_t>(roundf(x));
+  return static_cast<int32_t>(RoundHalfAway(x));
 }
 
 // in_tail: the element belongs to the last n % 8 of the row, which the NEON builds
@@ -93,9 +102,9 @@ __device__ __forceinline__ int32_t QuantizeAsym(float v, float inv, int32_t zp, 
   if (VARIANT == LRTFC_QUANT_PORTABLE) {
     // portable_tensor_utils.cc:112-118: float multiply, float add, then round half
     // away. An FMA here would change results.
-    q = static_cast<int32_t>(roundf(__fadd_rn(static_cast<float>(zp), __fmul_rn(v, inv))));
+    q = static_cast<int32_t>(RoundHalfAway(__fadd_rn(static_cast<float>(zp), __fmul_rn(v, inv))));
   } else if (in_tail) {
-    q = static_cast<int32_t>(__fadd_rn(static_cast<float>(zp), roundf(__fmul_rn(inv, v))));
+    q = static_cast<int32_t>(__fadd_rn(static_cast<float>(zp), RoundHalfAway(__fmul_rn(inv, v))));
   } else {
     q = RoundToNearest<VARIANT>(__fmul_rn(v, inv)) + zp;
   }
@@ -106,19 +115,27 @@ template <int VARIANT>
 __device__ __forceinline__ int32_t QuantizeSym(float v, float inv, bool in_tail) {
   int32_t q;
   if (VARIANT == LRTFC_QUANT_PORTABLE || in_tail) {
-    q = static_cast<int32_t>(roundf(__fmul_rn(v, inv)));
+    q = static_cast<int32_t>(RoundHalfAway(__fmul_rn(v, inv)));
   } else {
     q = RoundToNearest<VARIANT>(__fmul_rn(v, inv));
   }
   return min(127, max(-127, q));
 }
 
+// An all-zero row (scale 1, zero point 0, every value 0) needs no branch: callers pass
+// inv = 0 for it (see ElementwiseInv), and round(0 + v * 0) is 0 for the finite zeros of such
+// a row. With zero point 0 the asymmetric expression is also what the symmetric one computes,
+// up to its clamp at -127, so one code path serves both.
 template <int VARIANT>
 __device__ __forceinline__ int32_t QuantizeElement(float v, const RowQuantParams& p,
                                                    bool asymmetric, bool in_tail) {
-  if (p.all_zero) return 0;
-  return asymmetric ? QuantizeAsym<VARIANT>(v, p.inv, p.zero_point, in_tail)
-                    : QuantizeSym<VARIANT>(v, p.inv, in_tail);
+  const int32_t q = QuantizeAsym<VARIANT>(v, p.inv, p.zero_point, in_tail);
+  return asymmetric ? q : max(q, -127);
+}
+
+// The multiplier the elementwise pass should use for a row.
+__device__ __forceinline__ float ElementwiseInv(const RowQuantParams& p) {
+  return p.all_zero ? 0.0f : p.inv;
 }
 
 // Four quantized values packed little-endian into one dword.

@@ -225,7 +225,7 @@ class FullyConnectedBlockwiseInt4:
     """
 
     def __init__(self, packed_filter, scales_f16, depth, blocksize=32, bias=None,
-                 quant_variant=capi.QUANT_PORTABLE):
+                 quant_variant=capi.QUANT_PORTABLE, packed=True):
         _ensure_init()
         self.filter = _dev(packed_filter, torch.uint8)
         self.out_depth = self.filter.shape[0]
@@ -245,6 +245,17 @@ class FullyConnectedBlockwiseInt4:
             _ptr(self.filter), _ptr(self.scales), self.out_depth, self.depth, self.blocksize,
             _ptr(self.kfsum), _stream()))
         self._ws = None
+        # packed: one fused kernel on the re-tiled filter (block size 32 only); otherwise the
+        # two-kernel form on the reference layout.
+        self.retiled = None
+        if packed and self.blocksize == 32 and self.depth % 32 == 0:
+            lib = capi.load()
+            self.retiled = torch.empty(
+                lib.lrtfc_packed_int4_blockwise_bytes(self.out_depth, self.depth),
+                dtype=torch.uint8, device="cuda")
+            capi.check(lib.lrtfc_pack_int4_blockwise(_ptr(self.filter), _ptr(self.scales),
+                                                     self.out_depth, self.depth, 32,
+                                                     _ptr(self.retiled), _stream()))
 
     def _workspace(self, batches):
         need = capi.load().lrtfc_activation_workspace_bytes(batches, self.depth)
@@ -257,9 +268,29 @@ class FullyConnectedBlockwiseInt4:
         batches = x.numel() // self.depth
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
+        if self.retiled is not None:
+            capi.check(capi.load().lrtfc_fc_blockwise_int4_packed(
+                _ptr(x), _ptr(self.retiled), _ptr(self.kfsum), _ptr(self.bias), _ptr(out), batches,
+                self.depth, self.out_depth, self.variant, _stream()))
+            return out
         ws = self._workspace(batches)
         capi.check(capi.load().lrtfc_fc_blockwise_int4(
             _ptr(x), _ptr(self.filter), _ptr(self.scales), _ptr(self.kfsum), _ptr(self.bias),
             _ptr(out), batches, self.depth, self.out_depth, self.blocksize, self.variant,
             _ptr(ws), ws.numel(), _stream()))
+        return out
+
+    def call_split(self, x, out=None):
+        """Two launches on the re-tiled filter: the standalone row quantizer, then the
+        streaming kernel on its int8 output. Same results as the fused call."""
+        if self.retiled is None:
+            raise RuntimeError("call_split needs the re-tiled filter (packed=True, block size 32)")
+        x = x.contiguous()
+        batches = x.numel() // self.depth
+        if out is None:
+            out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
+        q, sf, zp = batch_quantize_floats(x.reshape(batches, self.depth), True, self.variant)
+        capi.check(capi.load().lrtfc_fc_blockwise_int4_packed_quantized(
+            _ptr(q), _ptr(sf), _ptr(zp), _ptr(self.retiled), _ptr(self.kfsum), _ptr(self.bias),
+            _ptr(out), batches, self.depth, self.out_depth, _stream()))
         return out

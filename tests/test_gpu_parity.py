@@ -302,10 +302,10 @@ def test_hybrid_full_size_properties(fc):
 
 # ---- blockwise int4 -------------------------------------------------------------------------
 
-def _run_int4(fc, c, bias=None):
+def _run_int4(fc, c, bias=None, packed=True):
     N = c["w"].shape[0]
     op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], c["w"].shape[1], c["blocksize"],
-                                        bias)
+                                        bias, packed=packed)
     y = op(_cuda(c["x"])).cpu().numpy()
     want = oracle.fc_blockwise_int4(c["x"], c["packed"], N, c["scales"].view(np.uint16),
                                     c["blocksize"], bias)
@@ -314,14 +314,28 @@ def _run_int4(fc, c, bias=None):
 
 @pytest.mark.parametrize("B,K,N", [(1, 4096, 1024), (4, 2048, 512), (1, 2048, 256), (4, 16384, 64),
                                    (1, 16384, 130), (2, 32, 4), (3, 96, 9), (8, 1024, 77),
-                                   (5, 4096, 40), (1, 8192, 31)])
-def test_blockwise_int4_shapes(fc, B, K, N):
+                                   (5, 4096, 40), (1, 8192, 31), (9, 2048, 20), (2, 6144, 24),
+                                   (3, 16384, 24), (2, 8192, 16), (1, 32768, 12), (2, 20480, 8)])
+@pytest.mark.parametrize("packed", [True, False])
+def test_blockwise_int4_shapes(fc, B, K, N, packed):
     """Config 3 / config 5 depths (2048, 4096, 16384) and ragged sizes, blocksize 32, with the
     full signed nibble range including -8."""
     c = wl.blockwise_int4_fc(B, K, N, seed=11 + B + K + N, lo=-8, hi=7)
     bias = np.random.default_rng(4).standard_normal(N).astype(np.float32) if N % 2 else None
-    y, want = _run_int4(fc, c, bias)
+    y, want = _run_int4(fc, c, bias, packed=packed)
     assert _close(y, want)
+    assert _bits_equal(y, want)
+
+
+@pytest.mark.parametrize("B,K,N", [(1, 4096, 72), (4, 2048, 33), (4, 16384, 16), (3, 8192, 9),
+                                   (7, 1056, 24), (2, 20480, 8)])
+def test_blockwise_int4_split_launch_matches_oracle(fc, B, K, N):
+    """Standalone quantizer + streaming kernel on pre-quantized rows (the form used for deep
+    rows with more than two batch rows)."""
+    c = wl.blockwise_int4_fc(B, K, N, seed=3 + B + K + N, lo=-8, hi=7)
+    op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], K, 32)
+    y = op.call_split(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_blockwise_int4(c["x"], c["packed"], N, c["scales"].view(np.uint16), 32)
     assert _bits_equal(y, want)
 
 
@@ -333,12 +347,24 @@ def test_blockwise_int4_other_block_sizes(fc, B, K, N, bs):
     assert _bits_equal(y, want)
 
 
-def test_blockwise_int4_subnormal_and_large_scales(fc):
+@pytest.mark.parametrize("variant", [1, 2])
+def test_blockwise_int4_fused_quantizer_variants(fc, variant):
+    c = wl.blockwise_int4_fc(3, 1056, 24, seed=8)
+    c["x"][0, :4] = [-125.0, 130.0, 2.5, -2.5]
+    op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], 1056, 32, quant_variant=variant)
+    y = op(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_blockwise_int4(c["x"], c["packed"], 24, c["scales"].view(np.uint16), 32,
+                                    variant=variant)
+    assert _bits_equal(y, want)
+
+
+@pytest.mark.parametrize("packed", [True, False])
+def test_blockwise_int4_subnormal_and_large_scales(fc, packed):
     c = wl.blockwise_int4_fc(2, 256, 16, seed=3)
     s = c["scales"].view(np.uint16).copy()
     s[0, :] = [0x0001, 0x03FF, 0x0400, 0x7BFF, 0x8001, 0x0000, 0x3C00, 0xBC00]  # subnormals, max, -0...
     c["scales"] = s.view(np.float16)
-    y, want = _run_int4(fc, c)
+    y, want = _run_int4(fc, c, packed=packed)
     assert _bits_equal(y, want)
 
 
