@@ -105,6 +105,19 @@ int lrtfc_blockwise_int4_kfsum(const uint8_t* packed_filter, const uint16_t* sca
                                int out_depth, int depth, int blocksize, float* kfsum,
                                void* stream);
 
+/* Which filter layout the Eval entry points run fastest on for a shape: the row-major
+ * tensor as the model stores it, or the re-tiled copy made by lrtfc_pack_int8_filter /
+ * lrtfc_pack_int4_blockwise. The choice stands where the reference picks a kernel path
+ * per shape (tflite/kernels/cpu_backend_gemm.h:116-160 routes matrix-vector products to
+ * a custom GEMV and the rest to ruy). Pure host functions; no device needed.
+ *   int8 / hybrid: row-major for prefill batches the MFMA GEMM tiles (batches a multiple
+ *   of 128, out_depth of 256, depth of 128, symmetric filter) and for per-tensor filters
+ *   with a non-zero zero point; packed otherwise. Hybrid callers pass filter_offset 0.
+ *   blockwise int4: packed for block size 32 dividing the depth. */
+enum { LRTFC_LAYOUT_ROW_MAJOR = 0, LRTFC_LAYOUT_PACKED = 1 };
+int lrtfc_fc_int8_preferred_layout(int batches, int depth, int out_depth, int32_t filter_offset);
+int lrtfc_fc_blockwise_int4_preferred_layout(int depth, int blocksize);
+
 /* Re-tiles a row-major int8 filter [out_depth, depth] for the matrix-core GEMV: tiles of
  * 16 output channels x 64 depth (1 KiB each, zero-padded at the edges), the 16 bytes of
  * lane L inside a tile being channel L % 16, depth 16 * (L / 16) .. +16; tiles of one
@@ -165,6 +178,16 @@ int lrtfc_fc_hybrid_int8(const int8_t* quantized_input, const float* scaling_fac
                          const float* per_channel_scales, float filter_scale,
                          const int32_t* filter_row_sums, const float* bias, float* output,
                          int batches, int depth, int out_depth, int activation, void* stream);
+
+/* lrtfc_fc_hybrid_int8 on a packed filter (lrtfc_pack_int8_filter): the form for batches
+ * whose rows were quantized by a separate lrtfc_batch_quantize_floats launch. Replaces the
+ * same reference functions as lrtfc_fc_hybrid_int8. */
+int lrtfc_fc_hybrid_int8_packed(const int8_t* quantized_input, const float* scaling_factors,
+                                const int32_t* zero_points, const int8_t* packed_filter,
+                                const float* per_channel_scales, float filter_scale,
+                                const int32_t* filter_row_sums, const float* bias, float* output,
+                                int batches, int depth, int out_depth, int activation,
+                                void* stream);
 
 /* Bytes of device scratch lrtfc_fc_hybrid / lrtfc_fc_blockwise_int4 need for
  * (batches, depth): quantized activations, scaling factors and zero points. */

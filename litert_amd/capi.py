@@ -30,6 +30,8 @@ SYMBOLS = [
     ("lrtfc_row_sums_int8", _i, [_vp, _i, _i, _vp, _vp]),
     ("lrtfc_unpack_int4", _i, [_vp, _i64, _vp, _vp]),
     ("lrtfc_blockwise_int4_kfsum", _i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    ("lrtfc_fc_int8_preferred_layout", _i, [_i, _i, _i, _i]),
+    ("lrtfc_fc_blockwise_int4_preferred_layout", _i, [_i, _i]),
     ("lrtfc_packed_int8_filter_bytes", _sz, [_i, _i]),
     ("lrtfc_pack_int8_filter", _i, [_vp, _i, _i, _vp, _vp]),
     ("lrtfc_fc_int8_packed", _i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i32, _i32,
@@ -41,6 +43,8 @@ SYMBOLS = [
     ("lrtfc_batch_quantize_floats", _i, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp]),
     ("lrtfc_fc_hybrid_int8", _i, [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i,
                                   _vp]),
+    ("lrtfc_fc_hybrid_int8_packed", _i, [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i,
+                                         _i, _vp]),
     ("lrtfc_activation_workspace_bytes", _sz, [_i, _i]),
     ("lrtfc_fc_hybrid", _i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz,
                              _vp]),

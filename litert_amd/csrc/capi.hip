@@ -288,6 +288,21 @@ int lrtfc_fc_int8(const int8_t* input, const int8_t* filter, const int32_t* bias
       "int8 GEMV");
 }
 
+int lrtfc_fc_int8_preferred_layout(int batches, int depth, int out_depth, int32_t filter_offset) {
+  lrtfc::FcInt8Args a{};
+  a.batches = batches;
+  a.depth = depth;
+  a.out_depth = out_depth;
+  a.filter_offset = filter_offset;
+  if (batches >= kGemmMinBatches && lrtfc::FcInt8GemmMfmaSupports(a)) return LRTFC_LAYOUT_ROW_MAJOR;
+  return lrtfc::FcInt8PackedGemvSupports(a) ? LRTFC_LAYOUT_PACKED : LRTFC_LAYOUT_ROW_MAJOR;
+}
+
+int lrtfc_fc_blockwise_int4_preferred_layout(int depth, int blocksize) {
+  return lrtfc::FcInt4PackedSupports(depth, blocksize) ? LRTFC_LAYOUT_PACKED
+                                                       : LRTFC_LAYOUT_ROW_MAJOR;
+}
+
 size_t lrtfc_packed_int8_filter_bytes(int out_depth, int depth) {
   if (out_depth <= 0 || depth <= 0) return 0;
   return lrtfc::PackedInt8FilterBytes(out_depth, depth);
@@ -370,6 +385,41 @@ int lrtfc_fc_hybrid_packed(const float* input, const int8_t* packed_filter,
   return FromHip(lrtfc::LaunchFcInt8PackedGemv(a, lrtfc::Int8Epilogue::kHybrid, input,
                                                asymmetric_quantize_inputs, quant_variant,
                                                AsStream(stream)),
+                 "packed hybrid GEMV");
+}
+
+int lrtfc_fc_hybrid_int8_packed(const int8_t* quantized_input, const float* scaling_factors,
+                                const int32_t* zero_points, const int8_t* packed_filter,
+                                const float* per_channel_scales, float filter_scale,
+                                const int32_t* filter_row_sums, const float* bias, float* output,
+                                int batches, int depth, int out_depth, int activation,
+                                void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(quantized_input && scaling_factors && packed_filter && output, "null pointer");
+  LRTFC_REQUIRE(!zero_points || filter_row_sums,
+                "filter_row_sums is required with activation zero points");
+  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(packed_filter) & 15) == 0,
+                "packed filter must be 16-byte aligned");
+  lrtfc::FcInt8Args a{};
+  a.input = quantized_input;
+  a.filter = packed_filter;
+  a.batches = batches;
+  a.depth = depth;
+  a.out_depth = out_depth;
+  a.filter_row_sums = filter_row_sums;
+  a.scaling_factors = scaling_factors;
+  a.zero_points = zero_points;
+  a.per_channel_scales = per_channel_scales;
+  a.filter_scale = filter_scale;
+  a.bias_f32 = bias;
+  a.activation = activation;
+  a.output_f32 = output;
+  return FromHip(lrtfc::LaunchFcInt8PackedGemv(a, lrtfc::Int8Epilogue::kHybrid, nullptr, 0,
+                                               LRTFC_QUANT_PORTABLE, AsStream(stream)),
                  "packed hybrid GEMV");
 }
 

@@ -217,10 +217,20 @@ struct FcNode {
   bool per_channel = false;
   float filter_scale = 1.0f;
   int32_t input_offset = 0, filter_offset = 0, output_offset = 0, act_min = 0, act_max = 0;
-  const void* uploaded_filter = nullptr;  // host pointer the device copy was made from
-  DeviceBuffer filter_dev, bias_dev, mult_dev, shift_dev, row_sums_dev, pcs_dev, scales_dev,
-      kfsum_dev;
+  const void* uploaded_filter = nullptr;  // host pointer the device copies were made from
+  // The filter lives on the device in the layout the node's shape runs fastest on: the
+  // model's own (row-major / nibble-packed rows) or the re-tiled copy. Only one is kept.
+  bool have_model_layout = false, have_retiled = false, use_retiled = false;
+  bool split_quantize = false;  // quantize rows in a launch of their own, not in the prologue
+  DeviceBuffer filter_dev, retiled_dev, bias_dev, mult_dev, shift_dev, row_sums_dev, pcs_dev,
+      scales_dev, kfsum_dev;
 };
+
+// Rows above which the fused kernels' prologue (every workgroup quantizes every row) costs
+// more than a separate quantization launch; deep int4 rows fuse at most two batch rows.
+constexpr int kHybridFusedMaxBatches = 4;
+constexpr int kInt4FusedMaxDepth = 4096;
+constexpr int kInt4DeepFusedMaxBatches = 2;
 
 struct PartitionKernel {
   DelegateState* state = nullptr;
@@ -310,6 +320,44 @@ void KernelFree(TfLiteContext* /*ctx*/, void* buffer) {
   if (buffer && buffer != reinterpret_cast<void*>(-1)) delete static_cast<PartitionKernel*>(buffer);
 }
 
+// The workspace of lrtfc_activation_workspace_bytes(batches, depth) bytes, carved as the
+// library carves it: quantized rows, then scaling factors, then zero points, each region
+// starting on a 256-byte boundary.
+struct ActivationScratch {
+  int8_t* q;
+  float* sf;
+  int32_t* zp;
+};
+
+ActivationScratch SplitScratch(void* workspace, int batches, int depth) {
+  auto round_up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+  auto* base = static_cast<uint8_t*>(workspace);
+  ActivationScratch w;
+  w.q = reinterpret_cast<int8_t*>(base);
+  const size_t q_bytes = round_up(static_cast<size_t>(batches) * depth);
+  w.sf = reinterpret_cast<float*>(base + q_bytes);
+  w.zp = reinterpret_cast<int32_t*>(base + q_bytes + round_up(static_cast<size_t>(batches) * 4));
+  return w;
+}
+
+#define RETURN_IF_OK(expr)                      \
+  do {                                          \
+    const TfLiteStatus st__ = (expr);           \
+    if (st__ != kTfLiteOk) return st__;         \
+  } while (0)
+
+// Makes the re-tiled copy of an int8 filter from the row-major one and drops the latter.
+TfLiteStatus RetileInt8(TfLiteContext* ctx, FcNode* n, hipStream_t s) {
+  RETURN_IF_HIP(ctx, n->retiled_dev.Ensure(lrtfc_packed_int8_filter_bytes(n->out_depth, n->depth)));
+  RETURN_IF_FC(ctx, lrtfc_pack_int8_filter(n->filter_dev.as<int8_t>(), n->out_depth, n->depth,
+                                           n->retiled_dev.as<int8_t>(), s));
+  RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+  n->have_retiled = true;
+  n->filter_dev.Release();
+  n->have_model_layout = false;
+  return kTfLiteOk;
+}
+
 TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
   const TfLiteTensor& input = ctx->tensors[n->input];
   const TfLiteTensor& filter = ctx->tensors[n->filter];
@@ -330,7 +378,7 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
     return kTfLiteError;
   }
   hipStream_t s = k->stream;
-  const bool reupload = n->uploaded_filter != filter.data.raw;
+  if (n->uploaded_filter != filter.data.raw) n->have_model_layout = n->have_retiled = false;
   const size_t weights = static_cast<size_t>(n->out_depth) * n->depth;
 
   if (n->kind == FcKind::kInt8) {
@@ -356,32 +404,46 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
     RETURN_IF_HIP(ctx, n->mult_dev.Upload(mult.data(), mult.size() * 4, s));
     RETURN_IF_HIP(ctx, n->shift_dev.Upload(shift.data(), shift.size() * 4, s));
     RETURN_IF_HIP(ctx, hipStreamSynchronize(s));  // mult/shift are stack-owned
-    if (reupload && weights > 0) {
-      if (filter.type == kTfLiteInt4) {
-        // Unpacked once here; the builtin unpacks on every Eval (fully_connected.cc:1670-1677).
-        DeviceBuffer packed;
-        RETURN_IF_HIP(ctx, packed.Upload(filter.data.raw, (weights + 1) / 2, s));
-        RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
-        RETURN_IF_FC(ctx, lrtfc_unpack_int4(packed.as<uint8_t>(), static_cast<int64_t>(weights),
-                                            n->filter_dev.as<int8_t>(), s));
-        RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
-      } else {
-        RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
+    n->use_retiled = weights > 0 &&
+                     lrtfc_fc_int8_preferred_layout(n->batches, n->depth, n->out_depth,
+                                                    n->filter_offset) == LRTFC_LAYOUT_PACKED;
+    if (weights > 0 && !(n->use_retiled ? n->have_retiled : n->have_model_layout)) {
+      if (!n->have_model_layout) {
+        if (filter.type == kTfLiteInt4) {
+          // Unpacked once here; the builtin unpacks on every Eval (fully_connected.cc:1670-1677).
+          DeviceBuffer packed;
+          RETURN_IF_HIP(ctx, packed.Upload(filter.data.raw, (weights + 1) / 2, s));
+          RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
+          RETURN_IF_FC(ctx, lrtfc_unpack_int4(packed.as<uint8_t>(), static_cast<int64_t>(weights),
+                                              n->filter_dev.as<int8_t>(), s));
+          RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+        } else {
+          RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
+        }
+        RETURN_IF_HIP(ctx, n->row_sums_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
+        RETURN_IF_FC(ctx, lrtfc_row_sums_int8(n->filter_dev.as<int8_t>(), n->out_depth, n->depth,
+                                              n->row_sums_dev.as<int32_t>(), s));
+        n->have_model_layout = true;
       }
-      RETURN_IF_HIP(ctx, n->row_sums_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
-      RETURN_IF_FC(ctx, lrtfc_row_sums_int8(n->filter_dev.as<int8_t>(), n->out_depth, n->depth,
-                                            n->row_sums_dev.as<int32_t>(), s));
+      if (n->use_retiled) RETURN_IF_OK(RetileInt8(ctx, n, s));
     }
     if (bias) RETURN_IF_HIP(ctx, n->bias_dev.Upload(bias->data.raw, static_cast<size_t>(n->out_depth) * 4, s));
   } else if (n->kind == FcKind::kHybrid) {
     const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
     n->per_channel = fq->scale->size > 1;  // VerifyPerChannelQuantization, fully_connected.cc:827
     n->filter_scale = filter.params.scale;
-    if (reupload) {
-      RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
-      RETURN_IF_HIP(ctx, n->row_sums_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
-      RETURN_IF_FC(ctx, lrtfc_row_sums_int8(n->filter_dev.as<int8_t>(), n->out_depth, n->depth,
-                                            n->row_sums_dev.as<int32_t>(), s));
+    n->use_retiled = weights > 0 && lrtfc_fc_int8_preferred_layout(1, n->depth, n->out_depth, 0) ==
+                                        LRTFC_LAYOUT_PACKED;
+    n->split_quantize = n->batches > kHybridFusedMaxBatches;
+    if (weights > 0 && !(n->use_retiled ? n->have_retiled : n->have_model_layout)) {
+      if (!n->have_model_layout) {
+        RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
+        RETURN_IF_HIP(ctx, n->row_sums_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
+        RETURN_IF_FC(ctx, lrtfc_row_sums_int8(n->filter_dev.as<int8_t>(), n->out_depth, n->depth,
+                                              n->row_sums_dev.as<int32_t>(), s));
+        n->have_model_layout = true;
+      }
+      if (n->use_retiled) RETURN_IF_OK(RetileInt8(ctx, n, s));
     }
     if (n->per_channel) {
       RETURN_IF_HIP(ctx, n->pcs_dev.Upload(fq->scale->data, static_cast<size_t>(n->out_depth) * 4, s));
@@ -392,15 +454,34 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
     n->blocksize = bq->blocksize;
     n->scales = bq->scale;
     const TfLiteTensor& scales = ctx->tensors[bq->scale];
-    if (reupload) {
-      RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights / 2, s));
-      RETURN_IF_HIP(ctx, n->scales_dev.Upload(scales.data.raw,
-                                              static_cast<size_t>(NumElements(scales.dims)) * 2, s));
-      RETURN_IF_HIP(ctx, n->kfsum_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
-      RETURN_IF_FC(ctx, lrtfc_blockwise_int4_kfsum(n->filter_dev.as<uint8_t>(),
-                                                   n->scales_dev.as<uint16_t>(), n->out_depth,
-                                                   n->depth, n->blocksize,
-                                                   n->kfsum_dev.as<float>(), s));
+    n->use_retiled = weights > 0 && lrtfc_fc_blockwise_int4_preferred_layout(
+                                        n->depth, n->blocksize) == LRTFC_LAYOUT_PACKED;
+    n->split_quantize = n->depth > kInt4FusedMaxDepth && n->batches > kInt4DeepFusedMaxBatches;
+    if (weights > 0 && !(n->use_retiled ? n->have_retiled : n->have_model_layout)) {
+      if (!n->have_model_layout) {
+        RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights / 2, s));
+        RETURN_IF_HIP(ctx, n->scales_dev.Upload(scales.data.raw,
+                                                static_cast<size_t>(NumElements(scales.dims)) * 2, s));
+        RETURN_IF_HIP(ctx, n->kfsum_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
+        RETURN_IF_FC(ctx, lrtfc_blockwise_int4_kfsum(n->filter_dev.as<uint8_t>(),
+                                                     n->scales_dev.as<uint16_t>(), n->out_depth,
+                                                     n->depth, n->blocksize,
+                                                     n->kfsum_dev.as<float>(), s));
+        n->have_model_layout = true;
+      }
+      if (n->use_retiled) {
+        RETURN_IF_HIP(ctx, n->retiled_dev.Ensure(
+                               lrtfc_packed_int4_blockwise_bytes(n->out_depth, n->depth)));
+        RETURN_IF_FC(ctx, lrtfc_pack_int4_blockwise(n->filter_dev.as<uint8_t>(),
+                                                    n->scales_dev.as<uint16_t>(), n->out_depth,
+                                                    n->depth, n->blocksize,
+                                                    n->retiled_dev.as<uint8_t>(), s));
+        RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+        n->have_retiled = true;
+        n->filter_dev.Release();  // the scales travel inside the re-tiled copy
+        n->scales_dev.Release();
+        n->have_model_layout = false;
+      }
     }
     if (bias) RETURN_IF_HIP(ctx, n->bias_dev.Upload(bias->data.raw, static_cast<size_t>(n->out_depth) * 4, s));
   }
@@ -409,7 +490,7 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
   // Device homes for this node's activations.
   RETURN_IF_HIP(ctx, k->activations[n->input].Ensure(input.bytes));
   RETURN_IF_HIP(ctx, k->activations[n->output].Ensure(output.bytes));
-  if (n->kind != FcKind::kInt8) {
+  if (n->kind != FcKind::kInt8 && (!n->use_retiled || n->split_quantize)) {
     RETURN_IF_HIP(ctx, k->workspace.Ensure(lrtfc_activation_workspace_bytes(n->batches, n->depth)));
   }
   return kTfLiteOk;
@@ -447,38 +528,86 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     }
     const void* in_dev = k->activations[n.input].get();
     const bool has_bias = n.bias != kTfLiteOptionalTensor;
+    const int variant = k->state->options.quant_variant;
+    const float* bias_f32 = has_bias ? n.bias_dev.as<float>() : nullptr;
     switch (n.kind) {
       case FcKind::kInt8:
-        RETURN_IF_FC(ctx, lrtfc_fc_int8(static_cast<const int8_t*>(in_dev),
-                                        n.filter_dev.as<int8_t>(),
-                                        has_bias ? n.bias_dev.as<int32_t>() : nullptr,
-                                        n.mult_dev.as<int32_t>(), n.shift_dev.as<int32_t>(),
-                                        n.per_channel, n.row_sums_dev.as<int32_t>(),
-                                        static_cast<int8_t*>(out_dev), n.batches, n.depth,
-                                        n.out_depth, n.input_offset, n.filter_offset,
-                                        n.output_offset, n.act_min, n.act_max, s));
-        break;
-      case FcKind::kHybrid:
-        RETURN_IF_FC(ctx, lrtfc_fc_hybrid(static_cast<const float*>(in_dev),
+        if (n.use_retiled) {
+          RETURN_IF_FC(ctx, lrtfc_fc_int8_packed(static_cast<const int8_t*>(in_dev),
+                                                 n.retiled_dev.as<int8_t>(),
+                                                 has_bias ? n.bias_dev.as<int32_t>() : nullptr,
+                                                 n.mult_dev.as<int32_t>(), n.shift_dev.as<int32_t>(),
+                                                 n.per_channel, n.row_sums_dev.as<int32_t>(),
+                                                 static_cast<int8_t*>(out_dev), n.batches, n.depth,
+                                                 n.out_depth, n.input_offset, n.output_offset,
+                                                 n.act_min, n.act_max, s));
+        } else {
+          RETURN_IF_FC(ctx, lrtfc_fc_int8(static_cast<const int8_t*>(in_dev),
                                           n.filter_dev.as<int8_t>(),
-                                          n.per_channel ? n.pcs_dev.as<float>() : nullptr,
-                                          n.filter_scale, n.row_sums_dev.as<int32_t>(),
-                                          has_bias ? n.bias_dev.as<float>() : nullptr,
-                                          static_cast<float*>(out_dev), n.batches, n.depth,
-                                          n.out_depth, n.params.asymmetric_quantize_inputs,
-                                          n.params.activation, k->state->options.quant_variant,
-                                          k->workspace.get(), k->workspace.bytes(), s));
+                                          has_bias ? n.bias_dev.as<int32_t>() : nullptr,
+                                          n.mult_dev.as<int32_t>(), n.shift_dev.as<int32_t>(),
+                                          n.per_channel, n.row_sums_dev.as<int32_t>(),
+                                          static_cast<int8_t*>(out_dev), n.batches, n.depth,
+                                          n.out_depth, n.input_offset, n.filter_offset,
+                                          n.output_offset, n.act_min, n.act_max, s));
+        }
         break;
+      case FcKind::kHybrid: {
+        const float* pcs = n.per_channel ? n.pcs_dev.as<float>() : nullptr;
+        const int asym = n.params.asymmetric_quantize_inputs;
+        if (!n.use_retiled) {
+          RETURN_IF_FC(ctx, lrtfc_fc_hybrid(static_cast<const float*>(in_dev),
+                                            n.filter_dev.as<int8_t>(), pcs, n.filter_scale,
+                                            n.row_sums_dev.as<int32_t>(), bias_f32,
+                                            static_cast<float*>(out_dev), n.batches, n.depth,
+                                            n.out_depth, asym, n.params.activation, variant,
+                                            k->workspace.get(), k->workspace.bytes(), s));
+        } else if (!n.split_quantize) {
+          RETURN_IF_FC(ctx, lrtfc_fc_hybrid_packed(static_cast<const float*>(in_dev),
+                                                   n.retiled_dev.as<int8_t>(), pcs, n.filter_scale,
+                                                   n.row_sums_dev.as<int32_t>(), bias_f32,
+                                                   static_cast<float*>(out_dev), n.batches,
+                                                   n.depth, n.out_depth, asym, n.params.activation,
+                                                   variant, s));
+        } else {
+          const ActivationScratch w = SplitScratch(k->workspace.get(), n.batches, n.depth);
+          RETURN_IF_FC(ctx, lrtfc_batch_quantize_floats(static_cast<const float*>(in_dev),
+                                                        n.batches, n.depth, w.q, w.sf, w.zp, asym,
+                                                        variant, s));
+          RETURN_IF_FC(ctx, lrtfc_fc_hybrid_int8_packed(w.q, w.sf, asym ? w.zp : nullptr,
+                                                        n.retiled_dev.as<int8_t>(), pcs,
+                                                        n.filter_scale, n.row_sums_dev.as<int32_t>(),
+                                                        bias_f32, static_cast<float*>(out_dev),
+                                                        n.batches, n.depth, n.out_depth,
+                                                        n.params.activation, s));
+        }
+        break;
+      }
       case FcKind::kInt4Blockwise:
-        RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4(static_cast<const float*>(in_dev),
-                                                  n.filter_dev.as<uint8_t>(),
-                                                  n.scales_dev.as<uint16_t>(),
-                                                  n.kfsum_dev.as<float>(),
-                                                  has_bias ? n.bias_dev.as<float>() : nullptr,
-                                                  static_cast<float*>(out_dev), n.batches, n.depth,
-                                                  n.out_depth, n.blocksize,
-                                                  k->state->options.quant_variant,
-                                                  k->workspace.get(), k->workspace.bytes(), s));
+        if (!n.use_retiled) {
+          RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4(static_cast<const float*>(in_dev),
+                                                    n.filter_dev.as<uint8_t>(),
+                                                    n.scales_dev.as<uint16_t>(),
+                                                    n.kfsum_dev.as<float>(), bias_f32,
+                                                    static_cast<float*>(out_dev), n.batches,
+                                                    n.depth, n.out_depth, n.blocksize, variant,
+                                                    k->workspace.get(), k->workspace.bytes(), s));
+        } else if (!n.split_quantize) {
+          RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4_packed(static_cast<const float*>(in_dev),
+                                                           n.retiled_dev.as<uint8_t>(),
+                                                           n.kfsum_dev.as<float>(), bias_f32,
+                                                           static_cast<float*>(out_dev), n.batches,
+                                                           n.depth, n.out_depth, variant, s));
+        } else {
+          const ActivationScratch w = SplitScratch(k->workspace.get(), n.batches, n.depth);
+          RETURN_IF_FC(ctx, lrtfc_batch_quantize_floats(static_cast<const float*>(in_dev),
+                                                        n.batches, n.depth, w.q, w.sf, w.zp, 1,
+                                                        variant, s));
+          RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4_packed_quantized(
+                                w.q, w.sf, w.zp, n.retiled_dev.as<uint8_t>(),
+                                n.kfsum_dev.as<float>(), bias_f32, static_cast<float*>(out_dev),
+                                n.batches, n.depth, n.out_depth, s));
+        }
         break;
       default:
         return kTfLiteError;

@@ -62,7 +62,7 @@ def test_int8_node_config1_through_delegate():
         assert np.array_equal(h.read(y), _oracle_int8(c, np.roll(c["x"], 7, axis=1)))
 
 
-@pytest.mark.parametrize("B", [1, 4])
+@pytest.mark.parametrize("B", [1, 4, 8, 19])  # up to 4 rows fuse the quantizer, more split it off
 def test_hybrid_node_through_delegate(B):
     c = wl.hybrid_fc(B, 4096, 1024)
     bias = np.random.default_rng(1).standard_normal(1024).astype(np.float32)
@@ -80,21 +80,24 @@ def test_hybrid_node_through_delegate(B):
         assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
 
 
-def test_blockwise_int4_node_through_delegate():
-    c = wl.blockwise_int4_fc(2, 2048, 512, lo=-8, hi=7)
-    bias = np.random.default_rng(2).standard_normal(512).astype(np.float32)
+@pytest.mark.parametrize("B,K,N", [(2, 2048, 512), (1, 16384, 40), (3, 8192, 24), (5, 1024, 16)])
+def test_blockwise_int4_node_through_delegate(B, K, N):
+    """Shallow rows and up to two deep rows run the fused kernel on the re-tiled filter; three
+    or more deep rows are quantized by a launch of their own first."""
+    c = wl.blockwise_int4_fc(B, K, N, lo=-8, hi=7)
+    bias = np.random.default_rng(2).standard_normal(N).astype(np.float32)
     with FakeHost() as h:
-        x = h.tensor(FLOAT32, (2, 2048), data=c["x"])
-        w = h.tensor(INT4, (512, 2048), data=c["packed"], const=True)
-        s = h.tensor(FLOAT16, (512, 64), data=c["scales"], const=True)
+        x = h.tensor(FLOAT32, (B, K), data=c["x"])
+        w = h.tensor(INT4, (N, K), data=c["packed"], const=True)
+        s = h.tensor(FLOAT16, (N, K // 32), data=c["scales"], const=True)
         h.blockwise(w, s, 32)
-        b = h.tensor(FLOAT32, (512,), data=bias, const=True)
-        y = h.tensor(FLOAT32, (2, 512))
+        b = h.tensor(FLOAT32, (N,), data=bias, const=True)
+        y = h.tensor(FLOAT32, (B, N))
         h.fc(x, w, b, y, activation=1)  # the reference ignores the fused activation on this path
         assert h.load_delegate() == 0, h.errors()
         assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
         assert h.invoke() == OK, h.errors()
-        want = oracle.fc_blockwise_int4(c["x"], c["packed"], 512, c["scales"].view(np.uint16), 32, bias)
+        want = oracle.fc_blockwise_int4(c["x"], c["packed"], N, c["scales"].view(np.uint16), 32, bias)
         assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
         assert (want < 0).any()  # so an applied RELU would have shown
 
@@ -212,6 +215,48 @@ def test_resize_then_reprepare():
         assert h.allocate_tensors() == OK, h.errors()  # prepare runs again after a resize
         assert h.invoke() == OK, h.errors()
         assert np.array_equal(h.read(y), oracle.fc_hybrid(c["x"], c["w"], c["pcs"]))
+
+
+def test_blockwise_int4_other_block_size_keeps_model_layout():
+    c = wl.blockwise_int4_fc(2, 256, 24, blocksize=64, lo=-8, hi=7)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (2, 256), data=c["x"])
+        w = h.tensor(INT4, (24, 256), data=c["packed"], const=True)
+        s = h.tensor(FLOAT16, (24, 4), data=c["scales"], const=True)
+        h.blockwise(w, s, 64)
+        y = h.tensor(FLOAT32, (2, 24))
+        h.fc(x, w, None, y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.invoke() == OK, h.errors()
+        want = oracle.fc_blockwise_int4(c["x"], c["packed"], 24, c["scales"].view(np.uint16), 64)
+        assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+
+
+def test_int8_resize_between_decode_and_prefill_switches_filter_layout():
+    """One row runs on the re-tiled filter; 128 rows on the row-major one (MFMA GEMM); going
+    back re-tiles again. Each step is checked against the oracle."""
+    c = wl.int8_fc(128, 256, 256, seed=9)
+    with FakeHost() as h:
+        B, K = c["x"].shape
+        N = c["w"].shape[0]
+        x = h.tensor(INT8, (1, K), data=c["x"][:1])
+        h.affine(x, [c["in_scale"]], [c["in_zp"]])
+        w = h.tensor(INT8, (N, K), data=c["w"], const=True)
+        h.affine(w, c["w_scale"])
+        b = h.tensor(INT32, (N,), data=c["bias"], const=True)
+        y = h.tensor(INT8, (1, N))
+        h.affine(y, [c["out_scale"]], [c["out_zp"]])
+        h.fc(x, w, b, y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        for rows in (1, 128, 3):
+            h.resize(x, (rows, K))
+            h.resize(y, (rows, N))
+            h.write(x, c["x"][:rows])
+            assert h.allocate_tensors() == OK, h.errors()
+            assert h.invoke() == OK, h.errors()
+            assert np.array_equal(h.read(y), _oracle_int8(c, c["x"][:rows])), rows
 
 
 def test_prepare_failure_is_reported_not_hidden():

@@ -213,15 +213,26 @@ def test_batch_quantize_reference_kats_through_hip(fc):
 
 # ---- hybrid ----------------------------------------------------------------------------
 
+def _hybrid_call(op, x, mode):
+    """mode: "fused" (one kernel whatever the batch), "split" (quantizer launch + GEMV on the
+    packed filter), True (the class's own choice between those two), False (row-major)."""
+    if mode == "fused":
+        op.FUSED_MAX_BATCHES = 1 << 30
+        return op(x)
+    if mode == "split":
+        return op.call_split(x)
+    return op(x)
+
+
 @pytest.mark.parametrize("B", [1, 4, 8])
-@pytest.mark.parametrize("packed", [True, False])
+@pytest.mark.parametrize("packed", ["fused", "split", True, False])
 def test_hybrid_config2_shape(fc, B, packed):
     """Config 2 at its real depth with a reduced number of output channels (the scalar
     oracle needs ~60 ms per 1000 channels per batch row); the fused single-kernel form on
     the re-tiled filter and the two-kernel form on the row-major one."""
     c = wl.hybrid_fc(B, 4096, 2048)
-    op = fc.FullyConnectedHybrid(c["w"], c["pcs"], packed=packed)
-    y = op(_cuda(c["x"])).cpu().numpy()
+    op = fc.FullyConnectedHybrid(c["w"], c["pcs"], packed=bool(packed))
+    y = _hybrid_call(op, _cuda(c["x"]), packed).cpu().numpy()
     want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"])
     assert _close(y, want)
     assert _bits_equal(y, want)
@@ -232,15 +243,15 @@ def test_hybrid_config2_shape(fc, B, packed):
 @pytest.mark.parametrize("asym", [True, False])
 @pytest.mark.parametrize("per_channel", [True, False])
 @pytest.mark.parametrize("activation", ["none", "relu", "relu_n1_to_1", "relu6"])
-@pytest.mark.parametrize("packed", [True, False])
+@pytest.mark.parametrize("packed", ["fused", "split", False])
 def test_hybrid_variants(fc, B, K, N, asym, per_channel, activation, packed):
     c = wl.hybrid_fc(B, K, N, seed=7 + B + K)
     bias = np.random.default_rng(3).standard_normal(N).astype(np.float32)
     pcs = c["pcs"] if per_channel else None
     op = fc.FullyConnectedHybrid(c["w"], pcs, filter_scale=0.005, bias=bias,
                                  asymmetric_quantize_inputs=asym, activation=activation,
-                                 packed=packed)
-    y = op(_cuda(c["x"])).cpu().numpy()
+                                 packed=bool(packed))
+    y = _hybrid_call(op, _cuda(c["x"]), packed).cpu().numpy()
     want = oracle.fc_hybrid(c["x"], c["w"], pcs, 0.005, bias, asym, fc._act(activation))
     assert _close(y, want)
     assert _bits_equal(y, want)
