@@ -56,6 +56,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-extras", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="launch only the dominant kernel (cold, 12 times) and a 64 MiB device "
+                         "copy (3 times), for a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the op shards "
@@ -76,6 +79,10 @@ def main():
     lib = capi.load()
     p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
     stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    if args.traffic_probe:
+        traffic_probe(torch, fc, wl)
+        return
 
     def timed_replays(graphs, reps):
         """Average milliseconds per replay, graphs[i % len] replayed reps times."""
@@ -160,16 +167,29 @@ def main():
                         op_gbps_cold=round(hybrid_bytes(b) / cold_us / 1e3, 1),
                         op_gbps_hot=round(hybrid_bytes(b) / hot_us / 1e3, 1),
                         frac_of_hbm_peak_cold=round(hybrid_bytes(b) / cold_us / 1e3 / HBM_PEAK_GBPS, 4))
+    # The op picks the fused kernel up to FUSED_MAX_BATCHES rows and quantizer + GEMV above;
+    # both forms timed at every batch size show where the crossover lies.
+    forms = {}
+    for b in BATCHES:
+        fused_max = fc.FullyConnectedHybrid.FUSED_MAX_BATCHES
+        try:
+            fc.FullyConnectedHybrid.FUSED_MAX_BATCHES = 1 << 30
+            fused_us = per_launch_us([(lambda o: lambda: o(xs[b], out=outs[b]))(op) for op in ops])
+        finally:
+            fc.FullyConnectedHybrid.FUSED_MAX_BATCHES = fused_max
+        split_us = per_launch_us([(lambda o: lambda: o.call_split(xs[b], out=outs[b]))(op)
+                                  for op in ops])
+        forms[b] = dict(fused_us_cold=round(fused_us, 3), split_us_cold=round(split_us, 3))
     b_dom = 1
     achieved = hybrid_bytes(b_dom) / per_b[b_dom]["op_us_cold"] / 1e3
     roofline = dict(bound="hbm",
                     kernel="FcInt8PackedGemvKernel<hybrid, fused quantize> (config 2, B=1, cold)",
                     achieved=round(achieved, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
-                    frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=None,
+                    frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=measured_traffic(),
                     algorithmic_bytes_per_launch=hybrid_bytes(b_dom),
                     avg_launch_us=per_b[b_dom]["op_us_cold"])
 
-    also = {"config2_hybrid_per_batch": per_b,
+    also = {"config2_hybrid_per_batch": per_b, "config2_fused_vs_split": forms,
             "config2_step_ms_hot": round(ms_hot, 5),
             "config2_step_gbps_hot": round(step_bytes / (ms_hot * 1e-3) / 1e9, 1)}
 
@@ -194,6 +214,41 @@ def main():
         "roofline": roofline, "cpu_baseline": cpu_baseline, "also": also,
     }
     print(json.dumps(line))
+
+
+def traffic_probe(torch, fc, wl):
+    """The launches a counter run needs and nothing else: the fused hybrid kernel at B = 1
+    on rotating weight copies (so every launch streams its filter from HBM) and a plain
+    device-to-device copy of 64 MiB, whose known 64 MiB read and 64 MiB written calibrate
+    the counters' unit."""
+    c = wl.hybrid_fc(1)
+    ops = [fc.FullyConnectedHybrid(np.roll(c["w"], i, axis=0) if i else c["w"], c["pcs"])
+           for i in range(WEIGHT_COPIES)]
+    x = torch.from_numpy(c["x"]).cuda()
+    y = torch.empty((1, N_OUT), dtype=torch.float32, device="cuda")
+    src = torch.ones(64 << 20, dtype=torch.int8, device="cuda")
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for i in range(12):
+        ops[i % len(ops)](x, out=y)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": "traffic", "hybrid_launches": 12, "copy_launches": 3,
+                      "copy_bytes": 64 << 20, "algorithmic_bytes": hybrid_bytes(1)}))
+
+
+def measured_traffic():
+    """HBM bytes per launch of the dominant kernel, from the committed counter summary
+    (two rocprofv3 --pmc runs of `bench.py --traffic-probe`); None when it is absent."""
+    path = os.path.join(ROOT, "profiles", "hybrid_gemv_fused_B1_hbm_traffic.txt")
+    try:
+        for ln in open(path):
+            if ln.startswith("traffic_bytes_per_launch:"):
+                return int(ln.split(":")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_launch_us):
@@ -223,20 +278,23 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
 
     def int4_kernel_only(op):
         def run():
-            capi.check(lib.lrtfc_fc_blockwise_int4_quantized(
-                p(q3[0]), p(q3[1]), p(q3[2]), p(op.filter), p(op.scales), p(op.kfsum), None, p(y3),
-                1, 4096, 14336, 32, stream()))
+            capi.check(lib.lrtfc_fc_blockwise_int4_packed_quantized(
+                p(q3[0]), p(q3[1]), p(q3[2]), p(op.retiled), p(op.kfsum), None, p(y3),
+                1, 4096, 14336, stream()))
         return run
 
-    k_cold = per_launch_us([int4_kernel_only(op) for op in ops3])
-    k_hot = per_launch_us([int4_kernel_only(ops3[0])] * len(ops3))
+    # op = one kernel (quantizer fused into the prologue); "prequantized" = the same kernel
+    # handed rows that were quantized beforehand, i.e. without the prologue's work.
     o_cold = per_launch_us([(lambda o: lambda: o(x3, out=y3))(op) for op in ops3])
+    o_hot = per_launch_us([lambda: ops3[0](x3, out=y3)] * len(ops3))
+    k_cold = per_launch_us([int4_kernel_only(op) for op in ops3])
     b3 = int4_bytes(1, 14336, 4096)
     out["config3_int4_gemv_14336x4096_B1"] = dict(
-        kernel_us_cold=round(k_cold, 3), kernel_us_hot=round(k_hot, 3), op_us_cold=round(o_cold, 3),
-        kernel_gbps_cold=round(b3 / k_cold / 1e3, 1), kernel_gbps_hot=round(b3 / k_hot / 1e3, 1),
-        op_gbps_cold=round(b3 / o_cold / 1e3, 1),
-        frac_of_hbm_peak_cold=round(b3 / k_cold / 1e3 / HBM_PEAK_GBPS, 4), algorithmic_bytes=b3)
+        op_us_cold=round(o_cold, 3), op_us_hot=round(o_hot, 3),
+        prequantized_kernel_us_cold=round(k_cold, 3),
+        op_gbps_cold=round(b3 / o_cold / 1e3, 1), op_gbps_hot=round(b3 / o_hot / 1e3, 1),
+        frac_of_hbm_peak_cold=round(b3 / o_cold / 1e3 / HBM_PEAK_GBPS, 4), algorithmic_bytes=b3,
+        kernel="FcInt4PackedKernel<fused quantize> on the re-tiled filter")
     del ops3
 
     # config 4: prefill int8 GEMM 2048 x 4096 x 4096, RELU6 off / on

@@ -304,6 +304,9 @@ class FullyConnectedBlockwiseInt4:
         batches = x.numel() // self.depth
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
+        if (self.retiled is not None and self.depth > self.FUSED_MAX_DEPTH
+                and batches > self.DEEP_FUSED_MAX_BATCHES):
+            return self.call_split(x, out)
         if self.retiled is not None:
             capi.check(capi.load().lrtfc_fc_blockwise_int4_packed(
                 _ptr(x), _ptr(self.retiled), _ptr(self.kfsum), _ptr(self.bias), _ptr(out), batches,
@@ -316,6 +319,11 @@ class FullyConnectedBlockwiseInt4:
             _ptr(ws), ws.numel(), _stream()))
         return out
 
+    # Rows deeper than FUSED_MAX_DEPTH fuse the quantizer for at most DEEP_FUSED_MAX_BATCHES
+    # batch rows (the prologue keeps the float rows in registers); more rows split it off.
+    FUSED_MAX_DEPTH = 4096
+    DEEP_FUSED_MAX_BATCHES = 2
+
     def call_split(self, x, out=None):
         """Two launches on the re-tiled filter: the standalone row quantizer, then the
         streaming kernel on its int8 output. Same results as the fused call."""
@@ -325,7 +333,16 @@ class FullyConnectedBlockwiseInt4:
         batches = x.numel() // self.depth
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
-        q, sf, zp = batch_quantize_floats(x.reshape(batches, self.depth), True, self.variant)
+        key = (batches, str(x.device))
+        if getattr(self, "_split_key", None) != key:
+            self._split_q = torch.empty((batches, self.depth), dtype=torch.int8, device=x.device)
+            self._split_sf = torch.empty(batches, dtype=torch.float32, device=x.device)
+            self._split_zp = torch.zeros(batches, dtype=torch.int32, device=x.device)
+            self._split_key = key
+        q, sf, zp = self._split_q, self._split_sf, self._split_zp
+        capi.check(capi.load().lrtfc_batch_quantize_floats(_ptr(x), batches, self.depth, _ptr(q),
+                                                           _ptr(sf), _ptr(zp), 1, self.variant,
+                                                           _stream()))
         capi.check(capi.load().lrtfc_fc_blockwise_int4_packed_quantized(
             _ptr(q), _ptr(sf), _ptr(zp), _ptr(self.retiled), _ptr(self.kfsum), _ptr(self.bias),
             _ptr(out), batches, self.depth, self.out_depth, _stream()))
