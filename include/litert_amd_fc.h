@@ -110,9 +110,10 @@ int lrtfc_blockwise_int4_kfsum(const uint8_t* packed_filter, const uint16_t* sca
  * lrtfc_pack_int4_blockwise. The choice stands where the reference picks a kernel path
  * per shape (tflite/kernels/cpu_backend_gemm.h:116-160 routes matrix-vector products to
  * a custom GEMV and the rest to ruy). Pure host functions; no device needed.
- *   int8 / hybrid: row-major for prefill batches the MFMA GEMM tiles (batches a multiple
- *   of 128, out_depth of 256, depth of 128, symmetric filter) and for per-tensor filters
- *   with a non-zero zero point; packed otherwise. Hybrid callers pass filter_offset 0.
+ *   int8 / hybrid: packed, except for per-tensor filters with a non-zero zero point (and
+ *   depths too large to stage a row in LDS), which need the row-major kernels. The answer
+ *   does not depend on `batches` today; the parameter is kept so that it may. Hybrid callers
+ *   pass filter_offset 0.
  *   blockwise int4: packed for block size 32 dividing the depth. */
 enum { LRTFC_LAYOUT_ROW_MAJOR = 0, LRTFC_LAYOUT_PACKED = 1 };
 int lrtfc_fc_int8_preferred_layout(int batches, int depth, int out_depth, int32_t filter_offset);
@@ -147,11 +148,13 @@ int lrtfc_fc_int8(const int8_t* input, const int8_t* filter, const int32_t* bias
                   int out_depth, int32_t input_offset, int32_t filter_offset,
                   int32_t output_offset, int32_t act_min, int32_t act_max, void* stream);
 
-/* lrtfc_fc_int8 for decode batches on a filter packed by lrtfc_pack_int8_filter: one
- * kernel on the int8 matrix cores whose cost does not grow with the batch up to 16 rows
- * (larger batches run in tiles of 16). Same arithmetic contract as lrtfc_fc_int8 with
- * filter_offset == 0; filter_row_sums (of the unpacked filter) is required when
- * input_offset != 0. */
+/* lrtfc_fc_int8 on a filter packed by lrtfc_pack_int8_filter, for every batch size: up to
+ * 32 rows one matrix-core GEMV kernel whose cost does not grow with the batch up to 16 rows
+ * (17..32 rows take two passes over the filter); above that an int8 MFMA GEMM that streams
+ * the filter once (any batch count and out_depth; depth a multiple of 16, input and filter
+ * 16-byte aligned -- other shapes keep the GEMV in tiles of 16 rows). Same arithmetic
+ * contract as lrtfc_fc_int8 with filter_offset == 0; filter_row_sums (of the unpacked
+ * filter) is required when input_offset != 0. */
 int lrtfc_fc_int8_packed(const int8_t* input, const int8_t* packed_filter, const int32_t* bias,
                          const int32_t* multipliers, const int32_t* shifts, int per_channel,
                          const int32_t* filter_row_sums, int8_t* output, int batches, int depth,
@@ -180,8 +183,9 @@ int lrtfc_fc_hybrid_int8(const int8_t* quantized_input, const float* scaling_fac
                          int batches, int depth, int out_depth, int activation, void* stream);
 
 /* lrtfc_fc_hybrid_int8 on a packed filter (lrtfc_pack_int8_filter): the form for batches
- * whose rows were quantized by a separate lrtfc_batch_quantize_floats launch. Replaces the
- * same reference functions as lrtfc_fc_hybrid_int8. */
+ * whose rows were quantized by a separate lrtfc_batch_quantize_floats launch (GEMV up to 32
+ * rows, MFMA GEMM with the same float epilogue above). Replaces the same reference
+ * functions as lrtfc_fc_hybrid_int8. */
 int lrtfc_fc_hybrid_int8_packed(const int8_t* quantized_input, const float* scaling_factors,
                                 const int32_t* zero_points, const int8_t* packed_filter,
                                 const float* per_channel_scales, float filter_scale,

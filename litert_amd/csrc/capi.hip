@@ -42,6 +42,9 @@ int RequireInit() {
 
 // Batches from this size on go to the MFMA GEMM when its tiling fits.
 constexpr int kGemmMinBatches = 128;
+// On the re-tiled filter: up to this many rows the GEMV (16 rows per pass over the filter)
+// wins; beyond it the GEMM, which streams the filter once.
+constexpr int kPackedGemmMinBatches = 32;
 
 // Workspace layout for the hybrid paths: quantized activations, then scaling
 // factors, then zero points, each 256-byte aligned.
@@ -294,7 +297,7 @@ int lrtfc_fc_int8_preferred_layout(int batches, int depth, int out_depth, int32_
   a.depth = depth;
   a.out_depth = out_depth;
   a.filter_offset = filter_offset;
-  if (batches >= kGemmMinBatches && lrtfc::FcInt8GemmMfmaSupports(a)) return LRTFC_LAYOUT_ROW_MAJOR;
+  (void)batches;  // the re-tiled form serves every batch size (GEMV up to 32 rows, GEMM above)
   return lrtfc::FcInt8PackedGemvSupports(a) ? LRTFC_LAYOUT_PACKED : LRTFC_LAYOUT_ROW_MAJOR;
 }
 
@@ -349,6 +352,11 @@ int lrtfc_fc_int8_packed(const int8_t* input, const int8_t* packed_filter, const
   a.act_min = act_min;
   a.act_max = act_max;
   a.output_i8 = output;
+  if (batches > kPackedGemmMinBatches && lrtfc::FcInt8PackedGemmSupports(a)) {
+    return FromHip(lrtfc::LaunchFcInt8PackedGemm(a, lrtfc::Int8Epilogue::kRequantize,
+                                                 AsStream(stream)),
+                   "packed int8 GEMM");
+  }
   return FromHip(lrtfc::LaunchFcInt8PackedGemv(a, lrtfc::Int8Epilogue::kRequantize, nullptr, 0, 0,
                                                AsStream(stream)),
                  "packed int8 GEMV");
@@ -418,6 +426,11 @@ int lrtfc_fc_hybrid_int8_packed(const int8_t* quantized_input, const float* scal
   a.bias_f32 = bias;
   a.activation = activation;
   a.output_f32 = output;
+  if (batches > kPackedGemmMinBatches && lrtfc::FcInt8PackedGemmSupports(a)) {
+    return FromHip(lrtfc::LaunchFcInt8PackedGemm(a, lrtfc::Int8Epilogue::kHybrid,
+                                                 AsStream(stream)),
+                   "packed hybrid GEMM");
+  }
   return FromHip(lrtfc::LaunchFcInt8PackedGemv(a, lrtfc::Int8Epilogue::kHybrid, nullptr, 0,
                                                LRTFC_QUANT_PORTABLE, AsStream(stream)),
                  "packed hybrid GEMV");

@@ -22,9 +22,11 @@ using i32x2 = int __attribute__((ext_vector_type(2)));
 // quotient equals floor((ab + 2^30) / 2^31), which needs no sign test: one 64-bit
 // multiply-add and an arithmetic shift.
 __device__ __forceinline__ int32_t Srdhm(int32_t a, int32_t b) {
-  if (a == b && a == INT32_MIN) return INT32_MAX;
   const int64_t t = static_cast<int64_t>(a) * static_cast<int64_t>(b) + (1ll << 30);
-  return static_cast<int32_t>(t >> 31);
+  const int32_t r = static_cast<int32_t>(t >> 31);
+  // The one product that does not fit (INT32_MIN squared) saturates; as a select, so that
+  // the epilogues stay free of branches.
+  return (a == INT32_MIN && b == INT32_MIN) ? INT32_MAX : r;
 }
 
 // RoundingDivideByPOT: shift right, nearest, ties away from zero.

@@ -63,6 +63,12 @@ hipError_t LaunchFcInt8PackedGemv(const FcInt8Args& a, Int8Epilogue epilogue,
                                   const float* input_f32, int asymmetric, int variant,
                                   hipStream_t stream);
 
+// Prefill batches on the same re-tiled filter: int8 MFMA GEMM (a.filter = packed, a.input =
+// int8 rows; the hybrid epilogue reads a.scaling_factors / a.zero_points). Any batch count,
+// any out_depth; depth a multiple of 16.
+bool FcInt8PackedGemmSupports(const FcInt8Args& a);
+hipError_t LaunchFcInt8PackedGemm(const FcInt8Args& a, Int8Epilogue epilogue, hipStream_t stream);
+
 struct FcInt4Args {
   const int8_t* input;           // [batches, depth] quantized activations
   const float* scaling_factors;  // [batches]

@@ -141,20 +141,18 @@ class FullyConnectedInt8:
         self.row_sums = torch.empty(self.out_depth, dtype=torch.int32, device="cuda")
         capi.check(lib.lrtfc_row_sums_int8(_ptr(self.filter), self.out_depth, self.depth,
                                            _ptr(self.row_sums), _stream()))
-        # Decode batches run on a re-tiled copy of the filter (matrix-core GEMV); prefill
-        # batches use the row-major filter (MFMA GEMM).
+        # packed: every batch size runs on a re-tiled copy of the filter (matrix-core GEMV up
+        # to 32 rows, MFMA GEMM above); otherwise the row-major kernels.
         self.packed_filter = None
         if packed and self.filter_offset == 0 and self.depth > 0:
             self.packed_filter = _pack_int8(self.filter)
-
-    GEMM_MIN_BATCHES = 128
 
     def __call__(self, x, out=None):
         x = x.contiguous()
         batches = x.numel() // self.depth if self.depth else 0
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.int8, device=x.device)
-        if self.packed_filter is not None and batches < self.GEMM_MIN_BATCHES:
+        if self.packed_filter is not None:
             capi.check(capi.load().lrtfc_fc_int8_packed(
                 _ptr(x), _ptr(self.packed_filter), _ptr(self.bias), _ptr(self.multipliers),
                 _ptr(self.shifts), int(self.per_channel), _ptr(self.row_sums), _ptr(out), batches,

@@ -233,9 +233,9 @@ def test_blockwise_int4_other_block_size_keeps_model_layout():
         assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
 
 
-def test_int8_resize_between_decode_and_prefill_switches_filter_layout():
-    """One row runs on the re-tiled filter; 128 rows on the row-major one (MFMA GEMM); going
-    back re-tiles again. Each step is checked against the oracle."""
+def test_int8_resize_between_decode_and_prefill():
+    """One row runs the GEMV, 128 rows the MFMA GEMM, 3 rows the GEMV again, all on the same
+    re-tiled filter; prepare runs after every resize. Each step is checked against the oracle."""
     c = wl.int8_fc(128, 256, 256, seed=9)
     with FakeHost() as h:
         B, K = c["x"].shape

@@ -141,11 +141,41 @@ def test_int8_int4_weights_kat(fc):
 def test_int8_prefill_gemm_bit_exact(fc, activation):
     """Config 4 shape class on the MFMA path, at a size the scalar oracle finishes in seconds."""
     c = wl.prefill_int8_fc(256, 512, 512, seed=77)
-    y, want = _run_int8(fc, c, activation)
-    assert np.array_equal(y, want)
+    for packed in (True, False):  # GEMM on the re-tiled filter / on the row-major one
+        y, want = _run_int8(fc, c, activation, packed=packed)
+        assert np.array_equal(y, want)
     c = wl.int8_fc(128, 256, 256, in_zp=-3, out_zp=5, seed=78)  # non-zero input offset on the GEMM
-    y, want = _run_int8(fc, c, activation)
+    for packed in (True, False):
+        y, want = _run_int8(fc, c, activation, packed=packed)
+        assert np.array_equal(y, want)
+
+
+@pytest.mark.parametrize("B,K,N", [(33, 64, 20), (128, 256, 256), (130, 272, 48), (200, 1040, 300),
+                                   (64, 16, 4), (257, 192, 513), (40, 4096, 70), (300, 80, 257),
+                                   (129, 128, 30), (96, 2048, 64)])
+@pytest.mark.parametrize("activation", ["none", "relu6"])
+def test_int8_packed_gemm_ragged_shapes_bit_exact(fc, B, K, N, activation):
+    """More than 32 rows on the re-tiled filter take the MFMA GEMM: batch and channel counts
+    off the 128 x 256 tile, depths that end inside a 64-deep slab or give an odd slab count,
+    channel counts that rule out vector stores."""
+    c = wl.int8_fc(B, K, N, in_zp=(-3 if N % 2 else 0), seed=300 + B + K + N)
+    y, want = _run_int8(fc, c, activation, bias=(N % 3 != 0))
     assert np.array_equal(y, want)
+
+
+@pytest.mark.parametrize("B,K,N", [(33, 64, 20), (128, 256, 256), (130, 272, 48), (65, 1040, 301)])
+@pytest.mark.parametrize("asym", [True, False])
+@pytest.mark.parametrize("per_channel", [True, False])
+def test_hybrid_packed_gemm_matches_oracle(fc, B, K, N, asym, per_channel):
+    """Hybrid rows beyond 32 run the same GEMM with the float epilogue."""
+    c = wl.hybrid_fc(B, K, N, seed=17 + B + K)
+    bias = np.random.default_rng(3).standard_normal(N).astype(np.float32)
+    pcs = c["pcs"] if per_channel else None
+    op = fc.FullyConnectedHybrid(c["w"], pcs, filter_scale=0.005, bias=bias,
+                                 asymmetric_quantize_inputs=asym, activation="relu6")
+    y = op(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_hybrid(c["x"], c["w"], pcs, 0.005, bias, asym, oracle.ACT_RELU6)
+    assert _bits_equal(y, want)
 
 
 def test_int8_prefill_full_size_properties(fc):
@@ -164,6 +194,10 @@ def test_int8_prefill_full_size_properties(fc):
         if activation == "none":
             y_gemv = op(x[:8]).cpu().numpy()  # 8 rows take the GEMV kernel
             assert np.array_equal(outs["none"][:8], y_gemv)
+            rowmajor = fc.FullyConnectedInt8(c["w"], c["bias"], float(c["in_scale"]), c["in_zp"],
+                                             c["w_scale"], float(c["out_scale"]), c["out_zp"],
+                                             packed=False)
+            assert np.array_equal(outs["none"], rowmajor(x).cpu().numpy())  # the other GEMM
     lo, hi = oracle.activation_range_int8(oracle.ACT_RELU6, 0.05, 0)
     assert np.array_equal(np.clip(outs["none"], lo, hi), outs["relu6"])
     mult, shift = oracle.fc_prepare_per_channel(0.03, c["w_scale"], 0.05)
