@@ -322,21 +322,60 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
             scales = (torch.rand((n, k // 32), device="cuda", generator=g) * 1.5e-2 + 5e-3).half()
             nodes.append(fc.FullyConnectedBlockwiseInt4(packed, scales, k, 32))
     chain_bytes = sum(int4_bytes(0, op.out_depth, op.depth) for op in nodes)
+    per_layer = len(wl.GEMMA2B_LAYER_FCS)
+    aux = [torch.cuda.Stream() for _ in range(3)]  # default priority, like the delegate's
+
+    def run_level(level, bufs):
+        """Nodes that do not depend on each other, spread round-robin over the current stream
+        and the auxiliary ones (what the delegate does inside a partition)."""
+        main = torch.cuda.current_stream()
+        lanes = [main] + aux[:max(0, min(len(level), 4) - 1)]
+        for st in lanes[1:]:
+            st.wait_stream(main)
+        for i, (op, key) in enumerate(level):
+            with torch.cuda.stream(lanes[i % len(lanes)]):
+                op(bufs["x"][op.depth], out=bufs["y"][key])
+        for st in lanes[1:]:
+            main.wait_stream(st)
+
     for b in (1, 4):
         xin = {k: torch.randn((b, k), device="cuda", generator=g) for k in (2048, 16384)}
-        yout = {n: torch.empty((b, n), dtype=torch.float32, device="cuda") for n in (256, 2048, 16384)}
+        # one output buffer per node of a layer, so that concurrent nodes never share one
+        yout = {i: torch.empty((b, n), dtype=torch.float32, device="cuda")
+                for i, (_, _, n) in enumerate(wl.GEMMA2B_LAYER_FCS)}
+        bufs = {"x": xin, "y": yout}
+        keyed = [(op, i % per_layer) for i, op in enumerate(nodes)]
 
-        def chain():
-            for op in nodes:
-                op(xin[op.depth], out=yout[op.out_depth])
+        def serial():
+            for op, key in keyed:
+                op(xin[op.depth], out=yout[key])
 
-        gc = capture(chain)
-        us = timed_replays([gc], 30) * 1e3
-        out["config5_gemma2b_fc_chain_B%d" % b] = dict(
-            us_per_token=round(us, 1), fc_nodes=len(nodes), weight_bytes=chain_bytes,
-            gbps=round(chain_bytes / us / 1e3, 1),
-            frac_of_hbm_peak=round(chain_bytes / us / 1e3 / HBM_PEAK_GBPS, 4))
-        del gc
+        def independent():
+            # As the configuration defines it (every node has its own input, outputs are
+            # discarded): no node depends on another, so all of them may overlap.
+            for l in range(wl.GEMMA2B_LAYERS):
+                run_level(keyed[l * per_layer:(l + 1) * per_layer], bufs)
+
+        def decoder_order():
+            # The dependency structure a real decoder layer imposes on the same nodes:
+            # {q, k, v} -> o -> {gate, up} -> down, layer after layer.
+            for l in range(wl.GEMMA2B_LAYERS):
+                layer = keyed[l * per_layer:(l + 1) * per_layer]
+                run_level(layer[0:3], bufs)
+                run_level(layer[3:4], bufs)
+                run_level(layer[4:6], bufs)
+                run_level(layer[6:7], bufs)
+
+        res = {}
+        for name, fn in (("one_stream", serial), ("independent_nodes_4_streams", independent),
+                         ("decoder_dependencies_4_streams", decoder_order)):
+            gc = capture(fn)
+            us = timed_replays([gc], 30) * 1e3
+            res[name] = dict(us_per_token=round(us, 1), gbps=round(chain_bytes / us / 1e3, 1),
+                             frac_of_hbm_peak=round(chain_bytes / us / 1e3 / HBM_PEAK_GBPS, 4))
+            del gc
+        res.update(fc_nodes=len(nodes), weight_bytes=chain_bytes)
+        out["config5_gemma2b_fc_chain_B%d" % b] = res
     return out
 
 

@@ -34,6 +34,7 @@ constexpr int kMaxFcVersion = 14;  // tflite/core/kernels/register.cc:84-86
 
 struct Options {
   int device = 0;
+  int streams = 4;  // HIP streams a partition spreads independent nodes over (1..4)
   int quant_variant = LRTFC_QUANT_PORTABLE;
   bool claim_int8 = true;
   bool claim_hybrid = true;
@@ -222,6 +223,11 @@ struct FcNode {
   // model's own (row-major / nibble-packed rows) or the re-tiled copy. Only one is kept.
   bool have_model_layout = false, have_retiled = false, use_retiled = false;
   bool split_quantize = false;  // quantize rows in a launch of their own, not in the prologue
+  // Scheduling inside the partition: the stream the node runs on, the node that produces its
+  // input (-1: the input is uploaded from the host), and whether a node on another stream
+  // waits for this one.
+  int lane = 0, producer = -1;
+  bool signal = false;
   DeviceBuffer filter_dev, retiled_dev, bias_dev, mult_dev, shift_dev, row_sums_dev, pcs_dev,
       scales_dev, kfsum_dev;
 };
@@ -238,10 +244,27 @@ struct PartitionKernel {
   std::map<int, DeviceBuffer> activations;  // tensor index -> device copy
   std::vector<int> uploads;                 // activation tensors read from the host each invoke
   std::vector<int> downloads;               // tensors written back to the host each invoke
-  DeviceBuffer workspace;
-  hipStream_t stream = nullptr;
+  // Nodes that do not depend on each other (the q/k/v or gate/up projections of a decoder
+  // layer, say) run on different streams so that their launch and prologue latencies overlap;
+  // a chain of dependent nodes stays on one stream. All streams have the default priority.
+  static constexpr int kMaxStreams = 4;
+  int num_streams = 1;
+  hipStream_t streams[kMaxStreams] = {};
+  hipStream_t stream = nullptr;  // streams[0]: uploads, downloads, prepare-time work
+  DeviceBuffer workspace[kMaxStreams];
+  hipEvent_t upload_done = nullptr;
+  hipEvent_t lane_done[kMaxStreams] = {};
+  std::vector<hipEvent_t> node_done;  // per node; only the signalling ones are created
+  bool lane_used[kMaxStreams] = {};
   ~PartitionKernel() {
-    if (stream) (void)hipStreamDestroy(stream);
+    for (hipEvent_t e : node_done) {
+      if (e) (void)hipEventDestroy(e);
+    }
+    if (upload_done) (void)hipEventDestroy(upload_done);
+    for (int i = 0; i < kMaxStreams; ++i) {
+      if (lane_done[i]) (void)hipEventDestroy(lane_done[i]);
+      if (streams[i]) (void)hipStreamDestroy(streams[i]);
+    }
   }
 };
 
@@ -272,12 +295,20 @@ void* KernelInit(TfLiteContext* ctx, const char* buffer, size_t /*length*/) {
   auto* state = static_cast<DelegateState*>(params->delegate->data_);
   auto kernel = std::make_unique<PartitionKernel>();
   kernel->state = state;
-  if (hipSetDevice(state->options.device) != hipSuccess ||
-      hipStreamCreate(&kernel->stream) != hipSuccess) {
-    ctx->ReportError(ctx, "litert_amd delegate: cannot create a HIP stream on device %d",
+  kernel->num_streams = state->options.streams;
+  bool streams_ok = hipSetDevice(state->options.device) == hipSuccess;
+  for (int i = 0; streams_ok && i < kernel->num_streams; ++i) {
+    streams_ok = hipStreamCreate(&kernel->streams[i]) == hipSuccess &&
+                 hipEventCreateWithFlags(&kernel->lane_done[i], hipEventDisableTiming) == hipSuccess;
+  }
+  streams_ok = streams_ok &&
+               hipEventCreateWithFlags(&kernel->upload_done, hipEventDisableTiming) == hipSuccess;
+  if (!streams_ok) {
+    ctx->ReportError(ctx, "litert_amd delegate: cannot create HIP streams on device %d",
                      state->options.device);
     return reinterpret_cast<void*>(-1);  // TfLiteKernelInitFailed(), tflite/core/c/common.cc:867
   }
+  kernel->stream = kernel->streams[0];
   std::map<int, bool> produced;
   for (int i = 0; i < params->nodes_to_replace->size; ++i) {
     const int node_index = params->nodes_to_replace->data[i];
@@ -308,6 +339,37 @@ void* KernelInit(TfLiteContext* ctx, const char* buffer, size_t /*length*/) {
     }
     produced[n.output] = true;
     kernel->nodes.push_back(std::move(n));
+  }
+  // Streams: a node continues on its producer's stream unless a sibling already did; nodes
+  // without a producer in the partition, and further siblings, take streams round-robin.
+  {
+    std::map<int, int> producer_of;  // tensor -> node that writes it
+    std::vector<bool> continued(kernel->nodes.size(), false);
+    int next_lane = 0;
+    for (size_t i = 0; i < kernel->nodes.size(); ++i) {
+      FcNode& n = kernel->nodes[i];
+      auto it = producer_of.find(n.input);
+      n.producer = it == producer_of.end() ? -1 : it->second;
+      if (n.producer >= 0 && !continued[n.producer]) {
+        n.lane = kernel->nodes[n.producer].lane;
+        continued[n.producer] = true;
+      } else {
+        n.lane = next_lane++ % kernel->num_streams;
+      }
+      if (n.producer >= 0 && kernel->nodes[n.producer].lane != n.lane) {
+        kernel->nodes[n.producer].signal = true;
+      }
+      kernel->lane_used[n.lane] = true;
+      producer_of[n.output] = static_cast<int>(i);
+    }
+    kernel->node_done.assign(kernel->nodes.size(), nullptr);
+    for (size_t i = 0; i < kernel->nodes.size(); ++i) {
+      if (kernel->nodes[i].signal &&
+          hipEventCreateWithFlags(&kernel->node_done[i], hipEventDisableTiming) != hipSuccess) {
+        ctx->ReportError(ctx, "litert_amd delegate: cannot create a HIP event");
+        return reinterpret_cast<void*>(-1);
+      }
+    }
   }
   // Every tensor the runtime lists as an output of the partition goes back to the host.
   for (int i = 0; i < params->output_tensors->size; ++i) {
@@ -491,7 +553,8 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
   RETURN_IF_HIP(ctx, k->activations[n->input].Ensure(input.bytes));
   RETURN_IF_HIP(ctx, k->activations[n->output].Ensure(output.bytes));
   if (n->kind != FcKind::kInt8 && (!n->use_retiled || n->split_quantize)) {
-    RETURN_IF_HIP(ctx, k->workspace.Ensure(lrtfc_activation_workspace_bytes(n->batches, n->depth)));
+    RETURN_IF_HIP(ctx, k->workspace[n->lane].Ensure(
+                           lrtfc_activation_workspace_bytes(n->batches, n->depth)));
   }
   return kTfLiteOk;
 }
@@ -510,15 +573,38 @@ TfLiteStatus KernelPrepare(TfLiteContext* ctx, TfLiteNode* node) {
 TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   auto* k = static_cast<PartitionKernel*>(node->user_data);
   RETURN_IF_HIP(ctx, hipSetDevice(k->state->options.device));
-  hipStream_t s = k->stream;
   // Tensor data pointers may move between invokes: read them from the context each time.
   for (int t : k->uploads) {
     const TfLiteTensor& tensor = ctx->tensors[t];
     if (tensor.bytes == 0) continue;
     RETURN_IF_HIP(ctx, hipMemcpyAsync(k->activations[t].get(), tensor.data.raw, tensor.bytes,
-                                      hipMemcpyHostToDevice, s));
+                                      hipMemcpyHostToDevice, k->stream));
   }
-  for (FcNode& n : k->nodes) {
+  bool multi = false;
+  for (int i = 1; i < k->num_streams; ++i) multi = multi || k->lane_used[i];
+  if (multi) {
+    RETURN_IF_HIP(ctx, hipEventRecord(k->upload_done, k->stream));
+    for (int i = 1; i < k->num_streams; ++i) {
+      if (k->lane_used[i]) RETURN_IF_HIP(ctx, hipStreamWaitEvent(k->streams[i], k->upload_done, 0));
+    }
+  }
+  for (size_t node_i = 0; node_i < k->nodes.size(); ++node_i) {
+    FcNode& n = k->nodes[node_i];
+    hipStream_t s = k->streams[n.lane];
+    DeviceBuffer& scratch = k->workspace[n.lane];
+    // Cross-stream edge: wait for the producer. (Runs before the early-outs below so that a
+    // consumer never waits on an event that was not recorded in this invoke.)
+    if (n.producer >= 0 && k->nodes[n.producer].lane != n.lane) {
+      RETURN_IF_HIP(ctx, hipStreamWaitEvent(s, k->node_done[n.producer], 0));
+    }
+    struct SignalOnExit {
+      PartitionKernel* k;
+      size_t i;
+      hipStream_t s;
+      ~SignalOnExit() {
+        if (k->nodes[i].signal) (void)hipEventRecord(k->node_done[i], s);
+      }
+    } signal_on_exit{k, node_i, s};
     const TfLiteTensor& output = ctx->tensors[n.output];
     if (NumElements(output.dims) == 0) continue;  // fully_connected.cc:1966-1968
     void* out_dev = k->activations[n.output].get();
@@ -561,7 +647,7 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                             n.row_sums_dev.as<int32_t>(), bias_f32,
                                             static_cast<float*>(out_dev), n.batches, n.depth,
                                             n.out_depth, asym, n.params.activation, variant,
-                                            k->workspace.get(), k->workspace.bytes(), s));
+                                            scratch.get(), scratch.bytes(), s));
         } else if (!n.split_quantize) {
           RETURN_IF_FC(ctx, lrtfc_fc_hybrid_packed(static_cast<const float*>(in_dev),
                                                    n.retiled_dev.as<int8_t>(), pcs, n.filter_scale,
@@ -570,7 +656,7 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                                    n.depth, n.out_depth, asym, n.params.activation,
                                                    variant, s));
         } else {
-          const ActivationScratch w = SplitScratch(k->workspace.get(), n.batches, n.depth);
+          const ActivationScratch w = SplitScratch(scratch.get(), n.batches, n.depth);
           RETURN_IF_FC(ctx, lrtfc_batch_quantize_floats(static_cast<const float*>(in_dev),
                                                         n.batches, n.depth, w.q, w.sf, w.zp, asym,
                                                         variant, s));
@@ -591,7 +677,7 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                                     n.kfsum_dev.as<float>(), bias_f32,
                                                     static_cast<float*>(out_dev), n.batches,
                                                     n.depth, n.out_depth, n.blocksize, variant,
-                                                    k->workspace.get(), k->workspace.bytes(), s));
+                                                    scratch.get(), scratch.bytes(), s));
         } else if (!n.split_quantize) {
           RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4_packed(static_cast<const float*>(in_dev),
                                                            n.retiled_dev.as<uint8_t>(),
@@ -599,7 +685,7 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                                            static_cast<float*>(out_dev), n.batches,
                                                            n.depth, n.out_depth, variant, s));
         } else {
-          const ActivationScratch w = SplitScratch(k->workspace.get(), n.batches, n.depth);
+          const ActivationScratch w = SplitScratch(scratch.get(), n.batches, n.depth);
           RETURN_IF_FC(ctx, lrtfc_batch_quantize_floats(static_cast<const float*>(in_dev),
                                                         n.batches, n.depth, w.q, w.sf, w.zp, 1,
                                                         variant, s));
@@ -612,6 +698,12 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
       default:
         return kTfLiteError;
     }
+  }
+  hipStream_t s = k->stream;
+  for (int i = 1; i < k->num_streams; ++i) {  // join: downloads follow every stream's work
+    if (!k->lane_used[i]) continue;
+    RETURN_IF_HIP(ctx, hipEventRecord(k->lane_done[i], k->streams[i]));
+    RETURN_IF_HIP(ctx, hipStreamWaitEvent(s, k->lane_done[i], 0));
   }
   for (int t : k->downloads) {
     TfLiteTensor& tensor = ctx->tensors[t];
@@ -680,6 +772,12 @@ bool ParseOptions(const char* const* keys, const char* const* values, size_t n, 
     const std::string val = values[i] ? values[i] : "";
     if (key == "device") {
       opt->device = std::atoi(val.c_str());
+    } else if (key == "streams") {
+      opt->streams = std::atoi(val.c_str());
+      if (opt->streams < 1 || opt->streams > 4) {
+        *error = "streams must be between 1 and 4, got '" + val + "'";
+        return false;
+      }
     } else if (key == "quant_variant") {
       if (val == "portable") {
         opt->quant_variant = LRTFC_QUANT_PORTABLE;

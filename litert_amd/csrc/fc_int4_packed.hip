@@ -104,20 +104,28 @@ struct Int4Shared {
   int32_t* zp;  // [BT]
   int32_t* zero;
   float* mm;    // [BT][kWaves][2]
-  __device__ Int4Shared(int8_t* base, int padded) {
+  // Floats of parked products: one tile per wavefront when a wavefront owns a channel group
+  // alone; every tile of the group when `ksplit` wavefronts share it (the ordered walk then
+  // needs them all).
+  __host__ __device__ static size_t ProductFloats(int chunks, int ksplit) {
+    const size_t tile = static_cast<size_t>(8) * BT * kPStride;
+    return ksplit == 1 ? kWaves * tile : (kWaves / ksplit) * static_cast<size_t>(chunks) * tile;
+  }
+  __device__ Int4Shared(int8_t* base, int padded, int chunks, int ksplit) {
     q = reinterpret_cast<int32_t*>(base);
     size_t off = static_cast<size_t>(BT) * padded;
     p = reinterpret_cast<float*>(base + off);
-    off += static_cast<size_t>(kWaves) * 8 * BT * kPStride * 4;
+    off += ProductFloats(chunks, ksplit) * 4;
     sf = reinterpret_cast<float*>(base + off);
     inv = sf + 8;
     zp = reinterpret_cast<int32_t*>(inv + 8);
     zero = zp + 8;
     mm = reinterpret_cast<float*>(zero + 8);
   }
-  static size_t Bytes(int padded) {
-    return static_cast<size_t>(BT) * padded + static_cast<size_t>(kWaves) * 8 * BT * kPStride * 4 +
-           4 * 8 * 4 + 8 * kWaves * 2 * 4;
+  static size_t Bytes(int padded, int ksplit) {
+    const int chunks = padded / (kTileBlocks * kBlock);
+    return static_cast<size_t>(BT) * padded + ProductFloats(chunks, ksplit) * 4 + 4 * 8 * 4 +
+           8 * kWaves * 2 * 4;
   }
 };
 
@@ -125,7 +133,7 @@ struct Int4Shared {
 // the prologue; the register form covers depth <= GPT * 256 * 8.
 template <int BT, bool FUSED, int VARIANT, int GPT>
 __global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a, int batch0,
-                                                               int bt) {
+                                                               int bt, int ksplit) {
   extern __shared__ __align__(16) int8_t smem[];
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
@@ -134,10 +142,14 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a,
   const int chunks = a.chunks;
   const int padded = chunks * kTileBlocks * kBlock;  // depth padded to whole tiles
   const int groups = (a.out_depth + kTileRows - 1) / kTileRows;
-  const int group = blockIdx.x * kWaves + wave;  // may run past the last group
+  // ksplit wavefronts share one channel group and take its tiles round-robin (deep, narrow
+  // filters would otherwise leave most of the chip without a wavefront).
+  const int kpart = wave % ksplit;
+  const int group_in_wg = wave / ksplit;
+  const int group = blockIdx.x * (kWaves / ksplit) + group_in_wg;  // may run past the last
   const i32x4* tbase = reinterpret_cast<const i32x4*>(a.packed) +
                        static_cast<size_t>(min(group, groups - 1)) * chunks * kTileVecs + lane;
-  Int4Shared<BT> sh(smem, padded);
+  Int4Shared<BT> sh(smem, padded, chunks, ksplit);
 
   // Activation loads first (raw, branch-free): whatever the prologue waits for must be
   // requested before the weight ring, because vector memory returns in issue order.
@@ -214,7 +226,7 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a,
   i32x4 ring[kRingTiles][kPlanes];
 #pragma unroll
   for (int t = 0; t < kRingTiles; ++t) {
-    const int c = min(t, chunks - 1);
+    const int c = min(kpart + t * ksplit, chunks - 1);
 #pragma unroll
     for (int j = 0; j < kPlanes; ++j) {
       ring[t][j] = __builtin_nontemporal_load(tbase + static_cast<size_t>(c) * kTileVecs + j * 64);
@@ -348,11 +360,35 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a,
   }
 
   // Tile loop. Lane L owns block L of the tile for each of the 8 channels.
-  float* pw = sh.p + static_cast<size_t>(wave) * 8 * BT * kPStride;
+  constexpr int kTileFloats = 8 * BT * kPStride;
+  float* pgroup = sh.p + static_cast<size_t>(group_in_wg) * chunks * kTileFloats;  // ksplit > 1
   float out = 0.0f;
   const int nblk = depth / kBlock;
-  for (int c = 0; c < chunks; ++c) {
-    const int slot = c % kRingTiles;
+  // One tile's 64 products per chain lane, added in block order.
+  auto walk_tile = [&](const float* tile, int c) {
+    const int count = min(kTileBlocks, nblk - c * kTileBlocks);
+    const float* line = tile + lane * kPStride;
+    if (count == kTileBlocks) {
+      // Whole tile: fetch the 64 products with back-to-back LDS reads, then add in order.
+      float4 v[kTileBlocks / 4];
+#pragma unroll
+      for (int j = 0; j < kTileBlocks / 4; ++j) v[j] = reinterpret_cast<const float4*>(line)[j];
+#pragma unroll
+      for (int j = 0; j < kTileBlocks / 4; ++j) {
+        out = __fadd_rn(out, v[j].x);
+        out = __fadd_rn(out, v[j].y);
+        out = __fadd_rn(out, v[j].z);
+        out = __fadd_rn(out, v[j].w);
+      }
+    } else {
+      for (int j = 0; j < count; ++j) out = __fadd_rn(out, line[j]);
+    }
+  };
+  int it = 0;
+  for (int c = kpart; c < chunks; c += ksplit, ++it) {
+    const int slot = it % kRingTiles;
+    float* pw = ksplit == 1 ? sh.p + static_cast<size_t>(wave) * kTileFloats
+                            : pgroup + static_cast<size_t>(c) * kTileFloats;
     // This block's activations (8 dwords per batch row) and 8 * sum(q).
     i32x4 qe[BT], qo[BT];
     int32_t qsum8[BT];
@@ -402,40 +438,29 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a,
             pw[(j * BT + b) * kPStride + lane] = __fmul_rn(static_cast<float>(acc), scale);
           }
         }
-        // Refill the slot with the tile two ahead.
-        if (c + kRingTiles < chunks) {
+        // Refill the slot with this wavefront's tile two turns ahead.
+        if (c + kRingTiles * ksplit < chunks) {
 #pragma unroll
           for (int j = 0; j < kPlanes; ++j) {
             ring[t][j] = __builtin_nontemporal_load(
-                tbase + static_cast<size_t>(c + kRingTiles) * kTileVecs + j * 64);
+                tbase + static_cast<size_t>(c + kRingTiles * ksplit) * kTileVecs + j * 64);
           }
         }
       }
     }
     // Ordered float32 accumulation over this tile's blocks (same wavefront wrote them).
-    if (chain_lane) {
-      const int count = min(kTileBlocks, nblk - c * kTileBlocks);
-      const float* line = pw + lane * kPStride;
-      if (count == kTileBlocks) {
-        // Whole tile: fetch the 64 products with back-to-back LDS reads, then add in order.
-        float4 v[kTileBlocks / 4];
-#pragma unroll
-        for (int j = 0; j < kTileBlocks / 4; ++j) v[j] = reinterpret_cast<const float4*>(line)[j];
-#pragma unroll
-        for (int j = 0; j < kTileBlocks / 4; ++j) {
-          out = __fadd_rn(out, v[j].x);
-          out = __fadd_rn(out, v[j].y);
-          out = __fadd_rn(out, v[j].z);
-          out = __fadd_rn(out, v[j].w);
-        }
-      } else {
-        for (int j = 0; j < count; ++j) out = __fadd_rn(out, line[j]);
-      }
+    if (ksplit == 1 && chain_lane) walk_tile(pw, c);
+  }
+  if (ksplit > 1) {
+    // Every tile of the group is parked; its first wavefront walks them in depth order.
+    __syncthreads();
+    if (kpart == 0 && chain_lane) {
+      for (int c = 0; c < chunks; ++c) walk_tile(pgroup + static_cast<size_t>(c) * kTileFloats, c);
     }
   }
 
   // fully_connected.cc:1078-1082.
-  if (chain_lane && chain_b < bt && group < groups) {
+  if (kpart == 0 && chain_lane && chain_b < bt && group < groups) {
     const int n = group * kTileRows + chain_row;
     if (n < a.out_depth) {
       out = __fsub_rn(out, __fmul_rn(row_zp, kfsum_n));
@@ -446,10 +471,20 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a,
   }
 }
 
+// Wavefronts per channel group: one while that already gives the chip ~1000 wavefronts;
+// otherwise the depth is shared out, as long as each wavefront keeps at least two tiles.
+int ChooseKsplit(int out_depth, int chunks) {
+  const int groups = (out_depth + kTileRows - 1) / kTileRows;
+  int ksplit = 1;
+  while (ksplit < kWaves && groups * ksplit < 1024 && chunks >= 4 * ksplit) ksplit *= 2;
+  return ksplit;
+}
+
 template <int BT, bool FUSED, int VARIANT, int GPT>
 hipError_t LaunchOne(const Int4PackedArgs& a, int batch0, int bt, hipStream_t stream) {
   const int padded = a.chunks * kTileBlocks * kBlock;
-  const size_t lds = Int4Shared<BT>::Bytes(padded);
+  const int ksplit = ChooseKsplit(a.out_depth, a.chunks);
+  const size_t lds = Int4Shared<BT>::Bytes(padded, ksplit);
   auto kernel = FcInt4PackedKernel<BT, FUSED, VARIANT, GPT>;
   if (lds > 48 * 1024) {
     static size_t granted = 0;
@@ -462,8 +497,9 @@ hipError_t LaunchOne(const Int4PackedArgs& a, int batch0, int bt, hipStream_t st
     }
   }
   const int groups = (a.out_depth + kTileRows - 1) / kTileRows;
-  const int grid = (groups + kWaves - 1) / kWaves;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, batch0, bt);
+  const int groups_per_wg = kWaves / ksplit;
+  const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, batch0, bt, ksplit);
   return hipGetLastError();
 }
 
@@ -530,7 +566,7 @@ hipError_t LaunchPackInt4Blockwise(const uint8_t* filter, const uint16_t* scales
 bool FcInt4PackedSupports(int depth, int blocksize) {
   if (blocksize != kBlock || depth <= 0 || depth % kBlock != 0) return false;
   const int chunks = (depth / kBlock + kTileBlocks - 1) / kTileBlocks;
-  return Int4Shared<1>::Bytes(chunks * kTileBlocks * kBlock) <= 150 * 1024;
+  return Int4Shared<1>::Bytes(chunks * kTileBlocks * kBlock, kWaves) <= 150 * 1024;
 }
 
 hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const float* input_f32,
@@ -555,8 +591,9 @@ hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const 
   while (batch0 < q.batches) {
     int bt = min(input_f32 ? MaxBatchTile<true>(q.depth) : MaxBatchTile<false>(q.depth),
                  q.batches - batch0);
-    while (bt > 1 && (bt > 2 ? Int4Shared<4>::Bytes(padded) : Int4Shared<2>::Bytes(padded)) >
-                         150 * 1024) {
+    const int ksplit = ChooseKsplit(q.out_depth, a.chunks);
+    while (bt > 1 && (bt > 2 ? Int4Shared<4>::Bytes(padded, ksplit)
+                             : Int4Shared<2>::Bytes(padded, ksplit)) > 150 * 1024) {
       bt = bt > 2 ? 2 : 1;
     }
     const hipError_t err = input_f32 ? LaunchTile<true>(a, variant, batch0, bt, stream)

@@ -139,6 +139,63 @@ def test_chain_stays_on_device_and_splits_around_cpu_nodes():
         assert np.array_equal(h.read(y2), w2) and np.array_equal(h.read(y3), w3)
 
 
+@pytest.mark.parametrize("streams", [1, 2, 4])
+def test_decoder_shaped_partition_on_several_streams(streams):
+    """x -> up -> {a, b, c} (three consumers of one tensor, on different streams) plus two
+    nodes fed straight from the host and a node that consumes `a`: every cross-stream edge
+    (upload -> node, node -> node, node -> download) carries data, so a missing wait shows
+    as a wrong result. Repeated invokes with new inputs check that events are re-armed."""
+    rng = np.random.default_rng(31)
+    B = 2
+    cu = wl.hybrid_fc(B, 256, 512, seed=41)
+    heads = [wl.hybrid_fc(B, 512, n, seed=42 + i) for i, n in enumerate((96, 64, 200))]
+    tail = wl.hybrid_fc(B, 96, 40, seed=50)
+    roots = [wl.hybrid_fc(B, 1024, 72, seed=60), wl.blockwise_int4_fc(B, 2048, 24, seed=61, lo=-8, hi=7)]
+    with FakeHost() as h:
+        def hybrid(x, c, n, k):
+            w = h.tensor(INT8, (n, k), data=c["w"], const=True)
+            h.affine(w, c["pcs"])
+            y = h.tensor(FLOAT32, (B, n))
+            h.fc(x, w, None, y, asymmetric=True)
+            return y
+        x = h.tensor(FLOAT32, (B, 256), data=cu["x"])
+        up = hybrid(x, cu, 512, 256)
+        ys = [hybrid(up, c, c["w"].shape[0], 512) for c in heads]
+        yt = hybrid(ys[0], tail, 40, 96)
+        xr0 = h.tensor(FLOAT32, (B, 1024), data=roots[0]["x"])
+        yr0 = hybrid(xr0, roots[0], 72, 1024)
+        xr1 = h.tensor(FLOAT32, (B, 2048), data=roots[1]["x"])
+        w4 = h.tensor(INT4, (24, 2048), data=roots[1]["packed"], const=True)
+        s4 = h.tensor(FLOAT16, (24, 64), data=roots[1]["scales"], const=True)
+        h.blockwise(w4, s4, 32)
+        yr1 = h.tensor(FLOAT32, (B, 24))
+        h.fc(xr1, w4, None, yr1)
+        assert h.load_delegate({"streams": streams}) == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert len(h.plan()) == 1  # one partition holds all seven nodes
+        for trial in range(3):
+            xin = cu["x"] if trial == 0 else rng.standard_normal((B, 256)).astype(np.float32)
+            h.write(x, xin)
+            assert h.invoke() == OK, h.errors()
+            w_up = oracle.fc_hybrid(xin, cu["w"], cu["pcs"])
+            wants = [oracle.fc_hybrid(w_up, c["w"], c["pcs"]) for c in heads]
+            want_tail = oracle.fc_hybrid(wants[0], tail["w"], tail["pcs"])
+            for y, want in zip(ys[1:] + [yt], wants[1:] + [want_tail]):
+                assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+            assert np.array_equal(h.read(yr0).view(np.uint32),
+                                  oracle.fc_hybrid(roots[0]["x"], roots[0]["w"], roots[0]["pcs"]).view(np.uint32))
+            assert np.array_equal(
+                h.read(yr1).view(np.uint32),
+                oracle.fc_blockwise_int4(roots[1]["x"], roots[1]["packed"], 24,
+                                         roots[1]["scales"].view(np.uint16), 32).view(np.uint32))
+
+
+def test_streams_option_is_validated():
+    with FakeHost() as h:
+        assert h.load_delegate({"streams": 9}) != 0
+        assert "streams" in h.errors()
+
+
 def test_shared_input_and_unclaimed_node_fall_back_to_cpu():
     """q/k/v-style fan-out from one input, plus a uint8 FC the delegate must leave alone."""
     c = wl.hybrid_fc(2, 512, 96, seed=9)

@@ -360,7 +360,8 @@ def _run_int4(fc, c, bias=None, packed=True):
 @pytest.mark.parametrize("B,K,N", [(1, 4096, 1024), (4, 2048, 512), (1, 2048, 256), (4, 16384, 64),
                                    (1, 16384, 130), (2, 32, 4), (3, 96, 9), (8, 1024, 77),
                                    (5, 4096, 40), (1, 8192, 31), (9, 2048, 20), (2, 6144, 24),
-                                   (3, 16384, 24), (2, 8192, 16), (1, 32768, 12), (2, 20480, 8)])
+                                   (3, 16384, 24), (2, 8192, 16), (1, 32768, 12), (2, 20480, 8),
+                                   (2, 17408, 10), (4, 16384, 2048), (1, 9216, 520)])
 @pytest.mark.parametrize("packed", [True, False])
 def test_blockwise_int4_shapes(fc, B, K, N, packed):
     """Config 3 / config 5 depths (2048, 4096, 16384) and ragged sizes, blocksize 32, with the
