@@ -366,14 +366,51 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
                 run_level(layer[4:6], bufs)
                 run_level(layer[6:7], bufs)
 
+        # Grouped launches: independent nodes of one depth run as ONE kernel.
+        def bound_group(keyed_nodes):
+            ops_ = [op for op, _ in keyed_nodes]
+            ys = [torch.empty((b, op.out_depth), dtype=torch.float32, device="cuda") for op in ops_]
+            return fc.GroupedBlockwiseInt4(ops_).bind([xin[op.depth] for op in ops_], ys)
+
+        layers = [keyed[l * per_layer:(l + 1) * per_layer] for l in range(wl.GEMMA2B_LAYERS)]
+        # As the configuration defines it, every node is independent: all nodes of one depth
+        # can share launches (groups of up to 32 nodes).
+        shallow = [kn for kn in keyed if kn[0].depth == 2048]
+        deep = [kn for kn in keyed if kn[0].depth != 2048]
+        mx = fc.GroupedBlockwiseInt4.MAX_NODES
+        all_groups = [bound_group(part[i:i + mx]) for part in (shallow, deep)
+                      for i in range(0, len(part), mx)]
+        # Decoder dependencies: {q, k, v} | o | {gate, up} | down, layer after layer.
+        decoder_groups = [[bound_group(layer[0:3]), bound_group(layer[3:4]),
+                           bound_group(layer[4:6]), bound_group(layer[6:7])] for layer in layers]
+
+        def grouped_independent():
+            for grp in all_groups:
+                grp()
+
+        def grouped_decoder_order():
+            for stages in decoder_groups:
+                for grp in stages:
+                    grp()
+
         res = {}
-        for name, fn in (("one_stream", serial), ("independent_nodes_4_streams", independent),
-                         ("decoder_dependencies_4_streams", decoder_order)):
+        for name, fn in (("one_launch_per_node_one_stream", serial),
+                         ("one_launch_per_node_4_streams_independent", independent),
+                         ("one_launch_per_node_4_streams_decoder_dependencies", decoder_order),
+                         ("grouped_launches_independent_nodes", grouped_independent),
+                         ("grouped_launches_decoder_dependencies", grouped_decoder_order)):
             gc = capture(fn)
             us = timed_replays([gc], 30) * 1e3
             res[name] = dict(us_per_token=round(us, 1), gbps=round(chain_bytes / us / 1e3, 1),
                              frac_of_hbm_peak=round(chain_bytes / us / 1e3 / HBM_PEAK_GBPS, 4))
             del gc
+        res["launches_per_token"] = {"per_node": len(nodes),
+                                     "grouped_independent": len(all_groups),
+                                     "grouped_decoder_dependencies": 4 * wl.GEMMA2B_LAYERS}
+        res["note"] = ("inputs are independent per node and outputs are discarded, as the "
+                       "configuration states; 'decoder_dependencies' imposes the order a real "
+                       "decoder layer would ({q,k,v} -> o -> {gate,up} -> down)")
+        del all_groups, decoder_groups
         res.update(fc_nodes=len(nodes), weight_bytes=chain_bytes)
         out["config5_gemma2b_fc_chain_B%d" % b] = res
     return out

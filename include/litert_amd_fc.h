@@ -256,6 +256,39 @@ int lrtfc_fc_blockwise_int4_packed_quantized(const int8_t* quantized_input,
                                              const float* bias, float* output, int batches,
                                              int depth, int out_depth, void* stream);
 
+/* ---- Several blockwise-int4 nodes in one launch ----------------------------------------
+ * Nodes of a graph that do not depend on each other (the q/k/v or the gate/up projections of
+ * a decoder layer) and share depth and batch count can run as ONE kernel: the gaps between
+ * launches disappear and small filters overlap large ones. The reference has no counterpart
+ * (its interpreter runs nodes one after another, tflite/core/subgraph.cc:1687-1693); every
+ * node computes exactly what lrtfc_fc_blockwise_int4_packed computes for it.
+ *   lrtfc_int4_group_prepare: once per group (and again when a pointer or shape changes);
+ *     writes a table of lrtfc_int4_group_table_bytes() into `device_table` (synchronously)
+ *     and fills `launch`. count at most LRTFC_INT4_GROUP_MAX; all pointers are device
+ *     pointers; bias may be NULL per node.
+ *   lrtfc_fc_blockwise_int4_packed_grouped: the launch (one kernel per 4 batch rows, per 2
+ *     above depth 4096); allocates and copies nothing. */
+#define LRTFC_INT4_GROUP_MAX 32
+typedef struct lrtfc_int4_group_node {
+  const float* input;            /* [batches, depth] */
+  const uint8_t* retiled_filter; /* from lrtfc_pack_int4_blockwise */
+  const float* kfsum;            /* [out_depth] */
+  const float* bias;             /* [out_depth] or NULL */
+  float* output;                 /* [batches, out_depth] */
+  int out_depth;
+} lrtfc_int4_group_node;
+typedef struct lrtfc_int4_group_launch {
+  int count, grid_blocks, ksplit, batches, depth;
+} lrtfc_int4_group_launch;
+size_t lrtfc_int4_group_table_bytes(void);
+int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,
+                             int depth, void* device_table, lrtfc_int4_group_launch* launch,
+                             void* stream);
+int lrtfc_fc_blockwise_int4_packed_grouped(const void* device_table,
+                                           const lrtfc_int4_group_launch* launch,
+                                           int quant_variant, void* stream);
+
+
 /* Same product on already-quantized activations (workspace layout not needed). */
 int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
                                       const float* scaling_factors, const int32_t* zero_points,

@@ -55,6 +55,9 @@ SYMBOLS = [
     ("lrtfc_fc_blockwise_int4_packed", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     ("lrtfc_fc_blockwise_int4_packed_quantized", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i,
                                                       _i, _vp]),
+    ("lrtfc_int4_group_table_bytes", _sz, []),
+    ("lrtfc_int4_group_prepare", _i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
+    ("lrtfc_fc_blockwise_int4_packed_grouped", _i, [_vp, _vp, _i, _vp]),
     ("lrtfc_fc_blockwise_int4_quantized", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
                                                _i, _vp]),
 ]
@@ -91,3 +94,15 @@ def check(status):
 
 def init(device=0):
     check(load().lrtfc_init(device))
+
+
+class Int4GroupNode(C.Structure):
+    """lrtfc_int4_group_node."""
+    _fields_ = [("input", C.c_void_p), ("retiled_filter", C.c_void_p), ("kfsum", C.c_void_p),
+                ("bias", C.c_void_p), ("output", C.c_void_p), ("out_depth", C.c_int)]
+
+
+class Int4GroupLaunch(C.Structure):
+    """lrtfc_int4_group_launch."""
+    _fields_ = [("count", C.c_int), ("grid_blocks", C.c_int), ("ksplit", C.c_int),
+                ("batches", C.c_int), ("depth", C.c_int)]

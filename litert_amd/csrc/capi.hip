@@ -623,6 +623,44 @@ int lrtfc_fc_blockwise_int4_packed_quantized(const int8_t* quantized_input,
                             kfsum, bias, output, batches, depth, out_depth, 0, stream);
 }
 
+size_t lrtfc_int4_group_table_bytes(void) { return lrtfc::Int4GroupTableBytes(); }
+
+int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,
+                             int depth, void* device_table, lrtfc_int4_group_launch* launch,
+                             void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(nodes && device_table && launch, "null pointer");
+  LRTFC_REQUIRE(count >= 1 && count <= LRTFC_INT4_GROUP_MAX, "a group holds 1..%d nodes, got %d",
+                LRTFC_INT4_GROUP_MAX, count);
+  LRTFC_REQUIRE(lrtfc::FcInt4PackedSupports(depth, 32), "depth %d is not a multiple of 32", depth);
+  LRTFC_REQUIRE(batches >= 1, "a grouped launch needs at least one batch row");
+  for (int i = 0; i < count; ++i) {
+    LRTFC_REQUIRE(nodes[i].input && nodes[i].retiled_filter && nodes[i].kfsum && nodes[i].output,
+                  "null pointer in node %d", i);
+    LRTFC_REQUIRE(nodes[i].out_depth >= 1, "node %d has no output channels", i);
+    LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(nodes[i].retiled_filter) & 15) == 0,
+                  "retiled filter of node %d must be 16-byte aligned", i);
+  }
+  const hipError_t err = lrtfc::PrepareInt4Group(nodes, count, batches, depth, device_table,
+                                                 launch, AsStream(stream));
+  return FromHip(err, "int4 group table upload");
+}
+
+int lrtfc_fc_blockwise_int4_packed_grouped(const void* device_table,
+                                           const lrtfc_int4_group_launch* launch,
+                                           int quant_variant, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(device_table && launch, "null pointer");
+  LRTFC_REQUIRE(launch->count >= 1 && launch->count <= LRTFC_INT4_GROUP_MAX &&
+                    launch->grid_blocks >= 1 && launch->ksplit >= 1 && launch->ksplit <= 4,
+                "launch record was not filled by lrtfc_int4_group_prepare");
+  LRTFC_REQUIRE(quant_variant >= 0 && quant_variant <= LRTFC_QUANT_NEON_LEGACY,
+                "unknown quantizer variant");
+  return FromHip(lrtfc::LaunchFcInt4PackedGrouped(device_table, *launch, quant_variant,
+                                                  AsStream(stream)),
+                 "grouped blockwise int4 GEMV");
+}
+
 int lrtfc_fc_blockwise_int4(const float* input, const uint8_t* packed_filter,
                             const uint16_t* scales_f16, const float* kfsum, const float* bias,
                             float* output, int batches, int depth, int out_depth, int blocksize,

@@ -35,6 +35,7 @@ constexpr int kTileBytes = kPlanes * 1024;
 constexpr int kTileVecs = kPlanes * 64;  // i32x4 per tile
 constexpr int kRingTiles = 2;
 constexpr int kPStride = kTileBlocks + 4;  // floats per (row, batch) line of parked products
+constexpr int kMaxGroupNodes = LRTFC_INT4_GROUP_MAX;
 
 __global__ __launch_bounds__(kThreads) void PackInt4BlockwiseKernel(
     const uint8_t* __restrict__ filter, const uint16_t* __restrict__ scales, int out_depth,
@@ -131,10 +132,10 @@ struct Int4Shared {
 
 // GPT: groups of 8 depth positions each thread keeps in registers between the two passes of
 // the prologue; the register form covers depth <= GPT * 256 * 8.
+// The work of one workgroup; `block` is its index among the workgroups of this filter.
 template <int BT, bool FUSED, int VARIANT, int GPT>
-__global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a, int batch0,
-                                                               int bt, int ksplit) {
-  extern __shared__ __align__(16) int8_t smem[];
+__device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int block, int batch0,
+                                                 int bt, int ksplit, int8_t* smem) {
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
   const int wave = tid / kWaveSize;
@@ -146,7 +147,7 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a,
   // filters would otherwise leave most of the chip without a wavefront).
   const int kpart = wave % ksplit;
   const int group_in_wg = wave / ksplit;
-  const int group = blockIdx.x * (kWaves / ksplit) + group_in_wg;  // may run past the last
+  const int group = block * (kWaves / ksplit) + group_in_wg;  // may run past the last
   const i32x4* tbase = reinterpret_cast<const i32x4*>(a.packed) +
                        static_cast<size_t>(min(group, groups - 1)) * chunks * kTileVecs + lane;
   Int4Shared<BT> sh(smem, padded, chunks, ksplit);
@@ -471,6 +472,39 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a,
   }
 }
 
+template <int BT, bool FUSED, int VARIANT, int GPT>
+__global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a, int batch0,
+                                                               int bt, int ksplit) {
+  extern __shared__ __align__(16) int8_t smem[];
+  FcInt4PackedBody<BT, FUSED, VARIANT, GPT>(a, blockIdx.x, batch0, bt, ksplit, smem);
+}
+
+// Several filters of the same depth in one launch (nodes of a graph that do not depend on
+// each other: the q/k/v or gate/up projections of a decoder layer). The table lives in device
+// memory: per node its arguments and the index of its first workgroup. One launch instead of
+// `count` removes count - 1 launch gaps and lets small filters overlap large ones.
+struct Int4GroupTable {
+  int first_block[kMaxGroupNodes + 1];
+  int reserved[3];
+  Int4PackedArgs node[kMaxGroupNodes];
+};
+
+template <int BT, int VARIANT, int GPT>
+__global__ __launch_bounds__(kThreads) void FcInt4PackedGroupedKernel(
+    const Int4GroupTable* __restrict__ table, int count, int batch0, int bt, int ksplit) {
+  extern __shared__ __align__(16) int8_t smem[];
+  // first_block is ascending: the node of this workgroup is the number of later nodes whose
+  // first workgroup is not beyond it. One vector load and a ballot instead of a scalar walk.
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int probe = min(lane + 1, count);
+  const bool not_beyond =
+      lane + 1 < count && static_cast<int>(blockIdx.x) >= table->first_block[probe];
+  const int node = __builtin_amdgcn_readfirstlane(__popcll(__ballot(not_beyond)));
+  const Int4PackedArgs a = table->node[node];
+  FcInt4PackedBody<BT, true, VARIANT, GPT>(a, blockIdx.x - table->first_block[node], batch0, bt,
+                                           ksplit, smem);
+}
+
 // Wavefronts per channel group: one while that already gives the chip ~1000 wavefronts;
 // otherwise the depth is shared out, as long as each wavefront keeps at least two tiles.
 int ChooseKsplit(int out_depth, int chunks) {
@@ -600,6 +634,114 @@ hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const 
                                      : LaunchTile<false>(a, variant, batch0, bt, stream);
     if (err != hipSuccess) return err;
     batch0 += bt;
+  }
+  return hipSuccess;
+}
+
+
+hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int batches, int depth,
+                            void* device_table, lrtfc_int4_group_launch* launch,
+                            hipStream_t stream) {
+  if (count < 1 || count > kMaxGroupNodes || !FcInt4PackedSupports(depth, kBlock)) {
+    return hipErrorInvalidValue;
+  }
+  if (batches < 1) return hipErrorInvalidValue;
+  const int chunks = (depth / kBlock + kTileBlocks - 1) / kTileBlocks;
+  int total_out = 0;
+  for (int i = 0; i < count; ++i) total_out += nodes[i].out_depth;
+  const int ksplit = ChooseKsplit(total_out, chunks);
+  const int groups_per_wg = kWaves / ksplit;
+  Int4GroupTable host{};
+  int next = 0;
+  for (int i = 0; i < count; ++i) {
+    host.first_block[i] = next;
+    Int4PackedArgs& a = host.node[i];
+    a.packed = nodes[i].retiled_filter;
+    a.input_f32 = nodes[i].input;
+    a.input_q = nullptr;
+    a.scaling_factors = nullptr;
+    a.zero_points = nullptr;
+    a.kfsum = nodes[i].kfsum;
+    a.bias = nodes[i].bias;
+    a.output = nodes[i].output;
+    a.batches = batches;
+    a.depth = depth;
+    a.out_depth = nodes[i].out_depth;
+    a.chunks = chunks;
+    const int groups = (nodes[i].out_depth + kTileRows - 1) / kTileRows;
+    next += (groups + groups_per_wg - 1) / groups_per_wg;
+  }
+  host.first_block[count] = next;
+  // Synchronous: the table is a stack object.
+  hipError_t err = hipMemcpyAsync(device_table, &host, sizeof(host), hipMemcpyHostToDevice, stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(stream);
+  if (err != hipSuccess) return err;
+  launch->count = count;
+  launch->grid_blocks = next;
+  launch->ksplit = ksplit;
+  launch->batches = batches;
+  launch->depth = depth;
+  return hipSuccess;
+}
+
+size_t Int4GroupTableBytes() { return sizeof(Int4GroupTable); }
+
+namespace {
+template <int BT, int VARIANT, int GPT>
+hipError_t LaunchGroupedOne(const void* table, const lrtfc_int4_group_launch& l, int batch0,
+                            int bt, hipStream_t stream) {
+  const int chunks = (l.depth / kBlock + kTileBlocks - 1) / kTileBlocks;
+  const int padded = chunks * kTileBlocks * kBlock;
+  const size_t lds = Int4Shared<BT>::Bytes(padded, l.ksplit);
+  auto kernel = FcInt4PackedGroupedKernel<BT, VARIANT, GPT>;
+  if (lds > 48 * 1024) {
+    static size_t granted = 0;
+    if (lds > granted) {
+      hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(lds));
+      if (err != hipSuccess) return err;
+      granted = lds;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3(l.grid_blocks), dim3(kThreads), lds, stream,
+                     static_cast<const Int4GroupTable*>(table), l.count, batch0, bt, l.ksplit);
+  return hipGetLastError();
+}
+
+template <int BT, int GPT>
+hipError_t LaunchGroupedVariant(const void* table, const lrtfc_int4_group_launch& l, int variant,
+                                int batch0, int bt, hipStream_t stream) {
+  switch (variant) {
+    case LRTFC_QUANT_NEON_V8:
+      return LaunchGroupedOne<BT, LRTFC_QUANT_NEON_V8, GPT>(table, l, batch0, bt, stream);
+    case LRTFC_QUANT_NEON_LEGACY:
+      return LaunchGroupedOne<BT, LRTFC_QUANT_NEON_LEGACY, GPT>(table, l, batch0, bt, stream);
+    default:
+      return LaunchGroupedOne<BT, LRTFC_QUANT_PORTABLE, GPT>(table, l, batch0, bt, stream);
+  }
+}
+}  // namespace
+
+hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_launch& l,
+                                     int variant, hipStream_t stream) {
+  if (l.count < 1 || l.grid_blocks < 1) return hipSuccess;
+  const bool deep = l.depth > kShallowDepth && l.depth <= kDeepDepth;
+  const int tile = MaxBatchTile<true>(l.depth);
+  for (int batch0 = 0; batch0 < l.batches; batch0 += tile) {  // more rows: one launch per tile
+    const int bt = min(tile, l.batches - batch0);
+    hipError_t err;
+    if (deep) {
+      err = bt <= 1 ? LaunchGroupedVariant<1, 8>(table, l, variant, batch0, bt, stream)
+                    : LaunchGroupedVariant<2, 8>(table, l, variant, batch0, bt, stream);
+    } else if (bt <= 1) {
+      err = LaunchGroupedVariant<1, 2>(table, l, variant, batch0, bt, stream);
+    } else if (bt <= 2) {
+      err = LaunchGroupedVariant<2, 2>(table, l, variant, batch0, bt, stream);
+    } else {
+      err = LaunchGroupedVariant<4, 2>(table, l, variant, batch0, bt, stream);
+    }
+    if (err != hipSuccess) return err;
   }
   return hipSuccess;
 }

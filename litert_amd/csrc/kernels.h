@@ -93,6 +93,13 @@ size_t PackedInt4BlockwiseBytes(int out_depth, int depth);
 hipError_t LaunchPackInt4Blockwise(const uint8_t* filter, const uint16_t* scales, int out_depth,
                                    int depth, uint8_t* packed, hipStream_t stream);
 bool FcInt4PackedSupports(int depth, int blocksize);
+// Grouped launch: several filters of one depth, one kernel (see lrtfc_int4_group_prepare).
+size_t Int4GroupTableBytes();
+hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int batches, int depth,
+                            void* device_table, lrtfc_int4_group_launch* launch,
+                            hipStream_t stream);
+hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_launch& launch,
+                                     int variant, hipStream_t stream);
 hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const float* input_f32,
                               int variant, hipStream_t stream);
 

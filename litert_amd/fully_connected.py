@@ -345,3 +345,57 @@ class FullyConnectedBlockwiseInt4:
             _ptr(q), _ptr(sf), _ptr(zp), _ptr(self.retiled), _ptr(self.kfsum), _ptr(self.bias),
             _ptr(out), batches, self.depth, self.out_depth, _stream()))
         return out
+
+
+class GroupedBlockwiseInt4:
+    """Several FullyConnectedBlockwiseInt4 nodes of one depth that do not depend on each other
+    (q/k/v, gate/up), run as ONE kernel. `bind` fixes the input and output tensors of every
+    node (the launch reads their addresses from a table in device memory); `__call__`
+    launches. Results are those of the nodes' own calls."""
+
+    MAX_NODES = 32
+
+    def __init__(self, ops):
+        if not 1 <= len(ops) <= self.MAX_NODES:
+            raise ValueError("a group holds 1..%d nodes" % self.MAX_NODES)
+        depth = ops[0].depth
+        for op in ops:
+            if op.retiled is None or op.depth != depth or op.variant != ops[0].variant:
+                raise ValueError("grouped nodes need the re-tiled filter, one depth, one variant")
+        self.ops = list(ops)
+        self.depth = depth
+        self.variant = ops[0].variant
+        self.table = torch.empty(capi.load().lrtfc_int4_group_table_bytes(), dtype=torch.uint8,
+                                 device="cuda")
+        self.launch = None
+        self._bound = None
+
+    def bind(self, inputs, outputs):
+        """inputs[i] [B, depth] float32, outputs[i] [B, out_depth_i] float32, CUDA, contiguous."""
+        batches = inputs[0].numel() // self.depth
+        nodes = (capi.Int4GroupNode * len(self.ops))()
+        for i, (op, x, y) in enumerate(zip(self.ops, inputs, outputs)):
+            if not (x.is_contiguous() and y.is_contiguous()):
+                raise ValueError("grouped inputs and outputs must be contiguous")
+            if x.numel() != batches * self.depth or y.numel() != batches * op.out_depth:
+                raise ValueError("node %d: tensor sizes do not match the group" % i)
+            nodes[i].input = x.data_ptr()
+            nodes[i].retiled_filter = op.retiled.data_ptr()
+            nodes[i].kfsum = op.kfsum.data_ptr()
+            nodes[i].bias = op.bias.data_ptr() if op.bias is not None else None
+            nodes[i].output = y.data_ptr()
+            nodes[i].out_depth = op.out_depth
+        launch = capi.Int4GroupLaunch()
+        capi.check(capi.load().lrtfc_int4_group_prepare(
+            C.byref(nodes), len(self.ops), batches, self.depth, _ptr(self.table),
+            C.byref(launch), _stream()))
+        self.launch = launch
+        self._bound = (list(inputs), list(outputs))  # keep the tensors alive
+        return self
+
+    def __call__(self):
+        if self.launch is None:
+            raise RuntimeError("bind() the group's tensors first")
+        capi.check(capi.load().lrtfc_fc_blockwise_int4_packed_grouped(
+            _ptr(self.table), C.byref(self.launch), self.variant, _stream()))
+        return self._bound[1]

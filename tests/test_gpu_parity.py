@@ -385,6 +385,40 @@ def test_blockwise_int4_split_launch_matches_oracle(fc, B, K, N):
     assert _bits_equal(y, want)
 
 
+@pytest.mark.parametrize("B,K,Ns", [(1, 2048, (64, 8, 24, 130, 520)), (3, 2048, (16, 256, 9)),
+                                    (4, 1024, (40,)), (1, 16384, (16, 40)), (2, 8192, (24, 8, 72)),
+                                    (9, 2048, (24, 80)), (5, 16384, (8, 16)),
+                                    (1, 64, tuple(range(4, 36)))])
+def test_blockwise_int4_grouped_launch_matches_oracle(fc, B, K, Ns):
+    """Several filters of one depth in one launch: every node against the oracle, with its
+    own input and, for odd channel counts, its own bias; then again after re-binding to new
+    inputs (the table is rewritten, the filters are not)."""
+    rng = np.random.default_rng(8)
+    cs = [wl.blockwise_int4_fc(B, K, n, seed=500 + i + n, lo=-8, hi=7) for i, n in enumerate(Ns)]
+    biases = [rng.standard_normal(n).astype(np.float32) if n % 2 else None for n in Ns]
+    ops = [fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], K, 32, b)
+           for c, b in zip(cs, biases)]
+    group = fc.GroupedBlockwiseInt4(ops)
+    for trial in range(2):
+        xs_np = [c["x"] if trial == 0 else rng.standard_normal((B, K)).astype(np.float32) for c in cs]
+        xs = [_cuda(x) for x in xs_np]
+        ys = [torch.full((B, n), float("nan"), dtype=torch.float32, device="cuda") for n in Ns]
+        group.bind(xs, ys)()
+        torch.cuda.synchronize()
+        for c, b, x, y, n in zip(cs, biases, xs_np, ys, Ns):
+            want = oracle.fc_blockwise_int4(x, c["packed"], n, c["scales"].view(np.uint16), 32, b)
+            assert _bits_equal(y.cpu().numpy(), want), (trial, n)
+
+
+def test_blockwise_int4_grouped_launch_needs_bind(fc):
+    c = wl.blockwise_int4_fc(1, 64, 8, seed=2, lo=-8, hi=7)
+    op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], 64, 32)
+    with pytest.raises(RuntimeError):
+        fc.GroupedBlockwiseInt4([op])()
+    with pytest.raises(ValueError):
+        fc.GroupedBlockwiseInt4([])
+
+
 @pytest.mark.parametrize("B,K,N,bs", [(2, 128, 6, 64), (1, 64, 5, 16), (3, 256, 4, 128), (2, 96, 8, 8)])
 def test_blockwise_int4_other_block_sizes(fc, B, K, N, bs):
     c = wl.blockwise_int4_fc(B, K, N, blocksize=bs, seed=5 + bs, lo=-8, hi=7)
