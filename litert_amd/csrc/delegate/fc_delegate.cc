@@ -228,6 +228,9 @@ struct FcNode {
   // waits for this one.
   int lane = 0, producer = -1;
   bool signal = false;
+  // Grouped launch (several independent int4 nodes of one depth in one kernel): index into
+  // PartitionKernel::groups, or -1.
+  int group = -1;
   DeviceBuffer filter_dev, retiled_dev, bias_dev, mult_dev, shift_dev, row_sums_dev, pcs_dev,
       scales_dev, kfsum_dev;
 };
@@ -256,6 +259,12 @@ struct PartitionKernel {
   hipEvent_t lane_done[kMaxStreams] = {};
   std::vector<hipEvent_t> node_done;  // per node; only the signalling ones are created
   bool lane_used[kMaxStreams] = {};
+  struct Group {
+    std::vector<int> members;  // node indices, consecutive
+    DeviceBuffer table;
+    lrtfc_int4_group_launch launch{};
+  };
+  std::vector<Group> groups;
   ~PartitionKernel() {
     for (hipEvent_t e : node_done) {
       if (e) (void)hipEventDestroy(e);
@@ -340,35 +349,13 @@ void* KernelInit(TfLiteContext* ctx, const char* buffer, size_t /*length*/) {
     produced[n.output] = true;
     kernel->nodes.push_back(std::move(n));
   }
-  // Streams: a node continues on its producer's stream unless a sibling already did; nodes
-  // without a producer in the partition, and further siblings, take streams round-robin.
   {
     std::map<int, int> producer_of;  // tensor -> node that writes it
-    std::vector<bool> continued(kernel->nodes.size(), false);
-    int next_lane = 0;
     for (size_t i = 0; i < kernel->nodes.size(); ++i) {
       FcNode& n = kernel->nodes[i];
       auto it = producer_of.find(n.input);
       n.producer = it == producer_of.end() ? -1 : it->second;
-      if (n.producer >= 0 && !continued[n.producer]) {
-        n.lane = kernel->nodes[n.producer].lane;
-        continued[n.producer] = true;
-      } else {
-        n.lane = next_lane++ % kernel->num_streams;
-      }
-      if (n.producer >= 0 && kernel->nodes[n.producer].lane != n.lane) {
-        kernel->nodes[n.producer].signal = true;
-      }
-      kernel->lane_used[n.lane] = true;
       producer_of[n.output] = static_cast<int>(i);
-    }
-    kernel->node_done.assign(kernel->nodes.size(), nullptr);
-    for (size_t i = 0; i < kernel->nodes.size(); ++i) {
-      if (kernel->nodes[i].signal &&
-          hipEventCreateWithFlags(&kernel->node_done[i], hipEventDisableTiming) != hipSuccess) {
-        ctx->ReportError(ctx, "litert_amd delegate: cannot create a HIP event");
-        return reinterpret_cast<void*>(-1);
-      }
     }
   }
   // Every tensor the runtime lists as an output of the partition goes back to the host.
@@ -552,9 +539,97 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
   // Device homes for this node's activations.
   RETURN_IF_HIP(ctx, k->activations[n->input].Ensure(input.bytes));
   RETURN_IF_HIP(ctx, k->activations[n->output].Ensure(output.bytes));
-  if (n->kind != FcKind::kInt8 && (!n->use_retiled || n->split_quantize)) {
-    RETURN_IF_HIP(ctx, k->workspace[n->lane].Ensure(
-                           lrtfc_activation_workspace_bytes(n->batches, n->depth)));
+  return kTfLiteOk;
+}
+
+// After every node is prepared (shapes and kernel forms known): which nodes share a launch,
+// which stream each unit runs on, which nodes other streams wait for.
+TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
+  const int count = static_cast<int>(k->nodes.size());
+  // Groups: runs of consecutive blockwise-int4 nodes on the fused re-tiled kernel with one
+  // depth and batch count, none of which reads what another of the run writes.
+  k->groups.clear();
+  for (FcNode& n : k->nodes) n.group = -1;
+  auto groupable = [&](const FcNode& n) {
+    return n.kind == FcKind::kInt4Blockwise && n.use_retiled && !n.split_quantize &&
+           n.depth > 0 && n.batches > 0 && n.out_depth > 0;
+  };
+  for (int i = 0; i < count;) {
+    int j = i;
+    if (groupable(k->nodes[i])) {
+      while (j + 1 < count && j + 1 - i < LRTFC_INT4_GROUP_MAX && groupable(k->nodes[j + 1]) &&
+             k->nodes[j + 1].depth == k->nodes[i].depth &&
+             k->nodes[j + 1].batches == k->nodes[i].batches && k->nodes[j + 1].producer < i) {
+        ++j;
+      }
+    }
+    if (j > i) {
+      PartitionKernel::Group g;
+      for (int m = i; m <= j; ++m) {
+        g.members.push_back(m);
+        k->nodes[m].group = static_cast<int>(k->groups.size());
+      }
+      k->groups.push_back(std::move(g));
+    }
+    i = j + 1;
+  }
+  // Streams: a unit (node or group) continues on the stream of its first node's producer
+  // unless a sibling already did; units without a producer in the partition, and further
+  // siblings, take streams round-robin.
+  std::vector<bool> continued(count, false);
+  int next_lane = 0;
+  for (int i = 0; i < k->kMaxStreams; ++i) k->lane_used[i] = false;
+  for (int i = 0; i < count; ++i) {
+    FcNode& n = k->nodes[i];
+    n.signal = false;
+    const bool follower = n.group >= 0 && k->groups[n.group].members.front() != i;
+    if (follower) {
+      n.lane = k->nodes[k->groups[n.group].members.front()].lane;
+    } else if (n.producer >= 0 && !continued[n.producer]) {
+      n.lane = k->nodes[n.producer].lane;
+      continued[n.producer] = true;
+    } else {
+      n.lane = next_lane++ % k->num_streams;
+    }
+    k->lane_used[n.lane] = true;
+  }
+  for (const FcNode& n : k->nodes) {
+    if (n.producer >= 0 && k->nodes[n.producer].lane != n.lane) k->nodes[n.producer].signal = true;
+  }
+  for (hipEvent_t& e : k->node_done) {
+    if (e) (void)hipEventDestroy(e);
+    e = nullptr;
+  }
+  k->node_done.assign(count, nullptr);
+  for (int i = 0; i < count; ++i) {
+    if (k->nodes[i].signal) {
+      RETURN_IF_HIP(ctx, hipEventCreateWithFlags(&k->node_done[i], hipEventDisableTiming));
+    }
+  }
+  // Scratch for the nodes that quantize in a launch of their own, per stream.
+  for (const FcNode& n : k->nodes) {
+    if (n.kind != FcKind::kInt8 && (!n.use_retiled || n.split_quantize)) {
+      RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(
+                             lrtfc_activation_workspace_bytes(n.batches, n.depth)));
+    }
+  }
+  // Group tables: device addresses of every member's tensors (stable until the next prepare).
+  for (PartitionKernel::Group& g : k->groups) {
+    std::vector<lrtfc_int4_group_node> nodes(g.members.size());
+    for (size_t m = 0; m < g.members.size(); ++m) {
+      const FcNode& n = k->nodes[g.members[m]];
+      nodes[m].input = k->activations[n.input].as<float>();
+      nodes[m].retiled_filter = n.retiled_dev.as<uint8_t>();
+      nodes[m].kfsum = n.kfsum_dev.as<float>();
+      nodes[m].bias = n.bias == kTfLiteOptionalTensor ? nullptr : n.bias_dev.as<float>();
+      nodes[m].output = k->activations[n.output].as<float>();
+      nodes[m].out_depth = n.out_depth;
+    }
+    const FcNode& first = k->nodes[g.members.front()];
+    RETURN_IF_HIP(ctx, g.table.Ensure(lrtfc_int4_group_table_bytes()));
+    RETURN_IF_FC(ctx, lrtfc_int4_group_prepare(nodes.data(), static_cast<int>(nodes.size()),
+                                               first.batches, first.depth, g.table.get(),
+                                               &g.launch, k->stream));
   }
   return kTfLiteOk;
 }
@@ -566,6 +641,7 @@ TfLiteStatus KernelPrepare(TfLiteContext* ctx, TfLiteNode* node) {
     const TfLiteStatus st = PrepareNode(ctx, k, &n);
     if (st != kTfLiteOk) return st;
   }
+  RETURN_IF_OK(PlanSchedule(ctx, k));
   RETURN_IF_HIP(ctx, hipStreamSynchronize(k->stream));
   return kTfLiteOk;
 }
@@ -596,6 +672,18 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     // consumer never waits on an event that was not recorded in this invoke.)
     if (n.producer >= 0 && k->nodes[n.producer].lane != n.lane) {
       RETURN_IF_HIP(ctx, hipStreamWaitEvent(s, k->node_done[n.producer], 0));
+    }
+    if (n.group >= 0) {
+      // The whole group launches when its last member is reached: by then the waits of every
+      // member are queued on the group's stream; members record their events after it.
+      PartitionKernel::Group& g = k->groups[n.group];
+      if (g.members.back() != static_cast<int>(node_i)) continue;
+      RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4_packed_grouped(
+                            g.table.get(), &g.launch, k->state->options.quant_variant, s));
+      for (int m : g.members) {
+        if (k->nodes[m].signal) RETURN_IF_HIP(ctx, hipEventRecord(k->node_done[m], s));
+      }
+      continue;
     }
     struct SignalOnExit {
       PartitionKernel* k;
@@ -863,6 +951,22 @@ int litert_amd_classify_node(const TfLiteContext* ctx, const TfLiteNode* node,
     std::snprintf(reason, reason_size, "%s", why.c_str());
   }
   return static_cast<int>(kind);
+}
+
+// Test and tooling hook: how a prepared partition (the user_data of its delegate-kernel
+// node) will run, as text: per node "index:kind/stream[/gN]", N = its grouped launch.
+int litert_amd_describe_partition(const void* user_data, char* out, size_t out_size) {
+  if (!user_data || user_data == reinterpret_cast<const void*>(-1) || !out || !out_size) return -1;
+  const auto* k = static_cast<const PartitionKernel*>(user_data);
+  std::string text = "groups=" + std::to_string(k->groups.size()) + " nodes=";
+  for (size_t i = 0; i < k->nodes.size(); ++i) {
+    const FcNode& n = k->nodes[i];
+    text += (i ? " " : "") + std::to_string(n.node_index) + ":" +
+            std::to_string(static_cast<int>(n.kind)) + "/s" + std::to_string(n.lane);
+    if (n.group >= 0) text += "/g" + std::to_string(n.group);
+  }
+  std::snprintf(out, out_size, "%s", text.c_str());
+  return static_cast<int>(k->groups.size());
 }
 
 }  // extern "C"

@@ -58,6 +58,8 @@ def lib():
             getattr(L, name).argtypes = [C.c_void_p, C.c_int]
         for name in ("fh_node_replaced", "fh_node_input", "fh_node_output"):
             getattr(L, name).argtypes = [C.c_void_p, C.c_int, C.c_int]
+        L.fh_node_user_data.argtypes = [C.c_void_p, C.c_int]
+        L.fh_node_user_data.restype = C.c_void_p
         L.fh_errors.argtypes = [C.c_void_p]
         L.fh_errors.restype = C.c_char_p
         L.fh_clear_errors.argtypes = [C.c_void_p]
@@ -168,6 +170,14 @@ class FakeHost:
             else:
                 out.append(("cpu", [n], n))
         return out
+
+    def describe_partition(self, node, path=DELEGATE_LIB):
+        """The delegate's own account of how it will run the partition behind `node`."""
+        lib = C.CDLL(path)
+        lib.litert_amd_describe_partition.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t]
+        buf = C.create_string_buffer(4096)
+        n = lib.litert_amd_describe_partition(self.L.fh_node_user_data(self.h, node), buf, 4096)
+        return n, buf.value.decode()
 
     def node_io(self, node):
         ins = [self.L.fh_node_input(self.h, node, i) for i in range(self.L.fh_node_num_inputs(self.h, node))]

@@ -428,6 +428,7 @@ int fh_node_output(void* hp, int node, int i) { return static_cast<Host*>(hp)->n
 int fh_tensor_has_delegate(void* hp, int tensor) {
   return static_cast<Host*>(hp)->tensors[tensor].delegate != nullptr;
 }
+void* fh_node_user_data(void* hp, int node) { return static_cast<Host*>(hp)->nodes[node]->node.user_data; }
 int fh_replace_calls(void* hp) { return static_cast<Host*>(hp)->replace_calls; }
 const char* fh_errors(void* hp) { return static_cast<Host*>(hp)->errors.c_str(); }
 void fh_clear_errors(void* hp) { static_cast<Host*>(hp)->errors.clear(); }

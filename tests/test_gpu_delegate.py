@@ -190,6 +190,53 @@ def test_decoder_shaped_partition_on_several_streams(streams):
                                          roots[1]["scales"].view(np.uint16), 32).view(np.uint32))
 
 
+@pytest.mark.parametrize("streams", [1, 3])
+@pytest.mark.parametrize("B", [1, 5])
+def test_int4_nodes_share_grouped_launches(streams, B):
+    """Blockwise-int4 nodes of one depth that do not depend on each other run as one kernel:
+    {a, b, c} read the same host tensor; d reads a's output and forms a second group with two
+    more host-fed nodes. Every output is compared with the oracle, over two invokes."""
+    K = 64
+    rng = np.random.default_rng(77)
+    shapes = {"a": 64, "b": 40, "c": 8, "d": 16, "e": 24, "f": 72}
+    cs = {k: wl.blockwise_int4_fc(B, K, n, seed=90 + i, lo=-8, hi=7) for i, (k, n) in enumerate(shapes.items())}
+    with FakeHost() as h:
+        def int4(x, c, n, bias=None):
+            w = h.tensor(INT4, (n, K), data=c["packed"], const=True)
+            s_ = h.tensor(FLOAT16, (n, K // 32), data=c["scales"], const=True)
+            h.blockwise(w, s_, 32)
+            b_ = h.tensor(FLOAT32, (n,), data=bias, const=True) if bias is not None else None
+            y = h.tensor(FLOAT32, (B, n))
+            h.fc(x, w, b_, y)
+            return y
+        bias_b = rng.standard_normal(40).astype(np.float32)
+        x = h.tensor(FLOAT32, (B, K), data=cs["a"]["x"])
+        ya = int4(x, cs["a"], 64)
+        yb = int4(x, cs["b"], 40, bias_b)
+        yc = int4(x, cs["c"], 8)
+        yd = int4(ya, cs["d"], 16)
+        xe = h.tensor(FLOAT32, (B, K), data=cs["e"]["x"])
+        ye = int4(xe, cs["e"], 24)
+        yf = int4(xe, cs["f"], 72)
+        assert h.load_delegate({"streams": streams}) == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert len(h.plan()) == 1
+        groups, text = h.describe_partition(h.plan()[0][2])
+        assert groups == 2 and text.count("/g0") == 3 and text.count("/g1") == 3, text
+
+        def ref(xin, c, n, bias=None):
+            return oracle.fc_blockwise_int4(xin, c["packed"], n, c["scales"].view(np.uint16), 32, bias)
+        for trial in range(2):
+            xin = cs["a"]["x"] if trial == 0 else rng.standard_normal((B, K)).astype(np.float32)
+            h.write(x, xin)
+            assert h.invoke() == OK, h.errors()
+            wa = ref(xin, cs["a"], 64)
+            for y, want in ((yb, ref(xin, cs["b"], 40, bias_b)), (yc, ref(xin, cs["c"], 8)),
+                            (yd, ref(wa, cs["d"], 16)), (ye, ref(cs["e"]["x"], cs["e"], 24)),
+                            (yf, ref(cs["e"]["x"], cs["f"], 72))):
+                assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+
+
 def test_streams_option_is_validated():
     with FakeHost() as h:
         assert h.load_delegate({"streams": 9}) != 0
