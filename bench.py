@@ -413,7 +413,45 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         del all_groups, decoder_groups
         res.update(fc_nodes=len(nodes), weight_bytes=chain_bytes)
         out["config5_gemma2b_fc_chain_B%d" % b] = res
+    try:
+        out["config5_through_delegate_B1"] = delegate_chain(torch, wl)
+    except Exception as e:  # the stand-in interpreter is test infrastructure; report, don't fail
+        out["config5_through_delegate_B1"] = {"error": repr(e)}
     return out
+
+
+def delegate_chain(torch, wl, b=1, invokes=20):
+    """Config 5 end to end through the delegate plugin, driven by the stand-in interpreter of
+    the tests: 126 FULLY_CONNECTED nodes, host tensors in, host tensors out. Wall-clock time of
+    Invoke(), i.e. including the upload of every node's input, the download of every node's
+    output (all 126 are graph outputs here) and the final synchronization."""
+    from tests.fake_host import FakeHost, FLOAT32, FLOAT16, INT4, OK
+    rng = np.random.default_rng(5)
+    with FakeHost() as h:
+        for layer in range(wl.GEMMA2B_LAYERS):
+            for name, k, n in wl.GEMMA2B_LAYER_FCS:
+                x = h.tensor(FLOAT32, (b, k), data=rng.standard_normal((b, k)).astype(np.float32))
+                w = h.tensor(INT4, (n, k), const=True,
+                             data=rng.integers(0, 256, (n, k // 2), dtype=np.uint8))
+                s_ = h.tensor(FLOAT16, (n, k // 32), const=True,
+                              data=(rng.random((n, k // 32), dtype=np.float32) * 1.5e-2 + 5e-3).astype(np.float16))
+                h.blockwise(w, s_, 32)
+                y = h.tensor(FLOAT32, (b, n))
+                h.fc(x, w, None, y)
+        if h.load_delegate() != 0 or h.modify_graph_with_delegate() != OK or h.allocate_tensors() != OK:
+            raise RuntimeError(h.errors())
+        plan = h.plan()
+        groups, _ = h.describe_partition(plan[0][2])
+        for _ in range(3):
+            if h.invoke() != OK:
+                raise RuntimeError(h.errors())
+        t0 = time.perf_counter()
+        for _ in range(invokes):
+            h.invoke()
+        us = (time.perf_counter() - t0) / invokes * 1e6
+    return {"invoke_wall_us": round(us, 1), "partitions": len(plan), "grouped_launches": groups,
+            "fc_nodes": wl.GEMMA2B_LAYERS * len(wl.GEMMA2B_LAYER_FCS),
+            "note": "host tensors in and out: 126 uploads + 126 downloads per invoke included"}
 
 
 def cpu_baseline_leg(c):

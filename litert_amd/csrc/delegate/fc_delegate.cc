@@ -209,6 +209,33 @@ class DeviceBuffer {
   size_t bytes_ = 0;
 };
 
+// Page-locked host memory (allocated, never registered): the staging area through which a
+// partition's inputs and outputs cross PCIe in one copy each.
+class PinnedBuffer {
+ public:
+  PinnedBuffer() = default;
+  PinnedBuffer(const PinnedBuffer&) = delete;
+  PinnedBuffer& operator=(const PinnedBuffer&) = delete;
+  ~PinnedBuffer() { Release(); }
+  void Release() {
+    if (ptr_) (void)hipHostFree(ptr_);
+    ptr_ = nullptr;
+    bytes_ = 0;
+  }
+  hipError_t Ensure(size_t bytes) {
+    if (bytes <= bytes_) return hipSuccess;
+    Release();
+    hipError_t err = hipHostMalloc(&ptr_, bytes, hipHostMallocDefault);
+    if (err == hipSuccess) bytes_ = bytes;
+    return err;
+  }
+  uint8_t* get() const { return static_cast<uint8_t*>(ptr_); }
+
+ private:
+  void* ptr_ = nullptr;
+  size_t bytes_ = 0;
+};
+
 struct FcNode {
   int node_index = -1;
   FcKind kind = FcKind::kNone;
@@ -244,7 +271,17 @@ constexpr int kInt4DeepFusedMaxBatches = 2;
 struct PartitionKernel {
   DelegateState* state = nullptr;
   std::vector<FcNode> nodes;
-  std::map<int, DeviceBuffer> activations;  // tensor index -> device copy
+  // Device homes of the activation tensors: one arena laid out at prepare, the uploaded
+  // tensors first, then the downloaded ones, then those that never leave the device. The two
+  // outer regions each cross PCIe in ONE copy per invoke, through page-locked staging.
+  DeviceBuffer arena;
+  std::map<int, size_t> arena_offset;  // tensor index -> byte offset in the arena
+  size_t upload_bytes = 0, download_offset = 0, download_bytes = 0;
+  PinnedBuffer upload_stage, download_stage;
+  void* Activation(int tensor) const {
+    auto it = arena_offset.find(tensor);
+    return it == arena_offset.end() ? nullptr : arena.as<uint8_t>() + it->second;
+  }
   std::vector<int> uploads;                 // activation tensors read from the host each invoke
   std::vector<int> downloads;               // tensors written back to the host each invoke
   // Nodes that do not depend on each other (the q/k/v or gate/up projections of a decoder
@@ -536,9 +573,6 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
   }
   n->uploaded_filter = filter.data.raw;
 
-  // Device homes for this node's activations.
-  RETURN_IF_HIP(ctx, k->activations[n->input].Ensure(input.bytes));
-  RETURN_IF_HIP(ctx, k->activations[n->output].Ensure(output.bytes));
   return kTfLiteOk;
 }
 
@@ -546,6 +580,28 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
 // which stream each unit runs on, which nodes other streams wait for.
 TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
   const int count = static_cast<int>(k->nodes.size());
+  // Arena layout (tensor sizes are final here).
+  {
+    k->arena_offset.clear();
+    size_t next = 0;
+    auto place = [&](int t) {
+      if (k->arena_offset.count(t)) return;
+      k->arena_offset[t] = next;
+      next += (ctx->tensors[t].bytes + 255) & ~static_cast<size_t>(255);
+    };
+    for (int t : k->uploads) place(t);
+    k->upload_bytes = next;
+    k->download_offset = next;
+    for (int t : k->downloads) place(t);
+    k->download_bytes = next - k->download_offset;
+    for (const FcNode& n : k->nodes) {
+      place(n.input);
+      place(n.output);
+    }
+    RETURN_IF_HIP(ctx, k->arena.Ensure(next));
+    RETURN_IF_HIP(ctx, k->upload_stage.Ensure(k->upload_bytes));
+    RETURN_IF_HIP(ctx, k->download_stage.Ensure(k->download_bytes));
+  }
   // Groups: runs of consecutive blockwise-int4 nodes on the fused re-tiled kernel with one
   // depth and batch count, none of which reads what another of the run writes.
   k->groups.clear();
@@ -618,11 +674,11 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
     std::vector<lrtfc_int4_group_node> nodes(g.members.size());
     for (size_t m = 0; m < g.members.size(); ++m) {
       const FcNode& n = k->nodes[g.members[m]];
-      nodes[m].input = k->activations[n.input].as<float>();
+      nodes[m].input = static_cast<const float*>(k->Activation(n.input));
       nodes[m].retiled_filter = n.retiled_dev.as<uint8_t>();
       nodes[m].kfsum = n.kfsum_dev.as<float>();
       nodes[m].bias = n.bias == kTfLiteOptionalTensor ? nullptr : n.bias_dev.as<float>();
-      nodes[m].output = k->activations[n.output].as<float>();
+      nodes[m].output = static_cast<float*>(k->Activation(n.output));
       nodes[m].out_depth = n.out_depth;
     }
     const FcNode& first = k->nodes[g.members.front()];
@@ -653,7 +709,10 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   for (int t : k->uploads) {
     const TfLiteTensor& tensor = ctx->tensors[t];
     if (tensor.bytes == 0) continue;
-    RETURN_IF_HIP(ctx, hipMemcpyAsync(k->activations[t].get(), tensor.data.raw, tensor.bytes,
+    std::memcpy(k->upload_stage.get() + k->arena_offset[t], tensor.data.raw, tensor.bytes);
+  }
+  if (k->upload_bytes > 0) {
+    RETURN_IF_HIP(ctx, hipMemcpyAsync(k->arena.get(), k->upload_stage.get(), k->upload_bytes,
                                       hipMemcpyHostToDevice, k->stream));
   }
   bool multi = false;
@@ -695,12 +754,12 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     } signal_on_exit{k, node_i, s};
     const TfLiteTensor& output = ctx->tensors[n.output];
     if (NumElements(output.dims) == 0) continue;  // fully_connected.cc:1966-1968
-    void* out_dev = k->activations[n.output].get();
+    void* out_dev = k->Activation(n.output);
     if (n.depth == 0) {                           // fully_connected.cc:1970-1973
       RETURN_IF_HIP(ctx, hipMemsetAsync(out_dev, 0, output.bytes, s));
       continue;
     }
-    const void* in_dev = k->activations[n.input].get();
+    const void* in_dev = k->Activation(n.input);
     const bool has_bias = n.bias != kTfLiteOptionalTensor;
     const int variant = k->state->options.quant_variant;
     const float* bias_f32 = has_bias ? n.bias_dev.as<float>() : nullptr;
@@ -793,16 +852,19 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     RETURN_IF_HIP(ctx, hipEventRecord(k->lane_done[i], k->streams[i]));
     RETURN_IF_HIP(ctx, hipStreamWaitEvent(s, k->lane_done[i], 0));
   }
-  for (int t : k->downloads) {
-    TfLiteTensor& tensor = ctx->tensors[t];
-    if (tensor.bytes == 0) continue;
-    auto it = k->activations.find(t);
-    if (it == k->activations.end()) continue;
-    RETURN_IF_HIP(ctx, hipMemcpyAsync(tensor.data.raw, it->second.get(), tensor.bytes,
-                                      hipMemcpyDeviceToHost, s));
+  if (k->download_bytes > 0) {
+    RETURN_IF_HIP(ctx, hipMemcpyAsync(k->download_stage.get(),
+                                      k->arena.as<uint8_t>() + k->download_offset,
+                                      k->download_bytes, hipMemcpyDeviceToHost, s));
   }
   // The runtime reads the outputs as soon as invoke returns.
   RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+  for (int t : k->downloads) {
+    TfLiteTensor& tensor = ctx->tensors[t];
+    if (tensor.bytes == 0) continue;
+    std::memcpy(tensor.data.raw,
+                k->download_stage.get() + (k->arena_offset[t] - k->download_offset), tensor.bytes);
+  }
   return kTfLiteOk;
 }
 
