@@ -61,8 +61,8 @@ def main():
                          "copy (3 times), for a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (the op shards "
-              "by output channel with no collective; see DESIGN.md). Run with --gpus 1.",
+        print("bench.py measures one GPU: this build has no multi-GPU path (the op would shard "
+              "by output channel with no collective). Run with --gpus 1.",
               file=sys.stderr)
         sys.exit(2)
 

@@ -1,0 +1,155 @@
+"""Writes tests/golden/reference_kats.json: the known-answer vectors that the reference's own
+tests hold for the quantized FULLY_CONNECTED path, as plain data (inputs and expected outputs).
+
+The numbers are transcribed from the reference's test sources (cited per entry); nothing of the
+reference is imported or executed. Float tensors of the op tests are quantized here with the
+restated test harness (tests/kat_harness.py, after tflite/kernels/test_util.h:198-222,
+1123-1190), so that a fixture holds exactly the integer tensors the kernels see.
+
+    python tests/golden/make_reference_kats.py
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from tests import kat_harness as kh  # noqa: E402
+
+W10 = [1, 2, 3, 4, 5, 6, 7, 8, 9, 10]
+X2 = [1, 2, 3, 4, 5, 6, 7, 8, -9, -10, 1, 2, 3, 4, 5, 6, 7, -8, 9, -10]
+W4 = [1, 2, 3, 4, 5, 6, 7, 6, 5, 4] * 3
+ACT = {"none": 0, "relu": 1}
+
+
+def per_tensor(source, in_range, out_range, weights, bias, x, units, act="none", int4=False):
+    in_s, in_zp = kh.quantization_params(*in_range)
+    out_s, out_zp = kh.quantization_params(*out_range)
+    if int4:
+        w_s, w_zp = kh.quantization_params(-7.0, 7.0, -7, 7)
+        wq = kh.quantize(weights, w_s, w_zp, -7, 7).reshape(units, -1)
+    else:
+        w_s, w_zp = kh.quantization_params(-63.5, 64)
+        wq = kh.quantize(weights, w_s, w_zp).reshape(units, -1)
+    xq = kh.quantize(x, in_s, in_zp).reshape(-1, wq.shape[1])
+    bias_scale = np.float32(in_s * w_s)
+    bq = None if bias is None else kh.quantize_bias(bias, bias_scale)
+    return dict(source=source, per_channel=False, int4=int4, activation=ACT[act],
+                input=xq.tolist(), filter=wq.tolist(), bias=None if bq is None else bq.tolist(),
+                input_scale=float(in_s), input_zero_point=int(in_zp),
+                filter_scales=[float(w_s)], filter_zero_point=int(w_zp),
+                bias_scale=None if bias is None else float(bias_scale),
+                output_scale=float(out_s), output_zero_point=int(out_zp))
+
+
+def per_channel(source, scales, weights, bias, x, units, depth, act="none", int4=False):
+    in_s, in_zp = kh.quantization_params(-63.5, 64)
+    out_s, out_zp = kh.quantization_params(-127, 128)
+    scales = np.asarray(scales, np.float32)
+    w = np.asarray(weights, np.float32).reshape(units, depth)
+    inv = (np.float32(1.0) / scales).astype(np.float32)
+    lim = 7 if int4 else 127
+    wq = np.clip(kh._round_half_away(w * inv[:, None]), -lim, lim).astype(np.int8)
+    xq = kh.quantize(x, in_s, in_zp).reshape(-1, depth)
+    bscale = (scales * in_s).astype(np.float32)
+    bq = kh._round_half_away(np.asarray(bias, np.float32) / bscale).astype(np.int32)
+    return dict(source=source, per_channel=True, int4=int4, activation=ACT[act],
+                input=xq.tolist(), filter=wq.tolist(), bias=bq.tolist(),
+                input_scale=float(in_s), input_zero_point=int(in_zp),
+                filter_scales=[float(s) for s in scales], filter_zero_point=0, bias_scale=None,
+                output_scale=float(out_s), output_zero_point=int(out_zp))
+
+
+def main():
+    t = "tflite/kernels/fully_connected_test.cc"
+    fc = []
+    for case, want in (
+            (per_tensor(t + ":816-840", (-63.5, 64), (-127, 128), W10 * 3, [1, 2, 3], X2, 3),
+             [23, 24, 25, 57, 58, 59]),
+            (per_tensor(t + ":1319-1347", (-63.5, 64), (-127, 128), W10 * 3, None, X2, 3, "relu"),
+             [22, 22, 22, 56, 56, 56]),
+            (per_tensor(t + ":1463-1487", (-63.5, 64), (-127, 128), W10 * 4, [1, 2, 3, 4], X2[10:], 4),
+             [57, 58, 59, 60]),
+            (per_tensor(t + ":1530-1562", (-127, 128), (-63.5, 64), W10 * 3, [1, 2, 3], X2, 3),
+             [47, 49, 51, 115, 117, 119]),
+            (per_tensor(t + ":756-782", (-63.5, 64), (-127, 128), W4, [1, 2, 3], X2, 3, "relu", True),
+             [103, 104, 105, 97, 98, 99]),
+            (per_channel(t + ":863-888", [0.2, 0.25, 0.5], W10 * 3, [1, 2, 3], X2, 3, 10),
+             [23, 24, 25, 57, 58, 59]),
+            (per_channel(t + ":890-948", [0.2, 0.25, 0.5], [1, 2, 3, 4, 5] * 3, [1, 2, 3],
+                         [1, 2, 3, 4, -5, 1, 2, 3, -4, 5, 1, 2, -3, 4, 5, 1, -2, 3, 4, 5], 3, 5, "relu"),
+             [5, 6, 7, 23, 24, 25, 37, 38, 39, 47, 48, 49]),
+            (per_channel(t + ":950-976", [1.0, 1.0, 1.0], W4, [1, 2, 3], X2, 3, 10, "relu", True),
+             [103, 104, 105, 97, 98, 99])):
+        case["expected_output"] = want
+        fc.append(case)
+
+    u = "tflite/kernels/internal/tensor_utils_test.cc"
+    a = [-640, -635.0, -630, 10.0, 2.0, -5.0, -10.0, 0.0, 1000.0]
+    small = [-1e-5, 3e-5, -7e-6, -9e-5, 1e-6, 4e-5, 9e-6, 2e-4, 0]
+    quantize = [
+        dict(source=u + ":220-236", asymmetric=False, values=a,
+             expected=[-81, -81, -80, 1, 0, -1, -1, 0, 127]),
+        dict(source=u + ":238-251", asymmetric=False, values=[0.0] * 9, expected=[0] * 9,
+             expected_scale=1.0),
+        dict(source=u + ":253-268", asymmetric=False, values=small,
+             expected=[-6, 19, -4, -57, 1, 25, 6, 127, 0]),
+        dict(source=u + ":270-290", asymmetric=True, values=a,
+             expected=[-128, -127, -126, -26, -28, -29, -30, -28, 127], expected_zero_point=-28),
+        dict(source=u + ":292-303", asymmetric=True, values=[0.0] * 9, expected=[0] * 9,
+             expected_scale=1.0, expected_zero_point=0),
+        dict(source=u + ":305-324", asymmetric=True, values=[2000.0] * 9, expected=[127] * 9,
+             expected_zero_point=-128),
+        dict(source=u + ":326-345", asymmetric=True, values=small,
+             expected=[-58, -23, -55, -128, -48, -14, -41, 127, -49], expected_zero_point=-49),
+    ]
+
+    q = "tflite/kernels/internal/quantization_util_test.cc"
+    multiplier = [dict(source=q + ":358-423", real=m, quantized=qm, shift=s) for m, qm, s in (
+        (0.25, 1073741824, -1), (0.50 - 5e-9, 2147483627, -1), (0.50 - 1e-10, 1073741824, 0),
+        (0.50, 1073741824, 0), (0.75, 1610612736, 0), (1 - 1e-9, 2147483646, 0),
+        (1 + 1e-11, 1073741824, 1), (1.25, 1342177280, 1), (1.50, 1610612736, 1),
+        (1.75, 1879048192, 1), (2 - 1e-9, 2147483647, 1), (2 - 1e-11, 1073741824, 2),
+        (2.0, 1073741824, 2), (2.0 ** -31, 1073741824, -30), (2.0 ** -32, 1073741824, -31),
+        (2.0 ** -33, 0, 0), (0.0, 0, 0))]
+    mbqm = [dict(source=q + ":447-485", x=x, real_multiplier=m, expected=e) for x, m, e in (
+        (0, 0.1, 0), (1, 0, 0), (10000, 0.00097656, 10), (-10000, 0.00097656, -10),
+        (-2 ** 31, 0.00001, -21475), (2 ** 31 - 1, 0.00001, 21475),
+        (10000, -0.00097656, -10), (-10000, -0.00097656, 10),
+        (-2 ** 31, -0.00001, 21475), (2 ** 31 - 1, -0.00001, -21475))]
+
+    # Hybrid dot goldens with per-channel scales and input offsets (u:1214-1231); the tensors
+    # are the test's generated data (u:1064-1150) for the 4 x 16 x 1 and 4 x 32 x 2 cases.
+    def mv(rows, cols, batch):
+        i = np.arange(rows * cols)
+        matrix = (i % 70).astype(np.int8).reshape(rows, cols)
+        j = np.arange(cols * batch)
+        vectors = (j % 50).astype(np.int32).reshape(batch, cols) + np.arange(batch)[:, None]
+        return dict(matrix=matrix.tolist(), vectors=vectors.astype(np.int8).tolist(),
+                    scaling_factors=[float(v) for v in np.arange(1, 9, dtype=np.float32)[:batch]],
+                    per_channel_scales=[0.5 if r % 2 == 0 else 1.0 for r in range(rows)],
+                    input_offsets=list(range(batch)))
+    hybrid_dot = []
+    for (rows, cols, batch), want in (((4, 16, 1), [620, 3160, 2540, 7000]),
+                                      ((4, 32, 2), [5208, 26288, 4245, 23312, 9138, 70756, 18708, 60916])):
+        case = mv(rows, cols, batch)
+        case.update(source=u + ":1214-1231", expected=want)
+        hybrid_dot.append(case)
+
+    out = dict(fully_connected_int8=fc, batch_quantize_floats=quantize,
+               quantize_multiplier=multiplier, multiply_by_quantized_multiplier=mbqm,
+               hybrid_dot_per_channel=hybrid_dot,
+               unpack_int4=[dict(source=u + ":2110-2119", packed=[0x38, 0xBE], count=4,
+                                 expected=[-8, 3, -2, -5]),
+                            dict(source=u + ":2121-2130", packed=[0x21, 0x43], count=3,
+                                 expected=[1, 2, 3])])
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_kats.json")
+    with open(path, "w") as f:
+        json.dump(out, f, indent=1)
+    print("wrote", path)
+
+
+if __name__ == "__main__":
+    main()
