@@ -84,6 +84,8 @@ def lib():
         L.orc_fc_hybrid_cached.argtypes = L.orc_fc_hybrid.argtypes + [_i32p, C.c_int]
         L.orc_fc_blockwise_int4.argtypes = [_f32p, C.c_int, C.c_int, _u8p, C.c_int, _u16p,
                                             C.c_int, _f32p, C.c_int, _f32p]
+        L.orc_fc_hybrid_int4_per_channel.argtypes = [_f32p, C.c_int, C.c_int, _u8p, C.c_int, _f32p,
+                                                     _f32p, C.c_int, _f32p]
         _LIB = L
     return _LIB
 
@@ -100,6 +102,9 @@ def ref_lib():
         R.ref_unpack_int4.argtypes = [_i8p, C.c_int, _i8p]
         for name in ("ref_apply_relu", "ref_apply_relu1", "ref_apply_relu6"):
             getattr(R, name).argtypes = [_f32p, C.c_int, _f32p]
+        if hasattr(R, "ref_fc_hybrid_int4"):
+            R.ref_fc_hybrid_int4.argtypes = [_f32p, C.c_int, C.c_int, _i8p, C.c_int, _f32p, _f32p,
+                                             _f32p]
         _REF = R
     return _REF
 
@@ -298,4 +303,24 @@ def fc_blockwise_int4(x, packed_w, out_depth, scales_f16_bits, blocksize, bias=N
     y = np.empty((B, out_depth), dtype=np.float32)
     lib().orc_fc_blockwise_int4(_p(x, _f32p), B, K, _p(pw, _u8p), out_depth, _p(sc, _u16p),
                                 blocksize, _p(bias, _f32p), variant, _p(y, _f32p))
+    return y
+
+
+# ---- per-channel int4 hybrid --------------------------------------------------
+
+def fc_hybrid_int4_per_channel(x, packed_w, out_depth, filter_scales, bias=None,
+                               activation=ACT_NONE):
+    """EvalHybridDense4Bit: x [B,K] float32, packed_w [N, K/2] nibbles (low = even k),
+    filter_scales [N] (or one value, broadcast as the op does)."""
+    x = _c(x, np.float32)
+    B, K = x.shape
+    pw = _c(packed_w, np.uint8).ravel()
+    fs = np.ascontiguousarray(np.broadcast_to(np.asarray(filter_scales, np.float32).ravel(),
+                                              (out_depth,)) if np.size(filter_scales) == 1
+                              else np.asarray(filter_scales, np.float32))
+    bias = _c(bias, np.float32)
+    y = np.empty((B, out_depth), dtype=np.float32)
+    lib().orc_fc_hybrid_int4_per_channel(_p(x, _f32p), B, K, _p(pw, _u8p), out_depth,
+                                         _p(fs, _f32p), _p(bias, _f32p), activation,
+                                         _p(y, _f32p))
     return y

@@ -611,4 +611,55 @@ void orc_fc_blockwise_int4(const float* input, int batches, int depth,
   }
 }
 
+// Per-channel int4 hybrid FULLY_CONNECTED: EvalHybridDense4Bit, tflite/kernels/fully_connected.cc
+// :1088-1178, in the arithmetic of its reference kernels
+// (tflite/kernels/internal/optimized/4bit/fully_connected_reference.cc):
+//   ReferenceBatchQuantizeFloats4Bit :121-180  symmetric per-row quantization, scale 127 / max|x|
+//     computed in double and stored as float, q = (int8)round(x * scale), and
+//     input_offset = sum(q) * zero_point_4bit (-7, fully_connected_common.h:27);
+//   ReferenceAssignBiasAndComputeOffsets :182-206  out = (offset * sf) * fs + bias;
+//   ReferenceRunKernel :290-329 with ReferenceUnpack :215-272
+//     out += (float(sum((w + 7) * q)) * sf) * fs, the weights being stored as w + 7;
+//   then ApplyActivationToVector. The tile layouts of the reference (4 x 32 boxes) only
+//   permute exact integer sums and are not restated. Weights are expected in [-7, 7], as the
+//   reference's prepacking assumes (merge(), fully_connected_common.h:36-42).
+void orc_fc_hybrid_int4_per_channel(const float* input, int batches, int depth,
+                                    const uint8_t* packed_filter, int out_depth,
+                                    const float* filter_scales, const float* bias,
+                                    int activation, float* output) {
+  const size_t k2 = (static_cast<size_t>(depth) + 1) & ~static_cast<size_t>(1);
+  std::vector<int8_t> q(depth);
+  for (int m = 0; m < batches; ++m) {
+    const float* x = input + static_cast<size_t>(m) * depth;
+    float scale_denom = 0;
+    for (int c = 0; c < depth; ++c) scale_denom = std::max(scale_denom, std::abs(x[c]));
+    if (scale_denom == 0) scale_denom = 127.0;
+    const float scale = 127.0 / scale_denom;           // double division, float store
+    const float batch_scale = scale_denom / 127.0;     // likewise
+    int32_t offset = 0;
+    for (int d = 0; d < depth; ++d) {
+      const float prod = x[d] * scale;
+      q[d] = static_cast<int8_t>(std::round(prod));
+      offset += q[d];
+    }
+    offset = offset * -7;
+    const float val = offset * batch_scale;
+    for (int n = 0; n < out_depth; ++n) {
+      int32_t acc = 0;
+      for (int k = 0; k < depth; ++k) {
+        const uint8_t byte = packed_filter[(static_cast<size_t>(n) * k2 + k) / 2];
+        const int nibble = (k % 2 == 0) ? (byte & 0xF) : (byte >> 4);
+        const int32_t w = (nibble ^ 0x8) - 8;
+        acc += (w + 7) * static_cast<int32_t>(q[k]);
+      }
+      float out = val * filter_scales[n];
+      if (bias) out = out + bias[n];
+      const float term = acc * batch_scale;
+      out = out + term * filter_scales[n];
+      output[static_cast<size_t>(m) * out_depth + n] = out;
+    }
+  }
+  orc_apply_activation(output, static_cast<int64_t>(batches) * out_depth, activation);
+}
+
 }  // extern "C"

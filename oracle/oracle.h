@@ -186,6 +186,12 @@ void orc_fc_blockwise_int4(const float* input, int batches, int depth,
                            const uint16_t* scales_f16, int blocksize, const float* bias,
                            int quant_variant, float* output);
 
+/* EvalHybridDense4Bit (per-channel int4 weights, symmetric activations); see oracle.cc. */
+void orc_fc_hybrid_int4_per_channel(const float* input, int batches, int depth,
+                                    const uint8_t* packed_filter, int out_depth,
+                                    const float* filter_scales, const float* bias,
+                                    int activation, float* output);
+
 #ifdef __cplusplus
 }
 #endif
