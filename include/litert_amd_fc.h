@@ -256,6 +256,28 @@ int lrtfc_fc_blockwise_int4_packed_quantized(const int8_t* quantized_input,
                                              const float* bias, float* output, int batches,
                                              int depth, int out_depth, void* stream);
 
+/* ---- Per-channel int4 hybrid FULLY_CONNECTED ------------------------------------------
+ * Replaces EvalHybridDense4Bit (tflite/kernels/fully_connected.cc:1088-1178) in the
+ * arithmetic of its reference kernels
+ * (tflite/kernels/internal/optimized/4bit/fully_connected_reference.cc): symmetric per-row
+ * quantization with scale max|x| / 127 (ReferenceBatchQuantizeFloats4Bit :121-180), input
+ * offsets -7 * sum(q), out = (offset * sf) * fs + bias, then += (float(sum((w + 7) q)) * sf)
+ * * fs (:182-272), then the fused activation. Weights are expected in [-7, 7] as the
+ * reference's prepacking assumes.
+ *   The filter is handed over as int8: unpack the model's nibbles with lrtfc_unpack_int4 and
+ *   re-tile with lrtfc_pack_int8_filter (the reference prepacks its own layout once,
+ *   fully_connected.cc:1109-1120). per_channel_scales NULL: filter_scale for every channel.
+ *   workspace: lrtfc_activation_workspace_bytes(batches, depth), 256-byte aligned. */
+int lrtfc_batch_quantize_floats_4bit(const float* values, int n_batch, int n_data,
+                                     int8_t* quantized, float* scaling_factors,
+                                     int32_t* input_offsets, void* stream);
+int lrtfc_fc_hybrid_int4_per_channel_packed(const float* input, const int8_t* packed_filter,
+                                            const float* per_channel_scales, float filter_scale,
+                                            const float* bias, float* output, int batches,
+                                            int depth, int out_depth, int activation,
+                                            void* workspace, size_t workspace_bytes,
+                                            void* stream);
+
 /* ---- Several blockwise-int4 nodes in one launch ----------------------------------------
  * Nodes of a graph that do not depend on each other (the q/k/v or the gate/up projections of
  * a decoder layer) and share depth and batch count can run as ONE kernel: the gaps between

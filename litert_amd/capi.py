@@ -55,6 +55,9 @@ SYMBOLS = [
     ("lrtfc_fc_blockwise_int4_packed", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     ("lrtfc_fc_blockwise_int4_packed_quantized", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i,
                                                       _i, _vp]),
+    ("lrtfc_batch_quantize_floats_4bit", _i, [_vp, _i, _i, _vp, _vp, _vp, _vp]),
+    ("lrtfc_fc_hybrid_int4_per_channel_packed", _i, [_vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i,
+                                                     _vp, _sz, _vp]),
     ("lrtfc_int4_group_table_bytes", _sz, []),
     ("lrtfc_int4_group_prepare", _i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_fc_blockwise_int4_packed_grouped", _i, [_vp, _vp, _i, _vp]),

@@ -623,6 +623,64 @@ int lrtfc_fc_blockwise_int4_packed_quantized(const int8_t* quantized_input,
                             kfsum, bias, output, batches, depth, out_depth, 0, stream);
 }
 
+int lrtfc_batch_quantize_floats_4bit(const float* values, int n_batch, int n_data,
+                                     int8_t* quantized, float* scaling_factors,
+                                     int32_t* input_offsets, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(n_batch >= 0 && n_data >= 0, "negative dimension");
+  if (n_batch == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(values && quantized && scaling_factors && input_offsets, "null pointer");
+  LRTFC_REQUIRE(n_data > 0, "empty rows cannot be quantized");
+  return FromHip(lrtfc::LaunchBatchQuantize4Bit(values, n_batch, n_data, quantized,
+                                                scaling_factors, input_offsets, AsStream(stream)),
+                 "4-bit path row quantizer");
+}
+
+int lrtfc_fc_hybrid_int4_per_channel_packed(const float* input, const int8_t* packed_filter,
+                                            const float* per_channel_scales, float filter_scale,
+                                            const float* bias, float* output, int batches,
+                                            int depth, int out_depth, int activation,
+                                            void* workspace, size_t workspace_bytes,
+                                            void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(input && packed_filter && output && workspace, "null pointer");
+  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  LRTFC_REQUIRE(workspace_bytes >= WorkspaceBytes(batches, depth),
+                "workspace too small: %zu < %zu bytes", workspace_bytes,
+                WorkspaceBytes(batches, depth));
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
+                "workspace must be 256-byte aligned");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(packed_filter) & 15) == 0,
+                "packed filter must be 16-byte aligned");
+  const Workspace w = SplitWorkspace(workspace, batches, depth);
+  int rc = lrtfc_batch_quantize_floats_4bit(input, batches, depth, w.q, w.sf, w.zp, stream);
+  if (rc != LRTFC_OK) return rc;
+  lrtfc::FcInt8Args a{};
+  a.input = w.q;
+  a.filter = packed_filter;
+  a.batches = batches;
+  a.depth = depth;
+  a.out_depth = out_depth;
+  a.scaling_factors = w.sf;
+  a.zero_points = w.zp;  // the rows' input offsets on this path
+  a.per_channel_scales = per_channel_scales;
+  a.filter_scale = filter_scale;
+  a.bias_f32 = bias;
+  a.activation = activation;
+  a.output_f32 = output;
+  if (batches > kPackedGemmMinBatches && lrtfc::FcInt8PackedGemmSupports(a)) {
+    return FromHip(lrtfc::LaunchFcInt8PackedGemm(a, lrtfc::Int8Epilogue::kHybrid4Bit,
+                                                 AsStream(stream)),
+                   "packed int4 per-channel hybrid GEMM");
+  }
+  return FromHip(lrtfc::LaunchFcInt8PackedGemv(a, lrtfc::Int8Epilogue::kHybrid4Bit, nullptr, 0,
+                                               LRTFC_QUANT_PORTABLE, AsStream(stream)),
+                 "packed int4 per-channel hybrid GEMV");
+}
+
 size_t lrtfc_int4_group_table_bytes(void) { return lrtfc::Int4GroupTableBytes(); }
 
 int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,

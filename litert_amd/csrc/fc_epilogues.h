@@ -28,6 +28,21 @@ __device__ __forceinline__ float HybridCore(int32_t dot, float batch_scale, floa
   return ApplyFloatActivation(out, activation);
 }
 
+// Output value of the per-channel int4 hybrid path: ReferenceAssignBiasAndComputeOffsets and
+// ReferenceUnpack (tflite/kernels/internal/optimized/4bit/fully_connected_reference.cc:182-272)
+// followed by ApplyActivationToVector. `dot` is sum(w * q) over the depth with the signed
+// weights; the reference accumulates sum((w + 7) * q) = dot + 7 * sum(q) = dot - input_offset.
+__device__ __forceinline__ float Hybrid4BitCore(int32_t dot, float batch_scale,
+                                                float channel_scale, int32_t input_offset,
+                                                float bias, bool has_bias, int activation) {
+  const float val = __fmul_rn(static_cast<float>(input_offset), batch_scale);
+  float out = __fmul_rn(val, channel_scale);
+  if (has_bias) out = __fadd_rn(out, bias);
+  const float term = __fmul_rn(static_cast<float>(dot - input_offset), batch_scale);
+  out = __fadd_rn(out, __fmul_rn(term, channel_scale));
+  return ApplyFloatActivation(out, activation);
+}
+
 // Pointer forms used by the row-major kernels.
 __device__ __forceinline__ void StoreRequantized(const FcInt8Args& a, int b, int n, int32_t dot,
                                                  int32_t xsum) {

@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
     } else {
       p[0] = __float_as_int(a.per_channel_scales ? a.per_channel_scales[n] : a.filter_scale);
       p[1] = __float_as_int(a.bias_f32 ? a.bias_f32[n] : 0.0f);
-      p[2] = a.zero_points ? a.filter_row_sums[n] : 0;
+      p[2] = (EPI == Int8Epilogue::kHybrid && a.zero_points) ? a.filter_row_sums[n] : 0;
     }
     chan_p = p;
   }
@@ -299,8 +299,11 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
           float v[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            v[r] = HybridCore(acc[i][j][4 * g + r], bscale, cscale[r], bzp, rsum[r], base[r],
-                              a.activation);
+            v[r] = EPI == Int8Epilogue::kHybrid4Bit
+                       ? Hybrid4BitCore(acc[i][j][4 * g + r], bscale, cscale[r], bzp, base[r],
+                                        a.bias_f32 != nullptr, a.activation)
+                       : HybridCore(acc[i][j][4 * g + r], bscale, cscale[r], bzp, rsum[r],
+                                    base[r], a.activation);
           }
           if (kFull || m < M) {
             float* dst = a.output_f32 + static_cast<size_t>(m) * N + c0;
@@ -339,9 +342,12 @@ hipError_t LaunchFcInt8PackedGemm(const FcInt8Args& a, Int8Epilogue epilogue, hi
   if (epilogue == Int8Epilogue::kRequantize) {
     hipLaunchKernelGGL(FcInt8PackedGemmKernel<Int8Epilogue::kRequantize>, dim3(grid),
                        dim3(kThreads), 0, stream, a);
-  } else {
+  } else if (epilogue == Int8Epilogue::kHybrid) {
     hipLaunchKernelGGL(FcInt8PackedGemmKernel<Int8Epilogue::kHybrid>, dim3(grid), dim3(kThreads),
                        0, stream, a);
+  } else {
+    hipLaunchKernelGGL(FcInt8PackedGemmKernel<Int8Epilogue::kHybrid4Bit>, dim3(grid),
+                       dim3(kThreads), 0, stream, a);
   }
   return hipGetLastError();
 }

@@ -419,8 +419,12 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
     } else {
       const float batch_scale = FUSED ? sh.sf[col] : a.scaling_factors[b];
       const int32_t batch_zp = FUSED ? sh.zp[col] : (a.zero_points ? a.zero_points[b] : 0);
-      a.output_f32[static_cast<size_t>(b) * a.out_depth + n] = HybridCore(
-          acc[i], batch_scale, ep_f0[i], batch_zp, ep_i0[i], ep_f1[i], a.activation);
+      a.output_f32[static_cast<size_t>(b) * a.out_depth + n] =
+          EPI == Int8Epilogue::kHybrid4Bit
+              ? Hybrid4BitCore(acc[i], batch_scale, ep_f0[i], batch_zp, ep_f1[i],
+                               a.bias_f32 != nullptr, a.activation)
+              : HybridCore(acc[i], batch_scale, ep_f0[i], batch_zp, ep_i0[i], ep_f1[i],
+                           a.activation);
     }
   }
 }
@@ -517,6 +521,8 @@ hipError_t LaunchFcInt8PackedGemv(const FcInt8Args& a, Int8Epilogue epilogue,
     hipError_t err;
     if (epilogue == Int8Epilogue::kRequantize) {
       err = LaunchVariant<Int8Epilogue::kRequantize, false>(p, variant, batch0, bt, stream);
+    } else if (epilogue == Int8Epilogue::kHybrid4Bit) {
+      err = LaunchVariant<Int8Epilogue::kHybrid4Bit, false>(p, variant, batch0, bt, stream);
     } else if (input_f32) {
       err = LaunchVariant<Int8Epilogue::kHybrid, true>(p, variant, batch0, bt, stream);
     } else {

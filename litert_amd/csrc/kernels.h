@@ -34,12 +34,17 @@ struct FcInt8Args {
   float* output_f32;
 };
 
-enum class Int8Epilogue { kRequantize, kHybrid };
+// kHybrid4Bit: the float epilogue of the per-channel int4 hybrid path; a.zero_points then
+// holds the rows' input offsets (-7 * sum(q)) and a.filter_row_sums is unused.
+enum class Int8Epilogue { kRequantize, kHybrid, kHybrid4Bit };
 
 hipError_t LaunchBatchQuantize(const float* values, int n_batch, int n_data, int8_t* quantized,
                                float* scaling_factors, int32_t* zero_points, int do_asymmetric,
                                int variant, hipStream_t stream);
 
+hipError_t LaunchBatchQuantize4Bit(const float* values, int n_batch, int n_data, int8_t* quantized,
+                                   float* scaling_factors, int32_t* input_offsets,
+                                   hipStream_t stream);
 hipError_t LaunchZeroFill(void* dst, size_t bytes, hipStream_t stream);
 hipError_t LaunchRowSumsInt8(const int8_t* filter, int out_depth, int depth, int32_t* row_sums,
                              hipStream_t stream);

@@ -116,7 +116,55 @@ __global__ __launch_bounds__(kThreads) void BatchQuantizeKernel(
   }
 }
 
+// The row quantizer of the per-channel int4 hybrid path (ReferenceBatchQuantizeFloats4Bit,
+// tflite/kernels/internal/optimized/4bit/fully_connected_reference.cc:121-180): symmetric,
+// scale_denom = max|x| (127 for an all-zero row), multiplier 127.0 / scale_denom and stored
+// scale scale_denom / 127.0 both divided in double and rounded to float, q = (int8)round(x *
+// multiplier) without a clamp, and input_offsets = sum(q) * zero_point_4bit (-7).
+__global__ __launch_bounds__(kThreads) void BatchQuantize4BitKernel(
+    const float* __restrict__ values, int n_data, int8_t* __restrict__ quantized,
+    float* __restrict__ scaling_factors, int32_t* __restrict__ input_offsets) {
+  __shared__ int32_t s_sum[kThreads / kWaveSize];
+  const int row = blockIdx.x;
+  const float* v = values + static_cast<size_t>(row) * n_data;
+  int8_t* q = quantized + static_cast<size_t>(row) * n_data;
+  float mn = 0.0f, mx = 0.0f;
+  for (int i = threadIdx.x; i < n_data; i += kThreads) {
+    mn = fminf(mn, v[i]);
+    mx = fmaxf(mx, v[i]);
+  }
+  const RowRange range = BlockMinMax(mn, mx);
+  float scale_denom = fmaxf(fabsf(range.mn), fabsf(range.mx));
+  if (scale_denom == 0.0f) scale_denom = 127.0f;
+  const float multiplier = static_cast<float>(127.0 / static_cast<double>(scale_denom));
+  int32_t sum = 0;
+  for (int i = threadIdx.x; i < n_data; i += kThreads) {
+    const int32_t o = static_cast<int8_t>(RoundHalfAway(__fmul_rn(v[i], multiplier)));
+    q[i] = static_cast<int8_t>(o);
+    sum += o;
+  }
+  sum = WaveSumI32(sum);
+  if ((threadIdx.x & (kWaveSize - 1)) == 0) s_sum[threadIdx.x / kWaveSize] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t total = 0;
+#pragma unroll
+    for (int w = 0; w < kThreads / kWaveSize; ++w) total += s_sum[w];
+    scaling_factors[row] = static_cast<float>(static_cast<double>(scale_denom) / 127.0);
+    input_offsets[row] = total * -7;
+  }
+}
+
 }  // namespace
+
+hipError_t LaunchBatchQuantize4Bit(const float* values, int n_batch, int n_data, int8_t* quantized,
+                                   float* scaling_factors, int32_t* input_offsets,
+                                   hipStream_t stream) {
+  if (n_batch == 0 || n_data == 0) return hipSuccess;
+  hipLaunchKernelGGL(BatchQuantize4BitKernel, dim3(n_batch), dim3(kThreads), 0, stream, values,
+                     n_data, quantized, scaling_factors, input_offsets);
+  return hipGetLastError();
+}
 
 hipError_t LaunchBatchQuantize(const float* values, int n_batch, int n_data, int8_t* quantized,
                                float* scaling_factors, int32_t* zero_points, int do_asymmetric,

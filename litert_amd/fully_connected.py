@@ -347,6 +347,46 @@ class FullyConnectedBlockwiseInt4:
         return out
 
 
+class FullyConnectedHybridInt4PerChannel:
+    """Per-channel int4 hybrid FC: EvalHybridDense4Bit, fully_connected.cc:1088-1178.
+
+    packed_filter: uint8 [N, K/2] as the model stores it (low nibble = even k); filter_scales:
+    [N], or one value for every channel; bias float32 [N] or None."""
+
+    def __init__(self, packed_filter, depth, filter_scales, bias=None, activation="none"):
+        _ensure_init()
+        lib = capi.load()
+        nibbles = _dev(packed_filter, torch.uint8)
+        self.out_depth = nibbles.shape[0]
+        self.depth = int(depth)
+        if self.depth % 2:
+            raise ValueError("the 4-bit path needs an even depth")
+        unpacked = torch.empty((self.out_depth, self.depth), dtype=torch.int8, device="cuda")
+        capi.check(lib.lrtfc_unpack_int4(_ptr(nibbles), self.out_depth * self.depth,
+                                         _ptr(unpacked), _stream()))
+        self.packed_filter = _pack_int8(unpacked)
+        fs = np.atleast_1d(np.asarray(filter_scales, dtype=np.float32))
+        self.pcs = _dev(fs, torch.float32) if fs.size > 1 else None
+        self.filter_scale = float(fs[0])
+        self.bias = _dev(bias, torch.float32)
+        self.activation = _act(activation)
+        self._ws = None
+
+    def __call__(self, x, out=None):
+        x = x.contiguous()
+        batches = x.numel() // self.depth
+        if out is None:
+            out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
+        need = capi.load().lrtfc_activation_workspace_bytes(batches, self.depth)
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        capi.check(capi.load().lrtfc_fc_hybrid_int4_per_channel_packed(
+            _ptr(x), _ptr(self.packed_filter), _ptr(self.pcs), self.filter_scale, _ptr(self.bias),
+            _ptr(out), batches, self.depth, self.out_depth, self.activation, _ptr(self._ws),
+            self._ws.numel(), _stream()))
+        return out
+
+
 class GroupedBlockwiseInt4:
     """Several FullyConnectedBlockwiseInt4 nodes of one depth that do not depend on each other
     (q/k/v, gate/up), run as ONE kernel. `bind` fixes the input and output tensors of every

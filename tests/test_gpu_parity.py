@@ -485,3 +485,47 @@ def test_empty_and_zero_depth(fc):
     rc = lib.lrtfc_fc_int8(p(out), p(out), None, p(one), p(one), 0, None, p(out), 2, 16, 3, 5, 0, 0,
                            -128, 127, None)
     assert rc == capi.INVALID_ARGUMENT and b"filter_row_sums" in lib.lrtfc_last_error()
+
+
+# ---- per-channel int4 hybrid (EvalHybridDense4Bit) ----------------------------------------
+
+@pytest.mark.parametrize("B,K,N", [(1, 32, 4), (4, 40, 5), (3, 46, 7), (2, 256, 17), (1, 4096, 512),
+                                   (8, 2048, 130), (16, 1000, 33), (40, 512, 72), (130, 272, 48)])
+@pytest.mark.parametrize("activation", ["none", "relu", "relu6"])
+def test_hybrid_int4_per_channel_matches_oracle(fc, B, K, N, activation):
+    """Bit-identical floats against the oracle (itself bit-identical to the reference's 4-bit
+    kernels): decode batches on the GEMV, more than 32 rows on the GEMM, ragged shapes, an
+    all-zero row, per-channel scales with and without bias."""
+    from tests import kat_harness as kh
+    rng = np.random.default_rng(700 + B + K + N)
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    if B > 2:
+        x[1] = 0
+    w = rng.integers(-7, 8, (N, K)).astype(np.int8)
+    packed = np.stack([kh.pack_int4(r) for r in w])
+    fs = rng.uniform(0.01, 0.1, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32) if N % 2 else None
+    op = fc.FullyConnectedHybridInt4PerChannel(packed, K, fs, bias, activation)
+    y = op(_cuda(x)).cpu().numpy()
+    want = oracle.fc_hybrid_int4_per_channel(x, packed, N, fs, bias, fc._act(activation))
+    assert _bits_equal(y, want)
+
+
+def test_hybrid_int4_per_channel_reference_kat_and_scalar_scale(fc):
+    """tflite/kernels/fully_connected_4bit_test.cc:102-190 through the HIP path (the test's own
+    tolerance), with the single filter scale the test model uses."""
+    from tests import kat_harness as kh
+    a = [-1, 2, 3, 4, 5, 6, 7, 1, 2, 3] * 2
+    b = [1, 2, 3, 4, 5, 6, 7, 1, 2, -3] + [-1, 2, 3, 4, 5, 6, 7, 1, 2, 3]
+    w = np.array([a + a, b + a, b + a, b + a, a + a], np.int8)
+    xa = [1, 2, 3, 4, 5, 6, 7, 8, -9, -10] * 4
+    xb = [1, 2, 3, 4, 5, 6, 7, -8, 9, -10] + [1, 2, 3, 4, 5, 6, 7, 8, -9, -10] * 3
+    x = np.array([xa, xb, xa, [0] * 40], np.float32)
+    packed = np.stack([kh.pack_int4(r) for r in w])
+    op = fc.FullyConnectedHybridInt4PerChannel(packed, 40, [1.0], np.array([1, 2, 3, 1, 2], np.float32),
+                                               "relu")
+    y = op(_cuda(x)).cpu().numpy()
+    want = np.array([[393., 456., 457., 455., 394.], [413., 476., 477., 475., 414.],
+                     [393., 456., 457., 455., 394.]])
+    assert np.abs(y[:3] - want).max() <= 1.3
+    assert y[3].tolist() == [1, 2, 3, 1, 2]
