@@ -39,6 +39,7 @@ struct Options {
   bool claim_int8 = true;
   bool claim_hybrid = true;
   bool claim_int4_blockwise = true;
+  bool claim_int4_per_channel = true;
 };
 
 struct DelegateState {
@@ -46,7 +47,7 @@ struct DelegateState {
   TfLiteDelegate delegate;
 };
 
-enum class FcKind { kNone, kInt8, kHybrid, kInt4Blockwise };
+enum class FcKind { kNone, kInt8, kHybrid, kInt4Blockwise, kHybridInt4 };
 
 int64_t NumElements(const TfLiteIntArray* dims) {
   int64_t n = 1;
@@ -162,6 +163,20 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
         return no("scale count != channels x blocks");
       }
       return FcKind::kInt4Blockwise;
+    }
+    if (filter.type == kTfLiteInt4 && filter.quantization.type == kTfLiteAffineQuantization) {
+      // The builtin's optimized 4-bit path (EvalHybridDense4Bit); outside its gate
+      // (fully_connected.cc:609-613) the builtin unpacks to int8 and runs the ordinary hybrid
+      // kernels, which quantize differently: those shapes stay on the CPU.
+      if (!opt.claim_int4_per_channel) return no("int4 per-channel path disabled by option");
+      if (!ClippingActivation(params->activation)) return no("activation not a clamp");
+      if (depth % 2 != 0 || out_depth < 4 || depth < 32) return no("shape outside 4-bit gate");
+      const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
+      if (!fq || !fq->scale || fq->scale->size < 1) return no("filter has no scales");
+      if (fq->scale->size > 1 && fq->scale->size != out_depth) {
+        return no("per-channel scales do not match output channels");
+      }
+      return FcKind::kHybridInt4;
     }
     return no("float activations with this filter type are left to the CPU kernels");
   }
@@ -535,6 +550,26 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
       RETURN_IF_HIP(ctx, n->pcs_dev.Upload(fq->scale->data, static_cast<size_t>(n->out_depth) * 4, s));
     }
     if (bias) RETURN_IF_HIP(ctx, n->bias_dev.Upload(bias->data.raw, static_cast<size_t>(n->out_depth) * 4, s));
+  } else if (n->kind == FcKind::kHybridInt4) {
+    // EvalHybridDense4Bit: the filter scales (one, or one per channel) follow
+    // fully_connected.cc:1146-1158; the nibbles are unpacked and re-tiled once.
+    const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
+    n->per_channel = fq->scale->size > 1;
+    n->filter_scale = fq->scale->data[0];
+    n->use_retiled = true;
+    if (weights > 0 && !n->have_retiled) {
+      DeviceBuffer nibbles;
+      RETURN_IF_HIP(ctx, nibbles.Upload(filter.data.raw, (weights + 1) / 2, s));
+      RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
+      RETURN_IF_FC(ctx, lrtfc_unpack_int4(nibbles.as<uint8_t>(), static_cast<int64_t>(weights),
+                                          n->filter_dev.as<int8_t>(), s));
+      RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+      RETURN_IF_OK(RetileInt8(ctx, n, s));
+    }
+    if (n->per_channel) {
+      RETURN_IF_HIP(ctx, n->pcs_dev.Upload(fq->scale->data, static_cast<size_t>(n->out_depth) * 4, s));
+    }
+    if (bias) RETURN_IF_HIP(ctx, n->bias_dev.Upload(bias->data.raw, static_cast<size_t>(n->out_depth) * 4, s));
   } else {  // blockwise int4
     const auto* bq = static_cast<const TfLiteBlockwiseQuantization*>(filter.quantization.params);
     n->blocksize = bq->blocksize;
@@ -664,7 +699,8 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
   }
   // Scratch for the nodes that quantize in a launch of their own, per stream.
   for (const FcNode& n : k->nodes) {
-    if (n.kind != FcKind::kInt8 && (!n.use_retiled || n.split_quantize)) {
+    if (n.kind == FcKind::kHybridInt4 ||
+        (n.kind != FcKind::kInt8 && (!n.use_retiled || n.split_quantize))) {
       RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(
                              lrtfc_activation_workspace_bytes(n.batches, n.depth)));
     }
@@ -816,6 +852,13 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
         }
         break;
       }
+      case FcKind::kHybridInt4:
+        RETURN_IF_FC(ctx, lrtfc_fc_hybrid_int4_per_channel_packed(
+                              static_cast<const float*>(in_dev), n.retiled_dev.as<int8_t>(),
+                              n.per_channel ? n.pcs_dev.as<float>() : nullptr, n.filter_scale,
+                              bias_f32, static_cast<float*>(out_dev), n.batches, n.depth,
+                              n.out_depth, n.params.activation, scratch.get(), scratch.bytes(), s));
+        break;
       case FcKind::kInt4Blockwise:
         if (!n.use_retiled) {
           RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4(static_cast<const float*>(in_dev),
@@ -941,6 +984,7 @@ bool ParseOptions(const char* const* keys, const char* const* values, size_t n, 
       }
     } else if (key == "claim") {
       opt->claim_int8 = opt->claim_hybrid = opt->claim_int4_blockwise = false;
+      opt->claim_int4_per_channel = false;
       size_t pos = 0;
       while (pos <= val.size()) {
         const size_t comma = val.find(',', pos);
@@ -951,8 +995,10 @@ bool ParseOptions(const char* const* keys, const char* const* values, size_t n, 
           opt->claim_hybrid = true;
         } else if (item == "int4_blockwise") {
           opt->claim_int4_blockwise = true;
+        } else if (item == "int4_per_channel") {
+          opt->claim_int4_per_channel = true;
         } else if (!item.empty()) {
-          *error = "claim accepts int8, hybrid, int4_blockwise; got '" + item + "'";
+          *error = "claim accepts int8, hybrid, int4_blockwise, int4_per_channel; got '" + item + "'";
           return false;
         }
         if (comma == std::string::npos) break;
@@ -1002,7 +1048,7 @@ void tflite_plugin_destroy_delegate(TfLiteDelegate* delegate) {
 }
 
 // Test and tooling hook: the claim predicate on its own (no device needed). Returns
-// 0 = declined, 1 = int8, 2 = hybrid, 3 = int4 blockwise; `reason` (may be NULL)
+// 0 = declined, 1 = int8, 2 = hybrid, 3 = int4 blockwise, 4 = int4 per-channel hybrid; `reason` (may be NULL)
 // receives why a node was declined.
 int litert_amd_classify_node(const TfLiteContext* ctx, const TfLiteNode* node,
                              const TfLiteRegistration* registration, char* reason,

@@ -17,7 +17,7 @@ DELEGATE_LIB = os.path.join(ROOT, "litert_amd", "lib", "liblitert_amd_delegate.s
 FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, INT16 = 1, 2, 3, 9, 10, 18, 7
 MMAP_RO, ARENA_RW = 1, 2
 OK, ERROR, DELEGATE_ERROR = 0, 1, 2
-KIND = {0: None, 1: "int8", 2: "hybrid", 3: "int4_blockwise"}
+KIND = {0: None, 1: "int8", 2: "hybrid", 3: "int4_blockwise", 4: "int4_per_channel"}
 
 _NP = {FLOAT32: np.float32, INT32: np.int32, UINT8: np.uint8, INT8: np.int8, FLOAT16: np.float16,
        INT16: np.int16, INT4: np.uint8}

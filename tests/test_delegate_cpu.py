@@ -84,8 +84,12 @@ def test_claim_predicate_float_activations():
         assert h.classify(_float_node(h, blockwise=True, K=16, bs=16)) == (None, "shape outside 4-bit gate")
         assert h.classify(_float_node(h, blockwise=True, K=96, bs=64)) == (None, "bad blocksize")
         assert h.classify(_float_node(h, blockwise=True, scale_type=FLOAT32)) == (None, "scales not const fp16")
-        # per-channel int4 hybrid (EvalHybridDense4Bit) is a different algorithm: declined
-        assert h.classify(_float_node(h, filter_type=INT4))[0] is None
+        # per-channel int4 hybrid (EvalHybridDense4Bit): claimed inside the builtin's 4-bit gate
+        assert h.classify(_float_node(h, filter_type=INT4))[0] == "int4_per_channel"
+        assert h.classify(_float_node(h, filter_type=INT4, per_channel=False))[0] == "int4_per_channel"
+        assert h.classify(_float_node(h, filter_type=INT4, N=2)) == (None, "shape outside 4-bit gate")
+        assert h.classify(_float_node(h, filter_type=INT4, K=16)) == (None, "shape outside 4-bit gate")
+        assert h.classify(_float_node(h, filter_type=INT4, activation=4)) == (None, "activation not a clamp")
 
 
 def test_bad_options_are_rejected_before_touching_the_device():

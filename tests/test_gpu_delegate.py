@@ -237,6 +237,33 @@ def test_int4_nodes_share_grouped_launches(streams, B):
                 assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("B,per_channel", [(1, True), (4, False), (40, True)])
+def test_int4_per_channel_hybrid_node_through_delegate(B, per_channel):
+    """EvalHybridDense4Bit: float in/out, int4 filter with affine (not blockwise) quantization."""
+    from tests import kat_harness as kh
+    rng = np.random.default_rng(5 + B)
+    K, N = 256, 24
+    x_np = rng.standard_normal((B, K)).astype(np.float32)
+    w_np = rng.integers(-7, 8, (N, K)).astype(np.int8)
+    packed = np.stack([kh.pack_int4(r) for r in w_np])
+    fs = rng.uniform(0.01, 0.1, N).astype(np.float32) if per_channel else np.array([0.05], np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (B, K), data=x_np)
+        w = h.tensor(INT4, (N, K), data=packed, const=True)
+        h.affine(w, fs)
+        b = h.tensor(FLOAT32, (N,), data=bias, const=True)
+        y = h.tensor(FLOAT32, (B, N))
+        node = h.fc(x, w, b, y, activation=1)
+        assert h.classify(node)[0] == "int4_per_channel"
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.plan()[0][:2] == ("delegate", [node])
+        assert h.invoke() == OK, h.errors()
+        want = oracle.fc_hybrid_int4_per_channel(x_np, packed, N, fs, bias, oracle.ACT_RELU)
+        assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+
+
 def test_streams_option_is_validated():
     with FakeHost() as h:
         assert h.load_delegate({"streams": 9}) != 0
