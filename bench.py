@@ -159,11 +159,28 @@ def main():
         g, n = many(fns)
         return timed_replays([g], replays) * 1e3 / n
 
+    def per_launch_stats(fns, replays=25):
+        """(median, min) microseconds per launch over `replays` separately timed replays."""
+        g, n = many(fns)
+        g.replay()
+        samples = []
+        for _ in range(replays):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            samples.append(e0.elapsed_time(e1) * 1e3 / n)
+        samples.sort()
+        return samples[len(samples) // 2], samples[0]
+
     per_b = {}
     for b in BATCHES:
         cold_us = per_launch_us([(lambda o: lambda: o(xs[b], out=outs[b]))(op) for op in ops])
         hot_us = per_launch_us([lambda: ops[0](xs[b], out=outs[b])] * len(ops))
-        per_b[b] = dict(op_us_cold=round(cold_us, 3), op_us_hot=round(hot_us, 3),
+        med_us, min_us = per_launch_stats([(lambda o: lambda: o(xs[b], out=outs[b]))(op) for op in ops])
+        per_b[b] = dict(op_us_cold=round(cold_us, 3), op_us_cold_median=round(med_us, 3),
+                        op_us_cold_min=round(min_us, 3), op_us_hot=round(hot_us, 3),
                         op_gbps_cold=round(hybrid_bytes(b) / cold_us / 1e3, 1),
                         op_gbps_hot=round(hybrid_bytes(b) / hot_us / 1e3, 1),
                         frac_of_hbm_peak_cold=round(hybrid_bytes(b) / cold_us / 1e3 / HBM_PEAK_GBPS, 4))
