@@ -1,0 +1,131 @@
+"""The LiteRT accelerator skin: the exported LiteRtAcceleratorImpl object as the LiteRT runtime
+would consume it (litert/runtime/accelerators/registration_helper.cc:34-86): ABI header, the
+five mandatory callbacks, and create_delegate against a stand-in runtime context whose
+wrap_delegate records what it is handed."""
+import ctypes as C
+import os
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "litert_amd", "lib", "liblitert_amd_delegate.so")
+
+
+class AbiHeader(C.Structure):
+    _fields_ = [("struct_size", C.c_uint16), ("major_version", C.c_uint16),
+                ("minor_version", C.c_uint16), ("reserved", C.c_uint16)]
+
+
+class BufferHandlers(C.Structure):
+    _fields_ = [("abi_header", AbiHeader)] + [(n, C.c_void_p) for n in (
+        "create_func", "destroy_func", "lock_func", "unlock_func", "clear_func", "import_func")] + [
+        ("device_tag", C.c_int), ("queue_tag", C.c_int), ("num_supported_buffer_types", C.c_size_t),
+        ("supported_buffer_types", C.c_int * 16)]
+
+
+class ApiVersion(C.Structure):
+    _fields_ = [("major", C.c_int), ("minor", C.c_int), ("patch", C.c_int)]
+
+
+DELETER = C.CFUNCTYPE(None, C.c_void_p)
+WRAP = C.CFUNCTYPE(C.c_int, C.c_void_p, DELETER, C.POINTER(C.c_void_p))
+UNWRAP = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_void_p))
+
+
+class RuntimeContext(C.Structure):
+    _fields_ = [("abi_header", AbiHeader), ("before", C.c_void_p * 17), ("wrap_delegate", WRAP),
+                ("unwrap_delegate", UNWRAP)]
+
+
+class AcceleratorDef(C.Structure):
+    _fields_ = [("abi_header", AbiHeader),
+                ("get_name", C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_char_p))),
+                ("get_version", C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(ApiVersion))),
+                ("get_hardware_support", C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_int))),
+                ("is_jit", C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_bool))),
+                ("create_delegate", C.CFUNCTYPE(C.c_int, C.POINTER(RuntimeContext), C.c_void_p,
+                                                C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p))),
+                ("start_metrics_collection", C.c_void_p), ("stop_metrics_collection", C.c_void_p),
+                ("buffer_handlers", BufferHandlers)]
+
+
+def _impl():
+    lib = C.CDLL(LIB)
+    return lib, AcceleratorDef.in_dll(lib, "LiteRtAcceleratorImpl")
+
+
+def test_layout_constants_of_the_reference():
+    # litert_accelerator_def.h:74-97, litert_custom_tensor_buffer_handlers_def.h:52-68,
+    # litert_runtime_context.h:259-262
+    assert C.sizeof(AcceleratorDef) == 200 and AcceleratorDef.buffer_handlers.offset == 64
+    assert C.sizeof(BufferHandlers) == 136 and BufferHandlers.supported_buffer_types.offset == 72
+    assert RuntimeContext.wrap_delegate.offset == 144 and RuntimeContext.unwrap_delegate.offset == 152
+
+
+def test_exported_table_is_what_the_runtime_accepts():
+    _, d = _impl()
+    assert (d.abi_header.struct_size, d.abi_header.major_version) == (200, 1)
+    for f in ("get_name", "get_version", "get_hardware_support", "is_jit", "create_delegate"):
+        assert C.cast(getattr(d, f), C.c_void_p).value, f
+    assert d.buffer_handlers.num_supported_buffer_types < 16  # registration_helper.cc:48-49
+    name = C.c_char_p()
+    assert d.get_name(None, C.byref(name)) == 0 and name.value == b"litert_amd_fc_mi355x"
+    v = ApiVersion()
+    assert d.get_version(None, C.byref(v)) == 0 and (v.major, v.minor, v.patch) == (0, 1, 0)
+    hw = C.c_int()
+    assert d.get_hardware_support(None, C.byref(hw)) == 0 and hw.value == 2  # kLiteRtHwAcceleratorGpu
+    jit = C.c_bool(True)
+    assert d.is_jit(None, C.byref(jit)) == 0 and jit.value is False
+    assert d.get_name(None, None) == 1  # kLiteRtStatusErrorInvalidArgument
+
+
+def _context(record):
+    def wrap(delegate, deleter, out):
+        record["delegate"] = delegate
+        record["deleter"] = deleter
+        out[0] = 0xABC0
+        return 0
+    ctx = RuntimeContext()
+    ctx.abi_header = AbiHeader(C.sizeof(RuntimeContext), 1, 0, 0)
+    ctx.wrap_delegate = WRAP(wrap)
+    record["keepalive"] = ctx.wrap_delegate
+    return ctx
+
+
+def test_create_delegate_rejects_bad_arguments_without_touching_the_device():
+    _, d = _impl()
+    out = C.c_void_p()
+    assert d.create_delegate(None, None, None, None, C.byref(out)) == 1
+    rec = {}
+    ctx = _context(rec)
+    assert d.create_delegate(C.byref(ctx), None, None, None, None) == 1
+    short = _context({})
+    short.abi_header.struct_size = 100  # a table that ends before wrap_delegate
+    assert d.create_delegate(C.byref(short), None, None, None, C.byref(out)) == 1
+
+
+def test_create_delegate_without_gpu_fails_cleanly():
+    torch = pytest.importorskip("torch")
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    _, d = _impl()
+    rec, out = {}, C.c_void_p()
+    ctx = _context(rec)
+    assert d.create_delegate(C.byref(ctx), None, None, None, C.byref(out)) == 3  # runtime failure
+    assert "delegate" not in rec
+
+
+@pytest.mark.gpu
+def test_create_delegate_hands_a_working_delegate_to_the_runtime():
+    torch = pytest.importorskip("torch")
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a gfx950 device; none visible")
+    _, d = _impl()
+    rec, out = {}, C.c_void_p()
+    ctx = _context(rec)
+    assert d.create_delegate(C.byref(ctx), None, None, None, C.byref(out)) == 0
+    assert out.value == 0xABC0 and rec["delegate"]
+    # the wrapped object is a TfLiteDelegate whose Prepare is set (tflite/core/c/common.h:1442-1493)
+    prepare = C.cast(rec["delegate"] + 8, C.POINTER(C.c_void_p))[0]
+    assert prepare
+    rec["deleter"](rec["delegate"])  # what the runtime does when the wrapper dies
