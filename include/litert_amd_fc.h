@@ -300,7 +300,7 @@ typedef struct lrtfc_int4_group_node {
   int out_depth;
 } lrtfc_int4_group_node;
 typedef struct lrtfc_int4_group_launch {
-  int count, grid_blocks, ksplit, batches, depth;
+  int count, grid_blocks, ksplit, groups_per_wave, batches, depth;
 } lrtfc_int4_group_launch;
 size_t lrtfc_int4_group_table_bytes(void);
 int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,

@@ -108,4 +108,4 @@ class Int4GroupNode(C.Structure):
 class Int4GroupLaunch(C.Structure):
     """lrtfc_int4_group_launch."""
     _fields_ = [("count", C.c_int), ("grid_blocks", C.c_int), ("ksplit", C.c_int),
-                ("batches", C.c_int), ("depth", C.c_int)]
+                ("groups_per_wave", C.c_int), ("batches", C.c_int), ("depth", C.c_int)]

@@ -710,7 +710,9 @@ int lrtfc_fc_blockwise_int4_packed_grouped(const void* device_table,
   if (int rc = RequireInit()) return rc;
   LRTFC_REQUIRE(device_table && launch, "null pointer");
   LRTFC_REQUIRE(launch->count >= 1 && launch->count <= LRTFC_INT4_GROUP_MAX &&
-                    launch->grid_blocks >= 1 && launch->ksplit >= 1 && launch->ksplit <= 4,
+                    launch->grid_blocks >= 1 && launch->ksplit >= 1 && launch->ksplit <= 4 &&
+                    launch->groups_per_wave >= 1 && launch->groups_per_wave <= 8 &&
+                    (launch->ksplit == 1 || launch->groups_per_wave == 1),
                 "launch record was not filled by lrtfc_int4_group_prepare");
   LRTFC_REQUIRE(quant_variant >= 0 && quant_variant <= LRTFC_QUANT_NEON_LEGACY,
                 "unknown quantizer variant");

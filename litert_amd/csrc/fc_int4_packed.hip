@@ -19,11 +19,16 @@
 // of a row in block order in float32; that order is kept: the products of a tile are
 // parked in LDS and 8 x batch lanes walk them in order, tile after tile, each walk
 // overlapping the wait for the next tile's bytes.
+#include <type_traits>
+
 #include "kernels.h"
 #include "quantize_device.h"
 
 namespace lrtfc {
 namespace {
+
+#define LRTFC_GLOBAL __attribute__((address_space(1)))
+using f32x4 = float __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWaveSize;
@@ -36,6 +41,7 @@ constexpr int kTileVecs = kPlanes * 64;  // i32x4 per tile
 constexpr int kRingTiles = 2;
 constexpr int kPStride = kTileBlocks + 4;  // floats per (row, batch) line of parked products
 constexpr int kMaxGroupNodes = LRTFC_INT4_GROUP_MAX;
+constexpr int kMaxGroupsPerWave = 8;  // 64 channels: one lane each when their kfsum is staged
 
 __global__ __launch_bounds__(kThreads) void PackInt4BlockwiseKernel(
     const uint8_t* __restrict__ filter, const uint16_t* __restrict__ scales, int out_depth,
@@ -105,6 +111,8 @@ struct Int4Shared {
   int32_t* zp;  // [BT]
   int32_t* zero;
   float* mm;    // [BT][kWaves][2]
+  float* kb;    // [kWaves][2][64]: kfsum and bias of the channels a wavefront covers
+  float* ob;    // [kWaves][64 * BT]: finished outputs of those channels
   // Floats of parked products: one tile per wavefront when a wavefront owns a channel group
   // alone; every tile of the group when `ksplit` wavefronts share it (the ordered walk then
   // needs them all).
@@ -122,20 +130,36 @@ struct Int4Shared {
     zp = reinterpret_cast<int32_t*>(inv + 8);
     zero = zp + 8;
     mm = reinterpret_cast<float*>(zero + 8);
+    kb = mm + BT * kWaves * 2;
+    ob = kb + kWaves * 2 * 64;
   }
   static size_t Bytes(int padded, int ksplit) {
     const int chunks = padded / (kTileBlocks * kBlock);
     return static_cast<size_t>(BT) * padded + ProductFloats(chunks, ksplit) * 4 + 4 * 8 * 4 +
-           8 * kWaves * 2 * 4;
+           BT * kWaves * 2 * 4 + kWaves * 2 * 64 * 4 + kWaves * 64 * BT * 4;
   }
 };
 
 // GPT: groups of 8 depth positions each thread keeps in registers between the two passes of
 // the prologue; the register form covers depth <= GPT * 256 * 8.
 // The work of one workgroup; `block` is its index among the workgroups of this filter.
+// gpw: consecutive channel groups one wavefront works through (ksplit == 1 only). Their
+// tiles are one contiguous stretch of the filter, so the ring of loads runs on across group
+// boundaries and the prologue (the row quantizer) is paid once for all of them.
 template <int BT, bool FUSED, int VARIANT, int GPT>
 __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int block, int batch0,
-                                                 int bt, int ksplit, int8_t* smem) {
+                                                 int bt, int ksplit, int gpw, int8_t* smem) {
+  // Every tensor is in global memory. Pointers that a kernel read from a table in memory
+  // carry no address space, and accesses through them would go the flat path, whose waits
+  // cannot leave a ring of loads in flight; so the address space is stated here.
+  const LRTFC_GLOBAL i32x4* g_packed = (const LRTFC_GLOBAL i32x4*)a.packed;
+  const LRTFC_GLOBAL float* g_input_f32 = (const LRTFC_GLOBAL float*)a.input_f32;
+  const LRTFC_GLOBAL int8_t* g_input_q = (const LRTFC_GLOBAL int8_t*)a.input_q;
+  const LRTFC_GLOBAL float* g_scaling_factors = (const LRTFC_GLOBAL float*)a.scaling_factors;
+  const LRTFC_GLOBAL int32_t* g_zero_points = (const LRTFC_GLOBAL int32_t*)a.zero_points;
+  const LRTFC_GLOBAL float* g_kfsum = (const LRTFC_GLOBAL float*)a.kfsum;
+  const LRTFC_GLOBAL float* g_bias = (const LRTFC_GLOBAL float*)a.bias;
+  LRTFC_GLOBAL float* g_output = (LRTFC_GLOBAL float*)a.output;
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
   const int wave = tid / kWaveSize;
@@ -147,10 +171,18 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
   // filters would otherwise leave most of the chip without a wavefront).
   const int kpart = wave % ksplit;
   const int group_in_wg = wave / ksplit;
-  const int group = block * (kWaves / ksplit) + group_in_wg;  // may run past the last
-  const i32x4* tbase = reinterpret_cast<const i32x4*>(a.packed) +
-                       static_cast<size_t>(min(group, groups - 1)) * chunks * kTileVecs + lane;
+  const int group0 = (block * (kWaves / ksplit) + group_in_wg) * gpw;  // may run past the last
+  const int my_groups = max(0, min(gpw, groups - group0));
+  const int ntiles = my_groups * chunks;  // tiles of this wavefront and its depth partners
+  const int first_group = min(group0, groups - 1);
+  const LRTFC_GLOBAL i32x4* tbase = g_packed +
+                       static_cast<size_t>(first_group) * chunks * kTileVecs + lane;
   Int4Shared<BT> sh(smem, padded, chunks, ksplit);
+  // Per-channel epilogue inputs of every channel this wavefront covers (lane = channel),
+  // requested ahead of the weights and parked in LDS once the prologue is through.
+  const int my_n = min(first_group * kTileRows + lane, a.out_depth - 1);
+  const float kfsum_raw = g_kfsum[my_n];
+  const float bias_raw = a.bias ? g_bias[my_n] : 0.0f;
 
   // Activation loads first (raw, branch-free): whatever the prologue waits for must be
   // requested before the weight ring, because vector memory returns in issue order.
@@ -166,17 +198,19 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
     if (in_regs) {
 #pragma unroll
       for (int b = 0; b < BT; ++b) {
-        const float* x = a.input_f32 + static_cast<size_t>(batch0 + min(b, bt - 1)) * depth;
+        const LRTFC_GLOBAL float* x = g_input_f32 + static_cast<size_t>(batch0 + min(b, bt - 1)) * depth;
 #pragma unroll
         for (int j = 0; j < kGroupsPerThread; ++j) {
           const int g = min(j * kThreads + tid, groups8 - 1);
-          xr[b][j][0] = *reinterpret_cast<const float4*>(x + g * 8);
-          xr[b][j][1] = *reinterpret_cast<const float4*>(x + g * 8 + 4);
+          const f32x4 lo = *reinterpret_cast<const LRTFC_GLOBAL f32x4*>(x + g * 8);
+          const f32x4 hi = *reinterpret_cast<const LRTFC_GLOBAL f32x4*>(x + g * 8 + 4);
+          xr[b][j][0] = make_float4(lo.x, lo.y, lo.z, lo.w);
+          xr[b][j][1] = make_float4(hi.x, hi.y, hi.z, hi.w);
         }
       }
     } else {
       for (int b = 0; b < bt; ++b) {  // slow form: min/max from memory before the ring
-        const float* x = a.input_f32 + static_cast<size_t>(batch0 + b) * depth;
+        const LRTFC_GLOBAL float* x = g_input_f32 + static_cast<size_t>(batch0 + b) * depth;
         float mn = 0.0f, mx = 0.0f;
         for (int i = tid; i < depth; i += kThreads) {
           mn = fminf(mn, x[i]);
@@ -196,16 +230,16 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
     if (in_regs) {
 #pragma unroll
       for (int b = 0; b < BT; ++b) {
-        const int8_t* x = a.input_q + static_cast<size_t>(batch0 + min(b, bt - 1)) * depth;
+        const LRTFC_GLOBAL int8_t* x = g_input_q + static_cast<size_t>(batch0 + min(b, bt - 1)) * depth;
 #pragma unroll
         for (int j = 0; j < kGroupsPerThread; ++j) {
           const int g = min(j * kThreads + tid, groups8 - 1);
-          qr[b][j] = *reinterpret_cast<const i32x2*>(x + g * 8);
+          qr[b][j] = *reinterpret_cast<const LRTFC_GLOBAL i32x2*>(x + g * 8);
         }
       }
     } else {
       for (int b = 0; b < bt; ++b) {
-        const int8_t* x = a.input_q + static_cast<size_t>(batch0 + b) * depth;
+        const LRTFC_GLOBAL int8_t* x = g_input_q + static_cast<size_t>(batch0 + b) * depth;
         for (int g = tid; g < padded / 8; g += kThreads) {
           uint32_t lo = 0, hi = 0;
           if (g < groups8) {
@@ -229,22 +263,19 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
   // row the prologue is too short for that to pay (9.0 -> 9.5 us), so both go out at once.
   i32x4 ring[kRingTiles][kPlanes];
   auto request_tile = [&](int t) {
-    const int c = min(kpart + t * ksplit, chunks - 1);
+    const int lin = min(kpart + t * ksplit, max(ntiles, 1) - 1);
 #pragma unroll
     for (int j = 0; j < kPlanes; ++j) {
-      ring[t][j] = __builtin_nontemporal_load(tbase + static_cast<size_t>(c) * kTileVecs + j * 64);
+      ring[t][j] =
+          __builtin_nontemporal_load(tbase + static_cast<size_t>(lin) * kTileVecs + j * 64);
     }
   };
   request_tile(0);
   if (BT == 1) request_tile(1);
-  // Per-channel epilogue inputs of the chain lanes (lane = row * BT + batch).
+  // Chain lanes: lane = row * BT + batch.
   const int chain_row = lane / BT;
   const int chain_b = lane - chain_row * BT;
   const bool chain_lane = lane < kTileRows * BT;
-  const int chain_n = min(min(group, groups - 1) * kTileRows + min(chain_row, kTileRows - 1),
-                          a.out_depth - 1);
-  const float kfsum_n = a.kfsum[chain_n];
-  const float bias_n = a.bias ? a.bias[chain_n] : 0.0f;
 
   // Activation rows into LDS.
   if (FUSED) {
@@ -318,7 +349,7 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
       }
     } else {
       for (int b = 0; b < bt; ++b) {
-        const float* x = a.input_f32 + static_cast<size_t>(batch0 + b) * depth;
+        const LRTFC_GLOBAL float* x = g_input_f32 + static_cast<size_t>(batch0 + b) * depth;
         RowQuantParams qp;
         qp.scale = sh.sf[b];
         qp.inv = sh.inv[b];
@@ -359,11 +390,15 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
 
   if (BT > 1) request_tile(1);
 
+  float* kb = sh.kb + wave * 2 * 64;
+  kb[lane] = kfsum_raw;
+  kb[64 + lane] = bias_raw;
+
   float row_scale = 0.0f;
   float row_zp = 0.0f;
   if (chain_lane && chain_b < bt) {
-    row_scale = FUSED ? sh.sf[chain_b] : a.scaling_factors[batch0 + chain_b];
-    row_zp = static_cast<float>(FUSED ? sh.zp[chain_b] : a.zero_points[batch0 + chain_b]);
+    row_scale = FUSED ? sh.sf[chain_b] : g_scaling_factors[batch0 + chain_b];
+    row_zp = static_cast<float>(FUSED ? sh.zp[chain_b] : g_zero_points[batch0 + chain_b]);
   }
 
   // Tile loop. Lane L owns block L of the tile for each of the 8 channels.
@@ -391,9 +426,24 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
       for (int j = 0; j < count; ++j) out = __fadd_rn(out, line[j]);
     }
   };
-  int it = 0;
-  for (int c = kpart; c < chunks; c += ksplit, ++it) {
-    const int slot = it % kRingTiles;
+  // fully_connected.cc:1078-1082 for the channel group at offset `goff` from the first. The
+  // value is parked in LDS and leaves in one store at the end: a store inside the tile loop
+  // would make the number of outstanding memory operations depend on the path taken, and
+  // the waits for the ring would have to assume the worst.
+  float* ob = sh.ob + wave * (kMaxGroupsPerWave * kTileRows * BT);
+  auto finish_group = [&](int goff) {
+    float o = __fsub_rn(out, __fmul_rn(row_zp, kb[goff * kTileRows + chain_row]));
+    o = __fmul_rn(o, row_scale);
+    if (a.bias) o = __fadd_rn(o, kb[64 + goff * kTileRows + chain_row]);
+    ob[goff * kTileRows * BT + lane] = o;
+  };
+  // One tile: ring slot SLOT holds tile `lin` of this wavefront's stretch. REFILL requests the
+  // tile two turns ahead into the same slot -- always, so that every turn of the main loop
+  // issues the same number of loads and the wait for a slot can leave exactly the other slot's
+  // loads in flight; past the end the request goes to one hot cache line instead.
+  auto process = [&](auto slot_tag, auto refill_tag, int lin, int c) {
+    constexpr int SLOT = decltype(slot_tag)::value;
+    constexpr bool REFILL = decltype(refill_tag)::value;
     float* pw = ksplit == 1 ? sh.p + static_cast<size_t>(wave) * kTileFloats
                             : pgroup + static_cast<size_t>(c) * kTileFloats;
     // This block's activations (8 dwords per batch row) and 8 * sum(q).
@@ -416,73 +466,101 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
       s = Dot4(qo[b].w, 0x01010101, s);
       qsum8[b] = 8 * s;
     }
+    const i32x4 sc = ring[SLOT][kTileRows];
 #pragma unroll
-    for (int t = 0; t < kRingTiles; ++t) {
-      if (t == slot) {  // static ring indexing
-        const i32x4 sc = ring[t][kTileRows];
+    for (int j = 0; j < kTileRows; ++j) {
+      const uint32_t pair = static_cast<uint32_t>(sc[j >> 1]);
+      const float scale =
+          HalfBitsToFloatFast(static_cast<uint16_t>((j & 1) ? (pair >> 16) : (pair & 0xFFFF)));
+      const i32x4 wv = ring[SLOT][j];
+      uint32_t lo[4], hi[4];
 #pragma unroll
-        for (int j = 0; j < kTileRows; ++j) {
-          const uint32_t pair = static_cast<uint32_t>(sc[j >> 1]);
-          const float scale = HalfBitsToFloatFast(static_cast<uint16_t>((j & 1) ? (pair >> 16) : (pair & 0xFFFF)));
-          const i32x4 wv = ring[t][j];
-          uint32_t lo[4], hi[4];
-#pragma unroll
-          for (int d = 0; d < 4; ++d) {
-            lo[d] = static_cast<uint32_t>(wv[d]) & 0x0F0F0F0Fu;
-            hi[d] = (static_cast<uint32_t>(wv[d]) >> 4) & 0x0F0F0F0Fu;
-          }
-#pragma unroll
-          for (int b = 0; b < BT; ++b) {
-            int32_t acc = -qsum8[b];
-            acc = Dot4(lo[0], qe[b].x, acc);
-            acc = Dot4(hi[0], qe[b].y, acc);
-            acc = Dot4(lo[1], qe[b].z, acc);
-            acc = Dot4(hi[1], qe[b].w, acc);
-            acc = Dot4(lo[2], qo[b].x, acc);
-            acc = Dot4(hi[2], qo[b].y, acc);
-            acc = Dot4(lo[3], qo[b].z, acc);
-            acc = Dot4(hi[3], qo[b].w, acc);
-            pw[(j * BT + b) * kPStride + lane] = __fmul_rn(static_cast<float>(acc), scale);
-          }
-        }
-        // Refill the slot with this wavefront's tile two turns ahead.
-        if (c + kRingTiles * ksplit < chunks) {
-#pragma unroll
-          for (int j = 0; j < kPlanes; ++j) {
-            ring[t][j] = __builtin_nontemporal_load(
-                tbase + static_cast<size_t>(c + kRingTiles * ksplit) * kTileVecs + j * 64);
-          }
-        }
+      for (int d = 0; d < 4; ++d) {
+        lo[d] = static_cast<uint32_t>(wv[d]) & 0x0F0F0F0Fu;
+        hi[d] = (static_cast<uint32_t>(wv[d]) >> 4) & 0x0F0F0F0Fu;
       }
+#pragma unroll
+      for (int b = 0; b < BT; ++b) {
+        int32_t acc = -qsum8[b];
+        acc = Dot4(lo[0], qe[b].x, acc);
+        acc = Dot4(hi[0], qe[b].y, acc);
+        acc = Dot4(lo[1], qe[b].z, acc);
+        acc = Dot4(hi[1], qe[b].w, acc);
+        acc = Dot4(lo[2], qo[b].x, acc);
+        acc = Dot4(hi[2], qo[b].y, acc);
+        acc = Dot4(lo[3], qo[b].z, acc);
+        acc = Dot4(hi[3], qo[b].w, acc);
+        pw[(j * BT + b) * kPStride + lane] = __fmul_rn(static_cast<float>(acc), scale);
+      }
+    }
+    if (REFILL) {
+      const int next = lin + kRingTiles * ksplit;
+      const LRTFC_GLOBAL i32x4* src =
+          next < ntiles ? tbase + static_cast<size_t>(next) * kTileVecs : g_packed;
+#pragma unroll
+      for (int j = 0; j < kPlanes; ++j) ring[SLOT][j] = __builtin_nontemporal_load(src + j * 64);
     }
     // Ordered float32 accumulation over this tile's blocks (same wavefront wrote them).
     if (ksplit == 1 && chain_lane) walk_tile(pw, c);
+  };
+  // Moves on to the next tile of the stretch; closes a channel group after its last tile.
+#define LRTFC_INT4_ADVANCE()                      \
+  do {                                            \
+    if (ksplit == 1) {                            \
+      if (++c == chunks) {                        \
+        if (chain_lane) finish_group(goff);       \
+        out = 0.0f;                               \
+        c = 0;                                    \
+        ++goff;                                   \
+      }                                           \
+    } else {                                      \
+      c += ksplit;                                \
+    }                                             \
+  } while (0)
+  int c = kpart;  // tile index within the current channel group
+  int goff = 0;
+  using Slot0 = std::integral_constant<int, 0>;
+  using Slot1 = std::integral_constant<int, 1>;
+  int lin = kpart;
+  for (; lin + ksplit < ntiles; lin += kRingTiles * ksplit) {
+    process(Slot0{}, std::true_type{}, lin, c);
+    LRTFC_INT4_ADVANCE();
+    process(Slot1{}, std::true_type{}, lin + ksplit, c);
+    LRTFC_INT4_ADVANCE();
   }
+  if (lin < ntiles) {
+    process(Slot0{}, std::false_type{}, lin, c);
+    LRTFC_INT4_ADVANCE();
+  }
+#undef LRTFC_INT4_ADVANCE
   if (ksplit > 1) {
     // Every tile of the group is parked; its first wavefront walks them in depth order.
     __syncthreads();
-    if (kpart == 0 && chain_lane) {
-      for (int c = 0; c < chunks; ++c) walk_tile(pgroup + static_cast<size_t>(c) * kTileFloats, c);
+    if (kpart == 0 && chain_lane && my_groups > 0) {
+      for (int cc = 0; cc < chunks; ++cc) {
+        walk_tile(pgroup + static_cast<size_t>(cc) * kTileFloats, cc);
+      }
+      finish_group(0);
     }
   }
-
-  // fully_connected.cc:1078-1082.
-  if (kpart == 0 && chain_lane && chain_b < bt && group < groups) {
-    const int n = group * kTileRows + chain_row;
-    if (n < a.out_depth) {
-      out = __fsub_rn(out, __fmul_rn(row_zp, kfsum_n));
-      out = __fmul_rn(out, row_scale);
-      if (a.bias) out = __fadd_rn(out, bias_n);
-      a.output[static_cast<size_t>(batch0 + chain_b) * a.out_depth + n] = out;
+  // Outputs of this wavefront's channel groups: index = (group offset, row, batch).
+  if (kpart == 0) {
+    for (int i = lane; i < my_groups * kTileRows * BT; i += kWaveSize) {
+      const int b = i % BT;
+      const int row = i / BT;  // channel offset from the first group's first channel
+      const int n = group0 * kTileRows + row;
+      if (b < bt && n < a.out_depth) {
+        g_output[static_cast<size_t>(batch0 + b) * a.out_depth + n] = ob[i];
+      }
     }
   }
 }
 
 template <int BT, bool FUSED, int VARIANT, int GPT>
 __global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a, int batch0,
-                                                               int bt, int ksplit) {
+                                                               int bt, int ksplit, int gpw) {
   extern __shared__ __align__(16) int8_t smem[];
-  FcInt4PackedBody<BT, FUSED, VARIANT, GPT>(a, blockIdx.x, batch0, bt, ksplit, smem);
+  FcInt4PackedBody<BT, FUSED, VARIANT, GPT>(a, blockIdx.x, batch0, bt, ksplit, gpw, smem);
 }
 
 // Several filters of the same depth in one launch (nodes of a graph that do not depend on
@@ -497,7 +575,8 @@ struct Int4GroupTable {
 
 template <int BT, int VARIANT, int GPT>
 __global__ __launch_bounds__(kThreads) void FcInt4PackedGroupedKernel(
-    const Int4GroupTable* __restrict__ table, int count, int batch0, int bt, int ksplit) {
+    const Int4GroupTable* __restrict__ table, int count, int batch0, int bt, int ksplit,
+    int gpw) {
   extern __shared__ __align__(16) int8_t smem[];
   // first_block is ascending: the node of this workgroup is the number of later nodes whose
   // first workgroup is not beyond it. One vector load and a ballot instead of a scalar walk.
@@ -508,7 +587,7 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedGroupedKernel(
   const int node = __builtin_amdgcn_readfirstlane(__popcll(__ballot(not_beyond)));
   const Int4PackedArgs a = table->node[node];
   FcInt4PackedBody<BT, true, VARIANT, GPT>(a, blockIdx.x - table->first_block[node], batch0, bt,
-                                           ksplit, smem);
+                                           ksplit, gpw, smem);
 }
 
 // Wavefronts per channel group: one while that already gives the chip ~1000 wavefronts;
@@ -518,6 +597,19 @@ int ChooseKsplit(int out_depth, int chunks) {
   int ksplit = 1;
   while (ksplit < kWaves && groups * ksplit < 1024 && chunks >= 4 * ksplit) ksplit *= 2;
   return ksplit;
+}
+
+// Channel groups per wavefront. Measured on launches from 7 MB to 340 MB: a wavefront should
+// stream up to 8 tiles (its ring then runs long enough to amortize the prologue), as long as
+// the launch keeps about one workgroup per CU (224 of them) to spread over the chip.
+int ChooseGroupsPerWave(int total_groups, int chunks, int ksplit) {
+  if (ksplit > 1) return 1;
+  int gpw = 1;
+  while (gpw * 2 <= kMaxGroupsPerWave && gpw * 2 * chunks <= 8 &&
+         total_groups / (kWaves * gpw * 2) >= 224) {
+    gpw *= 2;
+  }
+  return gpw;
 }
 
 template <int BT, bool FUSED, int VARIANT, int GPT>
@@ -537,9 +629,10 @@ hipError_t LaunchOne(const Int4PackedArgs& a, int batch0, int bt, hipStream_t st
     }
   }
   const int groups = (a.out_depth + kTileRows - 1) / kTileRows;
-  const int groups_per_wg = kWaves / ksplit;
+  const int gpw = ChooseGroupsPerWave(groups, a.chunks, ksplit);
+  const int groups_per_wg = kWaves / ksplit * gpw;
   const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, batch0, bt, ksplit);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, batch0, bt, ksplit, gpw);
   return hipGetLastError();
 }
 
@@ -656,7 +749,8 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
   int total_out = 0;
   for (int i = 0; i < count; ++i) total_out += nodes[i].out_depth;
   const int ksplit = ChooseKsplit(total_out, chunks);
-  const int groups_per_wg = kWaves / ksplit;
+  const int gpw = ChooseGroupsPerWave((total_out + kTileRows - 1) / kTileRows, chunks, ksplit);
+  const int groups_per_wg = kWaves / ksplit * gpw;
   Int4GroupTable host{};
   int next = 0;
   for (int i = 0; i < count; ++i) {
@@ -685,6 +779,7 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
   launch->count = count;
   launch->grid_blocks = next;
   launch->ksplit = ksplit;
+  launch->groups_per_wave = gpw;
   launch->batches = batches;
   launch->depth = depth;
   return hipSuccess;
@@ -711,7 +806,8 @@ hipError_t LaunchGroupedOne(const void* table, const lrtfc_int4_group_launch& l,
     }
   }
   hipLaunchKernelGGL(kernel, dim3(l.grid_blocks), dim3(kThreads), lds, stream,
-                     static_cast<const Int4GroupTable*>(table), l.count, batch0, bt, l.ksplit);
+                     static_cast<const Int4GroupTable*>(table), l.count, batch0, bt, l.ksplit,
+                     l.groups_per_wave);
   return hipGetLastError();
 }
 

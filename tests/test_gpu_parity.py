@@ -410,6 +410,30 @@ def test_blockwise_int4_grouped_launch_matches_oracle(fc, B, K, Ns):
             assert _bits_equal(y.cpu().numpy(), want), (trial, n)
 
 
+@pytest.mark.parametrize("B", [1, 3])
+def test_blockwise_int4_wavefronts_spanning_channel_groups(fc, B):
+    """Launches large enough that one wavefront works through 8 consecutive channel groups
+    (7169 groups of 8 channels, depth 2048): a single node whose last wavefront and last group
+    are partial, then three nodes of the same total size in one launch."""
+    K = 2048
+    c = wl.blockwise_int4_fc(B, K, 57349, seed=77, lo=-8, hi=7)
+    bias = np.random.default_rng(3).standard_normal(57349).astype(np.float32)
+    op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], K, 32, bias)
+    y = op(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_blockwise_int4(c["x"], c["packed"], 57349, c["scales"].view(np.uint16), 32, bias)
+    assert _bits_equal(y, want)
+    Ns = (40000, 264, 17101)
+    cs = [wl.blockwise_int4_fc(B, K, n, seed=900 + n, lo=-8, hi=7) for n in Ns]
+    ops = [fc.FullyConnectedBlockwiseInt4(ci["packed"], ci["scales"], K, 32) for ci in cs]
+    xs = [_cuda(ci["x"]) for ci in cs]
+    ys = [torch.full((B, n), float("nan"), dtype=torch.float32, device="cuda") for n in Ns]
+    fc.GroupedBlockwiseInt4(ops).bind(xs, ys)()
+    torch.cuda.synchronize()
+    for ci, yi, n in zip(cs, ys, Ns):
+        want = oracle.fc_blockwise_int4(ci["x"], ci["packed"], n, ci["scales"].view(np.uint16), 32)
+        assert _bits_equal(yi.cpu().numpy(), want), n
+
+
 def test_blockwise_int4_grouped_launch_needs_bind(fc):
     c = wl.blockwise_int4_fc(1, 64, 8, seed=2, lo=-8, hi=7)
     op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], 64, 32)
