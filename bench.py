@@ -391,7 +391,7 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
 
         layers = [keyed[l * per_layer:(l + 1) * per_layer] for l in range(wl.GEMMA2B_LAYERS)]
         # As the configuration defines it, every node is independent: all nodes of one depth
-        # can share launches (groups of up to 32 nodes).
+        # can share launches (groups of up to 128 nodes: one launch per depth).
         shallow = [kn for kn in keyed if kn[0].depth == 2048]
         deep = [kn for kn in keyed if kn[0].depth != 2048]
         mx = fc.GroupedBlockwiseInt4.MAX_NODES

@@ -290,7 +290,7 @@ int lrtfc_fc_hybrid_int4_per_channel_packed(const float* input, const int8_t* pa
  *     pointers; bias may be NULL per node.
  *   lrtfc_fc_blockwise_int4_packed_grouped: the launch (one kernel per 4 batch rows, per 2
  *     above depth 4096); allocates and copies nothing. */
-#define LRTFC_INT4_GROUP_MAX 32
+#define LRTFC_INT4_GROUP_MAX 128
 typedef struct lrtfc_int4_group_node {
   const float* input;            /* [batches, depth] */
   const uint8_t* retiled_filter; /* from lrtfc_pack_int4_blockwise */

@@ -579,12 +579,17 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedGroupedKernel(
     int gpw) {
   extern __shared__ __align__(16) int8_t smem[];
   // first_block is ascending: the node of this workgroup is the number of later nodes whose
-  // first workgroup is not beyond it. One vector load and a ballot instead of a scalar walk.
+  // first workgroup is not beyond it. Vector loads and ballots (64 nodes per turn) instead of
+  // a scalar walk.
   const int lane = threadIdx.x & (kWaveSize - 1);
-  const int probe = min(lane + 1, count);
-  const bool not_beyond =
-      lane + 1 < count && static_cast<int>(blockIdx.x) >= table->first_block[probe];
-  const int node = __builtin_amdgcn_readfirstlane(__popcll(__ballot(not_beyond)));
+  int node = 0;
+  for (int base = 0; base + 1 < count; base += kWaveSize) {
+    const int probe = base + lane + 1;
+    const bool not_beyond =
+        probe < count && static_cast<int>(blockIdx.x) >= table->first_block[min(probe, count)];
+    node += __popcll(__ballot(not_beyond));
+  }
+  node = __builtin_amdgcn_readfirstlane(node);
   const Int4PackedArgs a = table->node[node];
   FcInt4PackedBody<BT, true, VARIANT, GPT>(a, blockIdx.x - table->first_block[node], batch0, bt,
                                            ksplit, gpw, smem);

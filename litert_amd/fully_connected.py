@@ -393,7 +393,7 @@ class GroupedBlockwiseInt4:
     node (the launch reads their addresses from a table in device memory); `__call__`
     launches. Results are those of the nodes' own calls."""
 
-    MAX_NODES = 32
+    MAX_NODES = 128  # LRTFC_INT4_GROUP_MAX
 
     def __init__(self, ops):
         if not 1 <= len(ops) <= self.MAX_NODES:

@@ -388,7 +388,7 @@ def test_blockwise_int4_split_launch_matches_oracle(fc, B, K, N):
 @pytest.mark.parametrize("B,K,Ns", [(1, 2048, (64, 8, 24, 130, 520)), (3, 2048, (16, 256, 9)),
                                     (4, 1024, (40,)), (1, 16384, (16, 40)), (2, 8192, (24, 8, 72)),
                                     (9, 2048, (24, 80)), (5, 16384, (8, 16)),
-                                    (1, 64, tuple(range(4, 36)))])
+                                    (1, 64, tuple(range(4, 36))), (2, 64, tuple(range(3, 103)))])
 def test_blockwise_int4_grouped_launch_matches_oracle(fc, B, K, Ns):
     """Several filters of one depth in one launch: every node against the oracle, with its
     own input and, for odd channel counts, its own bias; then again after re-binding to new
@@ -441,6 +441,8 @@ def test_blockwise_int4_grouped_launch_needs_bind(fc):
         fc.GroupedBlockwiseInt4([op])()
     with pytest.raises(ValueError):
         fc.GroupedBlockwiseInt4([])
+    with pytest.raises(ValueError):
+        fc.GroupedBlockwiseInt4([op] * (fc.GroupedBlockwiseInt4.MAX_NODES + 1))
 
 
 @pytest.mark.parametrize("B,K,N,bs", [(2, 128, 6, 64), (1, 64, 5, 16), (3, 256, 4, 128), (2, 96, 8, 8)])
