@@ -16,6 +16,7 @@
 // leave HBM.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -23,6 +24,7 @@
 #include <map>
 #include <memory>
 #include <string>
+#include <tuple>
 #include <vector>
 
 #include "litert_amd_fc.h"
@@ -311,8 +313,14 @@ struct PartitionKernel {
   hipEvent_t lane_done[kMaxStreams] = {};
   std::vector<hipEvent_t> node_done;  // per node; only the signalling ones are created
   bool lane_used[kMaxStreams] = {};
+  struct Unit {
+    int level;  // distance from the partition's inputs
+    int first;  // node index (of the group's first member)
+    int group;  // index into groups, or -1 for a node on its own
+  };
+  std::vector<Unit> order;  // launch order
   struct Group {
-    std::vector<int> members;  // node indices, consecutive
+    std::vector<int> members;  // node indices, ascending
     DeviceBuffer table;
     lrtfc_int4_group_launch launch{};
   };
@@ -637,52 +645,70 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
     RETURN_IF_HIP(ctx, k->upload_stage.Ensure(k->upload_bytes));
     RETURN_IF_HIP(ctx, k->download_stage.Ensure(k->download_bytes));
   }
-  // Groups: runs of consecutive blockwise-int4 nodes on the fused re-tiled kernel with one
-  // depth and batch count, none of which reads what another of the run writes.
+  // Levels: a node without a producer inside the partition is at level 0, a consumer one
+  // above its producer (an FC node has one activation input, so one producer at most).
+  std::vector<int> level(count, 0);
+  for (int i = 0; i < count; ++i) {
+    if (k->nodes[i].producer >= 0) level[i] = level[k->nodes[i].producer] + 1;
+  }
+  // Groups: blockwise-int4 nodes on the fused re-tiled kernel that share level, depth and
+  // batch count -- wherever they stand in the plan. Nodes of one level cannot depend on each
+  // other, so each such set (cut into pieces of LRTFC_INT4_GROUP_MAX) is one launch.
   k->groups.clear();
   for (FcNode& n : k->nodes) n.group = -1;
   auto groupable = [&](const FcNode& n) {
     return n.kind == FcKind::kInt4Blockwise && n.use_retiled && !n.split_quantize &&
            n.depth > 0 && n.batches > 0 && n.out_depth > 0;
   };
-  for (int i = 0; i < count;) {
-    int j = i;
-    if (groupable(k->nodes[i])) {
-      while (j + 1 < count && j + 1 - i < LRTFC_INT4_GROUP_MAX && groupable(k->nodes[j + 1]) &&
-             k->nodes[j + 1].depth == k->nodes[i].depth &&
-             k->nodes[j + 1].batches == k->nodes[i].batches && k->nodes[j + 1].producer < i) {
-        ++j;
+  {
+    std::map<std::tuple<int, int, int>, std::vector<int>> sets;  // (level, depth, batches)
+    for (int i = 0; i < count; ++i) {
+      const FcNode& n = k->nodes[i];
+      if (groupable(n)) sets[std::make_tuple(level[i], n.depth, n.batches)].push_back(i);
+    }
+    for (const auto& entry : sets) {
+      const std::vector<int>& all = entry.second;
+      for (size_t at = 0; at < all.size(); at += LRTFC_INT4_GROUP_MAX) {
+        const size_t end = std::min(all.size(), at + static_cast<size_t>(LRTFC_INT4_GROUP_MAX));
+        if (end - at < 2) continue;
+        PartitionKernel::Group g;
+        g.members.assign(all.begin() + at, all.begin() + end);
+        for (int m : g.members) k->nodes[m].group = static_cast<int>(k->groups.size());
+        k->groups.push_back(std::move(g));
       }
     }
-    if (j > i) {
-      PartitionKernel::Group g;
-      for (int m = i; m <= j; ++m) {
-        g.members.push_back(m);
-        k->nodes[m].group = static_cast<int>(k->groups.size());
-      }
-      k->groups.push_back(std::move(g));
-    }
-    i = j + 1;
   }
+  // Launch order: units (a group, or a node on its own) by level, then by first node. A unit
+  // only reads what lower levels wrote, so this is a topological order of the partition.
+  k->order.clear();
+  for (int i = 0; i < count; ++i) {
+    const int g = k->nodes[i].group;
+    if (g >= 0 && k->groups[g].members.front() != i) continue;  // listed with its group
+    k->order.push_back(PartitionKernel::Unit{level[i], i, g});
+  }
+  std::stable_sort(k->order.begin(), k->order.end(),
+                   [](const PartitionKernel::Unit& a, const PartitionKernel::Unit& b) {
+                     return a.level != b.level ? a.level < b.level : a.first < b.first;
+                   });
   // Streams: a unit (node or group) continues on the stream of its first node's producer
   // unless a sibling already did; units without a producer in the partition, and further
   // siblings, take streams round-robin.
   std::vector<bool> continued(count, false);
   int next_lane = 0;
   for (int i = 0; i < k->kMaxStreams; ++i) k->lane_used[i] = false;
-  for (int i = 0; i < count; ++i) {
-    FcNode& n = k->nodes[i];
-    n.signal = false;
-    const bool follower = n.group >= 0 && k->groups[n.group].members.front() != i;
-    if (follower) {
-      n.lane = k->nodes[k->groups[n.group].members.front()].lane;
-    } else if (n.producer >= 0 && !continued[n.producer]) {
+  for (FcNode& n : k->nodes) n.signal = false;
+  for (const PartitionKernel::Unit& u : k->order) {
+    FcNode& n = k->nodes[u.first];
+    if (n.producer >= 0 && !continued[n.producer]) {
       n.lane = k->nodes[n.producer].lane;
       continued[n.producer] = true;
     } else {
       n.lane = next_lane++ % k->num_streams;
     }
     k->lane_used[n.lane] = true;
+    if (u.group >= 0) {
+      for (int m : k->groups[u.group].members) k->nodes[m].lane = n.lane;
+    }
   }
   for (const FcNode& n : k->nodes) {
     if (n.producer >= 0 && k->nodes[n.producer].lane != n.lane) k->nodes[n.producer].signal = true;
@@ -759,26 +785,32 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
       if (k->lane_used[i]) RETURN_IF_HIP(ctx, hipStreamWaitEvent(k->streams[i], k->upload_done, 0));
     }
   }
-  for (size_t node_i = 0; node_i < k->nodes.size(); ++node_i) {
+  for (const PartitionKernel::Unit& unit : k->order) {
+    const size_t node_i = static_cast<size_t>(unit.first);
     FcNode& n = k->nodes[node_i];
     hipStream_t s = k->streams[n.lane];
     DeviceBuffer& scratch = k->workspace[n.lane];
-    // Cross-stream edge: wait for the producer. (Runs before the early-outs below so that a
-    // consumer never waits on an event that was not recorded in this invoke.)
-    if (n.producer >= 0 && k->nodes[n.producer].lane != n.lane) {
-      RETURN_IF_HIP(ctx, hipStreamWaitEvent(s, k->node_done[n.producer], 0));
-    }
-    if (n.group >= 0) {
-      // The whole group launches when its last member is reached: by then the waits of every
-      // member are queued on the group's stream; members record their events after it.
-      PartitionKernel::Group& g = k->groups[n.group];
-      if (g.members.back() != static_cast<int>(node_i)) continue;
+    if (unit.group >= 0) {
+      // One launch for the whole group, behind the producers of every member; members that
+      // other streams wait for record their events after it.
+      PartitionKernel::Group& g = k->groups[unit.group];
+      for (int m : g.members) {
+        const int producer = k->nodes[m].producer;
+        if (producer >= 0 && k->nodes[producer].lane != n.lane) {
+          RETURN_IF_HIP(ctx, hipStreamWaitEvent(s, k->node_done[producer], 0));
+        }
+      }
       RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4_packed_grouped(
                             g.table.get(), &g.launch, k->state->options.quant_variant, s));
       for (int m : g.members) {
         if (k->nodes[m].signal) RETURN_IF_HIP(ctx, hipEventRecord(k->node_done[m], s));
       }
       continue;
+    }
+    // Cross-stream edge: wait for the producer. (Runs before the early-outs below so that a
+    // consumer never waits on an event that was not recorded in this invoke.)
+    if (n.producer >= 0 && k->nodes[n.producer].lane != n.lane) {
+      RETURN_IF_HIP(ctx, hipStreamWaitEvent(s, k->node_done[n.producer], 0));
     }
     struct SignalOnExit {
       PartitionKernel* k;

@@ -222,7 +222,8 @@ def test_int4_nodes_share_grouped_launches(streams, B):
         assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
         assert len(h.plan()) == 1
         groups, text = h.describe_partition(h.plan()[0][2])
-        assert groups == 2 and text.count("/g0") == 3 and text.count("/g1") == 3, text
+        # a, b, c, e, f have no producer inside the partition: one launch; d follows on its own
+        assert groups == 1 and text.count("/g0") == 5, text
 
         def ref(xin, c, n, bias=None):
             return oracle.fc_blockwise_int4(xin, c["packed"], n, c["scales"].view(np.uint16), 32, bias)
@@ -234,6 +235,47 @@ def test_int4_nodes_share_grouped_launches(streams, B):
             for y, want in ((yb, ref(xin, cs["b"], 40, bias_b)), (yc, ref(xin, cs["c"], 8)),
                             (yd, ref(wa, cs["d"], 16)), (ye, ref(cs["e"]["x"], cs["e"], 24)),
                             (yf, ref(cs["e"]["x"], cs["f"], 72))):
+                assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("streams", [1, 4])
+def test_int4_groups_follow_dependency_levels(streams):
+    """Plan order a, c(a), b, d(b), e(c): the launches are {a, b}, then {c, d}, then e --
+    grouping goes by distance from the partition's inputs, not by position in the plan."""
+    B, K = 2, 64
+    shapes = {"a": 64, "c": 64, "b": 64, "d": 24, "e": 8}
+    cs = {k: wl.blockwise_int4_fc(B, K, n, seed=40 + i, lo=-8, hi=7) for i, (k, n) in enumerate(shapes.items())}
+    with FakeHost() as h:
+        def int4(x, c, n):
+            w = h.tensor(INT4, (n, K), data=c["packed"], const=True)
+            s_ = h.tensor(FLOAT16, (n, K // 32), data=c["scales"], const=True)
+            h.blockwise(w, s_, 32)
+            y = h.tensor(FLOAT32, (B, n))
+            h.fc(x, w, None, y)
+            return y
+        x = h.tensor(FLOAT32, (B, K), data=cs["a"]["x"])
+        ya = int4(x, cs["a"], 64)
+        yc = int4(ya, cs["c"], 64)
+        yb = int4(x, cs["b"], 64)
+        yd = int4(yb, cs["d"], 24)
+        ye = int4(yc, cs["e"], 8)
+        assert h.load_delegate({"streams": streams}) == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert len(h.plan()) == 1
+        groups, text = h.describe_partition(h.plan()[0][2])
+        assert groups == 2 and text.count("/g0") == 2 and text.count("/g1") == 2, text
+
+        def ref(xin, c, n):
+            return oracle.fc_blockwise_int4(xin, c["packed"], n, c["scales"].view(np.uint16), 32)
+        rng = np.random.default_rng(4)
+        for trial in range(2):
+            xin = cs["a"]["x"] if trial == 0 else rng.standard_normal((B, K)).astype(np.float32)
+            h.write(x, xin)
+            assert h.invoke() == OK, h.errors()
+            wa, wb = ref(xin, cs["a"], 64), ref(xin, cs["b"], 64)
+            wc = ref(wa, cs["c"], 64)
+            # ya, yb, yc stay inside the partition (device arena); d and e are its outputs
+            for y, want in ((yd, ref(wb, cs["d"], 24)), (ye, ref(wc, cs["e"], 8))):
                 assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
 
 
