@@ -135,6 +135,45 @@ class FakeHost:
     def mark_output(self, tensor):
         self.L.fh_mark_graph_output(self.h, tensor)
 
+    def add_fc_nodes_of(self, subgraph, inputs=None):
+        """Builds the FULLY_CONNECTED nodes of a parsed `.tflite` subgraph
+        (litert_amd.tflite_file.SubGraph): their tensors with the quantization the runtime would
+        attach (interpreter_builder.cc:500-519 for blockwise, :521-600 for affine) and the nodes
+        with the file's options. `inputs` maps a model tensor index to the data it starts with.
+        Returns {model tensor index: host tensor index}."""
+        inputs = inputs or {}
+        made = {}
+
+        def make(ti):
+            if ti < 0 or ti in made:
+                return made.get(ti, -1)
+            t = subgraph.tensors[ti]
+            const = t.data is not None
+            data = t.data if const else inputs.get(ti)
+            nbytes = None
+            if data is None and t.type_name in ("INT4",):
+                nbytes = (int(np.prod(t.shape)) + 1) // 2
+            made[ti] = self.tensor(t.tflite_type, t.shape, data=data, const=const, nbytes=nbytes)
+            q = t.quantization
+            if q.kind == "affine":
+                self.affine(made[ti], q.scale, q.zero_point.astype(np.int32), q.quantized_dimension)
+            elif q.kind == "blockwise":
+                self.blockwise(made[ti], make(q.scales_tensor), q.block_size,
+                               make(q.zero_points_tensor))
+            return made[ti]
+
+        for op in subgraph.operators:
+            if op.fully_connected is None:
+                continue
+            o = op.fully_connected
+            ins = [make(i) for i in op.inputs]
+            out = make(op.outputs[0])
+            self.fc(ins[0], ins[1], ins[2] if len(ins) > 2 and ins[2] >= 0 else None, out,
+                    activation=o["activation"], keep_num_dims=o["keep_num_dims"],
+                    asymmetric=o["asymmetric_quantize_inputs"], weights_format=o["weights_format"],
+                    version=op.version, optional_bias_slot=len(ins) > 2)
+        return made
+
     # ---- delegate application --------------------------------------------------------------
     def load_delegate(self, options=None, path=DELEGATE_LIB):
         options = options or {}
