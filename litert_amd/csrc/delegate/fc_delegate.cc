@@ -44,10 +44,30 @@ struct Options {
   bool claim_int4_per_channel = true;
 };
 
+// Device memory the application registered for a tensor (litert_amd_register_device_buffer);
+// a TfLiteBufferHandle is an index into DelegateState::buffers. The memory stays the
+// application's: freeing a handle only empties its slot.
+struct RegisteredBuffer {
+  void* device = nullptr;
+  size_t bytes = 0;
+};
+
 struct DelegateState {
   Options options;
   TfLiteDelegate delegate;
+  std::vector<RegisteredBuffer> buffers;
 };
+
+// The registered memory behind a tensor that carries one of this delegate's handles, or
+// null: the tensor then lives in host memory as usual.
+const RegisteredBuffer* BoundBuffer(const DelegateState* state, const TfLiteTensor& t) {
+  if (t.delegate != &state->delegate || t.buffer_handle == kTfLiteNullBufferHandle) return nullptr;
+  if (t.buffer_handle < 0 || static_cast<size_t>(t.buffer_handle) >= state->buffers.size()) {
+    return nullptr;
+  }
+  const RegisteredBuffer& b = state->buffers[t.buffer_handle];
+  return b.device ? &b : nullptr;
+}
 
 enum class FcKind { kNone, kInt8, kHybrid, kInt4Blockwise, kHybridInt4 };
 
@@ -768,14 +788,30 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   auto* k = static_cast<PartitionKernel*>(node->user_data);
   RETURN_IF_HIP(ctx, hipSetDevice(k->state->options.device));
   // Tensor data pointers may move between invokes: read them from the context each time.
+  // An input that carries a buffer handle of this delegate is already in device memory: it is
+  // copied device to device behind the (single) host upload of the others.
+  bool host_inputs = false;
   for (int t : k->uploads) {
     const TfLiteTensor& tensor = ctx->tensors[t];
-    if (tensor.bytes == 0) continue;
+    if (tensor.bytes == 0 || BoundBuffer(k->state, tensor)) continue;
     std::memcpy(k->upload_stage.get() + k->arena_offset[t], tensor.data.raw, tensor.bytes);
+    host_inputs = true;
   }
-  if (k->upload_bytes > 0) {
+  if (host_inputs) {
     RETURN_IF_HIP(ctx, hipMemcpyAsync(k->arena.get(), k->upload_stage.get(), k->upload_bytes,
                                       hipMemcpyHostToDevice, k->stream));
+  }
+  for (int t : k->uploads) {
+    const TfLiteTensor& tensor = ctx->tensors[t];
+    const RegisteredBuffer* bound = tensor.bytes ? BoundBuffer(k->state, tensor) : nullptr;
+    if (!bound) continue;
+    if (bound->bytes < tensor.bytes) {
+      ctx->ReportError(ctx, "litert_amd delegate: buffer handle %d holds %zu bytes, tensor %d needs %zu",
+                       tensor.buffer_handle, bound->bytes, t, tensor.bytes);
+      return kTfLiteError;
+    }
+    RETURN_IF_HIP(ctx, hipMemcpyAsync(k->arena.as<uint8_t>() + k->arena_offset[t], bound->device,
+                                      tensor.bytes, hipMemcpyDeviceToDevice, k->stream));
   }
   bool multi = false;
   for (int i = 1; i < k->num_streams; ++i) multi = multi || k->lane_used[i];
@@ -927,16 +963,38 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     RETURN_IF_HIP(ctx, hipEventRecord(k->lane_done[i], k->streams[i]));
     RETURN_IF_HIP(ctx, hipStreamWaitEvent(s, k->lane_done[i], 0));
   }
-  if (k->download_bytes > 0) {
+  // An output that carries a buffer handle of this delegate stays in device memory: it goes
+  // to the registered buffer and the host copy is marked stale (the runtime fetches it
+  // through CopyFromBufferHandle if a CPU node or the application asks: subgraph.cc:876-889).
+  bool host_outputs = false;
+  for (int t : k->downloads) {
+    TfLiteTensor& tensor = ctx->tensors[t];
+    if (tensor.bytes == 0) continue;
+    const RegisteredBuffer* bound = BoundBuffer(k->state, tensor);
+    if (!bound) {
+      host_outputs = true;
+      continue;
+    }
+    if (bound->bytes < tensor.bytes) {
+      ctx->ReportError(ctx, "litert_amd delegate: buffer handle %d holds %zu bytes, tensor %d needs %zu",
+                       tensor.buffer_handle, bound->bytes, t, tensor.bytes);
+      return kTfLiteError;
+    }
+    RETURN_IF_HIP(ctx, hipMemcpyAsync(bound->device, k->arena.as<uint8_t>() + k->arena_offset[t],
+                                      tensor.bytes, hipMemcpyDeviceToDevice, s));
+    tensor.data_is_stale = true;
+  }
+  if (host_outputs) {
     RETURN_IF_HIP(ctx, hipMemcpyAsync(k->download_stage.get(),
                                       k->arena.as<uint8_t>() + k->download_offset,
                                       k->download_bytes, hipMemcpyDeviceToHost, s));
   }
-  // The runtime reads the outputs as soon as invoke returns.
+  // The runtime reads the outputs as soon as invoke returns; a consumer of a registered
+  // buffer (another partition, the application's own kernels) may start right away too.
   RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
   for (int t : k->downloads) {
     TfLiteTensor& tensor = ctx->tensors[t];
-    if (tensor.bytes == 0) continue;
+    if (tensor.bytes == 0 || BoundBuffer(k->state, tensor)) continue;
     std::memcpy(tensor.data.raw,
                 k->download_stage.get() + (k->arena_offset[t] - k->download_offset), tensor.bytes);
   }
@@ -988,6 +1046,54 @@ TfLiteStatus DelegatePrepare(TfLiteContext* ctx, TfLiteDelegate* delegate) {
       ctx->ReplaceNodeSubsetsWithDelegateKernels(ctx, KernelRegistration(), nodes, delegate);
   std::free(nodes);
   return st;
+}
+
+// ---- buffer handles (tflite/core/c/common.h:1458-1479) ---------------------------------
+
+TfLiteStatus CopyFromBufferHandle(TfLiteContext* ctx, TfLiteDelegate* delegate,
+                                  TfLiteBufferHandle handle, TfLiteTensor* tensor) {
+  auto* state = static_cast<DelegateState*>(delegate->data_);
+  if (handle < 0 || static_cast<size_t>(handle) >= state->buffers.size() ||
+      !state->buffers[handle].device || !tensor || !tensor->data.raw ||
+      state->buffers[handle].bytes < tensor->bytes) {
+    if (ctx && ctx->ReportError) {
+      ctx->ReportError(ctx, "litert_amd delegate: CopyFromBufferHandle: no buffer of %zu bytes behind handle %d",
+                       tensor ? tensor->bytes : size_t{0}, handle);
+    }
+    return kTfLiteError;
+  }
+  RETURN_IF_HIP(ctx, hipSetDevice(state->options.device));
+  RETURN_IF_HIP(ctx, hipMemcpy(tensor->data.raw, state->buffers[handle].device, tensor->bytes,
+                               hipMemcpyDeviceToHost));
+  return kTfLiteOk;
+}
+
+TfLiteStatus CopyToBufferHandle(TfLiteContext* ctx, TfLiteDelegate* delegate,
+                                TfLiteBufferHandle handle, TfLiteTensor* tensor) {
+  auto* state = static_cast<DelegateState*>(delegate->data_);
+  if (handle < 0 || static_cast<size_t>(handle) >= state->buffers.size() ||
+      !state->buffers[handle].device || !tensor || !tensor->data.raw ||
+      state->buffers[handle].bytes < tensor->bytes) {
+    if (ctx && ctx->ReportError) {
+      ctx->ReportError(ctx, "litert_amd delegate: CopyToBufferHandle: no buffer of %zu bytes behind handle %d",
+                       tensor ? tensor->bytes : size_t{0}, handle);
+    }
+    return kTfLiteError;
+  }
+  RETURN_IF_HIP(ctx, hipSetDevice(state->options.device));
+  RETURN_IF_HIP(ctx, hipMemcpy(state->buffers[handle].device, tensor->data.raw, tensor->bytes,
+                               hipMemcpyHostToDevice));
+  return kTfLiteOk;
+}
+
+// Frees the handle, not the memory behind it (common.h:1473-1479).
+void FreeBufferHandle(TfLiteContext*, TfLiteDelegate* delegate, TfLiteBufferHandle* handle) {
+  auto* state = static_cast<DelegateState*>(delegate->data_);
+  if (!handle) return;
+  if (*handle >= 0 && static_cast<size_t>(*handle) < state->buffers.size()) {
+    state->buffers[*handle] = RegisteredBuffer{};
+  }
+  *handle = kTfLiteNullBufferHandle;
 }
 
 bool ParseOptions(const char* const* keys, const char* const* values, size_t n, Options* opt,
@@ -1066,9 +1172,9 @@ TfLiteDelegate* tflite_plugin_create_delegate(const char* const* options_keys,
   state->delegate = TfLiteDelegate{};
   state->delegate.data_ = state.get();
   state->delegate.Prepare = DelegatePrepare;
-  state->delegate.CopyFromBufferHandle = nullptr;
-  state->delegate.CopyToBufferHandle = nullptr;
-  state->delegate.FreeBufferHandle = nullptr;
+  state->delegate.CopyFromBufferHandle = CopyFromBufferHandle;
+  state->delegate.CopyToBufferHandle = CopyToBufferHandle;
+  state->delegate.FreeBufferHandle = FreeBufferHandle;
   state->delegate.flags = kTfLiteDelegateFlagsNone;  // static shapes; re-prepared after a resize
   state->delegate.opaque_delegate_builder = nullptr;
   return &state.release()->delegate;
@@ -1077,6 +1183,27 @@ TfLiteDelegate* tflite_plugin_create_delegate(const char* const* options_keys,
 void tflite_plugin_destroy_delegate(TfLiteDelegate* delegate) {
   if (!delegate) return;
   delete static_cast<DelegateState*>(delegate->data_);
+}
+
+// Registers device memory (a hipMalloc'ed range of `bytes` bytes on the delegate's device)
+// and returns the buffer handle for it, or kTfLiteNullBufferHandle. The application then binds
+// it to an input or output tensor with Interpreter::SetBufferHandle (subgraph.h:1043-1057):
+// a bound input is read from that memory, a bound output is left there with data_is_stale
+// set. Counterpart of StatefulNnApiDelegate::RegisterNnapiMemory
+// (tflite/delegates/nnapi/nnapi_delegate.cc:6645-6660), free slots reused the same way.
+TfLiteBufferHandle litert_amd_register_device_buffer(TfLiteDelegate* delegate, void* device_memory,
+                                                     size_t bytes) {
+  if (!delegate || !delegate->data_ || !device_memory || bytes == 0) return kTfLiteNullBufferHandle;
+  auto* state = static_cast<DelegateState*>(delegate->data_);
+  if (&state->delegate != delegate) return kTfLiteNullBufferHandle;
+  for (size_t i = 0; i < state->buffers.size(); ++i) {
+    if (!state->buffers[i].device) {
+      state->buffers[i] = RegisteredBuffer{device_memory, bytes};
+      return static_cast<TfLiteBufferHandle>(i);
+    }
+  }
+  state->buffers.push_back(RegisteredBuffer{device_memory, bytes});
+  return static_cast<TfLiteBufferHandle>(state->buffers.size() - 1);
 }
 
 // Test and tooling hook: the claim predicate on its own (no device needed). Returns

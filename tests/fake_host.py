@@ -64,6 +64,13 @@ def lib():
         L.fh_errors.restype = C.c_char_p
         L.fh_clear_errors.argtypes = [C.c_void_p]
         L.fh_classify.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_char_p, C.c_size_t]
+        L.fh_set_buffer_handle.argtypes = [C.c_void_p, C.c_int, C.c_int]
+        L.fh_set_data_is_stale.argtypes = [C.c_void_p, C.c_int, C.c_int]
+        for name in ("fh_data_is_stale", "fh_buffer_handle", "fh_ensure_tensor_data_is_readable",
+                     "fh_copy_to_buffer_handle"):
+            getattr(L, name).argtypes = [C.c_void_p, C.c_int]
+        L.fh_delegate.argtypes = [C.c_void_p]
+        L.fh_delegate.restype = C.c_void_p
         _lib = L
     return _lib
 
@@ -173,6 +180,32 @@ class FakeHost:
                     asymmetric=o["asymmetric_quantize_inputs"], weights_format=o["weights_format"],
                     version=op.version, optional_bias_slot=len(ins) > 2)
         return made
+
+    # ---- buffer handles (Interpreter::SetBufferHandle, EnsureTensorDataIsReadable) -----------
+    def register_device_buffer(self, device_ptr, nbytes, path=DELEGATE_LIB):
+        """litert_amd_register_device_buffer on the loaded delegate; returns the handle."""
+        d = C.CDLL(path)
+        d.litert_amd_register_device_buffer.restype = C.c_int
+        d.litert_amd_register_device_buffer.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        return d.litert_amd_register_device_buffer(self.L.fh_delegate(self.h), device_ptr, nbytes)
+
+    def set_buffer_handle(self, tensor, handle):
+        return self.L.fh_set_buffer_handle(self.h, tensor, handle)
+
+    def buffer_handle(self, tensor):
+        return self.L.fh_buffer_handle(self.h, tensor)
+
+    def set_data_is_stale(self, tensor, stale=True):
+        self.L.fh_set_data_is_stale(self.h, tensor, int(stale))
+
+    def data_is_stale(self, tensor):
+        return bool(self.L.fh_data_is_stale(self.h, tensor))
+
+    def ensure_readable(self, tensor):
+        return self.L.fh_ensure_tensor_data_is_readable(self.h, tensor)
+
+    def copy_to_buffer_handle(self, tensor):
+        return self.L.fh_copy_to_buffer_handle(self.h, tensor)
 
     # ---- delegate application --------------------------------------------------------------
     def load_delegate(self, options=None, path=DELEGATE_LIB):

@@ -185,6 +185,22 @@ TfLiteStatus CtxReplaceNodeSubsets(TfLiteContext* ctx, TfLiteRegistration regist
 }
 
 
+// Subgraph::EnsureTensorDataIsReadable (tflite/core/subgraph.cc:876-889).
+TfLiteStatus EnsureReadable(Host* h, int tensor_index) {
+  TfLiteTensor* t = &h->tensors[tensor_index];
+  TfLiteStatus status = kTfLiteOk;
+  if (t->data_is_stale) {
+    if (!t->delegate || t->buffer_handle == kTfLiteNullBufferHandle ||
+        !t->delegate->CopyFromBufferHandle) {
+      h->errors += "stale tensor without a delegate buffer handle\n";
+      return kTfLiteError;
+    }
+    status = t->delegate->CopyFromBufferHandle(&h->ctx, t->delegate, t->buffer_handle, t);
+    t->data_is_stale = false;
+  }
+  return status;
+}
+
 void FreeDelegateKernels(Host* h) {
   for (auto& n : h->nodes) {
     if (n->is_delegate_kernel && n->initialised && n->reg.free) {
@@ -212,6 +228,11 @@ void* fh_create() {
 void fh_destroy(void* hp) {
   auto* h = static_cast<Host*>(hp);
   FreeDelegateKernels(h);
+  for (auto& t : h->tensors) {  // Subgraph::~Subgraph (subgraph.cc:310-316)
+    if (t.buffer_handle != kTfLiteNullBufferHandle && t.delegate && t.delegate->FreeBufferHandle) {
+      t.delegate->FreeBufferHandle(&h->ctx, t.delegate, &t.buffer_handle);
+    }
+  }
   if (h->delegate && h->destroy) h->destroy(h->delegate);
   for (auto& t : h->tensors) std::free(t.dims);
   for (auto& a : h->affine) {
@@ -374,6 +395,15 @@ int fh_invoke(void* hp) {
   auto* h = static_cast<Host*>(hp);
   for (int n : h->plan) {
     NodeRec& rec = *h->nodes[n];
+    // Inputs another party left in its own memory are fetched first (subgraph.cc:1724-1734).
+    for (int i = 0; i < rec.node.inputs->size; ++i) {
+      const int t = rec.node.inputs->data[i];
+      if (t == kTfLiteOptionalTensor) continue;
+      TfLiteTensor& tensor = h->tensors[t];
+      if (tensor.delegate && tensor.delegate != rec.node.delegate && tensor.data_is_stale) {
+        if (EnsureReadable(h, t) != kTfLiteOk) return kTfLiteError;
+      }
+    }
     if (rec.is_delegate_kernel) {
       const TfLiteStatus st = rec.reg.invoke(&h->ctx, &rec.node);
       if (st != kTfLiteOk) return st;
@@ -386,6 +416,37 @@ int fh_invoke(void* hp) {
     }
   }
   return kTfLiteOk;
+}
+
+// Interpreter::SetBufferHandle with the loaded delegate (subgraph.cc:2784-2800).
+int fh_set_buffer_handle(void* hp, int tensor, int handle) {
+  auto* h = static_cast<Host*>(hp);
+  TfLiteTensor& t = h->tensors[tensor];
+  if (!h->delegate || (t.delegate && t.delegate != h->delegate)) return kTfLiteError;
+  t.delegate = h->delegate;
+  if (t.buffer_handle != kTfLiteNullBufferHandle && h->delegate->FreeBufferHandle) {
+    h->delegate->FreeBufferHandle(&h->ctx, h->delegate, &t.buffer_handle);
+  }
+  t.buffer_handle = handle;
+  return kTfLiteOk;
+}
+void fh_set_data_is_stale(void* hp, int tensor, int stale) {
+  static_cast<Host*>(hp)->tensors[tensor].data_is_stale = stale != 0;
+}
+int fh_data_is_stale(void* hp, int tensor) {
+  return static_cast<Host*>(hp)->tensors[tensor].data_is_stale ? 1 : 0;
+}
+int fh_buffer_handle(void* hp, int tensor) { return static_cast<Host*>(hp)->tensors[tensor].buffer_handle; }
+int fh_ensure_tensor_data_is_readable(void* hp, int tensor) {
+  return EnsureReadable(static_cast<Host*>(hp), tensor);
+}
+void* fh_delegate(void* hp) { return static_cast<Host*>(hp)->delegate; }
+// TfLiteDelegate::CopyToBufferHandle on the tensor's own handle.
+int fh_copy_to_buffer_handle(void* hp, int tensor) {
+  auto* h = static_cast<Host*>(hp);
+  TfLiteTensor& t = h->tensors[tensor];
+  if (!t.delegate || !t.delegate->CopyToBufferHandle) return kTfLiteError;
+  return t.delegate->CopyToBufferHandle(&h->ctx, t.delegate, t.buffer_handle, &t);
 }
 
 void* fh_tensor_data(void* hp, int tensor) { return static_cast<Host*>(hp)->tensors[tensor].data.raw; }

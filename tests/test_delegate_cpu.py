@@ -13,8 +13,12 @@ from tests.fake_host import FakeHost, FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4
 def test_plugin_exports_entry_points():
     lib = C.CDLL(fhm.DELEGATE_LIB)
     for name in ("tflite_plugin_create_delegate", "tflite_plugin_destroy_delegate",
-                 "litert_amd_classify_node"):
+                 "litert_amd_classify_node", "litert_amd_describe_partition",
+                 "litert_amd_register_device_buffer", "LiteRtAcceleratorImpl"):
         assert hasattr(lib, name)
+    # no delegate, no handle (kTfLiteNullBufferHandle)
+    lib.litert_amd_register_device_buffer.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+    assert lib.litert_amd_register_device_buffer(None, None, 16) == -1
 
 
 def _int8_node(h, B=2, K=32, N=8, per_channel=True, filter_type=INT8, in_type=INT8, out_type=INT8,
