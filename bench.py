@@ -328,6 +328,38 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         out["config4_int8_gemm_2048x4096x4096_" + act] = dict(
             us=round(us, 2), tops=round(tops, 1),
             frac_of_int8_mfma_peak=round(tops / INT8_MFMA_PEAK_TOPS, 4))
+    # The same launch on constant operands (every x = 3, every w = 5). The kernel executes the same
+    # instructions in the same number of cycles; only the switching activity differs. The gap
+    # to the seeded U[-128,127] operands above is the clock the part sustains under that
+    # activity (power limit), not something the kernel's schedule can win back.
+    op4c = fc.FullyConnectedInt8(np.full_like(c4["w"], 5), c4["bias"], float(c4["in_scale"]),
+                                 c4["in_zp"], c4["w_scale"], float(c4["out_scale"]), c4["out_zp"])
+    x4c = torch.full_like(x4, 3)
+    us_c = per_launch_us([lambda: op4c(x4c, out=y4)] * 4)
+    out["config4_int8_gemm_constant_operands"] = dict(
+        us=round(us_c, 2), tops=round(ops_per_call / us_c / 1e6, 1),
+        frac_of_int8_mfma_peak=round(ops_per_call / us_c / 1e6 / INT8_MFMA_PEAK_TOPS, 4),
+        note="same kernel and launch, x = 3 and w = 5 everywhere: lower switching activity, higher sustained clock")
+    # Yardstick (not this library): the vendor int8 GEMM through torch._int_mm on the same
+    # operands, int32 output, no requantization.
+    try:
+        wt = dev(c4["w"]).t()
+        for _ in range(5):
+            torch._int_mm(x4, wt)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(50):
+            torch._int_mm(x4, wt)   # launched eagerly (the library may allocate a workspace)
+        e1.record()
+        torch.cuda.synchronize()
+        us_lib = e0.elapsed_time(e1) * 1e3 / 50
+        out["config4_yardstick_torch_int_mm"] = dict(
+            us=round(us_lib, 2), tops=round(ops_per_call / us_lib / 1e6, 1),
+            note="hipBLASLt via torch._int_mm(x[2048,4096], w^T): int32 out, no epilogue")
+    except Exception as e:  # a torch build without _int_mm on this device
+        out["config4_yardstick_torch_int_mm"] = dict(error=repr(e)[:120])
+    del op4c, x4c
 
     # config 5: FC chain of a Gemma-2B-shaped 18-layer decoder, blockwise int4, B = 1 and 4.
     # Each node gets its own seeded N(0,1) input (FC-only chain: outputs are discarded).
