@@ -82,6 +82,9 @@ def lib():
         L.orc_fc_hybrid.argtypes = [_f32p, C.c_int, C.c_int, _i8p, C.c_int, _f32p, C.c_float,
                                     _f32p, C.c_int, C.c_int, C.c_int, _f32p, _i8p, _f32p, _i32p]
         L.orc_fc_hybrid_cached.argtypes = L.orc_fc_hybrid.argtypes + [_i32p, C.c_int]
+        L.orc_matrix_batch_vector_multiply_accumulate_sse.argtypes = [
+            _i8p, C.c_int, C.c_int, _i8p, _f32p, C.c_int, _f32p, _f32p, _i32p, _i32p]
+        L.orc_matrix_batch_vector_multiply_accumulate_sse.restype = None
         L.orc_fc_blockwise_int4.argtypes = [_f32p, C.c_int, C.c_int, _u8p, C.c_int, _u16p,
                                             C.c_int, _f32p, C.c_int, _f32p]
         L.orc_fc_hybrid_int4_per_channel.argtypes = [_f32p, C.c_int, C.c_int, _u8p, C.c_int, _f32p,
@@ -263,6 +266,43 @@ def matrix_batch_vector_multiply_accumulate(matrix, vectors, scaling_factors, re
         _p(m, _i8p), rows, cols, _p(v, _i8p), _p(sf, _f32p), n_batch, _p(res, _f32p),
         _p(pcs, _f32p), _p(off, _i32p), _p(row_sums, _i32p), 1)
     return res
+
+
+def have_sse():
+    return bool(lib().orc_have_sse())
+
+
+def matrix_batch_vector_multiply_accumulate_sse(matrix, vectors, scaling_factors, result,
+                                                per_channel_scale=None, input_offset=None,
+                                                row_sums=None):
+    """The optimized-x86 tier (sse_tensor_utils.cc:308-379); row_sums are computed here when an
+    input_offset is given and none are passed (the op caches them after its first Eval)."""
+    m = _c(matrix, np.int8)
+    v = _c(vectors, np.int8)
+    rows, cols = m.shape
+    n_batch = v.size // cols
+    sf = _c(scaling_factors, np.float32)
+    res = np.array(result, dtype=np.float32).reshape(n_batch, rows).copy()
+    pcs = _c(per_channel_scale, np.float32)
+    off = _c(input_offset, np.int32)
+    if off is not None and row_sums is None:
+        row_sums = m.astype(np.int32).sum(1).astype(np.int32)
+    rs = _c(row_sums, np.int32)
+    lib().orc_matrix_batch_vector_multiply_accumulate_sse(
+        _p(m, _i8p), rows, cols, _p(v, _i8p), _p(sf, _f32p), n_batch, _p(res, _f32p),
+        _p(pcs, _f32p), _p(off, _i32p), _p(rs, _i32p))
+    return res
+
+
+def fc_hybrid_sse(x, w, per_channel_scales, row_sums, asymmetric=True, variant=QUANT_PORTABLE):
+    """EvalHybridDense with the optimized-x86 product (no bias, no activation: the form the CPU
+    baseline times): BatchQuantizeFloats, then the SSE kernel on a zeroed output."""
+    x = _c(x, np.float32)
+    w = _c(w, np.int8)
+    q, sf, zp = batch_quantize_floats(x.reshape(-1, w.shape[1]), asymmetric, variant)
+    out = np.zeros((q.shape[0], w.shape[0]), np.float32)
+    return matrix_batch_vector_multiply_accumulate_sse(
+        w, q, sf, out, per_channel_scales, zp if asymmetric else None, row_sums)
 
 
 def fc_hybrid(x, w, per_channel_scales=None, filter_scale=1.0, bias=None, asymmetric=True,

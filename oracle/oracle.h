@@ -141,6 +141,16 @@ void orc_batch_quantize_floats(const float* values, int n_batch, int n_data, int
 
 /* ---- hybrid (float activations, int8 weights) -------------------------- */
 
+/* The same product as the reference's optimized x86 build computes it
+ * (optimized/sse_tensor_utils.cc:308-379, SSE branch), in oracle_sse.cc; row_sums must be
+ * filled when input_offset is given. orc_have_sse() is 0 on other hosts (the function is
+ * then a no-op). */
+int orc_have_sse(void);
+void orc_matrix_batch_vector_multiply_accumulate_sse(
+    const int8_t* matrix, int m_rows, int m_cols, const int8_t* vectors,
+    const float* scaling_factors, int n_batch, float* result, const float* per_channel_scale,
+    const int32_t* input_offset, const int32_t* row_sums);
+
 /* reference/portable_tensor_utils.cc:165-206 (+ :140-163 when input_offset is
  * NULL). row_sums is recomputed when compute_row_sums is non-zero. */
 void orc_matrix_batch_vector_multiply_accumulate(const int8_t* matrix, int m_rows, int m_cols,

@@ -282,12 +282,59 @@ def _mv_data(rows, cols, batch, negative=False, per_channel=False, init_to_one=F
     return matrix, vectors.astype(np.int8), scale_factors, results, pcs, offs
 
 
+DOT_KERNELS = {"portable": oracle.matrix_batch_vector_multiply_accumulate,
+               "sse": oracle.matrix_batch_vector_multiply_accumulate_sse}
+_dot_kernel = "portable"
+
+
+@pytest.fixture(params=sorted(DOT_KERNELS))
+def dot_kernel(request):
+    """The reference runs these vectors against every build of the kernel (portable, NEON, SSE:
+    tensor_utils_test.cc is linked against each); so do the two tiers restated here."""
+    global _dot_kernel
+    if request.param == "sse" and not oracle.have_sse():
+        pytest.skip("not an x86 host")
+    _dot_kernel = request.param
+    yield request.param
+    _dot_kernel = "portable"
+
+
 def _dot(rows, cols, batch, negative=False, init_to_one=False, per_channel=False):
     m, v, sf, res, pcs, offs = _mv_data(rows, cols, batch, negative, per_channel, init_to_one)
-    return oracle.matrix_batch_vector_multiply_accumulate(m, v, sf, res, pcs, offs).ravel()
+    return DOT_KERNELS[_dot_kernel](m, v, sf, res, pcs, offs).ravel()
 
 
-def test_hybrid_dot_kat():
+def test_sse_dot_is_bit_identical_to_portable():
+    """The optimized-x86 tier of the CPU baseline (oracle_sse.cc) against the portable kernel on
+    ragged depths (vector body, 16-byte step, scalar tail), with and without input offsets,
+    activations over the whole int8 range, weights over [-127, 127] (the range symmetric weight
+    quantization produces; at -128 the kernel's sign transfer wraps, in the reference too)."""
+    if not oracle.have_sse():
+        pytest.skip("not an x86 host")
+    rng = np.random.default_rng(12)
+    for rows, cols, batch in ((3, 1, 1), (5, 15, 2), (4, 16, 1), (7, 31, 3), (2, 33, 1), (9, 100, 2),
+                              (6, 4096, 2)):
+        m = rng.integers(-127, 128, (rows, cols)).astype(np.int8)
+        v = rng.integers(-128, 128, (batch, cols)).astype(np.int8)
+        sf = rng.uniform(0.01, 0.1, batch).astype(np.float32)
+        pcs = rng.uniform(1e-3, 1e-2, rows).astype(np.float32)
+        res = rng.standard_normal((batch, rows)).astype(np.float32)
+        offsets = rng.integers(-128, 128, batch).astype(np.int32)
+        # the portable kernel's short form (no offsets) has no per-channel scale, so that
+        # pairing is not a call the op makes
+        for use_pcs, offs in ((None, None), (None, offsets), (pcs, offsets)):
+            a = oracle.matrix_batch_vector_multiply_accumulate(m, v, sf, res, use_pcs, offs)
+            b = oracle.matrix_batch_vector_multiply_accumulate_sse(m, v, sf, res, use_pcs, offs)
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (rows, cols, batch)
+    x = rng.standard_normal((3, 200)).astype(np.float32)
+    w = rng.integers(-127, 128, (11, 200)).astype(np.int8)
+    pcs = rng.uniform(1e-3, 1e-2, 11).astype(np.float32)
+    for asym in (True, False):
+        assert np.array_equal(oracle.fc_hybrid(x, w, pcs, asymmetric=asym).view(np.uint32),
+                              oracle.fc_hybrid_sse(x, w, pcs, None, asymmetric=asym).view(np.uint32))
+
+
+def test_hybrid_dot_kat(dot_kernel):
     assert _dot(4, 16, 1).tolist() == [1240, 3160, 5080, 7000]
     assert _dot(4, 32, 2).tolist() == [10416, 26288, 8490, 23312, 18276, 70756, 37416, 60916]
     r = _dot(32, 512, 5)
@@ -299,7 +346,7 @@ def test_hybrid_dot_kat():
     assert _dot(4, 32, 2, True, True).tolist() == [3437, 3523, 1591, 6973, 2517, 20521, 457, 10629]
 
 
-def test_hybrid_dot_per_channel_kat():
+def test_hybrid_dot_per_channel_kat(dot_kernel):
     assert _dot(4, 16, 1, per_channel=True).tolist() == [620, 3160, 2540, 7000]
     assert _dot(4, 32, 2, per_channel=True).tolist() == [5208, 26288, 4245, 23312, 9138, 70756,
                                                          18708, 60916]
