@@ -5,6 +5,9 @@
 #include <cstdio>
 #include <cstring>
 #include <limits>
+#include <map>
+#include <mutex>
+#include <utility>
 
 #include "kernels.h"
 
@@ -70,6 +73,26 @@ Workspace SplitWorkspace(void* base, int batches, int depth) {
 }
 
 }  // namespace
+
+namespace lrtfc {
+hipError_t EnsureDynamicLds(const void* kernel, size_t bytes) {
+  if (bytes <= 48 * 1024) return hipSuccess;
+  int device = 0;
+  if (hipError_t err = hipGetDevice(&device)) return err;
+  static std::mutex mu;
+  static std::map<std::pair<const void*, int>, size_t> granted;
+  std::lock_guard<std::mutex> lock(mu);
+  size_t& have = granted[std::make_pair(kernel, device)];
+  if (bytes > have) {
+    if (hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(bytes))) {
+      return err;
+    }
+    have = bytes;
+  }
+  return hipSuccess;
+}
+}  // namespace lrtfc
 
 extern "C" {
 

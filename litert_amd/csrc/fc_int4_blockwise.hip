@@ -205,16 +205,7 @@ hipError_t LaunchVariant(const FcInt4Args& a, int batch0, hipStream_t stream) {
   const size_t lds_bytes = static_cast<size_t>(BT) * a.depth +
                            static_cast<size_t>(R) * BT * (nblk | 1) * sizeof(float);
   auto kernel = FcBlockwiseInt4Kernel<R, BT, WC>;
-  if (lds_bytes > 48 * 1024) {
-    static size_t granted = 0;  // per instantiation
-    if (lds_bytes > granted) {
-      hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(lds_bytes));
-      if (err != hipSuccess) return err;
-      granted = lds_bytes;
-    }
-  }
+  if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds_bytes)) return err;
   const int grid = (a.out_depth + R - 1) / R;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds_bytes, stream, a, batch0);
   return hipGetLastError();

@@ -623,16 +623,7 @@ hipError_t LaunchOne(const Int4PackedArgs& a, int batch0, int bt, hipStream_t st
   const int ksplit = ChooseKsplit(a.out_depth, a.chunks);
   const size_t lds = Int4Shared<BT>::Bytes(padded, ksplit);
   auto kernel = FcInt4PackedKernel<BT, FUSED, VARIANT, GPT>;
-  if (lds > 48 * 1024) {
-    static size_t granted = 0;
-    if (lds > granted) {
-      hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(lds));
-      if (err != hipSuccess) return err;
-      granted = lds;
-    }
-  }
+  if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   const int groups = (a.out_depth + kTileRows - 1) / kTileRows;
   const int gpw = ChooseGroupsPerWave(groups, a.chunks, ksplit);
   const int groups_per_wg = kWaves / ksplit * gpw;
@@ -800,16 +791,7 @@ hipError_t LaunchGroupedOne(const void* table, const lrtfc_int4_group_launch& l,
   const int padded = chunks * kTileBlocks * kBlock;
   const size_t lds = Int4Shared<BT>::Bytes(padded, l.ksplit);
   auto kernel = FcInt4PackedGroupedKernel<BT, VARIANT, GPT>;
-  if (lds > 48 * 1024) {
-    static size_t granted = 0;
-    if (lds > granted) {
-      hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(lds));
-      if (err != hipSuccess) return err;
-      granted = lds;
-    }
-  }
+  if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   hipLaunchKernelGGL(kernel, dim3(l.grid_blocks), dim3(kThreads), lds, stream,
                      static_cast<const Int4GroupTable*>(table), l.count, batch0, bt, l.ksplit,
                      l.groups_per_wave);

@@ -434,16 +434,7 @@ hipError_t LaunchSized(const PackedArgs& p, int batch0, int bt, hipStream_t stre
   const int qstride = p.slabs * kSlabDepth + kQPad;
   const size_t lds = SharedBytes(bt, qstride);
   auto kernel = FcInt8PackedGemvKernel<EPI, FUSED, VARIANT, REG_ROWS>;
-  if (lds > 48 * 1024) {
-    static size_t granted = 0;
-    if (lds > granted) {
-      hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(lds));
-      if (err != hipSuccess) return err;
-      granted = lds;
-    }
-  }
+  if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
   // One wavefront per channel group when that already gives the chip ~2 wavefronts per
   // SIMD-pair; otherwise split the depth so that short filters still spread out.

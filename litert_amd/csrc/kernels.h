@@ -11,6 +11,12 @@
 
 namespace lrtfc {
 
+// Raises a kernel's dynamic-LDS limit when a launch needs more than the default 48 KiB. The
+// attribute belongs to the (kernel, device) pair, so what has been granted is remembered per
+// pair (defined in capi.hip; safe to call from several threads).
+hipError_t EnsureDynamicLds(const void* kernel, size_t bytes);
+
+
 // Arguments of the int8-weight kernels (full-integer and hybrid epilogues).
 struct FcInt8Args {
   const int8_t* input;   // [batches, depth] int8 (quantized activations)
