@@ -314,6 +314,25 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         kernel="FcInt4PackedKernel<fused quantize> on the re-tiled filter")
     del ops3
 
+    # Next-row op (not a BASELINE configuration): per-channel int4 hybrid FC (EvalHybridDense4Bit)
+    # at config 3's shape, B = 1, on the 4-bit-resident filter and on its int8 expansion.
+    g4 = torch.Generator(device="cuda").manual_seed(11)
+    nib = [torch.randint(0, 256, (14336, 2048), dtype=torch.uint8, device="cuda", generator=g4)
+           for _ in range(6)]
+    fs4 = np.random.default_rng(3).uniform(0.01, 0.1, 14336).astype(np.float32)
+    ops4b = [fc.FullyConnectedHybridInt4PerChannel(n, 4096, fs4) for n in nib]
+    y4b = torch.empty((1, 14336), dtype=torch.float32, device="cuda")
+    us_nib = per_launch_us([(lambda o: lambda: o(x3, out=y4b))(o) for o in ops4b])
+    us_i8 = per_launch_us([(lambda o: lambda: o(x3, out=y4b, force_int8=True))(o) for o in ops4b])
+    bytes_nib = 14336 * 2048 + 14336 * 4 + 4096 * 4 + 14336 * 4
+    out["next_int4_per_channel_hybrid_14336x4096_B1"] = dict(
+        us_cold_4bit_resident=round(us_nib, 3), us_cold_int8_expansion=round(us_i8, 3),
+        gbps_cold=round(bytes_nib / us_nib / 1e3, 1),
+        frac_of_hbm_peak_cold=round(bytes_nib / us_nib / 1e3 / HBM_PEAK_GBPS, 4),
+        algorithmic_bytes=bytes_nib,
+        note="two launches each (row quantizer + GEMV); per launch pair")
+    del ops4b, nib
+
     # config 4: prefill int8 GEMM 2048 x 4096 x 4096, RELU6 off / on
     c4 = wl.prefill_int8_fc()
     x4 = dev(c4["x"])

@@ -278,6 +278,22 @@ int lrtfc_fc_hybrid_int4_per_channel_packed(const float* input, const int8_t* pa
                                             void* workspace, size_t workspace_bytes,
                                             void* stream);
 
+/* The same op on a filter that stays 4 bits per weight in device memory (half the bytes to
+ * stream per decode step): lrtfc_pack_int4_per_channel re-tiles the model's nibble-packed rows
+ * ([out_depth, depth / 2] bytes, low nibble first; even depth) into
+ * lrtfc_packed_int4_per_channel_bytes(out_depth, depth) bytes, 16-byte aligned. Meant for
+ * decode batches (it makes one pass over the filter per 16 rows); prefill batches are faster on
+ * the int8 copy above. Results are identical bit for bit. */
+size_t lrtfc_packed_int4_per_channel_bytes(int out_depth, int depth);
+int lrtfc_pack_int4_per_channel(const uint8_t* packed_filter, int out_depth, int depth,
+                                uint8_t* retiled_filter, void* stream);
+int lrtfc_fc_hybrid_int4_per_channel_nibbles(const float* input, const uint8_t* retiled_filter,
+                                             const float* per_channel_scales, float filter_scale,
+                                             const float* bias, float* output, int batches,
+                                             int depth, int out_depth, int activation,
+                                             void* workspace, size_t workspace_bytes,
+                                             void* stream);
+
 /* ---- Several blockwise-int4 nodes in one launch ----------------------------------------
  * Nodes of a graph that do not depend on each other (the q/k/v or the gate/up projections of
  * a decoder layer) and share depth and batch count can run as ONE kernel: the gaps between

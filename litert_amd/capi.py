@@ -58,6 +58,10 @@ SYMBOLS = [
     ("lrtfc_batch_quantize_floats_4bit", _i, [_vp, _i, _i, _vp, _vp, _vp, _vp]),
     ("lrtfc_fc_hybrid_int4_per_channel_packed", _i, [_vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i,
                                                      _vp, _sz, _vp]),
+    ("lrtfc_packed_int4_per_channel_bytes", _sz, [_i, _i]),
+    ("lrtfc_pack_int4_per_channel", _i, [_vp, _i, _i, _vp, _vp]),
+    ("lrtfc_fc_hybrid_int4_per_channel_nibbles", _i, [_vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i,
+                                                      _vp, _sz, _vp]),
     ("lrtfc_int4_group_table_bytes", _sz, []),
     ("lrtfc_int4_group_prepare", _i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_fc_blockwise_int4_packed_grouped", _i, [_vp, _vp, _i, _vp]),

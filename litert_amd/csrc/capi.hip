@@ -704,6 +704,63 @@ int lrtfc_fc_hybrid_int4_per_channel_packed(const float* input, const int8_t* pa
                  "packed int4 per-channel hybrid GEMV");
 }
 
+size_t lrtfc_packed_int4_per_channel_bytes(int out_depth, int depth) {
+  if (out_depth <= 0 || depth <= 0) return 0;
+  return lrtfc::PackedInt4PerChannelBytes(out_depth, depth);
+}
+
+int lrtfc_pack_int4_per_channel(const uint8_t* packed_filter, int out_depth, int depth,
+                                uint8_t* retiled_filter, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(out_depth >= 0 && depth >= 0, "bad dimension");
+  if (out_depth == 0 || depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(depth % 2 == 0, "depth %d is odd: rows of nibbles must end on a byte", depth);
+  LRTFC_REQUIRE(packed_filter && retiled_filter, "null pointer");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(retiled_filter) & 15) == 0,
+                "re-tiled filter must be 16-byte aligned");
+  return FromHip(lrtfc::LaunchPackInt4PerChannel(packed_filter, out_depth, depth, retiled_filter,
+                                                 AsStream(stream)),
+                 "per-channel int4 filter re-tiling");
+}
+
+int lrtfc_fc_hybrid_int4_per_channel_nibbles(const float* input, const uint8_t* retiled_filter,
+                                             const float* per_channel_scales, float filter_scale,
+                                             const float* bias, float* output, int batches,
+                                             int depth, int out_depth, int activation,
+                                             void* workspace, size_t workspace_bytes,
+                                             void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(input && retiled_filter && output && workspace, "null pointer");
+  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  LRTFC_REQUIRE(lrtfc::FcInt4PerChannelGemvSupports(depth),
+                "depth %d is odd or too large for the nibble GEMV", depth);
+  LRTFC_REQUIRE(workspace_bytes >= WorkspaceBytes(batches, depth),
+                "workspace too small: %zu < %zu bytes", workspace_bytes,
+                WorkspaceBytes(batches, depth));
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
+                "workspace must be 256-byte aligned");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(retiled_filter) & 15) == 0,
+                "re-tiled filter must be 16-byte aligned");
+  if (lrtfc::FcInt4PerChannelGemvFuses(input, batches, depth)) {  // one kernel, no workspace use
+    return FromHip(lrtfc::LaunchFcInt4PerChannelGemv(retiled_filter, input, nullptr, nullptr,
+                                                     nullptr, per_channel_scales, filter_scale,
+                                                     bias, output, batches, depth, out_depth,
+                                                     activation, AsStream(stream)),
+                   "per-channel int4 hybrid GEMV (nibble layout, fused quantizer)");
+  }
+  const Workspace w = SplitWorkspace(workspace, batches, depth);
+  int rc = lrtfc_batch_quantize_floats_4bit(input, batches, depth, w.q, w.sf, w.zp, stream);
+  if (rc != LRTFC_OK) return rc;
+  return FromHip(lrtfc::LaunchFcInt4PerChannelGemv(retiled_filter, nullptr, w.q, w.sf, w.zp,
+                                                   per_channel_scales, filter_scale, bias, output,
+                                                   batches, depth, out_depth, activation,
+                                                   AsStream(stream)),
+                 "per-channel int4 hybrid GEMV (nibble layout)");
+}
+
 size_t lrtfc_int4_group_table_bytes(void) { return lrtfc::Int4GroupTableBytes(); }
 
 int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,

@@ -286,6 +286,9 @@ struct FcNode {
   // The filter lives on the device in the layout the node's shape runs fastest on: the
   // model's own (row-major / nibble-packed rows) or the re-tiled copy. Only one is kept.
   bool have_model_layout = false, have_retiled = false, use_retiled = false;
+  // Per-channel int4 hybrid nodes keep the filter at 4 bits per weight for decode batches
+  // (retiled_dev then holds nibble tiles) and as re-tiled int8 for prefill batches.
+  bool nibble_layout = false, have_nibbles = false;
   bool split_quantize = false;  // quantize rows in a launch of their own, not in the prologue
   // Scheduling inside the partition: the stream the node runs on, the node that produces its
   // input (-1: the input is uploaded from the host), and whether a node on another stream
@@ -304,6 +307,9 @@ struct FcNode {
 constexpr int kHybridFusedMaxBatches = 4;
 constexpr int kInt4FusedMaxDepth = 4096;
 constexpr int kInt4DeepFusedMaxBatches = 2;
+// Up to this many rows a per-channel int4 node streams its filter as nibbles (one pass per 16
+// rows); above, the MFMA GEMM on the int8 expansion streams it once.
+constexpr int kInt4PerChannelNibbleMaxBatches = 32;
 
 struct PartitionKernel {
   DelegateState* state = nullptr;
@@ -507,7 +513,9 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
     return kTfLiteError;
   }
   hipStream_t s = k->stream;
-  if (n->uploaded_filter != filter.data.raw) n->have_model_layout = n->have_retiled = false;
+  if (n->uploaded_filter != filter.data.raw) {
+    n->have_model_layout = n->have_retiled = n->have_nibbles = false;
+  }
   const size_t weights = static_cast<size_t>(n->out_depth) * n->depth;
 
   if (n->kind == FcKind::kInt8) {
@@ -585,14 +593,28 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
     n->per_channel = fq->scale->size > 1;
     n->filter_scale = fq->scale->data[0];
     n->use_retiled = true;
-    if (weights > 0 && !n->have_retiled) {
+    n->nibble_layout = n->batches <= kInt4PerChannelNibbleMaxBatches;
+    if (weights > 0 && !(n->nibble_layout ? n->have_nibbles : n->have_retiled)) {
       DeviceBuffer nibbles;
       RETURN_IF_HIP(ctx, nibbles.Upload(filter.data.raw, (weights + 1) / 2, s));
-      RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
-      RETURN_IF_FC(ctx, lrtfc_unpack_int4(nibbles.as<uint8_t>(), static_cast<int64_t>(weights),
-                                          n->filter_dev.as<int8_t>(), s));
-      RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
-      RETURN_IF_OK(RetileInt8(ctx, n, s));
+      if (n->nibble_layout) {
+        n->retiled_dev.Release();
+        RETURN_IF_HIP(ctx, n->retiled_dev.Ensure(
+                               lrtfc_packed_int4_per_channel_bytes(n->out_depth, n->depth)));
+        RETURN_IF_FC(ctx, lrtfc_pack_int4_per_channel(nibbles.as<uint8_t>(), n->out_depth, n->depth,
+                                                      n->retiled_dev.as<uint8_t>(), s));
+        RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+        n->have_nibbles = true;
+        n->have_retiled = false;
+      } else {
+        RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
+        RETURN_IF_FC(ctx, lrtfc_unpack_int4(nibbles.as<uint8_t>(), static_cast<int64_t>(weights),
+                                            n->filter_dev.as<int8_t>(), s));
+        RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+        n->retiled_dev.Release();
+        RETURN_IF_OK(RetileInt8(ctx, n, s));
+        n->have_nibbles = false;
+      }
     }
     if (n->per_channel) {
       RETURN_IF_HIP(ctx, n->pcs_dev.Upload(fq->scale->data, static_cast<size_t>(n->out_depth) * 4, s));
@@ -921,6 +943,14 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
         break;
       }
       case FcKind::kHybridInt4:
+        if (n.nibble_layout) {
+          RETURN_IF_FC(ctx, lrtfc_fc_hybrid_int4_per_channel_nibbles(
+                                static_cast<const float*>(in_dev), n.retiled_dev.as<uint8_t>(),
+                                n.per_channel ? n.pcs_dev.as<float>() : nullptr, n.filter_scale,
+                                bias_f32, static_cast<float*>(out_dev), n.batches, n.depth,
+                                n.out_depth, n.params.activation, scratch.get(), scratch.bytes(), s));
+          break;
+        }
         RETURN_IF_FC(ctx, lrtfc_fc_hybrid_int4_per_channel_packed(
                               static_cast<const float*>(in_dev), n.retiled_dev.as<int8_t>(),
                               n.per_channel ? n.pcs_dev.as<float>() : nullptr, n.filter_scale,

@@ -74,6 +74,23 @@ hipError_t LaunchFcInt8PackedGemv(const FcInt8Args& a, Int8Epilogue epilogue,
                                   const float* input_f32, int asymmetric, int variant,
                                   hipStream_t stream);
 
+// Per-channel int4 hybrid GEMV on the filter kept at 4 bits per weight (tile16x128n, made by
+// LaunchPackInt4PerChannel from the model's nibble-packed rows); rows quantized by
+// LaunchBatchQuantize4Bit. Any batch count (tiles of 16 rows), any out_depth, even depth.
+size_t PackedInt4PerChannelBytes(int out_depth, int depth);
+hipError_t LaunchPackInt4PerChannel(const uint8_t* filter, int out_depth, int depth,
+                                    uint8_t* packed, hipStream_t stream);
+bool FcInt4PerChannelGemvSupports(int depth);
+// input_f32 != nullptr: the fused form (row quantizer in the prologue; only where
+// FcInt4PerChannelGemvFuses says so), quantized_input / scaling_factors / input_offsets unused.
+bool FcInt4PerChannelGemvFuses(const float* input_f32, int batches, int depth);
+hipError_t LaunchFcInt4PerChannelGemv(const uint8_t* packed, const float* input_f32,
+                                      const int8_t* quantized_input,
+                                      const float* scaling_factors, const int32_t* input_offsets,
+                                      const float* per_channel_scales, float filter_scale,
+                                      const float* bias, float* output, int batches, int depth,
+                                      int out_depth, int activation, hipStream_t stream);
+
 // Prefill batches on the same re-tiled filter: int8 MFMA GEMM (a.filter = packed, a.input =
 // int8 rows; the hybrid epilogue reads a.scaling_factors / a.zero_points). Any batch count,
 // any out_depth; depth a multiple of 16.

@@ -361,10 +361,11 @@ class FullyConnectedHybridInt4PerChannel:
         self.depth = int(depth)
         if self.depth % 2:
             raise ValueError("the 4-bit path needs an even depth")
-        unpacked = torch.empty((self.out_depth, self.depth), dtype=torch.int8, device="cuda")
-        capi.check(lib.lrtfc_unpack_int4(_ptr(nibbles), self.out_depth * self.depth,
-                                         _ptr(unpacked), _stream()))
-        self.packed_filter = _pack_int8(unpacked)
+        # Two device layouts, each made on first use: the nibbles re-tiled (decode batches: half
+        # the bytes to stream) and the int8 expansion re-tiled (prefill batches: the MFMA GEMM).
+        self._nibbles = nibbles
+        self._retiled_nibbles = None
+        self._packed_int8 = None
         fs = np.atleast_1d(np.asarray(filter_scales, dtype=np.float32))
         self.pcs = _dev(fs, torch.float32) if fs.size > 1 else None
         self.filter_scale = float(fs[0])
@@ -372,7 +373,9 @@ class FullyConnectedHybridInt4PerChannel:
         self.activation = _act(activation)
         self._ws = None
 
-    def __call__(self, x, out=None):
+    NIBBLE_MAX_BATCHES = 32  # above: one pass of the MFMA GEMM over the int8 copy is cheaper
+
+    def __call__(self, x, out=None, force_int8=False):
         x = x.contiguous()
         batches = x.numel() // self.depth
         if out is None:
@@ -380,8 +383,27 @@ class FullyConnectedHybridInt4PerChannel:
         need = capi.load().lrtfc_activation_workspace_bytes(batches, self.depth)
         if self._ws is None or self._ws.numel() < need:
             self._ws = torch.empty(need, dtype=torch.uint8, device="cuda")
-        capi.check(capi.load().lrtfc_fc_hybrid_int4_per_channel_packed(
-            _ptr(x), _ptr(self.packed_filter), _ptr(self.pcs), self.filter_scale, _ptr(self.bias),
+        lib = capi.load()
+        if batches <= self.NIBBLE_MAX_BATCHES and not force_int8:
+            if self._retiled_nibbles is None:
+                self._retiled_nibbles = torch.empty(
+                    lib.lrtfc_packed_int4_per_channel_bytes(self.out_depth, self.depth),
+                    dtype=torch.uint8, device="cuda")
+                capi.check(lib.lrtfc_pack_int4_per_channel(
+                    _ptr(self._nibbles), self.out_depth, self.depth, _ptr(self._retiled_nibbles),
+                    _stream()))
+            capi.check(lib.lrtfc_fc_hybrid_int4_per_channel_nibbles(
+                _ptr(x), _ptr(self._retiled_nibbles), _ptr(self.pcs), self.filter_scale,
+                _ptr(self.bias), _ptr(out), batches, self.depth, self.out_depth, self.activation,
+                _ptr(self._ws), self._ws.numel(), _stream()))
+            return out
+        if self._packed_int8 is None:
+            unpacked = torch.empty((self.out_depth, self.depth), dtype=torch.int8, device="cuda")
+            capi.check(lib.lrtfc_unpack_int4(_ptr(self._nibbles), self.out_depth * self.depth,
+                                             _ptr(unpacked), _stream()))
+            self._packed_int8 = _pack_int8(unpacked)
+        capi.check(lib.lrtfc_fc_hybrid_int4_per_channel_packed(
+            _ptr(x), _ptr(self._packed_int8), _ptr(self.pcs), self.filter_scale, _ptr(self.bias),
             _ptr(out), batches, self.depth, self.out_depth, self.activation, _ptr(self._ws),
             self._ws.numel(), _stream()))
         return out

@@ -306,6 +306,34 @@ def test_int4_per_channel_hybrid_node_through_delegate(B, per_channel):
         assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
 
 
+def test_int4_per_channel_node_switches_layout_with_the_batch():
+    """Decode batches run on the filter kept as nibbles, prefill batches on its int8 expansion;
+    a resize moves the node from one to the other and back (prepare runs after every resize)."""
+    from tests import kat_harness as kh
+    rng = np.random.default_rng(21)
+    K, N = 512, 40
+    x_all = rng.standard_normal((48, K)).astype(np.float32)
+    w_np = rng.integers(-7, 8, (N, K)).astype(np.int8)
+    packed = np.stack([kh.pack_int4(r) for r in w_np])
+    fs = rng.uniform(0.01, 0.1, N).astype(np.float32)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (1, K), data=x_all[:1])
+        w = h.tensor(INT4, (N, K), data=packed, const=True)
+        h.affine(w, fs)
+        y = h.tensor(FLOAT32, (1, N))
+        h.fc(x, w, None, y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        for rows in (1, 48, 3, 20):
+            h.resize(x, (rows, K))
+            h.resize(y, (rows, N))
+            h.write(x, x_all[:rows])
+            assert h.allocate_tensors() == OK, h.errors()
+            assert h.invoke() == OK, h.errors()
+            want = oracle.fc_hybrid_int4_per_channel(x_all[:rows], packed, N, fs, None, 0)
+            assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32)), rows
+
+
 def test_streams_option_is_validated():
     with FakeHost() as h:
         assert h.load_delegate({"streams": 9}) != 0

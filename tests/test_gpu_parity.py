@@ -535,6 +535,27 @@ def test_hybrid_int4_per_channel_matches_oracle(fc, B, K, N, activation):
     y = op(_cuda(x)).cpu().numpy()
     want = oracle.fc_hybrid_int4_per_channel(x, packed, N, fs, bias, fc._act(activation))
     assert _bits_equal(y, want)
+    # both device layouts (nibbles for decode batches, int8 expansion for prefill) agree
+    assert _bits_equal(op(_cuda(x), force_int8=True).cpu().numpy(), want)
+
+
+def test_hybrid_int4_per_channel_nibble_layout_shapes(fc):
+    """The 4-bit-resident GEMV on its own entry point: a depth split over several wavefronts
+    (few channels, deep rows), 17..32 rows (two passes over the filter), a depth that is not a
+    multiple of 16 or 128, one filter scale for every channel."""
+    from tests import kat_harness as kh
+    rng = np.random.default_rng(99)
+    for B, K, N, per_channel in ((1, 8192, 24, True), (20, 640, 40, True), (32, 1024, 16, False),
+                                 (3, 34, 5, True), (2, 130, 9, False), (5, 16384, 8, True)):
+        x = rng.standard_normal((B, K)).astype(np.float32)
+        w = rng.integers(-7, 8, (N, K)).astype(np.int8)
+        packed = np.stack([kh.pack_int4(r) for r in w])
+        fs = rng.uniform(0.01, 0.1, N).astype(np.float32) if per_channel else np.array([0.03], np.float32)
+        op = fc.FullyConnectedHybridInt4PerChannel(packed, K, fs)
+        y = op(_cuda(x)).cpu().numpy()
+        assert op._retiled_nibbles is not None and op._packed_int8 is None
+        want = oracle.fc_hybrid_int4_per_channel(x, packed, N, np.broadcast_to(fs, (N,)).copy(), None, 0)
+        assert _bits_equal(y, want), (B, K, N)
 
 
 def test_hybrid_int4_per_channel_reference_kat_and_scalar_scale(fc):
