@@ -176,18 +176,24 @@ __global__ __launch_bounds__(kThreads) void FcInt4PerChannelGemvKernel(NibbleArg
     }
   }
 
+  // Per-channel epilogue inputs of this lane's four channels: requested after the activation
+  // rows and BEFORE the weights (behind the ring they would count as newer loads in the tile
+  // loop's first round and make the first MFMA wait for the whole ring). Unconditional loads: an
+  // absent array reads a valid dummy address and is ignored.
+  float ep_scale[4], ep_bias[4];
+  {
+    const float* dummy = reinterpret_cast<const float*>(a.packed);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = min(min(tile, tiles - 1) * kTileRows + 4 * kgroup + i, a.out_depth - 1);
+      ep_scale[i] = *(a.per_channel_scales ? a.per_channel_scales + n : dummy);
+      ep_bias[i] = *(a.bias ? a.bias + n : dummy);
+    }
+  }
   i32x4 ring[kRing];
 #pragma unroll
   for (int u = 0; u < kRing; ++u) {
     ring[u] = __builtin_nontemporal_load(wbase + static_cast<size_t>(min(s0 + u, slabs - 1)) * 64);
-  }
-  // Per-channel epilogue inputs of this lane's four channels, behind the ring.
-  float ep_scale[4], ep_bias[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int n = min(min(tile, tiles - 1) * kTileRows + 4 * kgroup + i, a.out_depth - 1);
-    ep_scale[i] = a.per_channel_scales ? a.per_channel_scales[n] : a.filter_scale;
-    ep_bias[i] = a.bias ? a.bias[n] : 0.0f;
   }
   if (FUSED) {
 #pragma unroll
@@ -324,7 +330,8 @@ __global__ __launch_bounds__(kThreads) void FcInt4PerChannelGemvKernel(NibbleArg
     if (n >= a.out_depth) continue;
     const int32_t dot = acc[i] - 8 * sum_q;  // sum(w * q) from sum((w + 8) * q)
     a.output[static_cast<size_t>(b) * a.out_depth + n] = Hybrid4BitCore(
-        dot, batch_scale, ep_scale[i], input_offset, ep_bias[i], a.bias != nullptr, a.activation);
+        dot, batch_scale, a.per_channel_scales ? ep_scale[i] : a.filter_scale, input_offset,
+        a.bias ? ep_bias[i] : 0.0f, a.bias != nullptr, a.activation);
   }
 }
 

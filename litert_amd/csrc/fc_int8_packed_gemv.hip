@@ -209,6 +209,37 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
     }
   }
 
+  // Per-channel epilogue parameters of this lane's four channels, requested here: after the
+  // activation rows (which the prologue waits for) and BEFORE the weights. Vector memory
+  // returns in issue order and the tile loop waits with a fixed count of newer loads allowed
+  // in flight; parameters requested behind the ring count as newer loads in the first round
+  // and make the first MFMA wait for the whole ring instead of its first tile (measured:
+  // 0.3-0.4 us per launch). Every load is unconditional -- an absent array reads a valid dummy
+  // address and is ignored -- so that the number of loads in flight does not depend on the
+  // path taken. (Scalar loads for these -- the 16 channels are uniform across the wavefront --
+  // were measured slower: dozens of serialized scalar-cache round trips in the prologue.)
+  // Loaded raw; combined in the epilogue.
+  int32_t ep_i0[4], ep_i1[4], ep_i2[4], ep_i3[4];  // requantize: multiplier, shift, bias, row sum
+  float ep_f0[4], ep_f1[4];                         // hybrid: channel scale, bias (+ ep_i0 row sum)
+  {
+    const int32_t* dummy_i = reinterpret_cast<const int32_t*>(a.filter);
+    const float* dummy_f = reinterpret_cast<const float*>(a.filter);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = min(min(tile, tiles - 1) * kTileRows + 4 * kgroup + i, a.out_depth - 1);
+      if (EPI == Int8Epilogue::kRequantize) {
+        ep_i0[i] = a.multipliers[a.per_channel ? n : 0];
+        ep_i1[i] = a.shifts[a.per_channel ? n : 0];
+        ep_i2[i] = *(a.bias_i32 ? a.bias_i32 + n : dummy_i);
+        ep_i3[i] = *(a.filter_row_sums ? a.filter_row_sums + n : dummy_i);
+      } else {
+        ep_i0[i] = *(a.filter_row_sums ? a.filter_row_sums + n : dummy_i);
+        ep_f0[i] = *(a.per_channel_scales ? a.per_channel_scales + n : dummy_f);
+        ep_f1[i] = *(a.bias_f32 ? a.bias_f32 + n : dummy_f);
+      }
+    }
+  }
+
   // 1. Fill the first half of the ring (branch-free; a share shorter than the ring re-reads
   // its last tile). Issuing loads blocks while the memory pipeline is full -- which it is from
   // the first microsecond on -- so the second half is issued after the prologue's arithmetic
@@ -339,27 +370,6 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
   for (int u = kRing / 2; u < kRing; ++u) {
     ring[u] = __builtin_nontemporal_load(wbase + static_cast<size_t>(min(s0 + u, slabs - 1)) * 64);
   }
-  // Per-channel epilogue parameters of this lane's four channels: requested right behind
-  // the ring of weights (they return in order, long before the last tile is consumed)
-  // so that no latency is left for the epilogue to wait for.
-  // Loaded raw: combining them here would wait for memory before the weights are requested.
-  int32_t ep_i0[4], ep_i1[4], ep_i2[4], ep_i3[4];  // requantize: multiplier, shift, bias, row sum
-  float ep_f0[4], ep_f1[4];                         // hybrid: channel scale, bias (+ ep_i0 row sum)
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int n = min(min(tile, tiles - 1) * kTileRows + 4 * kgroup + i, a.out_depth - 1);
-    if (EPI == Int8Epilogue::kRequantize) {
-      ep_i0[i] = a.per_channel ? a.multipliers[n] : a.multipliers[0];
-      ep_i1[i] = a.per_channel ? a.shifts[n] : a.shifts[0];
-      ep_i2[i] = a.bias_i32 ? a.bias_i32[n] : 0;
-      ep_i3[i] = a.input_offset != 0 ? a.filter_row_sums[n] : 0;
-    } else {
-      ep_i0[i] = a.filter_row_sums ? a.filter_row_sums[n] : 0;
-      ep_f0[i] = a.per_channel_scales ? a.per_channel_scales[n] : a.filter_scale;
-      ep_f1[i] = a.bias_f32 ? a.bias_f32[n] : 0.0f;
-    }
-  }
-
 
   // 3. Matrix-core loop. B operand: lane L supplies batch column (L % 16), the same 16
   // depth positions as its weight bytes. Columns past the tile read row 0; their
@@ -413,17 +423,22 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
     const int n = tile * kTileRows + 4 * kgroup + i;
     if (n >= a.out_depth) continue;
     if (EPI == Int8Epilogue::kRequantize) {
+      const int32_t bias = a.bias_i32 ? ep_i2[i] : 0;
+      const int32_t row_sum = a.filter_row_sums ? ep_i3[i] : 0;  // input_offset != 0 needs them
       a.output_i8[static_cast<size_t>(b) * a.out_depth + n] =
-          RequantizeCore(acc[i] + ep_i2[i] + a.input_offset * ep_i3[i], ep_i0[i], ep_i1[i],
+          RequantizeCore(acc[i] + bias + a.input_offset * row_sum, ep_i0[i], ep_i1[i],
                          a.output_offset, a.act_min, a.act_max);
     } else {
       const float batch_scale = FUSED ? sh.sf[col] : a.scaling_factors[b];
       const int32_t batch_zp = FUSED ? sh.zp[col] : (a.zero_points ? a.zero_points[b] : 0);
+      const float channel_scale = a.per_channel_scales ? ep_f0[i] : a.filter_scale;
+      const float bias = a.bias_f32 ? ep_f1[i] : 0.0f;
+      const int32_t row_sum = a.filter_row_sums ? ep_i0[i] : 0;
       a.output_f32[static_cast<size_t>(b) * a.out_depth + n] =
           EPI == Int8Epilogue::kHybrid4Bit
-              ? Hybrid4BitCore(acc[i], batch_scale, ep_f0[i], batch_zp, ep_f1[i],
+              ? Hybrid4BitCore(acc[i], batch_scale, channel_scale, batch_zp, bias,
                                a.bias_f32 != nullptr, a.activation)
-              : HybridCore(acc[i], batch_scale, ep_f0[i], batch_zp, ep_i0[i], ep_f1[i],
+              : HybridCore(acc[i], batch_scale, channel_scale, batch_zp, row_sum, bias,
                            a.activation);
     }
   }
