@@ -56,6 +56,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-extras", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--traffic-probe-int4", action="store_true",
+                    help="launch only what the int4 grouped kernel's counter runs need, then exit")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch only the dominant kernel (cold, 12 times) and a 64 MiB device "
                          "copy (3 times), for a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run")
@@ -82,6 +84,9 @@ def main():
 
     if args.traffic_probe:
         traffic_probe(torch, fc, wl)
+        return
+    if args.traffic_probe_int4:
+        traffic_probe_int4(torch, fc, wl)
         return
 
     def timed_replays(graphs, reps):
@@ -253,6 +258,34 @@ def traffic_probe(torch, fc, wl):
     torch.cuda.synchronize()
     print(json.dumps({"probe": "traffic", "hybrid_launches": 12, "copy_launches": 3,
                       "copy_bytes": 64 << 20, "algorithmic_bytes": hybrid_bytes(1)}))
+
+
+def traffic_probe_int4(torch, fc, wl):
+    """Counter-run launches for the grouped int4 kernel: config 5's 108 nodes of depth 2048 in
+    ONE launch (B = 1), four times, plus the 64 MiB copy that calibrates the counters."""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    ops, total = [], 0
+    for _ in range(wl.GEMMA2B_LAYERS):
+        for name, k, n in wl.GEMMA2B_LAYER_FCS:
+            if k != 2048:
+                continue
+            packed = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda", generator=g)
+            scales = (torch.rand((n, k // 32), device="cuda", generator=g) * 1.5e-2 + 5e-3).half()
+            ops.append(fc.FullyConnectedBlockwiseInt4(packed, scales, k, 32))
+            total += int4_bytes(1, n, k)
+    x = torch.randn((1, 2048), device="cuda", generator=g)
+    ys = [torch.empty((1, op.out_depth), dtype=torch.float32, device="cuda") for op in ops]
+    group = fc.GroupedBlockwiseInt4(ops).bind([x] * len(ops), ys)
+    src = torch.ones(64 << 20, dtype=torch.int8, device="cuda")
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(4):
+        group()
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": "traffic-int4", "grouped_launches": 4, "nodes": len(ops),
+                      "copy_launches": 3, "copy_bytes": 64 << 20, "algorithmic_bytes": total}))
 
 
 def measured_traffic():
