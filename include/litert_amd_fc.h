@@ -335,6 +335,37 @@ int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
                                       int batches, int depth, int out_depth, int blocksize,
                                       void* stream);
 
+/* ---- EMBEDDING_LOOKUP from quantized tables (the op that feeds a decoder's first
+ * FULLY_CONNECTED nodes) ------------------------------------------------------------------ */
+
+/* Output element types of the lookups below. */
+#define LRTFC_OUT_FLOAT32 0
+#define LRTFC_OUT_FLOAT16 1
+
+/* Blockwise Int4 table -> float rows. Replaces EvalBlockwise,
+ * tflite/kernels/embedding_lookup.cc:194-307 with Unpack4Bit :140-159: output[i, c] =
+ * float((int8)(nibble << 4)) * (scale[lookup[i], c / blocksize] / 16), converted to binary16 for
+ * LRTFC_OUT_FLOAT16. table: rows x cols/2 bytes, low nibble = even column; scales_f16:
+ * [rows, cols / blocksize] IEEE binary16; lookup: [count] int32; output: [count, cols].
+ * cols must be a multiple of blocksize (:269-275) and both even (the reference reads rows from
+ * byte boundaries). status: device int32[2] or NULL; every call rewrites it as {0, -1}, or
+ * {1, p} when lookup[p] is the first index outside [0, rows) -- where the reference fails the
+ * invoke (:280-286); rows with such an index are left unwritten. All pointers are device
+ * pointers; the call only enqueues work on `stream`. */
+int lrtfc_embedding_lookup_blockwise_int4(const int32_t* lookup, int count, const uint8_t* table,
+                                          int rows, int cols, const uint16_t* scales_f16,
+                                          int blocksize, int out_type, void* output,
+                                          int32_t* status, void* stream);
+
+/* Int8 (value_bits 8) or Int4 (4) table with one scale, or one per row when row_scales is not
+ * NULL -> float rows. Replaces EvalHybrid, tflite/kernels/embedding_lookup.cc:309-395:
+ * output[i, c] = float(value) * scale for Int8 and Unpack4Bit's arithmetic for Int4 (cols even).
+ * status as above (:365-371). */
+int lrtfc_embedding_lookup_hybrid(const int32_t* lookup, int count, const void* table,
+                                  int value_bits, int rows, int cols, float scale,
+                                  const float* row_scales, int out_type, void* output,
+                                  int32_t* status, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

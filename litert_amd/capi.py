@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "liblitert_amd_fc.so")
 OK, INVALID_ARGUMENT, NO_DEVICE, HIP_ERROR, UNSUPPORTED = range(5)
 ACT_NONE, ACT_RELU, ACT_RELU_N1_TO_1, ACT_RELU6 = range(4)
 QUANT_PORTABLE, QUANT_NEON_V8, QUANT_NEON_LEGACY = range(3)
+OUT_FLOAT32, OUT_FLOAT16 = range(2)
 
 # Every symbol include/litert_amd_fc.h declares: (name, restype, argtypes).
 _vp, _i, _i32, _i64, _f, _d, _sz = (C.c_void_p, C.c_int, C.c_int32, C.c_int64, C.c_float,
@@ -62,6 +63,8 @@ SYMBOLS = [
     ("lrtfc_pack_int4_per_channel", _i, [_vp, _i, _i, _vp, _vp]),
     ("lrtfc_fc_hybrid_int4_per_channel_nibbles", _i, [_vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i,
                                                       _vp, _sz, _vp]),
+    ("lrtfc_embedding_lookup_blockwise_int4", _i, [_vp, _i, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp]),
+    ("lrtfc_embedding_lookup_hybrid", _i, [_vp, _i, _vp, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp]),
     ("lrtfc_int4_group_table_bytes", _sz, []),
     ("lrtfc_int4_group_prepare", _i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_fc_blockwise_int4_packed_grouped", _i, [_vp, _vp, _i, _vp]),

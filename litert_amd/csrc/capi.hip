@@ -761,6 +761,54 @@ int lrtfc_fc_hybrid_int4_per_channel_nibbles(const float* input, const uint8_t* 
                  "per-channel int4 hybrid GEMV (nibble layout)");
 }
 
+int lrtfc_embedding_lookup_blockwise_int4(const int32_t* lookup, int count, const uint8_t* table,
+                                          int rows, int cols, const uint16_t* scales_f16,
+                                          int blocksize, int out_type, void* output,
+                                          int32_t* status, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(count >= 0 && rows >= 0 && cols >= 0, "bad dimension");
+  LRTFC_REQUIRE(out_type == LRTFC_OUT_FLOAT32 || out_type == LRTFC_OUT_FLOAT16,
+                "output type %d is neither float32 nor float16", out_type);
+  LRTFC_REQUIRE(blocksize > 0 && cols % blocksize == 0,
+                "lookup dimension %d must be divisible by blocksize %d", cols, blocksize);
+  LRTFC_REQUIRE(cols % 2 == 0 && blocksize % 2 == 0,
+                "Int4 rows and blocks must hold an even number of columns");
+  if (count > 0 && cols > 0) {
+    LRTFC_REQUIRE(lookup && table && scales_f16 && output, "null pointer");
+  } else {
+    LRTFC_REQUIRE(count == 0 || lookup, "null pointer");
+  }
+  return FromHip(lrtfc::LaunchEmbeddingLookup(lookup, count, table, 4, rows, cols, scales_f16,
+                                              blocksize, nullptr, 0.0f,
+                                              out_type == LRTFC_OUT_FLOAT16, output, status,
+                                              AsStream(stream)),
+                 "blockwise int4 embedding lookup");
+}
+
+int lrtfc_embedding_lookup_hybrid(const int32_t* lookup, int count, const void* table,
+                                  int value_bits, int rows, int cols, float scale,
+                                  const float* row_scales, int out_type, void* output,
+                                  int32_t* status, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(count >= 0 && rows >= 0 && cols >= 0, "bad dimension");
+  LRTFC_REQUIRE(value_bits == 4 || value_bits == 8, "value_bits %d is neither 4 nor 8",
+                value_bits);
+  LRTFC_REQUIRE(out_type == LRTFC_OUT_FLOAT32 || out_type == LRTFC_OUT_FLOAT16,
+                "output type %d is neither float32 nor float16", out_type);
+  LRTFC_REQUIRE(value_bits == 8 || cols % 2 == 0,
+                "Int4 rows must hold an even number of columns");
+  if (count > 0 && cols > 0) {
+    LRTFC_REQUIRE(lookup && table && output, "null pointer");
+  } else {
+    LRTFC_REQUIRE(count == 0 || lookup, "null pointer");
+  }
+  return FromHip(lrtfc::LaunchEmbeddingLookup(lookup, count, table, value_bits, rows, cols,
+                                              nullptr, 0, row_scales, scale,
+                                              out_type == LRTFC_OUT_FLOAT16, output, status,
+                                              AsStream(stream)),
+                 "hybrid embedding lookup");
+}
+
 size_t lrtfc_int4_group_table_bytes(void) { return lrtfc::Int4GroupTableBytes(); }
 
 int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,

@@ -364,3 +364,62 @@ def fc_hybrid_int4_per_channel(x, packed_w, out_depth, filter_scales, bias=None,
                                          _p(fs, _f32p), _p(bias, _f32p), activation,
                                          _p(y, _f32p))
     return y
+
+
+# ---- EMBEDDING_LOOKUP from quantized tables ------------------------------------
+
+class LookupOutOfBounds(ValueError):
+    """A lookup index outside [0, rows); `position` is its place in the lookup vector."""
+
+    def __init__(self, position):
+        super().__init__(f"lookup {position} out of bounds")
+        self.position = position
+
+
+def float_to_half_bits(values):
+    v = _c(values, np.float32).ravel()
+    L = lib()
+    L.orc_float_to_half.argtypes = [C.c_float]
+    L.orc_float_to_half.restype = C.c_uint16
+    return np.array([L.orc_float_to_half(float(f)) for f in v], dtype=np.uint16)
+
+
+def _lookup_output(count, cols, out_f16):
+    return np.zeros((count, cols), dtype=np.uint16 if out_f16 else np.float32)
+
+
+def embedding_lookup_blockwise_int4(lookup, packed_table, rows, cols, scales_f16_bits, blocksize,
+                                    out_f16=False):
+    """EvalBlockwise: packed_table [rows, cols/2] nibbles (low = even column), scales
+    [rows, cols/blocksize] as binary16 bit patterns. Returns float32 [count, cols], or binary16
+    bit patterns (uint16) when out_f16."""
+    lk = _c(lookup, np.int32).ravel()
+    tb = _c(packed_table, np.uint8).ravel()
+    sc = _c(scales_f16_bits, np.uint16).ravel()
+    y = _lookup_output(lk.size, cols, out_f16)
+    rc = lib().orc_embedding_lookup_blockwise_int4(
+        _p(lk, _i32p), lk.size, _p(tb, _u8p), rows, cols, _p(sc, _u16p), blocksize, int(out_f16),
+        y.ctypes.data_as(C.c_void_p))
+    if rc < 0:
+        raise LookupOutOfBounds(-rc - 1)
+    if rc:
+        raise ValueError("columns not divisible by the block size")
+    return y
+
+
+def embedding_lookup_hybrid(lookup, table, value_bits, rows, cols, scale=1.0, row_scales=None,
+                            out_f16=False):
+    """EvalHybrid: table int8 [rows, cols] (value_bits 8) or nibbles [rows*cols/2] (4)."""
+    lk = _c(lookup, np.int32).ravel()
+    tb = np.ascontiguousarray(table).view(np.uint8).ravel()
+    rs = _c(row_scales, np.float32)
+    y = _lookup_output(lk.size, cols, out_f16)
+    L = lib()
+    L.orc_embedding_lookup_hybrid.argtypes = [_i32p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                              C.c_float, _f32p, C.c_int, C.c_void_p]
+    rc = L.orc_embedding_lookup_hybrid(_p(lk, _i32p), lk.size, tb.ctypes.data_as(C.c_void_p),
+                                       value_bits, rows, cols, float(scale), _p(rs, _f32p),
+                                       int(out_f16), y.ctypes.data_as(C.c_void_p))
+    if rc < 0:
+        raise LookupOutOfBounds(-rc - 1)
+    return y

@@ -662,4 +662,116 @@ void orc_fc_hybrid_int4_per_channel(const float* input, int batches, int depth,
   orc_apply_activation(output, static_cast<int64_t>(batches) * out_depth, activation);
 }
 
+// IEEE binary32 -> binary16, round to nearest even, subnormals kept, overflow to infinity: what
+// `tflite::half(float)` does in either of its builds (tflite/types/half.h:69 through _Float16,
+// :129 through fp16_ieee_from_fp32_value).
+uint16_t orc_float_to_half(float f) {
+  uint32_t bits;
+  std::memcpy(&bits, &f, sizeof bits);
+  const uint16_t sign = static_cast<uint16_t>((bits >> 16) & 0x8000u);
+  const uint32_t abs = bits & 0x7FFFFFFFu;
+  if (abs >= 0x7F800000u) {  // inf / NaN (quiet, payload top bits kept)
+    return static_cast<uint16_t>(sign | 0x7C00u | (abs > 0x7F800000u ? 0x200u | ((abs >> 13) & 0x3FFu) : 0));
+  }
+  if (abs >= 0x477FF000u) return static_cast<uint16_t>(sign | 0x7C00u);  // rounds to >= 65520
+  const int exp = static_cast<int>(abs >> 23) - 127;
+  if (exp >= -14) {  // normal half
+    const uint32_t man = abs & 0x7FFFFFu;
+    uint32_t h = (static_cast<uint32_t>(exp + 15) << 10) | (man >> 13);
+    const uint32_t rem = man & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h;  // carry may bump the exponent
+    return static_cast<uint16_t>(sign | h);
+  }
+  if (exp < -25) return sign;  // below half of the smallest subnormal
+  // subnormal half: value = man24 * 2^(exp-23), unit 2^-24
+  const uint32_t man24 = (abs & 0x7FFFFFu) | 0x800000u;
+  const int shift = -exp - 1;  // 14..24
+  uint32_t h = man24 >> shift;
+  const uint32_t rem = man24 & ((1u << shift) - 1u);
+  const uint32_t half_way = 1u << (shift - 1);
+  if (rem > half_way || (rem == half_way && (h & 1u))) ++h;
+  return static_cast<uint16_t>(sign | h);
+}
+
+namespace {
+
+// Unpack4Bit, tflite/kernels/embedding_lookup.cc:140-159: the nibble is moved to the top of an
+// int8 (16 x its signed value) and multiplied by scale / 16.
+inline void EmbeddingStore(float v, int out_f16, void* output, size_t index) {
+  if (out_f16) {
+    static_cast<uint16_t*>(output)[index] = orc_float_to_half(v);
+  } else {
+    static_cast<float*>(output)[index] = v;
+  }
+}
+
+void EmbeddingUnpack4Bit(float scaling_factor, size_t col_size, const int8_t* value_ptr,
+                         int out_f16, void* output, size_t out_off) {
+  const float scaling_factor0 = scaling_factor / 16;
+  size_t j = 0, i4 = 0;
+  for (; j + 1 < col_size; j += 2, ++i4) {
+    const int8_t v = value_ptr[i4];
+    const int8_t lo = static_cast<int8_t>(v << 4);
+    const int8_t hi = static_cast<int8_t>(v & 0xF0);
+    EmbeddingStore(lo * scaling_factor0, out_f16, output, out_off + j);
+    EmbeddingStore(hi * scaling_factor0, out_f16, output, out_off + j + 1);
+  }
+  if (col_size & 1) {
+    const int8_t lo = static_cast<int8_t>(value_ptr[i4] << 4);
+    EmbeddingStore(lo * scaling_factor0, out_f16, output, out_off + j);
+  }
+}
+
+}  // namespace
+
+// EMBEDDING_LOOKUP on an Int4 table with blockwise quantization: EvalBlockwise,
+// tflite/kernels/embedding_lookup.cc:194-307. Rows are written in lookup order until an index
+// falls outside [0, rows): then -(position + 1) is returned, as the kernel fails there (:280-286).
+// A column count that the block size does not divide returns 1 (:269-275).
+int orc_embedding_lookup_blockwise_int4(const int32_t* lookup, int count, const uint8_t* table,
+                                        int rows, int cols, const uint16_t* scales_f16,
+                                        int blocksize, int out_f16, void* output) {
+  if (blocksize <= 0 || cols % blocksize != 0) return 1;
+  const size_t num_blocks = static_cast<size_t>(cols) / blocksize;
+  const int8_t* value_ptr = reinterpret_cast<const int8_t*>(table);
+  for (int i = 0; i < count; ++i) {
+    const int idx = lookup[i];
+    if (idx >= rows || idx < 0) return -(i + 1);
+    const size_t output_row_offset = static_cast<size_t>(i) * cols;
+    const size_t scale_offset = static_cast<size_t>(idx) * num_blocks;
+    const size_t value_offset = static_cast<size_t>(idx) * cols;
+    for (size_t j = 0; j < num_blocks; ++j) {
+      const float scaling_factor = orc_half_to_float(scales_f16[scale_offset + j]);
+      const size_t val_off = value_offset + j * blocksize;
+      EmbeddingUnpack4Bit(scaling_factor, blocksize, &value_ptr[val_off / 2], out_f16, output,
+                          output_row_offset + j * blocksize);
+    }
+  }
+  return 0;
+}
+
+// EMBEDDING_LOOKUP from an Int8 or Int4 table to floats: EvalHybrid,
+// tflite/kernels/embedding_lookup.cc:309-395. One scale for the table, or one per row
+// (row_scales, :376-383). value_bits is 8 or 4. Same return convention as above.
+int orc_embedding_lookup_hybrid(const int32_t* lookup, int count, const void* table, int value_bits,
+                                int rows, int cols, float scale, const float* row_scales,
+                                int out_f16, void* output) {
+  const int8_t* value_ptr = static_cast<const int8_t*>(table);
+  for (int i = 0; i < count; ++i) {
+    const int32_t idx = lookup[i];
+    if (idx >= rows || idx < 0) return -(i + 1);
+    const size_t out_off = static_cast<size_t>(i) * cols;
+    const float scaling_factor = row_scales ? row_scales[idx] : scale;
+    const size_t offset = static_cast<size_t>(cols) * idx;
+    if (value_bits == 4) {
+      EmbeddingUnpack4Bit(scaling_factor, cols, &value_ptr[offset >> 1], out_f16, output, out_off);
+    } else {
+      for (int j = 0; j < cols; ++j) {
+        EmbeddingStore(value_ptr[offset + j] * scaling_factor, out_f16, output, out_off + j);
+      }
+    }
+  }
+  return 0;
+}
+
 }  // extern "C"

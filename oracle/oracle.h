@@ -202,6 +202,24 @@ void orc_fc_hybrid_int4_per_channel(const float* input, int batches, int depth,
                                     const float* filter_scales, const float* bias,
                                     int activation, float* output);
 
+/* ---- EMBEDDING_LOOKUP from quantized tables ------------------------------ */
+
+/* IEEE binary32 -> binary16, round to nearest even (tflite/types/half.h:69, :129). */
+uint16_t orc_float_to_half(float f);
+
+/* tflite/kernels/embedding_lookup.cc:194-307 (EvalBlockwise, Int4 table, fp16 block scales
+ * [rows, cols/blocksize]). output: float32 or (out_f16) binary16 [count, cols]. Returns 0,
+ * -(position+1) of the first lookup outside [0, rows), or 1 when blocksize does not divide cols. */
+int orc_embedding_lookup_blockwise_int4(const int32_t* lookup, int count, const uint8_t* table,
+                                        int rows, int cols, const uint16_t* scales_f16,
+                                        int blocksize, int out_f16, void* output);
+
+/* tflite/kernels/embedding_lookup.cc:309-395 (EvalHybrid) for value_bits 8 or 4; one scale or
+ * row_scales[rows]. */
+int orc_embedding_lookup_hybrid(const int32_t* lookup, int count, const void* table, int value_bits,
+                                int rows, int cols, float scale, const float* row_scales,
+                                int out_f16, void* output);
+
 #ifdef __cplusplus
 }
 #endif

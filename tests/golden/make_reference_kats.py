@@ -62,6 +62,54 @@ def per_channel(source, scales, weights, bias, x, units, depth, act="none", int4
                 output_scale=float(out_s), output_zero_point=int(out_zp))
 
 
+def embedding_lookup_cases():
+    """tflite/kernels/embedding_lookup_test.cc: tables quantized as its harness does
+    (test_util.h:705-750 per block, :753-800 per row; round half away of value x float(1 / scale),
+    clamped to +-7 for Int4 and +-127 for Int8, quantization_utils.cc:394-437, 440-475), the
+    lookups and the float outputs the tests expect within their tolerances (7.41e-3, 1e-2 for
+    Float16 outputs, :35-36)."""
+    e = "tflite/kernels/embedding_lookup_test.cc"
+    small = [0.00, 0.007, 0.006, 0.005, 0.004, 0.003, 0.002, 0.001,
+             0.02, -0.02, 0.04, 0.06, 0.08, -0.04, -0.08, -0.06,
+             0.3, 0.6, 0.9, 1.2, 1.5, -0.3, -0.6, -0.9]
+    wide = [0.00, 0.01, 0.02, 0.03, 0.10, 0.11, 0.12, 0.13,
+            1.00, -1.01, 1.02, 1.03, 1.10, 1.11, 1.12, 1.13,
+            2.00, 2.01, 2.02, 2.03, 2.10, 2.11, 2.12, 2.13]
+    lookup = [1, 0, 2]
+
+    def rows_of(data, order):
+        d = np.asarray(data, np.float32).reshape(3, 8)
+        return d[order].ravel().tolist()
+
+    def quantize(data, scales_per_element, limit):
+        inv = (np.float32(1.0) / scales_per_element).astype(np.float32)
+        q = kh._round_half_away(np.asarray(data, np.float32) * inv)
+        return np.clip(q, -limit, limit).astype(np.int8)
+
+    cases = []
+    for lines, f16 in ((":509-534", False), (":569-596", True)):
+        bits16 = np.asarray([0.001, 0.001, 0.02, 0.02, 0.3, 0.3], np.float16)
+        per_element = np.repeat(bits16.astype(np.float32), 4)
+        q = quantize(small, per_element, 7)
+        cases.append(dict(source=e + lines, kind="blockwise", value_bits=4, rows=3, cols=8,
+                          blocksize=4, lookup=lookup, table=kh.pack_int4(q).tolist(),
+                          scales_f16_bits=bits16.view(np.uint16).tolist(), out_f16=f16,
+                          expected=rows_of(small, lookup), tolerance=1e-2 if f16 else 7.41e-3))
+    for lines, data, scales, bits, shape in (
+            (":420-440", wide, [0.00102, 0.0089, 0.016772], 8, [3, 8]),
+            (":442-462", wide, [0.00102, 0.0089, 0.016772], 8, [3, 2, 4]),
+            (":633-656", small, [0.001, 0.02, 0.3], 4, [3, 8]),
+            (":658-679", small, [0.001, 0.02, 0.3], 4, [3, 2, 4])):
+        sc = np.asarray(scales, np.float32)
+        q = quantize(data, np.repeat(sc, 8), 7 if bits == 4 else 127)
+        table = kh.pack_int4(q).tolist() if bits == 4 else q.tolist()
+        cases.append(dict(source=e + lines, kind="per_row", value_bits=bits, rows=3, cols=8,
+                          value_shape=shape, lookup=lookup, table=table,
+                          row_scales=[float(v) for v in sc], out_f16=False,
+                          expected=rows_of(data, lookup), tolerance=7.41e-3))
+    return cases
+
+
 def main():
     t = "tflite/kernels/fully_connected_test.cc"
     fc = []
@@ -138,7 +186,9 @@ def main():
         case.update(source=u + ":1214-1231", expected=want)
         hybrid_dot.append(case)
 
-    out = dict(fully_connected_int8=fc, batch_quantize_floats=quantize,
+    lookups = embedding_lookup_cases()
+
+    out = dict(embedding_lookup=lookups, fully_connected_int8=fc, batch_quantize_floats=quantize,
                quantize_multiplier=multiplier, multiply_by_quantized_multiplier=mbqm,
                hybrid_dot_per_channel=hybrid_dot,
                unpack_int4=[dict(source=u + ":2110-2119", packed=[0x38, 0xBE], count=4,
