@@ -348,9 +348,10 @@ int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
  * LRTFC_OUT_FLOAT16. table: rows x cols/2 bytes, low nibble = even column; scales_f16:
  * [rows, cols / blocksize] IEEE binary16; lookup: [count] int32; output: [count, cols].
  * cols must be a multiple of blocksize (:269-275) and both even (the reference reads rows from
- * byte boundaries). status: device int32[2] or NULL; every call rewrites it as {0, -1}, or
- * {1, p} when lookup[p] is the first index outside [0, rows) -- where the reference fails the
- * invoke (:280-286); rows with such an index are left unwritten. All pointers are device
+ * byte boundaries). status: device int32[3] or NULL; every call rewrites it as {0, -1, 0}, or
+ * {1, p, lookup[p]} when lookup[p] is the first index outside [0, rows) -- where the reference
+ * fails the invoke and reports that index (:280-286); rows with such an index are left
+ * unwritten. All pointers are device
  * pointers; the call only enqueues work on `stream`. */
 int lrtfc_embedding_lookup_blockwise_int4(const int32_t* lookup, int count, const uint8_t* table,
                                           int rows, int cols, const uint16_t* scales_f16,

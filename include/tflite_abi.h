@@ -300,6 +300,7 @@ typedef struct { /* builtin_op_data.h:191-211 */
 } TfLiteFullyConnectedParams;
 
 enum { /* builtin_ops.h:39,81 */
+  kTfLiteBuiltinEmbeddingLookup = 7,
   kTfLiteBuiltinFullyConnected = 9,
   kTfLiteBuiltinDelegate = 51,
 };

@@ -42,6 +42,7 @@ struct Options {
   bool claim_hybrid = true;
   bool claim_int4_blockwise = true;
   bool claim_int4_per_channel = true;
+  bool claim_embedding_lookup = true;
 };
 
 // Device memory the application registered for a tensor (litert_amd_register_device_buffer);
@@ -69,7 +70,7 @@ const RegisteredBuffer* BoundBuffer(const DelegateState* state, const TfLiteTens
   return b.device ? &b : nullptr;
 }
 
-enum class FcKind { kNone, kInt8, kHybrid, kInt4Blockwise, kHybridInt4 };
+enum class FcKind { kNone, kInt8, kHybrid, kInt4Blockwise, kHybridInt4, kEmbeddingLookup };
 
 int64_t NumElements(const TfLiteIntArray* dims) {
   int64_t n = 1;
@@ -94,6 +95,69 @@ bool ClippingActivation(TfLiteFusedActivation a) {
          a == kTfLiteActRelu6;
 }
 
+// EMBEDDING_LOOKUP nodes whose table is quantized and whose rows come out as floats: what
+// EvalBlockwise and EvalHybrid of the builtin accept (tflite/kernels/embedding_lookup.cc:49-100,
+// 194-225, 397-412) for Int4 and Int8 tables. Float tables (a plain row copy), UInt8 and Int2
+// tables stay on the CPU.
+FcKind ClassifyEmbeddingLookup(const TfLiteContext* ctx, const TfLiteNode* node,
+                               const Options& opt, std::string* why_not) {
+  auto no = [&](const char* reason) {
+    if (why_not) *why_not = reason;
+    return FcKind::kNone;
+  };
+  if (!opt.claim_embedding_lookup) return no("embedding lookup disabled by option");
+  if (node->inputs->size != 2 || node->outputs->size != 1) return no("needs 2 inputs, 1 output");
+  const TfLiteTensor& lookup = ctx->tensors[node->inputs->data[0]];
+  const TfLiteTensor& value = ctx->tensors[node->inputs->data[1]];
+  const TfLiteTensor& output = ctx->tensors[node->outputs->data[0]];
+  if (!lookup.dims || lookup.dims->size != 1 || lookup.type != kTfLiteInt32) {
+    return no("lookup is not a rank-1 int32 tensor");
+  }
+  if (!value.dims || value.dims->size < 2) return no("table has fewer than 2 dimensions");
+  if (!IsConstant(value)) return no("table is not a constant tensor");
+  if (output.type != kTfLiteFloat32 && output.type != kTfLiteFloat16) {
+    return no("output is not float32 or float16");
+  }
+  const int rows = value.dims->data[0];
+  int64_t cols = 1;
+  for (int i = 1; i < value.dims->size; ++i) cols *= value.dims->data[i];
+  if (cols > 0x7FFFFFFF) return no("row too long");
+  if (value.quantization.type == kTfLiteBlockwiseQuantization) {
+    if (value.type != kTfLiteInt4) return no("blockwise table is not Int4");
+    if (value.dims->size != 2) return no("blockwise table is not rank 2");
+    const auto* bq = static_cast<const TfLiteBlockwiseQuantization*>(value.quantization.params);
+    if (!bq || bq->blocksize <= 0 || cols % bq->blocksize != 0) return no("bad blocksize");
+    if (cols % 2 != 0 || bq->blocksize % 2 != 0) return no("odd row or block length");
+    if (bq->scale < 0 || static_cast<size_t>(bq->scale) >= ctx->tensors_size) {
+      return no("scale tensor index out of range");
+    }
+    const TfLiteTensor& scales = ctx->tensors[bq->scale];
+    if (scales.type != kTfLiteFloat16 || !IsConstant(scales)) return no("scales not const fp16");
+    if (NumElements(scales.dims) != static_cast<int64_t>(rows) * (cols / bq->blocksize)) {
+      return no("scale count != rows x blocks");
+    }
+    return FcKind::kEmbeddingLookup;
+  }
+  if (value.type != kTfLiteInt8 && value.type != kTfLiteInt4) {
+    return no("table type is left to the CPU kernels");
+  }
+  if (value.type == kTfLiteInt4 && cols % 2 != 0) return no("odd row length");
+  if (value.quantization.type == kTfLiteAffineQuantization) {
+    const auto* q = static_cast<const TfLiteAffineQuantization*>(value.quantization.params);
+    if (!q || !q->scale || !q->zero_point || q->scale->size < 1 || q->zero_point->size < 1) {
+      return no("table has no scales");
+    }
+    if (q->zero_point->data[0] != 0) return no("non-zero table zero point");
+    if (q->scale->size > 1) {
+      if (q->quantized_dimension != 0 || q->scale->size != rows) {
+        return no("per-row scales do not match the rows");
+      }
+      if (q->zero_point->size != rows && q->zero_point->size != 1) return no("bad zero points");
+    }
+  }
+  return FcKind::kEmbeddingLookup;
+}
+
 // The node-claim predicate: the same tensor / quantization-parameter / fused-activation
 // combinations the builtin kernel accepts for these three paths
 // (tflite/kernels/fully_connected.cc:254-308, 440-761), nothing else.
@@ -104,6 +168,9 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
     if (why_not) *why_not = reason;
     return FcKind::kNone;
   };
+  if (registration->builtin_code == kTfLiteBuiltinEmbeddingLookup) {
+    return ClassifyEmbeddingLookup(ctx, node, opt, why_not);
+  }
   if (registration->builtin_code != kTfLiteBuiltinFullyConnected) return no("not FULLY_CONNECTED");
   if (registration->version > kMaxFcVersion) return no("op version newer than 14");
   if (!node->builtin_data) return no("no builtin data");
@@ -290,6 +357,11 @@ struct FcNode {
   // (retiled_dev then holds nibble tiles) and as re-tiled int8 for prefill batches.
   bool nibble_layout = false, have_nibbles = false;
   bool split_quantize = false;  // quantize rows in a launch of their own, not in the prologue
+  // EMBEDDING_LOOKUP nodes: input = the lookup vector, filter = the table (filter_dev), batches =
+  // lookups, depth = out_depth = columns of a row; block scales in scales_dev or per-row scales
+  // in pcs_dev; status_slot = the node's place in PartitionKernel::lookup_status.
+  int table_rows = 0, value_bits = 0, status_slot = -1;
+  bool out_f16 = false;
   // Scheduling inside the partition: the stream the node runs on, the node that produces its
   // input (-1: the input is uploaded from the host), and whether a node on another stream
   // waits for this one.
@@ -325,6 +397,11 @@ struct PartitionKernel {
     auto it = arena_offset.find(tensor);
     return it == arena_offset.end() ? nullptr : arena.as<uint8_t>() + it->second;
   }
+  // Three int32 per EMBEDDING_LOOKUP node, in page-locked host memory the lookup kernels write
+  // straight into: {0 or 1, first offending position, the index found there}.
+  PinnedBuffer lookup_status;
+  int32_t* lookup_status_dev = nullptr;
+  int lookup_nodes = 0;
   std::vector<int> uploads;                 // activation tensors read from the host each invoke
   std::vector<int> downloads;               // tensors written back to the host each invoke
   // Nodes that do not depend on each other (the q/k/v or gate/up projections of a decoder
@@ -424,9 +501,13 @@ void* KernelInit(TfLiteContext* ctx, const char* buffer, size_t /*length*/) {
     n.kind = kind;
     n.input = node->inputs->data[0];
     n.filter = node->inputs->data[1];
-    n.bias = (node->inputs->size == 3) ? node->inputs->data[2] : kTfLiteOptionalTensor;
+    n.bias = (kind != FcKind::kEmbeddingLookup && node->inputs->size == 3)
+                 ? node->inputs->data[2]
+                 : kTfLiteOptionalTensor;
     n.output = node->outputs->data[0];
-    n.params = *static_cast<const TfLiteFullyConnectedParams*>(node->builtin_data);
+    if (kind != FcKind::kEmbeddingLookup) {
+      n.params = *static_cast<const TfLiteFullyConnectedParams*>(node->builtin_data);
+    }
     if (!produced.count(n.input)) {
       bool listed = false;
       for (int t : kernel->uploads) listed = listed || (t == n.input);
@@ -493,7 +574,57 @@ TfLiteStatus RetileInt8(TfLiteContext* ctx, FcNode* n, hipStream_t s) {
   return kTfLiteOk;
 }
 
+// EMBEDDING_LOOKUP: shapes as embedding_lookup.cc:49-100 leaves them (output = lookups x the
+// table's row shape), the table and its scales uploaded once.
+TfLiteStatus PrepareLookupNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
+  const TfLiteTensor& lookup = ctx->tensors[n->input];
+  const TfLiteTensor& value = ctx->tensors[n->filter];
+  const TfLiteTensor& output = ctx->tensors[n->output];
+  n->table_rows = value.dims->data[0];
+  int64_t cols = 1;
+  for (int i = 1; i < value.dims->size; ++i) cols *= value.dims->data[i];
+  n->depth = n->out_depth = static_cast<int>(cols);
+  n->batches = static_cast<int>(NumElements(lookup.dims));
+  n->value_bits = value.type == kTfLiteInt4 ? 4 : 8;
+  n->out_f16 = output.type == kTfLiteFloat16;
+  n->use_retiled = true;  // no activation workspace, no grouping
+  if (NumElements(output.dims) != static_cast<int64_t>(n->batches) * cols) {
+    ctx->ReportError(ctx, "litert_amd delegate: node %d output shape does not hold %d x %lld values",
+                     n->node_index, n->batches, static_cast<long long>(cols));
+    return kTfLiteError;
+  }
+  hipStream_t s = k->stream;
+  n->blocksize = 0;
+  n->per_channel = false;
+  n->filter_scale = value.params.scale;
+  const bool fresh = n->uploaded_filter != value.data.raw;
+  if (value.quantization.type == kTfLiteBlockwiseQuantization) {
+    const auto* bq = static_cast<const TfLiteBlockwiseQuantization*>(value.quantization.params);
+    n->blocksize = bq->blocksize;
+    n->scales = bq->scale;
+    const TfLiteTensor& scales = ctx->tensors[bq->scale];
+    if (fresh) {
+      RETURN_IF_HIP(ctx, n->scales_dev.Upload(scales.data.raw,
+                                              static_cast<size_t>(NumElements(scales.dims)) * 2, s));
+    }
+  } else if (value.quantization.type == kTfLiteAffineQuantization) {
+    const auto* q = static_cast<const TfLiteAffineQuantization*>(value.quantization.params);
+    n->per_channel = q->scale->size > 1;  // one scale per row, embedding_lookup.cc:376-383
+    if (n->per_channel && fresh) {
+      RETURN_IF_HIP(ctx, n->pcs_dev.Upload(q->scale->data, static_cast<size_t>(n->table_rows) * 4, s));
+    }
+  }
+  if (fresh && value.bytes > 0) {
+    RETURN_IF_HIP(ctx, n->filter_dev.Upload(value.data.raw, value.bytes, s));
+    RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+  }
+  n->have_model_layout = true;
+  n->uploaded_filter = value.data.raw;
+  return kTfLiteOk;
+}
+
 TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
+  if (n->kind == FcKind::kEmbeddingLookup) return PrepareLookupNode(ctx, k, n);
   const TfLiteTensor& input = ctx->tensors[n->input];
   const TfLiteTensor& filter = ctx->tensors[n->filter];
   const TfLiteTensor* bias = n->bias == kTfLiteOptionalTensor ? nullptr : &ctx->tensors[n->bias];
@@ -766,7 +897,18 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
     }
   }
   // Scratch for the nodes that quantize in a launch of their own, per stream.
+  k->lookup_nodes = 0;
+  for (FcNode& n : k->nodes) {
+    if (n.kind == FcKind::kEmbeddingLookup) n.status_slot = k->lookup_nodes++;
+  }
+  if (k->lookup_nodes > 0) {
+    RETURN_IF_HIP(ctx, k->lookup_status.Ensure(static_cast<size_t>(k->lookup_nodes) * 12));
+    void* dev = nullptr;
+    RETURN_IF_HIP(ctx, hipHostGetDevicePointer(&dev, k->lookup_status.get(), 0));
+    k->lookup_status_dev = static_cast<int32_t*>(dev);
+  }
   for (const FcNode& n : k->nodes) {
+    if (n.kind == FcKind::kEmbeddingLookup) continue;
     if (n.kind == FcKind::kHybridInt4 ||
         (n.kind != FcKind::kInt8 && (!n.use_retiled || n.split_quantize))) {
       RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(
@@ -983,6 +1125,24 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                 n.batches, n.depth, n.out_depth, s));
         }
         break;
+      case FcKind::kEmbeddingLookup: {
+        int32_t* status = k->lookup_status_dev + 3 * n.status_slot;
+        const int out_type = n.out_f16 ? LRTFC_OUT_FLOAT16 : LRTFC_OUT_FLOAT32;
+        if (n.blocksize > 0) {
+          RETURN_IF_FC(ctx, lrtfc_embedding_lookup_blockwise_int4(
+                                static_cast<const int32_t*>(in_dev), n.batches,
+                                n.filter_dev.as<uint8_t>(), n.table_rows, n.depth,
+                                n.scales_dev.as<uint16_t>(), n.blocksize, out_type, out_dev, status,
+                                s));
+        } else {
+          RETURN_IF_FC(ctx, lrtfc_embedding_lookup_hybrid(
+                                static_cast<const int32_t*>(in_dev), n.batches, n.filter_dev.get(),
+                                n.value_bits, n.table_rows, n.depth, n.filter_scale,
+                                n.per_channel ? n.pcs_dev.as<float>() : nullptr, out_type, out_dev,
+                                status, s));
+        }
+        break;
+      }
       default:
         return kTfLiteError;
     }
@@ -1022,6 +1182,18 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   // The runtime reads the outputs as soon as invoke returns; a consumer of a registered
   // buffer (another partition, the application's own kernels) may start right away too.
   RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+  // A lookup outside the table fails the invoke, with the builtin's message
+  // (tflite/kernels/embedding_lookup.cc:280-286, 365-371).
+  for (const FcNode& n : k->nodes) {
+    if (n.kind != FcKind::kEmbeddingLookup || n.batches == 0 || n.depth == 0) continue;
+    const int32_t* status =
+        reinterpret_cast<const int32_t*>(k->lookup_status.get()) + 3 * n.status_slot;
+    if (status[0] != 0) {
+      ctx->ReportError(ctx, "Embedding Lookup: index out of bounds. Got %d, and bounds are [0, %d]",
+                       status[2], n.table_rows - 1);
+      return kTfLiteError;
+    }
+  }
   for (int t : k->downloads) {
     TfLiteTensor& tensor = ctx->tensors[t];
     if (tensor.bytes == 0 || BoundBuffer(k->state, tensor)) continue;
@@ -1152,7 +1324,7 @@ bool ParseOptions(const char* const* keys, const char* const* values, size_t n, 
       }
     } else if (key == "claim") {
       opt->claim_int8 = opt->claim_hybrid = opt->claim_int4_blockwise = false;
-      opt->claim_int4_per_channel = false;
+      opt->claim_int4_per_channel = opt->claim_embedding_lookup = false;
       size_t pos = 0;
       while (pos <= val.size()) {
         const size_t comma = val.find(',', pos);
@@ -1165,8 +1337,11 @@ bool ParseOptions(const char* const* keys, const char* const* values, size_t n, 
           opt->claim_int4_blockwise = true;
         } else if (item == "int4_per_channel") {
           opt->claim_int4_per_channel = true;
+        } else if (item == "embedding_lookup") {
+          opt->claim_embedding_lookup = true;
         } else if (!item.empty()) {
-          *error = "claim accepts int8, hybrid, int4_blockwise, int4_per_channel; got '" + item + "'";
+          *error = "claim accepts int8, hybrid, int4_blockwise, int4_per_channel, embedding_lookup; got '" +
+                   item + "'";
           return false;
         }
         if (comma == std::string::npos) break;
@@ -1237,7 +1412,8 @@ TfLiteBufferHandle litert_amd_register_device_buffer(TfLiteDelegate* delegate, v
 }
 
 // Test and tooling hook: the claim predicate on its own (no device needed). Returns
-// 0 = declined, 1 = int8, 2 = hybrid, 3 = int4 blockwise, 4 = int4 per-channel hybrid; `reason` (may be NULL)
+// 0 = declined, 1 = int8, 2 = hybrid, 3 = int4 blockwise, 4 = int4 per-channel hybrid,
+// 5 = EMBEDDING_LOOKUP from a quantized table; `reason` (may be NULL)
 // receives why a node was declined.
 int litert_amd_classify_node(const TfLiteContext* ctx, const TfLiteNode* node,
                              const TfLiteRegistration* registration, char* reason,

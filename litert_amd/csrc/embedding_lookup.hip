@@ -18,8 +18,8 @@
 //
 // Indices outside [0, rows) make the reference fail at the first such lookup (:280-286,
 // :365-371). Here the first workgroup scans the lookup vector and records the first offending
-// position in `status` (a device int32 pair: {0 or 1, position or -1}), rewritten in full by
-// every launch; rows with such an index are not written.
+// position in `status` (three device int32: {0 or 1, position or -1, the index found there or
+// 0}), rewritten in full by every launch; rows with such an index are not written.
 #include "kernels.h"
 
 namespace lrtfc {
@@ -87,6 +87,7 @@ __device__ __forceinline__ void ScanLookups(const LookupArgs& a) {
     const bool bad = first_bad != 0x7FFFFFFF;
     a.status[0] = bad ? 1 : 0;
     a.status[1] = bad ? first_bad : -1;
+    a.status[2] = bad ? a.lookup[first_bad] : 0;
   }
 }
 
@@ -176,7 +177,7 @@ hipError_t LaunchEmbeddingLookup(const int32_t* lookup, int count, const void* t
   a.cols = cols;
   a.blocksize = block_scales ? blocksize : cols;
   if (count == 0 || cols == 0) {
-    // nothing to gather; the status pair is still rewritten
+    // nothing to gather; the status words are still rewritten
     if (status == nullptr) return hipSuccess;
     LookupStatusOnlyKernel<<<1, kThreads, 0, stream>>>(a);
     return hipGetLastError();

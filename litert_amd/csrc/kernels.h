@@ -133,8 +133,8 @@ hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const 
 
 // EMBEDDING_LOOKUP from an Int4 (value_bits 4) or Int8 (8) table to float32 / binary16 rows.
 // block_scales != nullptr: blockwise fp16 scales [rows, cols / blocksize]; otherwise row_scales
-// [rows] or `scale`. status: device int32 pair {0 or 1, first offending position or -1},
-// rewritten by every launch; may be nullptr. Int4 tables need even cols and blocksize.
+// [rows] or `scale`. status: three device int32 {0 or 1, first offending position or -1, the
+// index there or 0}, rewritten by every launch; may be nullptr. Int4 tables need even cols and blocksize.
 hipError_t LaunchEmbeddingLookup(const int32_t* lookup, int count, const void* table,
                                  int value_bits, int rows, int cols, const uint16_t* block_scales,
                                  int blocksize, const float* row_scales, float scale, int out_f16,

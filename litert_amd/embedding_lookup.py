@@ -5,7 +5,8 @@ kernel through the C-ABI and leave the rows in device memory, ready to feed FULL
 An index outside [0, rows) fails the reference's invoke at the first such lookup (:280-286,
 :365-371). The kernel records it in a device status pair; `__call__` reads that pair back (one
 stream synchronization) and raises IndexError with the reference's message, unless
-`check=False` leaves the check to the caller (`status` holds {0 or 1, position or -1}).
+`check=False` leaves the check to the caller (`status` holds {0 or 1, position or -1, the
+index found there or 0}).
 """
 import numpy as np
 import torch
@@ -23,13 +24,13 @@ class _Lookup:
             raise ValueError("output tensor does not match the lookup")
         return out
 
-    def _finish(self, lookup, check):
+    def _finish(self, check):
         if not check:
             return
-        flag, position = self.status.tolist()  # synchronizes the stream
+        flag, _, index = self.status.tolist()  # synchronizes the stream
         if flag:
             raise IndexError("Embedding Lookup: index out of bounds. Got %d, and bounds are [0, %d]"
-                             % (int(lookup[position]), self.rows - 1))
+                             % (index, self.rows - 1))
 
 
 class EmbeddingLookupBlockwiseInt4(_Lookup):
@@ -48,7 +49,7 @@ class EmbeddingLookupBlockwiseInt4(_Lookup):
             scales_f16 = scales_f16.view(torch.int16)
         self.scales = _dev(scales_f16, torch.int16)
         self.out_f16 = bool(out_f16)
-        self.status = torch.zeros(2, dtype=torch.int32, device="cuda")
+        self.status = torch.zeros(3, dtype=torch.int32, device="cuda")
 
     def __call__(self, lookup, out=None, check=True):
         lookup = _dev(lookup, torch.int32)
@@ -57,7 +58,7 @@ class EmbeddingLookupBlockwiseInt4(_Lookup):
             _ptr(lookup), lookup.numel(), _ptr(self.table), self.rows, self.cols, _ptr(self.scales),
             self.blocksize, capi.OUT_FLOAT16 if self.out_f16 else capi.OUT_FLOAT32, _ptr(out),
             _ptr(self.status), _stream()))
-        self._finish(lookup, check)
+        self._finish(check)
         return out
 
 
@@ -76,7 +77,7 @@ class EmbeddingLookupHybrid(_Lookup):
         self.scale = float(scale)
         self.row_scales = _dev(row_scales, torch.float32)
         self.out_f16 = bool(out_f16)
-        self.status = torch.zeros(2, dtype=torch.int32, device="cuda")
+        self.status = torch.zeros(3, dtype=torch.int32, device="cuda")
 
     def __call__(self, lookup, out=None, check=True):
         lookup = _dev(lookup, torch.int32)
@@ -86,5 +87,5 @@ class EmbeddingLookupHybrid(_Lookup):
             self.scale, _ptr(self.row_scales),
             capi.OUT_FLOAT16 if self.out_f16 else capi.OUT_FLOAT32, _ptr(out), _ptr(self.status),
             _stream()))
-        self._finish(lookup, check)
+        self._finish(check)
         return out

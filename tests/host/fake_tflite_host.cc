@@ -334,6 +334,19 @@ int fh_add_other_node(void* hp, int builtin_code, int input, int output) {
   return static_cast<int>(h->nodes.size()) - 1;
 }
 
+// EMBEDDING_LOOKUP (builtin code 7): inputs {lookup, table}, no builtin options.
+int fh_add_embedding_lookup_node(void* hp, int lookup, int value, int output) {
+  auto* h = static_cast<Host*>(hp);
+  auto rec = std::make_unique<NodeRec>();
+  rec->node.inputs = MakeIntArray({lookup, value});
+  rec->node.outputs = MakeIntArray({output});
+  rec->reg.builtin_code = 7;
+  rec->reg.version = 1;
+  h->nodes.push_back(std::move(rec));
+  h->plan.push_back(static_cast<int>(h->nodes.size()) - 1);
+  return static_cast<int>(h->nodes.size()) - 1;
+}
+
 void fh_mark_graph_output(void* hp, int tensor) { static_cast<Host*>(hp)->graph_outputs.insert(tensor); }
 void fh_set_cpu_callback(void* hp, CpuCallback cb) { static_cast<Host*>(hp)->cpu = cb; }
 

@@ -118,3 +118,46 @@ def test_no_gpu_means_no_delegate():
         assert "HIP device" in h.errors()
         # the graph is untouched: every node still belongs to the CPU
         assert [kind for kind, _, _ in h.plan()] == ["cpu"]
+
+
+def _lookup_node(h, rows=16, cols=64, count=3, value_type=INT4, blockwise=True, bs=32, per_row=True,
+                 out_type=FLOAT32, lookup_type=INT32, const_table=True, zero_point=0,
+                 scale_type=FLOAT16, value_shape=None):
+    lk = h.tensor(lookup_type, (count,))
+    shape = value_shape or (rows, cols)
+    nbytes = rows * cols // 2 if value_type == INT4 else rows * cols
+    v = h.tensor(value_type, shape, data=np.zeros(nbytes, np.uint8), const=const_table)
+    if blockwise:
+        s = h.tensor(scale_type, (rows, cols // bs),
+                     data=np.ones((rows, cols // bs), np.float16 if scale_type == FLOAT16 else np.float32),
+                     const=True)
+        h.blockwise(v, s, bs)
+    else:
+        h.affine(v, np.full(rows if per_row else 1, 0.01), np.full(rows if per_row else 1, zero_point))
+    y = h.tensor(out_type, (count,) + tuple(shape[1:]))
+    return h.embedding_lookup(lk, v, y)
+
+
+def test_claim_predicate_embedding_lookup():
+    """What EvalBlockwise / EvalHybrid accept for Int4 and Int8 tables
+    (tflite/kernels/embedding_lookup.cc:49-100, 194-225, 397-412), nothing else."""
+    with FakeHost() as h:
+        assert h.classify(_lookup_node(h))[0] == "embedding_lookup"
+        assert h.classify(_lookup_node(h, out_type=FLOAT16))[0] == "embedding_lookup"
+        assert h.classify(_lookup_node(h, blockwise=False))[0] == "embedding_lookup"
+        assert h.classify(_lookup_node(h, blockwise=False, per_row=False))[0] == "embedding_lookup"
+        assert h.classify(_lookup_node(h, blockwise=False, value_type=INT8))[0] == "embedding_lookup"
+        assert h.classify(_lookup_node(h, blockwise=False, value_type=INT8,
+                                       value_shape=(16, 4, 16)))[0] == "embedding_lookup"
+        # declined: left to the CPU kernel
+        assert h.classify(_lookup_node(h, bs=24)) == (None, "bad blocksize")
+        assert h.classify(_lookup_node(h, scale_type=FLOAT32)) == (None, "scales not const fp16")
+        assert h.classify(_lookup_node(h, const_table=False)) == (None, "table is not a constant tensor")
+        assert h.classify(_lookup_node(h, lookup_type=FLOAT32))[1] == "lookup is not a rank-1 int32 tensor"
+        assert h.classify(_lookup_node(h, out_type=INT8))[1] == "output is not float32 or float16"
+        assert h.classify(_lookup_node(h, blockwise=False, value_type=UINT8))[1] == (
+            "table type is left to the CPU kernels")
+        assert h.classify(_lookup_node(h, blockwise=False, zero_point=3))[1] == "non-zero table zero point"
+        assert h.classify(_lookup_node(h, blockwise=False, cols=7, rows=2))[1] == "odd row length"
+        assert h.load_delegate({"claim": "int8,lookup"}) == 1
+        assert "embedding_lookup; got 'lookup'" in h.errors()

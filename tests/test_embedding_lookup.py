@@ -207,7 +207,7 @@ def test_hip_lookup_out_of_bounds_and_empty():
     out = torch.full((6, cols), 7.0, device="cuda")
     with pytest.raises(IndexError, match=r"Got 16, and bounds are \[0, 15\]"):
         op(lookup, out=out)
-    assert op.status.tolist() == [1, 2]
+    assert op.status.tolist() == [1, 2, 16]
     got = out.cpu().numpy()
     good = [0, 1, 3, 5]
     want = oracle.embedding_lookup_blockwise_int4(lookup[good], table, rows, cols, sbits, bs)
@@ -215,16 +215,16 @@ def test_hip_lookup_out_of_bounds_and_empty():
     assert np.all(got[[2, 4]] == 7.0)  # rows of offending lookups are left alone
     # the next good call rewrites the status pair
     op(lookup[good])
-    assert op.status.tolist() == [0, -1]
+    assert op.status.tolist() == [0, -1, 0]
     # the failing position may lie beyond the first 256 lookups
     many = np.zeros(1000, np.int32)
     many[[700, 900]] = rows
     with pytest.raises(IndexError):
         op(many)
-    assert op.status.tolist() == [1, 700]
+    assert op.status.tolist() == [1, 700, 16]
     # empty lookup vector: nothing written, status cleared
     assert op(np.zeros(0, np.int32)).shape == (0, cols)
-    assert op.status.tolist() == [0, -1]
+    assert op.status.tolist() == [0, -1, 0]
     hy = el.EmbeddingLookupHybrid(np.zeros((4, 8), np.int8), 8, 8, scale=0.5)
     with pytest.raises(IndexError, match=r"Got -1, and bounds are \[0, 3\]"):
         hy(np.array([-1], np.int32))

@@ -483,3 +483,111 @@ def test_empty_graph_and_nothing_to_claim():
         assert h.load_delegate() == 0
         assert h.modify_graph_with_delegate() == OK
         assert [k for k, _, _ in h.plan()] == ["cpu"]
+
+
+# ---- EMBEDDING_LOOKUP from quantized tables ---------------------------------------------------
+
+def _lookup_table(rng, rows, cols, bs):
+    packed = rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8)
+    scales = (rng.random((rows, cols // bs), dtype=np.float32) * 2e-2 + 1e-3).astype(np.float16)
+    return packed, scales
+
+
+@pytest.mark.parametrize("out_f16", [False, True])
+@pytest.mark.parametrize("count", [1, 37])
+def test_blockwise_embedding_lookup_node_through_delegate(count, out_f16):
+    rng = np.random.default_rng(21 + count)
+    rows, cols, bs = 500, 2048, 32
+    packed, scales = _lookup_table(rng, rows, cols, bs)
+    lookup = rng.integers(0, rows, count).astype(np.int32)
+    with FakeHost() as h:
+        lk = h.tensor(INT32, (count,), data=lookup)
+        v = h.tensor(INT4, (rows, cols), data=packed, const=True)
+        s = h.tensor(FLOAT16, (rows, cols // bs), data=scales, const=True)
+        h.blockwise(v, s, bs)
+        y = h.tensor(FLOAT16 if out_f16 else FLOAT32, (count, cols))
+        node = h.embedding_lookup(lk, v, y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.plan()[0][:2] == ("delegate", [node])
+        assert h.invoke() == OK, h.errors()
+        want = oracle.embedding_lookup_blockwise_int4(lookup, packed, rows, cols,
+                                                      scales.view(np.uint16), bs, out_f16)
+        assert np.array_equal(h.read(y).view(want.dtype), want)
+        # other tokens on the next invoke; a token outside the table fails it as the builtin does
+        lookup2 = rng.integers(0, rows, count).astype(np.int32)
+        h.write(lk, lookup2)
+        assert h.invoke() == OK, h.errors()
+        want = oracle.embedding_lookup_blockwise_int4(lookup2, packed, rows, cols,
+                                                      scales.view(np.uint16), bs, out_f16)
+        assert np.array_equal(h.read(y).view(want.dtype), want)
+        lookup2[-1] = rows
+        h.write(lk, lookup2)
+        assert h.invoke() != OK
+        assert "Embedding Lookup: index out of bounds. Got 500, and bounds are [0, 499]" in h.errors()
+        lookup2[-1] = 0
+        h.write(lk, lookup2)
+        assert h.invoke() == OK, h.errors()
+
+
+@pytest.mark.parametrize("bits,per_row,shape", [(8, True, (40, 96)), (8, False, (40, 4, 24)),
+                                                (4, True, (40, 96)), (4, False, (40, 50))])
+def test_affine_embedding_lookup_node_through_delegate(bits, per_row, shape):
+    rng = np.random.default_rng(bits + shape[-1])
+    rows, cols = shape[0], int(np.prod(shape[1:]))
+    table = (rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8) if bits == 4
+             else rng.integers(-128, 128, (rows, cols), dtype=np.int8))
+    scales = (rng.random(rows if per_row else 1, dtype=np.float32) * 0.02 + 1e-3)
+    lookup = rng.integers(0, rows, 9).astype(np.int32)
+    with FakeHost() as h:
+        lk = h.tensor(INT32, (9,), data=lookup)
+        v = h.tensor(INT4 if bits == 4 else INT8, shape, data=table, const=True)
+        h.affine(v, scales)
+        y = h.tensor(FLOAT32, (9,) + shape[1:])
+        h.embedding_lookup(lk, v, y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.invoke() == OK, h.errors()
+        got = h.read(y)
+    want = oracle.embedding_lookup_hybrid(lookup, table, bits, rows, cols, scale=float(scales[0]),
+                                          row_scales=scales if per_row else None)
+    assert got.shape == (9,) + shape[1:]
+    assert np.array_equal(got.reshape(9, cols).view(np.uint32), want.view(np.uint32))
+
+
+def test_embedding_lookup_feeds_projections_inside_one_partition():
+    """Token ids -> embedding rows -> the q/k/v projections of a decoder's first layer, all
+    blockwise Int4: one partition, the rows never leave the device, results as the oracle's
+    chain of the two builtins."""
+    rng = np.random.default_rng(77)
+    rows, K, bs, B = 1000, 2048, 32, 4
+    packed, scales = _lookup_table(rng, rows, K, bs)
+    lookup = rng.integers(0, rows, B).astype(np.int32)
+    projections = [wl.blockwise_int4_fc(B, K, n, seed=5 + i) for i, n in enumerate((2048, 256, 256))]
+    with FakeHost() as h:
+        lk = h.tensor(INT32, (B,), data=lookup)
+        v = h.tensor(INT4, (rows, K), data=packed, const=True)
+        s = h.tensor(FLOAT16, (rows, K // bs), data=scales, const=True)
+        h.blockwise(v, s, bs)
+        x = h.tensor(FLOAT32, (B, K))
+        h.embedding_lookup(lk, v, x)
+        outs = []
+        for c in projections:
+            n = c["packed"].shape[0]
+            w = h.tensor(INT4, (n, K), data=c["packed"], const=True)
+            ws = h.tensor(FLOAT16, (n, K // 32), data=c["scales"], const=True)
+            h.blockwise(w, ws, 32)
+            y = h.tensor(FLOAT32, (B, n))
+            h.fc(x, w, None, y)
+            h.mark_output(y)
+            outs.append(y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert len(h.plan()) == 1 and h.plan()[0][0] == "delegate"
+        assert h.invoke() == OK, h.errors()
+        rows_f32 = oracle.embedding_lookup_blockwise_int4(lookup, packed, rows, K,
+                                                          scales.view(np.uint16), bs)
+        for c, y in zip(projections, outs):
+            want = oracle.fc_blockwise_int4(rows_f32, c["packed"], c["packed"].shape[0],
+                                            c["scales"].view(np.uint16), 32)
+            assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
