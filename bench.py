@@ -366,6 +366,31 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         note="two launches each (row quantizer + GEMV); per launch pair")
     del ops4b, nib
 
+    # Next-row op: EMBEDDING_LOOKUP from a blockwise Int4 table of a 256000-token vocabulary,
+    # 2048 columns, block size 32 (what feeds config 5's first layer): one decode token and a
+    # prefill batch of 2048 tokens. Bytes per looked-up row: 1024 of nibbles + 128 of scales
+    # read, 8192 of float32 written.
+    from litert_amd import embedding_lookup as el
+    g5 = torch.Generator(device="cuda").manual_seed(13)
+    table = torch.randint(0, 256, (256000, 1024), dtype=torch.uint8, device="cuda", generator=g5)
+    tscales = (torch.rand((256000, 64), device="cuda", generator=g5) * 2e-2 + 1e-3).half()
+    lookup_op = el.EmbeddingLookupBlockwiseInt4(table, tscales, 2048, 32)
+    entry = {}
+    for count in (1, 2048):
+        ids = [torch.randint(0, 256000, (count,), dtype=torch.int32, device="cuda", generator=g5)
+               for _ in range(8)]
+        rows_out = torch.empty((count, 2048), dtype=torch.float32, device="cuda")
+        us = per_launch_us([(lambda t: lambda: lookup_op(t, out=rows_out, check=False))(t) for t in ids])
+        moved = count * (1024 + 128 + 8192 + 4)
+        entry["us_%d_tokens" % count] = round(us, 3)
+        entry["gbps_%d_tokens" % count] = round(moved / us / 1e3, 1)
+        if count == 2048:
+            entry["frac_of_hbm_peak_2048_tokens"] = round(moved / us / 1e3 / HBM_PEAK_GBPS, 4)
+            entry["algorithmic_bytes_2048_tokens"] = moved
+    entry["kernel"] = "EmbeddingLookupKernel<Int4, float32, 8 columns per thread>"
+    out["next_embedding_lookup_blockwise_int4_256000x2048"] = entry
+    del table, tscales, lookup_op
+
     # config 4: prefill int8 GEMM 2048 x 4096 x 4096, RELU6 off / on
     c4 = wl.prefill_int8_fc()
     x4 = dev(c4["x"])
