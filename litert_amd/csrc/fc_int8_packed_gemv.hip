@@ -451,10 +451,15 @@ hipError_t LaunchSized(const PackedArgs& p, int batch0, int bt, hipStream_t stre
   auto kernel = FcInt8PackedGemvKernel<EPI, FUSED, VARIANT, REG_ROWS>;
   if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
-  // One wavefront per channel group when that already gives the chip ~2 wavefronts per
-  // SIMD-pair; otherwise split the depth so that short filters still spread out.
+  // How many wavefronts share one channel group's depth. What the memory system rewards is
+  // bytes in flight: a wavefront keeps kRing tiles outstanding whatever its share, so shares
+  // of about two rings (32 tiles) put twice the wavefronts -- and twice the outstanding
+  // loads -- on each CU compared with one wavefront per group at depth 4096 (measured at
+  // 14336 x 4096, B = 1: 13.5 -> 12.7 us; 8192 x 8192: 19.6 -> 17.2 us; shares of 16 tiles are
+  // slower again). Short filters split further until the chip has a wavefront per SIMD.
   int ksplit = 1;
-  while (ksplit < kWaves && tiles * ksplit < 512 && p.slabs / (ksplit * 2) >= 4) ksplit *= 2;
+  while (ksplit < kWaves && p.slabs / (ksplit * 2) >= 2 * kRing) ksplit *= 2;
+  while (ksplit < kWaves && tiles * ksplit < 1024 && p.slabs / (ksplit * 2) >= 4) ksplit *= 2;
   const int tiles_per_wg = kWaves / ksplit;
   const int grid = (tiles + tiles_per_wg - 1) / tiles_per_wg;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, p, batch0, bt, ksplit);
