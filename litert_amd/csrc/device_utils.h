@@ -97,16 +97,42 @@ __device__ __forceinline__ int32_t WaveSumI32(int32_t v) {
   return v;
 }
 
+// Float min / max over the 64 lanes; every lane receives the result (it is wave-uniform).
+// Four data-parallel-primitive steps reduce each row of 16 lanes inside the vector ALU (lane
+// swaps within quads, then the half-row and row mirrors), and the four row results are read
+// out as scalars: 10 short instructions, where a butterfly of cross-lane shuffles goes
+// through the LDS crossbar six times in sequence. min and max are exact and order-free.
+template <int CTRL>
+__device__ __forceinline__ float DppMoveF32(float v) {
+  const int i = __float_as_int(v);
+  return __int_as_float(__builtin_amdgcn_update_dpp(i, i, CTRL, 0xF, 0xF, false));
+}
+
+__device__ __forceinline__ float ReadLaneF32(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+constexpr int kDppQuadSwap1 = 0xB1;       // quad_perm [1, 0, 3, 2]
+constexpr int kDppQuadSwap2 = 0x4E;       // quad_perm [2, 3, 0, 1]
+constexpr int kDppRowHalfMirror = 0x141;  // lane i <-> 7 - i within each 8
+constexpr int kDppRowMirror = 0x140;      // lane i <-> 15 - i within each 16
+
 __device__ __forceinline__ float WaveMinF32(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, kWaveSize));
-  return v;
+  v = fminf(v, DppMoveF32<kDppQuadSwap1>(v));
+  v = fminf(v, DppMoveF32<kDppQuadSwap2>(v));
+  v = fminf(v, DppMoveF32<kDppRowHalfMirror>(v));
+  v = fminf(v, DppMoveF32<kDppRowMirror>(v));
+  return fminf(fminf(ReadLaneF32(v, 0), ReadLaneF32(v, 16)),
+               fminf(ReadLaneF32(v, 32), ReadLaneF32(v, 48)));
 }
 
 __device__ __forceinline__ float WaveMaxF32(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWaveSize));
-  return v;
+  v = fmaxf(v, DppMoveF32<kDppQuadSwap1>(v));
+  v = fmaxf(v, DppMoveF32<kDppQuadSwap2>(v));
+  v = fmaxf(v, DppMoveF32<kDppRowHalfMirror>(v));
+  v = fmaxf(v, DppMoveF32<kDppRowMirror>(v));
+  return fmaxf(fmaxf(ReadLaneF32(v, 0), ReadLaneF32(v, 16)),
+               fmaxf(ReadLaneF32(v, 32), ReadLaneF32(v, 48)));
 }
 
 // 4-way int8 dot product with int32 accumulate (v_dot4_i32_i8).

@@ -333,14 +333,8 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
               if (g < groups8) {
                 const float4 lo = xr[b][j][0], hi = xr[b][j][1];
                 const bool tail = g * 8 >= vector_end;
-                even = PackBytes(QuantizeElement<VARIANT>(lo.x, qp, true, tail),
-                                 QuantizeElement<VARIANT>(lo.z, qp, true, tail),
-                                 QuantizeElement<VARIANT>(hi.x, qp, true, tail),
-                                 QuantizeElement<VARIANT>(hi.z, qp, true, tail));
-                odd = PackBytes(QuantizeElement<VARIANT>(lo.y, qp, true, tail),
-                                QuantizeElement<VARIANT>(lo.w, qp, true, tail),
-                                QuantizeElement<VARIANT>(hi.y, qp, true, tail),
-                                QuantizeElement<VARIANT>(hi.w, qp, true, tail));
+                even = QuantizePack4<VARIANT>(lo.x, lo.z, hi.x, hi.z, qp, tail);
+                odd = QuantizePack4<VARIANT>(lo.y, lo.w, hi.y, hi.w, qp, tail);
               }
               *reinterpret_cast<i32x2*>(sh.q + b * (padded / 4) + 2 * g) = i32x2{even, odd};
             }

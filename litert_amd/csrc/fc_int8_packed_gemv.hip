@@ -308,10 +308,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
               if (i < depth) {
                 const float4 t = xr[b][j];
                 const bool tail = i >= vector_end;
-                packed = PackBytes(QuantizeElement<VARIANT>(t.x, qp, p.asymmetric, tail),
-                                   QuantizeElement<VARIANT>(t.y, qp, p.asymmetric, tail),
-                                   QuantizeElement<VARIANT>(t.z, qp, p.asymmetric, tail),
-                                   QuantizeElement<VARIANT>(t.w, qp, p.asymmetric, tail));
+                packed = QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, tail);
               }
               *reinterpret_cast<int32_t*>(qrow + i) = packed;
             }
@@ -335,10 +332,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
             if (i < depth) {
               const float4 t = *reinterpret_cast<const float4*>(x + i);
               const bool tail = i >= vector_end;
-              packed = PackBytes(QuantizeElement<VARIANT>(t.x, qp, p.asymmetric, tail),
-                                 QuantizeElement<VARIANT>(t.y, qp, p.asymmetric, tail),
-                                 QuantizeElement<VARIANT>(t.z, qp, p.asymmetric, tail),
-                                 QuantizeElement<VARIANT>(t.w, qp, p.asymmetric, tail));
+              packed = QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, tail);
             }
             *reinterpret_cast<int32_t*>(qrow + i) = packed;
           }

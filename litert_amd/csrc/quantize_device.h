@@ -75,13 +75,14 @@ __device__ __forceinline__ RowQuantParams SymmetricRowParams(float mn, float mx)
   return p;
 }
 
-// std::round (nearest, ties away from zero) in five VALU operations. trunc, the
-// subtraction and the +-1 step are all exact in float, so this is bit-identical to roundf.
+// std::round (nearest, ties away from zero) in five VALU operations: x = t + frac with
+// t = trunc(x), and trunc(2 * frac) is exactly the step to add (-1, 0 or +1: it leaves zero
+// as soon as |frac| reaches one half). trunc, the subtraction, the doubling and the final sum
+// are all exact in float, so this is bit-identical to roundf.
 __device__ __forceinline__ float RoundHalfAway(float x) {
   const float t = truncf(x);
-  const float frac = x - t;
-  const float step = copysignf(1.0f, x);
-  return fabsf(frac) >= 0.5f ? t + step : t;
+  const float frac = __fsub_rn(x, t);
+  return __fadd_rn(t, truncf(__fadd_rn(frac, frac)));
 }
 
 // The rounding used inside the NEON loops (neon_tensor_utils.cc:2347-2359).
@@ -131,6 +132,44 @@ __device__ __forceinline__ int32_t QuantizeElement(float v, const RowQuantParams
                                                    bool asymmetric, bool in_tail) {
   const int32_t q = QuantizeAsym<VARIANT>(v, p.inv, p.zero_point, in_tail);
   return asymmetric ? q : max(q, -127);
+}
+
+// The quantized value of one element as an integral float, zero point included and not yet
+// clamped: the same expressions as QuantizeAsym (adding the zero point to an integral float is
+// exact, so the NEON forms' integer addition may happen in float).
+template <int VARIANT>
+__device__ __forceinline__ float QuantizedFloat(float v, float inv, float zp, bool in_tail) {
+  if (VARIANT == LRTFC_QUANT_PORTABLE) {
+    return RoundHalfAway(__fadd_rn(zp, __fmul_rn(v, inv)));
+  }
+  if (in_tail) return __fadd_rn(zp, RoundHalfAway(__fmul_rn(inv, v)));
+  const float x = __fmul_rn(v, inv);
+  if (VARIANT == LRTFC_QUANT_NEON_LEGACY) {
+    const float nudge = __fadd_rn(x < 0.0f ? -1.0f : 0.0f, 0.5f);
+    return __fadd_rn(truncf(__fadd_rn(x, nudge)), zp);
+  }
+  return __fadd_rn(RoundHalfAway(x), zp);
+}
+
+// Four elements quantized, clamped to [-128, 127] and packed little-endian into one dword.
+// The clamp is the saturation of v_cvt_pk_u8_f32 on value + 128 (integral, so the
+// instruction's own rounding never acts); flipping the four top bits afterwards takes the 128
+// back out. A symmetric row (zero point 0, multiplier 127 / max|v|) cannot reach -128: every
+// |v * inv| stays below 127.5, so its clamp at -127 never binds and needs no instruction.
+template <int VARIANT>
+__device__ __forceinline__ int32_t QuantizePack4(float a, float b, float c, float d,
+                                                 const RowQuantParams& p, bool in_tail) {
+  const float zp = static_cast<float>(p.zero_point);
+  uint32_t w = 0;
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      __fadd_rn(QuantizedFloat<VARIANT>(a, p.inv, zp, in_tail), 128.0f), 0, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      __fadd_rn(QuantizedFloat<VARIANT>(b, p.inv, zp, in_tail), 128.0f), 1, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      __fadd_rn(QuantizedFloat<VARIANT>(c, p.inv, zp, in_tail), 128.0f), 2, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      __fadd_rn(QuantizedFloat<VARIANT>(d, p.inv, zp, in_tail), 128.0f), 3, w);
+  return static_cast<int32_t>(w ^ 0x80808080u);
 }
 
 // The multiplier the elementwise pass should use for a row.
