@@ -103,7 +103,8 @@ size_t SharedBytes(int bt, int qstride) {
 constexpr int kRing = 16;  // weight tiles in flight per wavefront
 
 // REG_ROWS: how many float rows the fused prologue may keep in registers (1, 2 or 4); a
-// smaller value frees registers. ksplit: wavefronts sharing one channel group (1, 2, 4).
+// smaller value frees registers. Without the fused prologue it scales the registers that hold
+// already quantized rows on their way to LDS (4 KiB of int8 per workgroup and unit). ksplit: wavefronts sharing one channel group (1, 2, 4).
 template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS>
 __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p, int batch0,
                                                                    int bt, int ksplit) {
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(PackedArgs p,
   // activation tiles are therefore fetched into registers first (kXRegs float4 per row per
   // thread for up to REG_ROWS rows, or kQRegs 16-byte chunks of int8), without branches;
   // larger ones are staged completely before the weights are requested.
-  constexpr int kXRegs = 4, kQRegs = 4;
+  constexpr int kXRegs = 4, kQRegs = 4 * REG_ROWS;
   const int padded = slabs * kSlabDepth;
   const int vector_end = depth - (depth % 8);
   float4 xr[REG_ROWS][kXRegs];
@@ -462,7 +463,15 @@ hipError_t LaunchSized(const PackedArgs& p, int batch0, int bt, hipStream_t stre
 
 template <Int8Epilogue EPI, bool FUSED, int VARIANT>
 hipError_t LaunchOne(const PackedArgs& p, int batch0, int bt, hipStream_t stream) {
-  if (!FUSED || bt <= 1) return LaunchSized<EPI, FUSED, VARIANT, 1>(p, batch0, bt, stream);
+  if (!FUSED) {
+    // Quantized rows that fit the registers are requested before the weights and need no
+    // wait of their own: up to 16 rows of depth 4096.
+    const int64_t row_bytes = static_cast<int64_t>(bt) * p.slabs * kSlabDepth;
+    if (row_bytes <= 16 * kThreads * 4) return LaunchSized<EPI, false, VARIANT, 1>(p, batch0, bt, stream);
+    if (row_bytes <= 16 * kThreads * 8) return LaunchSized<EPI, false, VARIANT, 2>(p, batch0, bt, stream);
+    return LaunchSized<EPI, false, VARIANT, 4>(p, batch0, bt, stream);
+  }
+  if (bt <= 1) return LaunchSized<EPI, FUSED, VARIANT, 1>(p, batch0, bt, stream);
   if (bt <= 2) return LaunchSized<EPI, FUSED, VARIANT, 2>(p, batch0, bt, stream);
   return LaunchSized<EPI, FUSED, VARIANT, 4>(p, batch0, bt, stream);
 }
