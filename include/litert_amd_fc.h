@@ -304,8 +304,11 @@ int lrtfc_fc_hybrid_int4_per_channel_nibbles(const float* input, const uint8_t* 
  *     writes a table of lrtfc_int4_group_table_bytes() into `device_table` (synchronously)
  *     and fills `launch`. count at most LRTFC_INT4_GROUP_MAX; all pointers are device
  *     pointers; bias may be NULL per node.
- *   lrtfc_fc_blockwise_int4_packed_grouped: the launch (one kernel per 4 batch rows, per 2
- *     above depth 4096); allocates and copies nothing. */
+ *   lrtfc_fc_blockwise_int4_packed_grouped: the launch (one kernel per 4 batch rows; above
+ *     depth 4096 per 2 rows, or -- when every node brought a `workspace` and there are more
+ *     than 2 rows -- one launch that quantizes all rows of all nodes into the workspaces and
+ *     one kernel per 4 rows on them, so that every filter is streamed once); allocates and
+ *     copies nothing. */
 #define LRTFC_INT4_GROUP_MAX 128
 typedef struct lrtfc_int4_group_node {
   const float* input;            /* [batches, depth] */
@@ -314,9 +317,12 @@ typedef struct lrtfc_int4_group_node {
   const float* bias;             /* [out_depth] or NULL */
   float* output;                 /* [batches, out_depth] */
   int out_depth;
+  void* workspace;               /* NULL, or lrtfc_activation_workspace_bytes(batches, depth)
+                                    bytes of this node's own, 256-byte aligned */
 } lrtfc_int4_group_node;
 typedef struct lrtfc_int4_group_launch {
   int count, grid_blocks, ksplit, groups_per_wave, batches, depth;
+  int split_quantize;            /* rows are quantized by a launch of their own */
 } lrtfc_int4_group_launch;
 size_t lrtfc_int4_group_table_bytes(void);
 int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,

@@ -109,10 +109,12 @@ def init(device=0):
 class Int4GroupNode(C.Structure):
     """lrtfc_int4_group_node."""
     _fields_ = [("input", C.c_void_p), ("retiled_filter", C.c_void_p), ("kfsum", C.c_void_p),
-                ("bias", C.c_void_p), ("output", C.c_void_p), ("out_depth", C.c_int)]
+                ("bias", C.c_void_p), ("output", C.c_void_p), ("out_depth", C.c_int),
+                ("workspace", C.c_void_p)]
 
 
 class Int4GroupLaunch(C.Structure):
     """lrtfc_int4_group_launch."""
     _fields_ = [("count", C.c_int), ("grid_blocks", C.c_int), ("ksplit", C.c_int),
-                ("groups_per_wave", C.c_int), ("batches", C.c_int), ("depth", C.c_int)]
+                ("groups_per_wave", C.c_int), ("batches", C.c_int), ("depth", C.c_int),
+                ("split_quantize", C.c_int)]

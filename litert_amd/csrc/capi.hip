@@ -49,27 +49,13 @@ constexpr int kGemmMinBatches = 128;
 // wins; beyond it the GEMM, which streams the filter once.
 constexpr int kPackedGemmMinBatches = 32;
 
-// Workspace layout for the hybrid paths: quantized activations, then scaling
-// factors, then zero points, each 256-byte aligned.
-size_t AlignUp(size_t v, size_t a) { return (v + a - 1) / a * a; }
-struct Workspace {
-  int8_t* q;
-  float* sf;
-  int32_t* zp;
-};
+// Workspace layout for the hybrid paths (kernels.h).
+using Workspace = lrtfc::ActivationWorkspace;
 size_t WorkspaceBytes(int batches, int depth) {
-  return AlignUp(static_cast<size_t>(batches) * depth, 256) +
-         2 * AlignUp(static_cast<size_t>(batches) * 4, 256);
+  return lrtfc::ActivationWorkspaceBytes(batches, depth);
 }
 Workspace SplitWorkspace(void* base, int batches, int depth) {
-  char* p = static_cast<char*>(base);
-  Workspace w;
-  w.q = reinterpret_cast<int8_t*>(p);
-  p += AlignUp(static_cast<size_t>(batches) * depth, 256);
-  w.sf = reinterpret_cast<float*>(p);
-  p += AlignUp(static_cast<size_t>(batches) * 4, 256);
-  w.zp = reinterpret_cast<int32_t*>(p);
-  return w;
+  return lrtfc::SplitActivationWorkspace(base, batches, depth);
 }
 
 }  // namespace
@@ -826,6 +812,8 @@ int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int 
     LRTFC_REQUIRE(nodes[i].out_depth >= 1, "node %d has no output channels", i);
     LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(nodes[i].retiled_filter) & 15) == 0,
                   "retiled filter of node %d must be 16-byte aligned", i);
+    LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(nodes[i].workspace) & 255) == 0,
+                  "workspace of node %d must be 256-byte aligned", i);
   }
   const hipError_t err = lrtfc::PrepareInt4Group(nodes, count, batches, depth, device_table,
                                                  launch, AsStream(stream));
@@ -840,7 +828,8 @@ int lrtfc_fc_blockwise_int4_packed_grouped(const void* device_table,
   LRTFC_REQUIRE(launch->count >= 1 && launch->count <= LRTFC_INT4_GROUP_MAX &&
                     launch->grid_blocks >= 1 && launch->ksplit >= 1 && launch->ksplit <= 4 &&
                     launch->groups_per_wave >= 1 && launch->groups_per_wave <= 8 &&
-                    (launch->ksplit == 1 || launch->groups_per_wave == 1),
+                    (launch->ksplit == 1 || launch->groups_per_wave == 1) &&
+                    (launch->split_quantize == 0 || launch->split_quantize == 1),
                 "launch record was not filled by lrtfc_int4_group_prepare");
   LRTFC_REQUIRE(quant_variant >= 0 && quant_variant <= LRTFC_QUANT_NEON_LEGACY,
                 "unknown quantizer variant");

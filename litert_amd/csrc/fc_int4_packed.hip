@@ -567,7 +567,7 @@ struct Int4GroupTable {
   Int4PackedArgs node[kMaxGroupNodes];
 };
 
-template <int BT, int VARIANT, int GPT>
+template <int BT, bool FUSED, int VARIANT, int GPT>
 __global__ __launch_bounds__(kThreads) void FcInt4PackedGroupedKernel(
     const Int4GroupTable* __restrict__ table, int count, int batch0, int bt, int ksplit,
     int gpw) {
@@ -585,8 +585,23 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedGroupedKernel(
   }
   node = __builtin_amdgcn_readfirstlane(node);
   const Int4PackedArgs a = table->node[node];
-  FcInt4PackedBody<BT, true, VARIANT, GPT>(a, blockIdx.x - table->first_block[node], batch0, bt,
-                                           ksplit, gpw, smem);
+  FcInt4PackedBody<BT, FUSED, VARIANT, GPT>(a, blockIdx.x - table->first_block[node], batch0, bt,
+                                            ksplit, gpw, smem);
+}
+
+// The row quantizer for a whole group: workgroup r quantizes row r % batches of node
+// r / batches into that node's workspace (EvalBlockwise4Bit always quantizes asymmetrically,
+// tflite/kernels/fully_connected.cc:1044-1047).
+template <int VARIANT>
+__global__ __launch_bounds__(kQuantizeThreads) void QuantizeGroupRowsKernel(
+    const Int4GroupTable* __restrict__ table, int batches) {
+  const int node = blockIdx.x / batches;
+  const int row = blockIdx.x - node * batches;
+  const Int4PackedArgs& a = table->node[node];
+  QuantizeRow<VARIANT>(a.input_f32 + static_cast<size_t>(row) * a.depth, a.depth,
+                       const_cast<int8_t*>(a.input_q) + static_cast<size_t>(row) * a.depth,
+                       const_cast<float*>(a.scaling_factors) + row,
+                       const_cast<int32_t*>(a.zero_points) + row, /*do_asymmetric=*/1);
 }
 
 // Wavefronts per channel group: one while that already gives the chip ~1000 wavefronts;
@@ -741,6 +756,10 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
   const int ksplit = ChooseKsplit(total_out, chunks);
   const int gpw = ChooseGroupsPerWave((total_out + kTileRows - 1) / kTileRows, chunks, ksplit);
   const int groups_per_wg = kWaves / ksplit * gpw;
+  // Deep rows keep at most two in registers through the fused prologue; more rows are
+  // quantized by a launch of their own when every node has a workspace to receive them.
+  bool split = depth > kShallowDepth && depth <= kDeepDepth && batches > 2;
+  for (int i = 0; i < count; ++i) split = split && nodes[i].workspace != nullptr;
   Int4GroupTable host{};
   int next = 0;
   for (int i = 0; i < count; ++i) {
@@ -751,6 +770,12 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
     a.input_q = nullptr;
     a.scaling_factors = nullptr;
     a.zero_points = nullptr;
+    if (split) {
+      const ActivationWorkspace w = SplitActivationWorkspace(nodes[i].workspace, batches, depth);
+      a.input_q = w.q;
+      a.scaling_factors = w.sf;
+      a.zero_points = w.zp;
+    }
     a.kfsum = nodes[i].kfsum;
     a.bias = nodes[i].bias;
     a.output = nodes[i].output;
@@ -772,19 +797,20 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
   launch->groups_per_wave = gpw;
   launch->batches = batches;
   launch->depth = depth;
+  launch->split_quantize = split ? 1 : 0;
   return hipSuccess;
 }
 
 size_t Int4GroupTableBytes() { return sizeof(Int4GroupTable); }
 
 namespace {
-template <int BT, int VARIANT, int GPT>
+template <int BT, bool FUSED, int VARIANT, int GPT>
 hipError_t LaunchGroupedOne(const void* table, const lrtfc_int4_group_launch& l, int batch0,
                             int bt, hipStream_t stream) {
   const int chunks = (l.depth / kBlock + kTileBlocks - 1) / kTileBlocks;
   const int padded = chunks * kTileBlocks * kBlock;
   const size_t lds = Int4Shared<BT>::Bytes(padded, l.ksplit);
-  auto kernel = FcInt4PackedGroupedKernel<BT, VARIANT, GPT>;
+  auto kernel = FcInt4PackedGroupedKernel<BT, FUSED, VARIANT, GPT>;
   if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   hipLaunchKernelGGL(kernel, dim3(l.grid_blocks), dim3(kThreads), lds, stream,
                      static_cast<const Int4GroupTable*>(table), l.count, batch0, bt, l.ksplit,
@@ -797,18 +823,51 @@ hipError_t LaunchGroupedVariant(const void* table, const lrtfc_int4_group_launch
                                 int batch0, int bt, hipStream_t stream) {
   switch (variant) {
     case LRTFC_QUANT_NEON_V8:
-      return LaunchGroupedOne<BT, LRTFC_QUANT_NEON_V8, GPT>(table, l, batch0, bt, stream);
+      return LaunchGroupedOne<BT, true, LRTFC_QUANT_NEON_V8, GPT>(table, l, batch0, bt, stream);
     case LRTFC_QUANT_NEON_LEGACY:
-      return LaunchGroupedOne<BT, LRTFC_QUANT_NEON_LEGACY, GPT>(table, l, batch0, bt, stream);
+      return LaunchGroupedOne<BT, true, LRTFC_QUANT_NEON_LEGACY, GPT>(table, l, batch0, bt, stream);
     default:
-      return LaunchGroupedOne<BT, LRTFC_QUANT_PORTABLE, GPT>(table, l, batch0, bt, stream);
+      return LaunchGroupedOne<BT, true, LRTFC_QUANT_PORTABLE, GPT>(table, l, batch0, bt, stream);
   }
+}
+
+hipError_t LaunchGroupQuantizer(const void* table, const lrtfc_int4_group_launch& l, int variant,
+                                hipStream_t stream) {
+  const auto* t = static_cast<const Int4GroupTable*>(table);
+  const dim3 grid(static_cast<unsigned>(l.count) * l.batches), block(kQuantizeThreads);
+  switch (variant) {
+    case LRTFC_QUANT_NEON_V8:
+      hipLaunchKernelGGL(QuantizeGroupRowsKernel<LRTFC_QUANT_NEON_V8>, grid, block, 0, stream, t,
+                         l.batches);
+      break;
+    case LRTFC_QUANT_NEON_LEGACY:
+      hipLaunchKernelGGL(QuantizeGroupRowsKernel<LRTFC_QUANT_NEON_LEGACY>, grid, block, 0, stream,
+                         t, l.batches);
+      break;
+    default:
+      hipLaunchKernelGGL(QuantizeGroupRowsKernel<LRTFC_QUANT_PORTABLE>, grid, block, 0, stream, t,
+                         l.batches);
+      break;
+  }
+  return hipGetLastError();
 }
 }  // namespace
 
 hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_launch& l,
                                      int variant, hipStream_t stream) {
   if (l.count < 1 || l.grid_blocks < 1) return hipSuccess;
+  if (l.split_quantize) {
+    if (hipError_t err = LaunchGroupQuantizer(table, l, variant, stream)) return err;
+    for (int batch0 = 0; batch0 < l.batches; batch0 += 4) {
+      const int bt = min(4, l.batches - batch0);
+      const hipError_t err =
+          bt <= 1   ? LaunchGroupedOne<1, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream)
+          : bt <= 2 ? LaunchGroupedOne<2, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream)
+                    : LaunchGroupedOne<4, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream);
+      if (err != hipSuccess) return err;
+    }
+    return hipSuccess;
+  }
   const bool deep = l.depth > kShallowDepth && l.depth <= kDeepDepth;
   const int tile = MaxBatchTile<true>(l.depth);
   for (int batch0 = 0; batch0 < l.batches; batch0 += tile) {  // more rows: one launch per tile

@@ -17,6 +17,29 @@ namespace lrtfc {
 hipError_t EnsureDynamicLds(const void* kernel, size_t bytes);
 
 
+// Layout of the activation workspace of lrtfc_activation_workspace_bytes(batches, depth):
+// quantized rows, then scaling factors, then zero points, each region on a 256-byte boundary.
+struct ActivationWorkspace {
+  int8_t* q;
+  float* sf;
+  int32_t* zp;
+};
+inline size_t AlignUp256(size_t v) { return (v + 255) / 256 * 256; }
+inline size_t ActivationWorkspaceBytes(int batches, int depth) {
+  return AlignUp256(static_cast<size_t>(batches) * depth) +
+         2 * AlignUp256(static_cast<size_t>(batches) * 4);
+}
+inline ActivationWorkspace SplitActivationWorkspace(void* base, int batches, int depth) {
+  char* p = static_cast<char*>(base);
+  ActivationWorkspace w;
+  w.q = reinterpret_cast<int8_t*>(p);
+  p += AlignUp256(static_cast<size_t>(batches) * depth);
+  w.sf = reinterpret_cast<float*>(p);
+  p += AlignUp256(static_cast<size_t>(batches) * 4);
+  w.zp = reinterpret_cast<int32_t*>(p);
+  return w;
+}
+
 // Arguments of the int8-weight kernels (full-integer and hybrid epilogues).
 struct FcInt8Args {
   const int8_t* input;   // [batches, depth] int8 (quantized activations)

@@ -182,6 +182,115 @@ __device__ __forceinline__ int32_t PackBytes(int32_t a, int32_t b, int32_t c, in
   return (a & 0xFF) | ((b & 0xFF) << 8) | ((c & 0xFF) << 16) | (static_cast<uint32_t>(d) << 24);
 }
 
+// ---- one row by one workgroup (the standalone quantizer kernels) ------------------------
+
+constexpr int kQuantizeThreads = 256;
+
+struct RowRange {
+  float mn;
+  float mx;
+};
+
+// Block-wide min and max. Every thread returns the same pair.
+__device__ __forceinline__ RowRange BlockMinMax(float mn, float mx) {
+  __shared__ float s_min[kQuantizeThreads / kWaveSize];
+  __shared__ float s_max[kQuantizeThreads / kWaveSize];
+  mn = WaveMinF32(mn);
+  mx = WaveMaxF32(mx);
+  const int wave = threadIdx.x / kWaveSize;
+  if ((threadIdx.x & (kWaveSize - 1)) == 0) {
+    s_min[wave] = mn;
+    s_max[wave] = mx;
+  }
+  __syncthreads();
+  RowRange r{s_min[0], s_max[0]};
+#pragma unroll
+  for (int w = 1; w < kQuantizeThreads / kWaveSize; ++w) {
+    r.mn = fminf(r.mn, s_min[w]);
+    r.mx = fmaxf(r.mx, s_max[w]);
+  }
+  return r;
+}
+
+// One row through BatchQuantizeFloats by one workgroup of kQuantizeThreads threads: v[n_data]
+// -> q[n_data], *scaling_factor, *zero_point (may be null).
+template <int VARIANT>
+__device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_data,
+                                            int8_t* __restrict__ q,
+                                            float* __restrict__ scaling_factor,
+                                            int32_t* __restrict__ zero_point, int do_asymmetric) {
+  const bool vec_ok = (n_data % 4 == 0) && ((reinterpret_cast<uintptr_t>(v) & 15) == 0) &&
+                      ((reinterpret_cast<uintptr_t>(q) & 3) == 0);
+
+  // Pass 1: range of the row. Starting from 0 gives min(0, min v) / max(0, max v),
+  // which is also what max(|min|, |max|) needs for the symmetric case.
+  float mn = 0.0f, mx = 0.0f;
+  if (vec_ok) {
+    const float4* v4 = reinterpret_cast<const float4*>(v);
+    for (int i = threadIdx.x; i < n_data / 4; i += kQuantizeThreads) {
+      const float4 t = v4[i];
+      mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
+      mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
+    }
+  } else {
+    for (int i = threadIdx.x; i < n_data; i += kQuantizeThreads) {
+      mn = fminf(mn, v[i]);
+      mx = fmaxf(mx, v[i]);
+    }
+  }
+  const RowRange range = BlockMinMax(mn, mx);
+
+  // Scale and zero point, every thread redundantly (a few dozen flops).
+  const RowQuantParams qp = do_asymmetric ? AsymmetricRowParams<VARIANT>(range.mn, range.mx)
+                                          : SymmetricRowParams(range.mn, range.mx);
+  const float sf = qp.scale;
+  const float inv = qp.inv;
+  const int32_t zp = qp.zero_point;
+  const bool all_zero = qp.all_zero;
+  if (threadIdx.x == 0) {
+    *scaling_factor = sf;
+    if (zero_point) *zero_point = zp;
+  }
+
+  // Pass 2: elementwise. The NEON builds process 8 floats per step and finish
+  // the remaining n_data % 8 with a scalar expression that rounds differently.
+  const int vector_end = n_data - (n_data % 8);
+  if (vec_ok) {
+    const float4* v4 = reinterpret_cast<const float4*>(v);
+    char4* q4 = reinterpret_cast<char4*>(q);
+    for (int i = threadIdx.x; i < n_data / 4; i += kQuantizeThreads) {
+      char4 o;
+      if (all_zero) {
+        o = make_char4(0, 0, 0, 0);
+      } else {
+        const float4 t = v4[i];
+        const bool tail = 4 * i >= vector_end;
+        if (do_asymmetric) {
+          const int32_t packed = QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, tail);
+          o = make_char4(static_cast<char>(packed), static_cast<char>(packed >> 8),
+                         static_cast<char>(packed >> 16), static_cast<char>(packed >> 24));
+        } else {
+          o.x = static_cast<char>(QuantizeSym<VARIANT>(t.x, inv, tail));
+          o.y = static_cast<char>(QuantizeSym<VARIANT>(t.y, inv, tail));
+          o.z = static_cast<char>(QuantizeSym<VARIANT>(t.z, inv, tail));
+          o.w = static_cast<char>(QuantizeSym<VARIANT>(t.w, inv, tail));
+        }
+      }
+      q4[i] = o;
+    }
+  } else {
+    for (int i = threadIdx.x; i < n_data; i += kQuantizeThreads) {
+      int8_t o = 0;
+      if (!all_zero) {
+        const bool tail = i >= vector_end;
+        o = static_cast<int8_t>(do_asymmetric ? QuantizeAsym<VARIANT>(v[i], inv, zp, tail)
+                                              : QuantizeSym<VARIANT>(v[i], inv, tail));
+      }
+      q[i] = o;
+    }
+  }
+}
+
 }  // namespace lrtfc
 
 #endif  // LITERT_AMD_CSRC_QUANTIZE_DEVICE_H_

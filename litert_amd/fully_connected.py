@@ -436,6 +436,14 @@ class GroupedBlockwiseInt4:
         """inputs[i] [B, depth] float32, outputs[i] [B, out_depth_i] float32, CUDA, contiguous."""
         batches = inputs[0].numel() // self.depth
         nodes = (capi.Int4GroupNode * len(self.ops))()
+        # Deep rows beyond two per launch are quantized into per-node workspaces first, so that
+        # every filter is streamed once (same rule as FullyConnectedBlockwiseInt4.__call__).
+        workspaces = None
+        if (self.depth > FullyConnectedBlockwiseInt4.FUSED_MAX_DEPTH
+                and batches > FullyConnectedBlockwiseInt4.DEEP_FUSED_MAX_BATCHES):
+            need = capi.load().lrtfc_activation_workspace_bytes(batches, self.depth)
+            workspaces = torch.empty((len(self.ops), (need + 255) // 256 * 256), dtype=torch.uint8,
+                                     device="cuda")
         for i, (op, x, y) in enumerate(zip(self.ops, inputs, outputs)):
             if not (x.is_contiguous() and y.is_contiguous()):
                 raise ValueError("grouped inputs and outputs must be contiguous")
@@ -447,12 +455,13 @@ class GroupedBlockwiseInt4:
             nodes[i].bias = op.bias.data_ptr() if op.bias is not None else None
             nodes[i].output = y.data_ptr()
             nodes[i].out_depth = op.out_depth
+            nodes[i].workspace = workspaces[i].data_ptr() if workspaces is not None else None
         launch = capi.Int4GroupLaunch()
         capi.check(capi.load().lrtfc_int4_group_prepare(
             C.byref(nodes), len(self.ops), batches, self.depth, _ptr(self.table),
             C.byref(launch), _stream()))
         self.launch = launch
-        self._bound = (list(inputs), list(outputs))  # keep the tensors alive
+        self._bound = (list(inputs), list(outputs), workspaces)  # keep the tensors alive
         return self
 
     def __call__(self):

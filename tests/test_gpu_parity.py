@@ -388,6 +388,8 @@ def test_blockwise_int4_split_launch_matches_oracle(fc, B, K, N):
 @pytest.mark.parametrize("B,K,Ns", [(1, 2048, (64, 8, 24, 130, 520)), (3, 2048, (16, 256, 9)),
                                     (4, 1024, (40,)), (1, 16384, (16, 40)), (2, 8192, (24, 8, 72)),
                                     (9, 2048, (24, 80)), (5, 16384, (8, 16)),
+                                    # deep rows beyond two: quantized by the group's own launch
+                                    (3, 8192, (24, 40, 8)), (4, 16384, (16, 264)), (9, 8192, (8, 72)),
                                     (1, 64, tuple(range(4, 36))), (2, 64, tuple(range(3, 103)))])
 def test_blockwise_int4_grouped_launch_matches_oracle(fc, B, K, Ns):
     """Several filters of one depth in one launch: every node against the oracle, with its
@@ -432,6 +434,27 @@ def test_blockwise_int4_wavefronts_spanning_channel_groups(fc, B):
     for ci, yi, n in zip(cs, ys, Ns):
         want = oracle.fc_blockwise_int4(ci["x"], ci["packed"], n, ci["scales"].view(np.uint16), 32)
         assert _bits_equal(yi.cpu().numpy(), want), n
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+def test_blockwise_int4_grouped_deep_rows_quantizer_variants(fc, variant):
+    """The group's row quantizer launch (deep rows, more than two per node) in the two NEON
+    flavours, with elements on rounding ties."""
+    B, K, Ns = 4, 8200 - 8, (16, 24)
+    cs = [wl.blockwise_int4_fc(B, K, n, seed=40 + n) for n in Ns]
+    for c in cs:
+        c["x"][0, :4] = [-125.0, 130.0, 2.5, -2.5]
+    ops = [fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], K, 32, quant_variant=variant)
+           for c in cs]
+    ys = [torch.empty((B, n), dtype=torch.float32, device="cuda") for n in Ns]
+    group = fc.GroupedBlockwiseInt4(ops).bind([_cuda(c["x"]) for c in cs], ys)
+    assert group.launch.split_quantize == 1
+    group()
+    torch.cuda.synchronize()
+    for c, y, n in zip(cs, ys, Ns):
+        want = oracle.fc_blockwise_int4(c["x"], c["packed"], n, c["scales"].view(np.uint16), 32,
+                                        variant=variant)
+        assert _bits_equal(y.cpu().numpy(), want), n
 
 
 def test_blockwise_int4_grouped_launch_needs_bind(fc):
