@@ -42,6 +42,7 @@ constexpr int kRingTiles = 2;
 constexpr int kPStride = kTileBlocks + 4;  // floats per (row, batch) line of parked products
 constexpr int kMaxGroupNodes = LRTFC_INT4_GROUP_MAX;
 constexpr int kMaxGroupsPerWave = 8;  // 64 channels: one lane each when their kfsum is staged
+constexpr int kSplitShallowMinBlocks = 1024;  // grouped launches: see PrepareInt4Group
 
 __global__ __launch_bounds__(kThreads) void PackInt4BlockwiseKernel(
     const uint8_t* __restrict__ filter, const uint16_t* __restrict__ scales, int out_depth,
@@ -758,7 +759,16 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
   const int groups_per_wg = kWaves / ksplit * gpw;
   // Deep rows keep at most two in registers through the fused prologue; more rows are
   // quantized by a launch of their own when every node has a workspace to receive them.
-  bool split = depth > kShallowDepth && depth <= kDeepDepth && batches > 2;
+  // Shallow rows do the same only in launches of many workgroups, where quantizing each row
+  // once instead of once per workgroup outweighs the extra launch (config 5, B = 4: the 108
+  // nodes of depth 2048 in 272 instead of 280 us per token; groups of one to three nodes lose).
+  int total_blocks = 0;
+  for (int i = 0; i < count; ++i) {
+    const int groups = (nodes[i].out_depth + kTileRows - 1) / kTileRows;
+    total_blocks += (groups + groups_per_wg - 1) / groups_per_wg;
+  }
+  bool split = batches > 2 && depth <= kDeepDepth &&
+               (depth > kShallowDepth || total_blocks >= kSplitShallowMinBlocks);
   for (int i = 0; i < count; ++i) split = split && nodes[i].workspace != nullptr;
   Int4GroupTable host{};
   int next = 0;
@@ -858,12 +868,19 @@ hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_l
   if (l.count < 1 || l.grid_blocks < 1) return hipSuccess;
   if (l.split_quantize) {
     if (hipError_t err = LaunchGroupQuantizer(table, l, variant, stream)) return err;
+    const bool deep_rows = l.depth > kShallowDepth;
     for (int batch0 = 0; batch0 < l.batches; batch0 += 4) {
       const int bt = min(4, l.batches - batch0);
-      const hipError_t err =
-          bt <= 1   ? LaunchGroupedOne<1, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream)
-          : bt <= 2 ? LaunchGroupedOne<2, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream)
-                    : LaunchGroupedOne<4, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream);
+      hipError_t err;
+      if (deep_rows) {
+        err = bt <= 1   ? LaunchGroupedOne<1, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream)
+              : bt <= 2 ? LaunchGroupedOne<2, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream)
+                        : LaunchGroupedOne<4, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream);
+      } else {
+        err = bt <= 1   ? LaunchGroupedOne<1, false, LRTFC_QUANT_PORTABLE, 2>(table, l, batch0, bt, stream)
+              : bt <= 2 ? LaunchGroupedOne<2, false, LRTFC_QUANT_PORTABLE, 2>(table, l, batch0, bt, stream)
+                        : LaunchGroupedOne<4, false, LRTFC_QUANT_PORTABLE, 2>(table, l, batch0, bt, stream);
+      }
       if (err != hipSuccess) return err;
     }
     return hipSuccess;

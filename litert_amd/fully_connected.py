@@ -439,8 +439,7 @@ class GroupedBlockwiseInt4:
         # Deep rows beyond two per launch are quantized into per-node workspaces first, so that
         # every filter is streamed once (same rule as FullyConnectedBlockwiseInt4.__call__).
         workspaces = None
-        if (self.depth > FullyConnectedBlockwiseInt4.FUSED_MAX_DEPTH
-                and batches > FullyConnectedBlockwiseInt4.DEEP_FUSED_MAX_BATCHES):
+        if batches > FullyConnectedBlockwiseInt4.DEEP_FUSED_MAX_BATCHES:
             need = capi.load().lrtfc_activation_workspace_bytes(batches, self.depth)
             workspaces = torch.empty((len(self.ops), (need + 255) // 256 * 256), dtype=torch.uint8,
                                      device="cuda")
