@@ -425,6 +425,7 @@ struct PartitionKernel {
   struct Group {
     std::vector<int> members;  // node indices, ascending
     DeviceBuffer table;
+    DeviceBuffer workspace;  // one activation workspace per member when rows exceed two
     lrtfc_int4_group_launch launch{};
   };
   std::vector<Group> groups;
@@ -829,9 +830,11 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
   // other, so each such set (cut into pieces of LRTFC_INT4_GROUP_MAX) is one launch.
   k->groups.clear();
   for (FcNode& n : k->nodes) n.group = -1;
+  // (Nodes whose rows are quantized by a launch of their own group too: the group then has
+  // one such launch for all its rows, into per-node workspaces.)
   auto groupable = [&](const FcNode& n) {
-    return n.kind == FcKind::kInt4Blockwise && n.use_retiled && !n.split_quantize &&
-           n.depth > 0 && n.batches > 0 && n.out_depth > 0;
+    return n.kind == FcKind::kInt4Blockwise && n.use_retiled && n.depth > 0 && n.batches > 0 &&
+           n.out_depth > 0;
   };
   {
     std::map<std::tuple<int, int, int>, std::vector<int>> sets;  // (level, depth, batches)
@@ -908,7 +911,7 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
     k->lookup_status_dev = static_cast<int32_t*>(dev);
   }
   for (const FcNode& n : k->nodes) {
-    if (n.kind == FcKind::kEmbeddingLookup) continue;
+    if (n.kind == FcKind::kEmbeddingLookup || n.group >= 0) continue;
     if (n.kind == FcKind::kHybridInt4 ||
         (n.kind != FcKind::kInt8 && (!n.use_retiled || n.split_quantize))) {
       RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(
@@ -918,6 +921,12 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
   // Group tables: device addresses of every member's tensors (stable until the next prepare).
   for (PartitionKernel::Group& g : k->groups) {
     std::vector<lrtfc_int4_group_node> nodes(g.members.size());
+    const FcNode& head = k->nodes[g.members.front()];
+    size_t per_node = 0;
+    if (head.batches > kInt4DeepFusedMaxBatches) {
+      per_node = (lrtfc_activation_workspace_bytes(head.batches, head.depth) + 255) & ~size_t{255};
+      RETURN_IF_HIP(ctx, g.workspace.Ensure(per_node * g.members.size()));
+    }
     for (size_t m = 0; m < g.members.size(); ++m) {
       const FcNode& n = k->nodes[g.members[m]];
       nodes[m].input = static_cast<const float*>(k->Activation(n.input));
@@ -926,6 +935,7 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
       nodes[m].bias = n.bias == kTfLiteOptionalTensor ? nullptr : n.bias_dev.as<float>();
       nodes[m].output = static_cast<float*>(k->Activation(n.output));
       nodes[m].out_depth = n.out_depth;
+      nodes[m].workspace = per_node ? g.workspace.as<uint8_t>() + per_node * m : nullptr;
     }
     const FcNode& first = k->nodes[g.members.front()];
     RETURN_IF_HIP(ctx, g.table.Ensure(lrtfc_int4_group_table_bytes()));

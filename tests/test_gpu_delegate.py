@@ -591,3 +591,36 @@ def test_embedding_lookup_feeds_projections_inside_one_partition():
             want = oracle.fc_blockwise_int4(rows_f32, c["packed"], c["packed"].shape[0],
                                             c["scales"].view(np.uint16), 32)
             assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("B,K", [(3, 8192), (4, 2048)])
+def test_int4_grouped_nodes_with_more_than_two_rows(B, K):
+    """Independent blockwise-int4 nodes with three or four batch rows share one launch as well;
+    above depth 4096 the group quantizes all its rows in a launch of its own (per-node
+    workspaces owned by the partition). Outputs bit-identical to the oracle over two invokes."""
+    Ns = (16, 24, 8)
+    cs = [wl.blockwise_int4_fc(B, K, n, seed=300 + n, lo=-8, hi=7) for n in Ns]
+    rng = np.random.default_rng(5)
+    with FakeHost() as h:
+        xs, ys = [], []
+        for c, n in zip(cs, Ns):
+            x = h.tensor(FLOAT32, (B, K), data=c["x"])
+            w = h.tensor(INT4, (n, K), data=c["packed"], const=True)
+            s_ = h.tensor(FLOAT16, (n, K // 32), data=c["scales"], const=True)
+            h.blockwise(w, s_, 32)
+            y = h.tensor(FLOAT32, (B, n))
+            h.fc(x, w, None, y)
+            xs.append(x)
+            ys.append(y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        groups, text = h.describe_partition(h.plan()[0][2])
+        assert groups == 1 and text.count("/g0") == 3, text
+        for trial in range(2):
+            ins = [c["x"] if trial == 0 else rng.standard_normal((B, K)).astype(np.float32) for c in cs]
+            for x, v in zip(xs, ins):
+                h.write(x, v)
+            assert h.invoke() == OK, h.errors()
+            for c, n, y, v in zip(cs, Ns, ys, ins):
+                want = oracle.fc_blockwise_int4(v, c["packed"], n, c["scales"].view(np.uint16), 32)
+                assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32)), (trial, n)
