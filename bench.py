@@ -363,7 +363,7 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         gbps_cold=round(bytes_nib / us_nib / 1e3, 1),
         frac_of_hbm_peak_cold=round(bytes_nib / us_nib / 1e3 / HBM_PEAK_GBPS, 4),
         algorithmic_bytes=bytes_nib,
-        note="two launches each (row quantizer + GEMV); per launch pair")
+        note="4-bit-resident: one kernel (row quantizer fused into the prologue); int8 expansion: row quantizer launch + GEMV launch")
     del ops4b, nib
 
     # Next-row op: EMBEDDING_LOOKUP from a blockwise Int4 table of a 256000-token vocabulary,
