@@ -60,3 +60,13 @@ def test_no_device_is_an_error_not_a_fallback():
     # compute entry points refuse to run before a successful init
     rc = lib.lrtfc_row_sums_int8(None, 4, 16, None, None)
     assert rc == capi.NO_DEVICE
+    rc = lib.lrtfc_embedding_lookup_blockwise_int4(None, 1, None, 4, 64, None, 32, capi.OUT_FLOAT32,
+                                                   None, None, None)
+    assert rc == capi.NO_DEVICE
+    rc = lib.lrtfc_embedding_lookup_hybrid(None, 1, None, 8, 4, 64, 0.5, None, capi.OUT_FLOAT16, None,
+                                           None, None)
+    assert rc == capi.NO_DEVICE
+    # the host mirrors raise instead of computing anywhere else
+    from litert_amd import embedding_lookup as el
+    with pytest.raises(Exception):
+        el.EmbeddingLookupHybrid(np.zeros((4, 8), np.int8), 8)
