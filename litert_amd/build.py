@@ -21,6 +21,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall",
           "-Wno-unused-function", "-I" + os.path.join(ROOT, "include")]
+# Kernel-argument preloading (gfx940 and later): the leading scalar arguments of a kernel
+# arrive in registers with the wavefront instead of through a first round of scalar loads.
+COMMON += ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
 COMMON += os.environ.get("LITERT_AMD_EXTRA_HIPCC_FLAGS", "").split()
 
 FC_SOURCES = ["capi.hip", "quantize.hip", "fc_int8_gemv.hip", "fc_int8_packed_gemv.hip", "fc_int8_packed_gemm.hip",
