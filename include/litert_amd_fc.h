@@ -341,6 +341,27 @@ int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
                                       int batches, int depth, int out_depth, int blocksize,
                                       void* stream);
 
+/* ---- Blockwise-int4 FULLY_CONNECTED for prefill batches ---------------------------------
+ * EvalBlockwise4Bit (tflite/kernels/fully_connected.cc:1014-1086) as a matrix-core GEMM: the
+ * filter streams once for the whole batch instead of once per four rows. Same results, bit for
+ * bit, as lrtfc_fc_blockwise_int4 (every output adds its blocks' `float(int32 sum) * scale` in
+ * block order). Block size 32.
+ *   lrtfc_gemm_int4_blockwise_bytes / lrtfc_pack_int4_blockwise_gemm: the filter re-tiled for
+ *     this kernel (16 channels x one block per 512-byte tile, sign-extended to int8, then the
+ *     scales as float32); made once, like the other re-tilings.
+ *   lrtfc_fc_blockwise_int4_gemm_workspace_bytes: device scratch for the quantized rows in
+ *     both their forms (256-byte aligned).
+ *   lrtfc_fc_blockwise_int4_gemm: row quantizer launch, row re-tiling launch, GEMM launch. */
+size_t lrtfc_gemm_int4_blockwise_bytes(int out_depth, int depth);
+int lrtfc_pack_int4_blockwise_gemm(const uint8_t* packed_filter, const uint16_t* scales_f16,
+                                   int out_depth, int depth, int blocksize, uint8_t* gemm_filter,
+                                   void* stream);
+size_t lrtfc_fc_blockwise_int4_gemm_workspace_bytes(int batches, int depth);
+int lrtfc_fc_blockwise_int4_gemm(const float* input, const uint8_t* gemm_filter,
+                                 const float* kfsum, const float* bias, float* output,
+                                 int batches, int depth, int out_depth, int quant_variant,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- EMBEDDING_LOOKUP from quantized tables (the op that feeds a decoder's first
  * FULLY_CONNECTED nodes) ------------------------------------------------------------------ */
 

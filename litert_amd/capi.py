@@ -63,6 +63,10 @@ SYMBOLS = [
     ("lrtfc_pack_int4_per_channel", _i, [_vp, _i, _i, _vp, _vp]),
     ("lrtfc_fc_hybrid_int4_per_channel_nibbles", _i, [_vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i,
                                                       _vp, _sz, _vp]),
+    ("lrtfc_gemm_int4_blockwise_bytes", _sz, [_i, _i]),
+    ("lrtfc_pack_int4_blockwise_gemm", _i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    ("lrtfc_fc_blockwise_int4_gemm_workspace_bytes", _sz, [_i, _i]),
+    ("lrtfc_fc_blockwise_int4_gemm", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
     ("lrtfc_embedding_lookup_blockwise_int4", _i, [_vp, _i, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_embedding_lookup_hybrid", _i, [_vp, _i, _vp, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp]),
     ("lrtfc_int4_group_table_bytes", _sz, []),

@@ -747,6 +747,61 @@ int lrtfc_fc_hybrid_int4_per_channel_nibbles(const float* input, const uint8_t* 
                  "per-channel int4 hybrid GEMV (nibble layout)");
 }
 
+size_t lrtfc_gemm_int4_blockwise_bytes(int out_depth, int depth) {
+  if (out_depth <= 0 || depth <= 0) return 0;
+  return lrtfc::GemmInt4BlockwiseBytes(out_depth, depth);
+}
+
+int lrtfc_pack_int4_blockwise_gemm(const uint8_t* packed_filter, const uint16_t* scales_f16,
+                                   int out_depth, int depth, int blocksize, uint8_t* gemm_filter,
+                                   void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(out_depth >= 0 && depth >= 0, "negative dimension");
+  if (out_depth == 0 || depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(packed_filter && scales_f16 && gemm_filter, "null pointer");
+  LRTFC_REQUIRE(lrtfc::FcInt4BlockwiseGemmSupports(depth, blocksize),
+                "the int4 GEMM needs block size 32 and a depth that is a multiple of 32");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(gemm_filter) & 15) == 0,
+                "re-tiled filter must be 16-byte aligned");
+  return FromHip(lrtfc::LaunchPackInt4BlockwiseGemm(packed_filter, scales_f16, out_depth, depth,
+                                                    gemm_filter, AsStream(stream)),
+                 "int4 GEMM filter re-tiling");
+}
+
+size_t lrtfc_fc_blockwise_int4_gemm_workspace_bytes(int batches, int depth) {
+  if (batches <= 0 || depth <= 0) return 0;
+  return WorkspaceBytes(batches, depth) + lrtfc::AlignUp256(lrtfc::TiledRowsBytes(batches, depth));
+}
+
+int lrtfc_fc_blockwise_int4_gemm(const float* input, const uint8_t* gemm_filter,
+                                 const float* kfsum, const float* bias, float* output,
+                                 int batches, int depth, int out_depth, int quant_variant,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(input && gemm_filter && kfsum && output && workspace, "null pointer");
+  LRTFC_REQUIRE(lrtfc::FcInt4BlockwiseGemmSupports(depth, 32), "depth %d is not a multiple of 32",
+                depth);
+  LRTFC_REQUIRE(workspace_bytes >= lrtfc_fc_blockwise_int4_gemm_workspace_bytes(batches, depth),
+                "workspace too small: %zu < %zu bytes", workspace_bytes,
+                lrtfc_fc_blockwise_int4_gemm_workspace_bytes(batches, depth));
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
+                "workspace must be 256-byte aligned");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(gemm_filter) & 15) == 0,
+                "re-tiled filter must be 16-byte aligned");
+  const Workspace w = SplitWorkspace(workspace, batches, depth);
+  void* tiled = static_cast<char*>(workspace) + WorkspaceBytes(batches, depth);
+  // EvalBlockwise4Bit always quantizes asymmetrically (fully_connected.cc:1044-1047).
+  int rc = lrtfc_batch_quantize_floats(input, batches, depth, w.q, w.sf, w.zp,
+                                       /*do_asymmetric=*/1, quant_variant, stream);
+  if (rc != LRTFC_OK) return rc;
+  return FromHip(lrtfc::LaunchFcInt4BlockwiseGemm(w.q, w.sf, w.zp, gemm_filter, kfsum, bias,
+                                                  output, batches, depth, out_depth, tiled,
+                                                  AsStream(stream)),
+                 "blockwise int4 GEMM");
+}
+
 int lrtfc_embedding_lookup_blockwise_int4(const int32_t* lookup, int count, const uint8_t* table,
                                           int rows, int cols, const uint16_t* scales_f16,
                                           int blocksize, int out_type, void* output,

@@ -1,0 +1,328 @@
+// Blockwise-int4 FULLY_CONNECTED for prefill batches on gfx950: EvalBlockwise4Bit
+// (tflite/kernels/fully_connected.cc:1014-1086) as a matrix-core GEMM.
+//
+// The decode kernel (fc_int4_packed.hip) streams the whole filter once per four batch rows,
+// which is right for one to a few rows and hopeless for hundreds. Here every (row, channel)
+// output keeps its float32 accumulator in a register and walks the blocks of 32 depth
+// positions in order: one v_mfma_i32_16x16x32_i8 per block and 16 x 16 tile gives the exact
+// int32 block sums (its K is exactly one block), and three vector operations per output add
+// `float(sum) * scale[channel][block]` to the accumulator -- the reference's own order of
+// float operations (:1069-1077), unfused, so the results are bit-identical to the decode
+// kernel's and the oracle's. Those three operations per output and block, not the matrix
+// cores, bound the kernel (the MFMA of a block takes 16 cycles, its 4 outputs per lane 48).
+//
+// Layouts, made once at prepare (filter) or per call (activations):
+//   filter `tile16x32s`: for channel tile t (16 channels) and block b, 512 bytes: lane L's 8
+//     bytes are channel 16 t + L % 16, depths 32 b + 8 (L / 16) ... + 8, sign-extended to
+//     int8 -- the A operand of the MFMA as one 8-byte load per lane; after all tiles, the block
+//     scales as float32, 16 per (t, b), so that a lane reads the scales of its four output
+//     channels in one 16-byte load.
+//   activations `tile16x32`: the same with batch rows in place of channels (B operand), made
+//     from the row-major int8 rows of the standalone quantizer.
+// No LDS: a wavefront owns CT x RT tiles (16 to 32 channels x 16 to 64 rows, by batch size)
+// and requests the operands of the next blocks while it works on the current one (a ring of
+// kStages blocks in registers); both operands are re-read by other wavefronts from L2.
+#include "kernels.h"
+
+namespace lrtfc {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kBlock = 32;    // depth positions per quantization block
+constexpr int kTile = 16;     // channels / rows per MFMA tile
+// A wavefront owns CT x RT tiles of 16 channels x 16 rows (template parameters of the kernel);
+// a workgroup is 2 x 2 wavefronts.
+
+using i64 = long;
+
+__device__ __forceinline__ int SignedNibble(uint32_t byte, int high) {
+  const int n = high ? (byte >> 4) : (byte & 0xF);
+  return (n ^ 8) - 8;
+}
+
+// Model layout (rows of depth / 2 bytes, low nibble = even depth; fp16 scales [N, nb]) ->
+// tile16x32s + float32 scales. One thread per 8-byte lane slot of the tile array.
+__global__ __launch_bounds__(kThreads) void PackInt4BlockwiseGemmKernel(
+    const uint8_t* __restrict__ filter, const uint16_t* __restrict__ scales_f16, int out_depth,
+    int depth, int tiles, int nb, uint8_t* __restrict__ dst) {
+  const int64_t slot = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t slots = static_cast<int64_t>(tiles) * nb * 64;
+  if (slot < slots) {
+    const int lane = static_cast<int>(slot & 63);
+    const int64_t tb = slot >> 6;
+    const int b = static_cast<int>(tb % nb);
+    const int t = static_cast<int>(tb / nb);
+    const int n = t * kTile + (lane & 15);
+    const int k0 = b * kBlock + 8 * (lane >> 4);
+    uint32_t lo = 0, hi = 0;
+    if (n < out_depth) {
+      const uint8_t* src = filter + static_cast<size_t>(n) * (depth / 2) + k0 / 2;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t byte = src[j];
+        const uint32_t pair = (static_cast<uint32_t>(SignedNibble(byte, 0)) & 0xFF) |
+                              (static_cast<uint32_t>(SignedNibble(byte, 1)) & 0xFF) << 8;
+        if (j < 2) {
+          lo |= pair << (16 * j);
+        } else {
+          hi |= pair << (16 * (j - 2));
+        }
+      }
+    }
+    reinterpret_cast<uint2*>(dst)[slot] = make_uint2(lo, hi);
+  }
+  // scales: one thread per (tile, block, channel)
+  const int64_t scale_slots = static_cast<int64_t>(tiles) * nb * kTile;
+  if (slot < scale_slots) {
+    const int c = static_cast<int>(slot & 15);
+    const int64_t tb = slot >> 4;
+    const int b = static_cast<int>(tb % nb);
+    const int t = static_cast<int>(tb / nb);
+    const int n = t * kTile + c;
+    float* out = reinterpret_cast<float*>(dst + slots * 8);
+    out[slot] = n < out_depth ? HalfBitsToFloatFast(scales_f16[static_cast<size_t>(n) * nb + b]) : 0.0f;
+  }
+}
+
+// Row-major int8 rows [batches, depth] -> tile16x32 (rows past the batch are zero).
+__global__ __launch_bounds__(kThreads) void TileQuantizedRowsKernel(
+    const int8_t* __restrict__ rows, int batches, int depth, int row_tiles, int nb,
+    uint2* __restrict__ dst) {
+  const int64_t slot = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (slot >= static_cast<int64_t>(row_tiles) * nb * 64) return;
+  const int lane = static_cast<int>(slot & 63);
+  const int64_t tb = slot >> 6;
+  const int b = static_cast<int>(tb % nb);
+  const int t = static_cast<int>(tb / nb);
+  const int m = t * kTile + (lane & 15);
+  uint2 v = make_uint2(0, 0);
+  if (m < batches) {
+    v = *reinterpret_cast<const uint2*>(rows + static_cast<size_t>(m) * depth + b * kBlock +
+                                        8 * (lane >> 4));
+  }
+  dst[slot] = v;
+}
+
+struct GemmArgs {
+  const i64* filter;        // tile16x32s
+  const float4* scales;     // float32 [tiles][nb][16] viewed as float4
+  const i64* activations;   // tile16x32
+  const float* scaling_factors;  // [batches]
+  const int32_t* zero_points;    // [batches]
+  const float* kfsum;            // [out_depth]
+  const float* bias;             // [out_depth] or nullptr
+  float* output;                 // [batches, out_depth]
+  int batches, out_depth, nb;
+  int channel_tiles, row_tiles;  // of 16
+  int vector_store;              // rows of the output start on 16-byte boundaries
+};
+
+template <int CT, int RT>
+struct Stage {
+  i64 w[CT];      // channel tiles
+  float4 s[CT];   // their scales for this lane's four channels
+  i64 x[RT];      // row tiles
+};
+
+// WROWS: wavefronts of a workgroup along the batch rows (1 or 2); the others along the channels.
+template <int CT, int RT, int WROWS>
+__global__ __launch_bounds__(kThreads) void FcInt4BlockwiseGemmKernel(GemmArgs a) {
+  constexpr int WCH = 4 / WROWS;
+  // Blocks in flight per wavefront: one or two tiles per block are bound by the filter stream
+  // and want many (16 rows: 33 us with 4, 27 us with 16); larger tiles are bound by their
+  // arithmetic and run best with 4.
+  constexpr int kStages = CT * RT <= 2 ? 16 : 4;
+  const int lane = threadIdx.x & 63;
+  // The wavefront index as a scalar: tile addresses then stay in scalar registers and every
+  // load is "scalar base + lane offset".
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // Workgroups walk the channel direction fastest: neighbours share activation tiles in L2.
+  const int wg_c = blockIdx.x, wg_r = blockIdx.y;
+  const int ct0 = (wg_c * WCH + wave % WCH) * CT;
+  const int rt0 = (wg_r * WROWS + wave / WCH) * RT;
+  if (ct0 >= a.channel_tiles || rt0 >= a.row_tiles) return;
+  // Tiles past the edge re-read the last valid one; their outputs are never stored.
+  int ct[CT], rt[RT];
+#pragma unroll
+  for (int j = 0; j < CT; ++j) ct[j] = min(ct0 + j, a.channel_tiles - 1);
+#pragma unroll
+  for (int j = 0; j < RT; ++j) rt[j] = min(rt0 + j, a.row_tiles - 1);
+  const int nb = a.nb;
+  const i64* wp[CT];
+  const float4* sp[CT];
+  const i64* xp[RT];
+#pragma unroll
+  for (int j = 0; j < CT; ++j) {
+    wp[j] = a.filter + static_cast<size_t>(ct[j]) * nb * 64 + lane;
+    sp[j] = a.scales + static_cast<size_t>(ct[j]) * nb * 4 + (lane >> 4);
+  }
+#pragma unroll
+  for (int j = 0; j < RT; ++j) xp[j] = a.activations + static_cast<size_t>(rt[j]) * nb * 64 + lane;
+  auto fetch = [&](int b) {
+    const int bb = min(b, nb - 1);  // past the end: a hot line, result unused
+    Stage<CT, RT> st;
+#pragma unroll
+    for (int j = 0; j < CT; ++j) {
+      st.w[j] = wp[j][static_cast<size_t>(bb) * 64];
+      st.s[j] = sp[j][static_cast<size_t>(bb) * 4];
+    }
+#pragma unroll
+    for (int j = 0; j < RT; ++j) st.x[j] = xp[j][static_cast<size_t>(bb) * 64];
+    return st;
+  };
+  Stage<CT, RT> ring[kStages];
+#pragma unroll
+  for (int s = 0; s < kStages; ++s) ring[s] = fetch(s);
+
+  // out[cj][rj][i]: channel 16 ct[cj] + 4 (lane / 16) + i, batch row 16 rt[rj] + lane % 16.
+  float out[CT][RT][4];
+#pragma unroll
+  for (int cj = 0; cj < CT; ++cj)
+#pragma unroll
+    for (int rj = 0; rj < RT; ++rj)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[cj][rj][i] = 0.0f;
+
+  const i32x4 zero = {0, 0, 0, 0};
+  for (int base = 0; base < nb; base += kStages) {
+#pragma unroll
+    for (int s = 0; s < kStages; ++s) {
+      const Stage<CT, RT> st = ring[s];
+      ring[s] = fetch(base + kStages + s);
+      if (base + s < nb) {
+#pragma unroll
+        for (int cj = 0; cj < CT; ++cj) {
+          const float sc[4] = {st.s[cj].x, st.s[cj].y, st.s[cj].z, st.s[cj].w};
+#pragma unroll
+          for (int rj = 0; rj < RT; ++rj) {
+            const i32x4 acc =
+                __builtin_amdgcn_mfma_i32_16x16x32_i8(st.w[cj], st.x[rj], zero, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              out[cj][rj][i] =
+                  __fadd_rn(out[cj][rj][i], __fmul_rn(static_cast<float>(acc[i]), sc[i]));
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // fully_connected.cc:1078-1082: zero-point term, row scale, bias.
+#pragma unroll
+  for (int rj = 0; rj < RT; ++rj) {
+    if (rt0 + rj >= a.row_tiles) break;
+    const int m = rt[rj] * kTile + (lane & 15);
+    if (m >= a.batches) continue;
+    const float zp = static_cast<float>(a.zero_points[m]);
+    const float row_scale = a.scaling_factors[m];
+#pragma unroll
+    for (int cj = 0; cj < CT; ++cj) {
+      if (ct0 + cj >= a.channel_tiles) break;
+      const int n0 = ct[cj] * kTile + 4 * (lane >> 4);
+      float o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = min(n0 + i, a.out_depth - 1);
+        float v = __fsub_rn(out[cj][rj][i], __fmul_rn(zp, a.kfsum[n]));
+        v = __fmul_rn(v, row_scale);
+        if (a.bias) v = __fadd_rn(v, a.bias[n]);
+        o[i] = v;
+      }
+      float* dst = a.output + static_cast<size_t>(m) * a.out_depth + n0;
+      if (n0 + 3 < a.out_depth && a.vector_store) {
+        *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (n0 + i < a.out_depth) dst[i] = o[i];
+        }
+      }
+    }
+  }
+}
+
+}  // namespace
+
+size_t GemmInt4BlockwiseBytes(int out_depth, int depth) {
+  const size_t tiles = (static_cast<size_t>(out_depth) + kTile - 1) / kTile;
+  const size_t nb = static_cast<size_t>(depth) / kBlock;
+  return tiles * nb * (512 + kTile * sizeof(float));
+}
+
+bool FcInt4BlockwiseGemmSupports(int depth, int blocksize) {
+  return blocksize == kBlock && depth > 0 && depth % kBlock == 0;
+}
+
+hipError_t LaunchPackInt4BlockwiseGemm(const uint8_t* filter, const uint16_t* scales_f16,
+                                       int out_depth, int depth, uint8_t* packed,
+                                       hipStream_t stream) {
+  if (out_depth == 0 || depth == 0) return hipSuccess;
+  const int tiles = (out_depth + kTile - 1) / kTile;
+  const int nb = depth / kBlock;
+  const int64_t slots = static_cast<int64_t>(tiles) * nb * 64;
+  const unsigned grid = static_cast<unsigned>((slots + kThreads - 1) / kThreads);
+  hipLaunchKernelGGL(PackInt4BlockwiseGemmKernel, dim3(grid), dim3(kThreads), 0, stream, filter,
+                     scales_f16, out_depth, depth, tiles, nb, packed);
+  return hipGetLastError();
+}
+
+size_t TiledRowsBytes(int batches, int depth) {
+  const size_t row_tiles = (static_cast<size_t>(batches) + kTile - 1) / kTile;
+  return row_tiles * kTile * static_cast<size_t>(depth);
+}
+
+hipError_t LaunchFcInt4BlockwiseGemm(const int8_t* quantized_rows, const float* scaling_factors,
+                                     const int32_t* zero_points, const uint8_t* gemm_filter,
+                                     const float* kfsum, const float* bias, float* output,
+                                     int batches, int depth, int out_depth, void* tiled_rows,
+                                     hipStream_t stream) {
+  if (batches == 0 || out_depth == 0) return hipSuccess;
+  const int nb = depth / kBlock;
+  const int row_tiles = (batches + kTile - 1) / kTile;
+  const int channel_tiles = (out_depth + kTile - 1) / kTile;
+  {
+    const int64_t slots = static_cast<int64_t>(row_tiles) * nb * 64;
+    const unsigned grid = static_cast<unsigned>((slots + kThreads - 1) / kThreads);
+    hipLaunchKernelGGL(TileQuantizedRowsKernel, dim3(grid), dim3(kThreads), 0, stream,
+                       quantized_rows, batches, depth, row_tiles, nb,
+                       static_cast<uint2*>(tiled_rows));
+    if (hipError_t err = hipGetLastError()) return err;
+  }
+  GemmArgs a;
+  a.filter = reinterpret_cast<const i64*>(gemm_filter);
+  a.scales = reinterpret_cast<const float4*>(gemm_filter +
+                                             static_cast<size_t>(channel_tiles) * nb * 512);
+  a.activations = static_cast<const i64*>(tiled_rows);
+  a.scaling_factors = scaling_factors;
+  a.zero_points = zero_points;
+  a.kfsum = kfsum;
+  a.bias = bias;
+  a.output = output;
+  a.batches = batches;
+  a.out_depth = out_depth;
+  a.nb = nb;
+  a.channel_tiles = channel_tiles;
+  a.row_tiles = row_tiles;
+  a.vector_store = (out_depth % 4 == 0) && (reinterpret_cast<uintptr_t>(output) % 16 == 0);
+  // Tiles per wavefront (channels x rows), the four wavefronts of a workgroup side by side
+  // along the channels. Measured at 14336 x 4096: up to 64 rows the filter stream decides and
+  // one channel tile per wavefront spreads it over the most wavefronts; beyond, 2 x 4 tiles
+  // re-read the least (2048 rows: 584 us against 767 us with 2 x 2).
+  const int CT = row_tiles <= 4 ? 1 : 2;
+  const int RT = row_tiles <= 1 ? 1 : row_tiles <= 2 ? 2 : 4;
+  const dim3 grid((channel_tiles + 4 * CT - 1) / (4 * CT), (row_tiles + RT - 1) / RT);
+  if (grid.y > 65535) return hipErrorInvalidValue;
+  if (CT == 2) {
+    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<2, 4, 1>), grid, dim3(kThreads), 0, stream, a);
+  } else if (RT == 4) {
+    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 4, 1>), grid, dim3(kThreads), 0, stream, a);
+  } else if (RT == 2) {
+    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 2, 1>), grid, dim3(kThreads), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 1, 1>), grid, dim3(kThreads), 0, stream, a);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace lrtfc

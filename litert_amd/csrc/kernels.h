@@ -154,6 +154,23 @@ hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_l
 hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const float* input_f32,
                               int variant, hipStream_t stream);
 
+// Blockwise-int4 FULLY_CONNECTED for prefill batches: matrix-core GEMM with one float32
+// accumulator per output walking the blocks in order (block size 32). The filter is re-tiled by
+// LaunchPackInt4BlockwiseGemm (GemmInt4BlockwiseBytes bytes: int8 tiles, then float32 scales);
+// the rows arrive quantized (row-major int8 + scaling factors + zero points) and are re-tiled
+// into `tiled_rows` (TiledRowsBytes bytes) by the launch itself.
+size_t GemmInt4BlockwiseBytes(int out_depth, int depth);
+bool FcInt4BlockwiseGemmSupports(int depth, int blocksize);
+hipError_t LaunchPackInt4BlockwiseGemm(const uint8_t* filter, const uint16_t* scales_f16,
+                                       int out_depth, int depth, uint8_t* packed,
+                                       hipStream_t stream);
+size_t TiledRowsBytes(int batches, int depth);
+hipError_t LaunchFcInt4BlockwiseGemm(const int8_t* quantized_rows, const float* scaling_factors,
+                                     const int32_t* zero_points, const uint8_t* gemm_filter,
+                                     const float* kfsum, const float* bias, float* output,
+                                     int batches, int depth, int out_depth, void* tiled_rows,
+                                     hipStream_t stream);
+
 // EMBEDDING_LOOKUP from an Int4 (value_bits 4) or Int8 (8) table to float32 / binary16 rows.
 // block_scales != nullptr: blockwise fp16 scales [rows, cols / blocksize]; otherwise row_scales
 // [rows] or `scale`. status: three device int32 {0 or 1, first offending position or -1, the

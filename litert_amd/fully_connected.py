@@ -279,6 +279,8 @@ class FullyConnectedBlockwiseInt4:
             _ptr(self.filter), _ptr(self.scales), self.out_depth, self.depth, self.blocksize,
             _ptr(self.kfsum), _stream()))
         self._ws = None
+        self._gemm_filter = None
+        self._gemm_ws = None
         # packed: one fused kernel on the re-tiled filter (block size 32 only); otherwise the
         # two-kernel form on the reference layout.
         self.retiled = None
@@ -297,9 +299,41 @@ class FullyConnectedBlockwiseInt4:
             self._ws = torch.empty(need, dtype=torch.uint8, device="cuda")
         return self._ws
 
+    # From this many rows on the matrix-core GEMM streams the filter once for the whole batch;
+    # below, the decode kernel (one pass over the filter per four rows) is faster.
+    GEMM_MIN_BATCHES = 16
+
+    def call_gemm(self, x, out=None):
+        """Prefill form: row quantizer, row re-tiling and the blockwise GEMM on a filter
+        re-tiled for it (made on first use and kept). Same results as the other forms."""
+        if self.blocksize != 32 or self.depth % 32:
+            raise RuntimeError("call_gemm needs block size 32")
+        lib = capi.load()
+        x = x.contiguous()
+        batches = x.numel() // self.depth
+        if out is None:
+            out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
+        if self._gemm_filter is None:
+            self._gemm_filter = torch.empty(
+                lib.lrtfc_gemm_int4_blockwise_bytes(self.out_depth, self.depth), dtype=torch.uint8,
+                device="cuda")
+            capi.check(lib.lrtfc_pack_int4_blockwise_gemm(
+                _ptr(self.filter), _ptr(self.scales), self.out_depth, self.depth, 32,
+                _ptr(self._gemm_filter), _stream()))
+        need = lib.lrtfc_fc_blockwise_int4_gemm_workspace_bytes(batches, self.depth)
+        if self._gemm_ws is None or self._gemm_ws.numel() < need:
+            self._gemm_ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        capi.check(lib.lrtfc_fc_blockwise_int4_gemm(
+            _ptr(x), _ptr(self._gemm_filter), _ptr(self.kfsum), _ptr(self.bias), _ptr(out), batches,
+            self.depth, self.out_depth, self.variant, _ptr(self._gemm_ws), self._gemm_ws.numel(),
+            _stream()))
+        return out
+
     def __call__(self, x, out=None):
         x = x.contiguous()
         batches = x.numel() // self.depth
+        if batches >= self.GEMM_MIN_BATCHES and self.blocksize == 32 and self.depth % 32 == 0:
+            return self.call_gemm(x, out)
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
         if (self.retiled is not None and self.depth > self.FUSED_MAX_DEPTH

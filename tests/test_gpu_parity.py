@@ -436,6 +436,42 @@ def test_blockwise_int4_wavefronts_spanning_channel_groups(fc, B):
         assert _bits_equal(yi.cpu().numpy(), want), n
 
 
+@pytest.mark.parametrize("B,K,N,bias", [(16, 64, 8, False), (33, 128, 20, True), (64, 256, 70, False),
+                                        (100, 2048, 264, True), (17, 4096, 130, False),
+                                        (128, 1024, 64, True), (65, 96, 5, True), (1, 64, 4, False),
+                                        (250, 32, 33, False)])
+def test_blockwise_int4_gemm_matches_oracle(fc, B, K, N, bias):
+    """Prefill form (matrix-core GEMM, one float accumulator per output walking the blocks in
+    order): bit-identical to the oracle, edges in every direction (rows and channels that do
+    not fill their tiles, one block, odd channel counts with scalar stores)."""
+    c = wl.blockwise_int4_fc(B, K, N, seed=11 + B + K + N, lo=-8, hi=7)
+    b = np.random.default_rng(B).standard_normal(N).astype(np.float32) if bias else None
+    op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], K, 32, b)
+    y = op.call_gemm(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_blockwise_int4(c["x"], c["packed"], N, c["scales"].view(np.uint16), 32, b)
+    assert _bits_equal(y, want)
+    if B >= op.GEMM_MIN_BATCHES:  # the op picks this form by itself from 16 rows on
+        assert _bits_equal(op(_cuda(c["x"])).cpu().numpy(), want)
+
+
+def test_blockwise_int4_gemm_full_width_agrees_with_decode_kernel(fc):
+    """256 rows against the full-size filter of config 3 (14336 x 4096): the GEMM and the
+    decode kernel (64 passes of four rows) must agree bit for bit; a sample of channels is
+    also checked against the oracle."""
+    c = wl.blockwise_int4_fc(4)
+    x = np.random.default_rng(12).standard_normal((256, 4096)).astype(np.float32)
+    op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], 4096, 32)
+    xd = _cuda(x)
+    gemm = op.call_gemm(xd).cpu().numpy()
+    decode = torch.cat([op(xd[i:i + 4]) for i in range(0, 256, 4)]).cpu().numpy()
+    assert _bits_equal(gemm, decode)
+    rows = [0, 100, 255]
+    sample = np.arange(0, 14336, 449)
+    want = oracle.fc_blockwise_int4(x[rows], c["packed"][sample], sample.size,
+                                    c["scales"][sample].view(np.uint16), 32)
+    assert _bits_equal(gemm[rows][:, sample], want)
+
+
 @pytest.mark.parametrize("variant", [1, 2])
 def test_blockwise_int4_grouped_deep_rows_quantizer_variants(fc, variant):
     """The group's row quantizer launch (deep rows, more than two per node) in the two NEON
