@@ -345,6 +345,24 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         op_gbps_cold=round(b3 / o_cold / 1e3, 1), op_gbps_hot=round(b3 / o_hot / 1e3, 1),
         frac_of_hbm_peak_cold=round(b3 / o_cold / 1e3 / HBM_PEAK_GBPS, 4), algorithmic_bytes=b3,
         kernel="FcInt4PackedKernel<fused quantize> on the re-tiled filter")
+    # Prefill batches on the blockwise int4 path (not a BASELINE configuration): config 3's filter
+    # against 2048 and 128 rows through the matrix-core GEMM (row quantizer + row re-tiling +
+    # GEMM launches), and what the decode kernel needs for the same rows in passes of four.
+    op3 = fc.FullyConnectedBlockwiseInt4(c3["packed"], c3["scales"], 4096, 32)
+    entry = {}
+    for rows in (128, 2048):
+        xg = torch.randn((rows, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(rows))
+        yg = torch.empty((rows, 14336), dtype=torch.float32, device="cuda")
+        us = per_launch_us([lambda: op3.call_gemm(xg, out=yg)] * 4, replays=5)
+        entry["us_%d_rows" % rows] = round(us, 1)
+        entry["tops_%d_rows" % rows] = round(2.0 * rows * 4096 * 14336 / us / 1e6, 1)
+    passes = per_launch_us([lambda: [ops3[0](xg[i:i + 4], out=yg[i:i + 4]) for i in range(0, 128, 4)]],
+                           replays=5)
+    entry["us_128_rows_decode_kernel_passes"] = round(passes, 1)
+    entry["kernel"] = "FcInt4BlockwiseGemmKernel (v_mfma_i32_16x16x32_i8 per block, float32 accumulators in block order)"
+    out["next_int4_blockwise_prefill_14336x4096"] = entry
+    del op3
+
     del ops3
 
     # Next-row op (not a BASELINE configuration): per-channel int4 hybrid FC (EvalHybridDense4Bit)

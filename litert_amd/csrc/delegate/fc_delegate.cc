@@ -356,6 +356,9 @@ struct FcNode {
   // Per-channel int4 hybrid nodes keep the filter at 4 bits per weight for decode batches
   // (retiled_dev then holds nibble tiles) and as re-tiled int8 for prefill batches.
   bool nibble_layout = false, have_nibbles = false;
+  // Blockwise-int4 nodes run prefill batches on the filter re-tiled for the matrix-core GEMM
+  // (retiled_dev then holds that form) and decode batches on the streaming form.
+  bool gemm_layout = false, have_gemm = false;
   bool split_quantize = false;  // quantize rows in a launch of their own, not in the prologue
   // EMBEDDING_LOOKUP nodes: input = the lookup vector, filter = the table (filter_dev), batches =
   // lookups, depth = out_depth = columns of a row; block scales in scales_dev or per-row scales
@@ -382,6 +385,9 @@ constexpr int kInt4DeepFusedMaxBatches = 2;
 // Up to this many rows a per-channel int4 node streams its filter as nibbles (one pass per 16
 // rows); above, the MFMA GEMM on the int8 expansion streams it once.
 constexpr int kInt4PerChannelNibbleMaxBatches = 32;
+// From this many rows on a blockwise-int4 node streams its filter once through the GEMM instead
+// of once per four rows.
+constexpr int kInt4BlockwiseGemmMinBatches = 16;
 
 struct PartitionKernel {
   DelegateState* state = nullptr;
@@ -646,7 +652,7 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
   }
   hipStream_t s = k->stream;
   if (n->uploaded_filter != filter.data.raw) {
-    n->have_model_layout = n->have_retiled = n->have_nibbles = false;
+    n->have_model_layout = n->have_retiled = n->have_nibbles = n->have_gemm = false;
   }
   const size_t weights = static_cast<size_t>(n->out_depth) * n->depth;
 
@@ -760,7 +766,33 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
     n->use_retiled = weights > 0 && lrtfc_fc_blockwise_int4_preferred_layout(
                                         n->depth, n->blocksize) == LRTFC_LAYOUT_PACKED;
     n->split_quantize = n->depth > kInt4FusedMaxDepth && n->batches > kInt4DeepFusedMaxBatches;
-    if (weights > 0 && !(n->use_retiled ? n->have_retiled : n->have_model_layout)) {
+    n->gemm_layout = n->use_retiled && n->batches >= kInt4BlockwiseGemmMinBatches;
+    if (n->gemm_layout) {
+      if (!n->have_gemm) {
+        DeviceBuffer nibbles, block_scales;
+        RETURN_IF_HIP(ctx, nibbles.Upload(filter.data.raw, weights / 2, s));
+        RETURN_IF_HIP(ctx, block_scales.Upload(
+                               scales.data.raw, static_cast<size_t>(NumElements(scales.dims)) * 2, s));
+        RETURN_IF_HIP(ctx, n->kfsum_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
+        RETURN_IF_FC(ctx, lrtfc_blockwise_int4_kfsum(nibbles.as<uint8_t>(),
+                                                     block_scales.as<uint16_t>(), n->out_depth,
+                                                     n->depth, n->blocksize,
+                                                     n->kfsum_dev.as<float>(), s));
+        n->retiled_dev.Release();
+        RETURN_IF_HIP(ctx, n->retiled_dev.Ensure(
+                               lrtfc_gemm_int4_blockwise_bytes(n->out_depth, n->depth)));
+        RETURN_IF_FC(ctx, lrtfc_pack_int4_blockwise_gemm(nibbles.as<uint8_t>(),
+                                                         block_scales.as<uint16_t>(), n->out_depth,
+                                                         n->depth, n->blocksize,
+                                                         n->retiled_dev.as<uint8_t>(), s));
+        RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+        n->filter_dev.Release();
+        n->scales_dev.Release();
+        n->have_gemm = true;
+        n->have_retiled = n->have_model_layout = false;
+      }
+    } else if (weights > 0 && !(n->use_retiled ? n->have_retiled : n->have_model_layout)) {
+      n->have_gemm = false;
       if (!n->have_model_layout) {
         RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights / 2, s));
         RETURN_IF_HIP(ctx, n->scales_dev.Upload(scales.data.raw,
@@ -833,8 +865,8 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
   // (Nodes whose rows are quantized by a launch of their own group too: the group then has
   // one such launch for all its rows, into per-node workspaces.)
   auto groupable = [&](const FcNode& n) {
-    return n.kind == FcKind::kInt4Blockwise && n.use_retiled && n.depth > 0 && n.batches > 0 &&
-           n.out_depth > 0;
+    return n.kind == FcKind::kInt4Blockwise && n.use_retiled && !n.gemm_layout && n.depth > 0 &&
+           n.batches > 0 && n.out_depth > 0;
   };
   {
     std::map<std::tuple<int, int, int>, std::vector<int>> sets;  // (level, depth, batches)
@@ -912,6 +944,11 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
   }
   for (const FcNode& n : k->nodes) {
     if (n.kind == FcKind::kEmbeddingLookup || n.group >= 0) continue;
+    if (n.kind == FcKind::kInt4Blockwise && n.gemm_layout) {
+      RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(
+                             lrtfc_fc_blockwise_int4_gemm_workspace_bytes(n.batches, n.depth)));
+      continue;
+    }
     if (n.kind == FcKind::kHybridInt4 ||
         (n.kind != FcKind::kInt8 && (!n.use_retiled || n.split_quantize))) {
       RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(
@@ -1110,7 +1147,13 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                               n.out_depth, n.params.activation, scratch.get(), scratch.bytes(), s));
         break;
       case FcKind::kInt4Blockwise:
-        if (!n.use_retiled) {
+        if (n.gemm_layout) {
+          RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4_gemm(
+                                static_cast<const float*>(in_dev), n.retiled_dev.as<uint8_t>(),
+                                n.kfsum_dev.as<float>(), bias_f32, static_cast<float*>(out_dev),
+                                n.batches, n.depth, n.out_depth, variant, scratch.get(),
+                                scratch.bytes(), s));
+        } else if (!n.use_retiled) {
           RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4(static_cast<const float*>(in_dev),
                                                     n.filter_dev.as<uint8_t>(),
                                                     n.scales_dev.as<uint16_t>(),

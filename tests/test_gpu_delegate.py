@@ -624,3 +624,37 @@ def test_int4_grouped_nodes_with_more_than_two_rows(B, K):
             for c, n, y, v in zip(cs, Ns, ys, ins):
                 want = oracle.fc_blockwise_int4(v, c["packed"], n, c["scales"].view(np.uint16), 32)
                 assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32)), (trial, n)
+
+
+def test_blockwise_int4_resize_between_decode_and_prefill():
+    """Two rows run the streaming kernel, 40 rows the matrix-core GEMM (the filter is re-tiled
+    for it at that prepare), 3 rows the streaming kernel again. Every step bit-identical to the
+    oracle; two independent nodes, so the decode steps share a grouped launch."""
+    K, Ns = 256, (24, 72)
+    cs = [wl.blockwise_int4_fc(40, K, n, seed=60 + n, lo=-8, hi=7) for n in Ns]
+    with FakeHost() as h:
+        xs, ys = [], []
+        for c, n in zip(cs, Ns):
+            x = h.tensor(FLOAT32, (2, K), data=c["x"][:2])
+            w = h.tensor(INT4, (n, K), data=c["packed"], const=True)
+            s_ = h.tensor(FLOAT16, (n, K // 32), data=c["scales"], const=True)
+            h.blockwise(w, s_, 32)
+            y = h.tensor(FLOAT32, (2, n))
+            h.fc(x, w, None, y)
+            xs.append(x)
+            ys.append(y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        for rows in (2, 40, 3, 16):
+            for c, n, x, y in zip(cs, Ns, xs, ys):
+                h.resize(x, (rows, K))
+                h.resize(y, (rows, n))
+                h.write(x, c["x"][:rows])
+            assert h.allocate_tensors() == OK, h.errors()
+            groups, _ = h.describe_partition(h.plan()[0][2])
+            assert groups == (0 if rows >= 16 else 1), rows
+            assert h.invoke() == OK, h.errors()
+            for c, n, y in zip(cs, Ns, ys):
+                want = oracle.fc_blockwise_int4(c["x"][:rows], c["packed"], n,
+                                                c["scales"].view(np.uint16), 32)
+                assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32)), (rows, n)
