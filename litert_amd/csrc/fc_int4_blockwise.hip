@@ -181,22 +181,39 @@ __global__ __launch_bounds__(kThreads) void FcBlockwiseInt4GenericKernel(FcInt4A
   a.output[idx] = out;
 }
 
+// kfsum[n] = sum over blocks, in block order, of scale * float(sum of the block's weights)
+// (tflite/kernels/fully_connected.cc:1056-1077). One wavefront per channel: lane L forms the
+// products of blocks L, L + 64, ... in parallel, and the products are then added one by one in
+// block order (each read out of its lane as a scalar), which is the order the result depends on.
 __global__ __launch_bounds__(kThreads) void BlockwiseInt4KfsumKernel(
     const uint8_t* __restrict__ packed_filter, const uint16_t* __restrict__ scales_f16,
     int out_depth, int depth, int blocksize, float* __restrict__ kfsum) {
-  const int n = blockIdx.x * kThreads + threadIdx.x;
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int n = blockIdx.x * (kThreads / kWaveSize) +
+                __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
   if (n >= out_depth) return;
   const int nblk = depth / blocksize;
   const size_t k2 = (static_cast<size_t>(depth) + 1) & ~static_cast<size_t>(1);
   const uint8_t* row = packed_filter + n * (k2 / 2);
   float total = 0.0f;
-  for (int bi = 0; bi < nblk; ++bi) {
-    int32_t ksum = 0;
-    for (int ki = 0; ki < blocksize; ++ki) ksum += NibbleAt(row, bi * blocksize + ki);
-    const float scale = HalfBitsToFloat(scales_f16[static_cast<size_t>(n) * nblk + bi]);
-    total = __fadd_rn(total, __fmul_rn(scale, static_cast<float>(ksum)));
+  for (int base = 0; base < nblk; base += kWaveSize) {
+    const int bi = base + lane;
+    float product = 0.0f;
+    if (bi < nblk) {
+      int32_t ksum = 0;
+      for (int ki = 0; ki < blocksize; ++ki) ksum += NibbleAt(row, bi * blocksize + ki);
+      const float scale = HalfBitsToFloat(scales_f16[static_cast<size_t>(n) * nblk + bi]);
+      product = __fmul_rn(scale, static_cast<float>(ksum));
+    }
+    const int count = min(kWaveSize, nblk - base);
+#pragma unroll
+    for (int j = 0; j < kWaveSize; ++j) {
+      if (j < count) {
+        total = __fadd_rn(total, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(product), j)));
+      }
+    }
   }
-  kfsum[n] = total;
+  if (lane == 0) kfsum[n] = total;
 }
 
 template <int R, int BT, int WC>
@@ -237,7 +254,8 @@ hipError_t LaunchBlockwiseInt4Kfsum(const uint8_t* packed_filter, const uint16_t
                                     int out_depth, int depth, int blocksize, float* kfsum,
                                     hipStream_t stream) {
   if (out_depth == 0) return hipSuccess;
-  const int grid = (out_depth + kThreads - 1) / kThreads;
+  const int channels_per_wg = kThreads / kWaveSize;
+  const int grid = (out_depth + channels_per_wg - 1) / channels_per_wg;
   hipLaunchKernelGGL(BlockwiseInt4KfsumKernel, dim3(grid), dim3(kThreads), 0, stream,
                      packed_filter, scales_f16, out_depth, depth, blocksize, kfsum);
   return hipGetLastError();
