@@ -36,13 +36,20 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
+# Per-file additions. The blockwise int4 GEMM reads every MFMA result with the vector ALU right
+# away (one MFMA per quantization block), so its results should land in ordinary vector
+# registers: with the default choice of accumulation registers each of them costs a copy
+# instruction first (a quarter of the kernel's vector work).
+FILE_FLAGS = {"fc_int4_blockwise_gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def build_fc():
     os.makedirs(LIB, exist_ok=True)
     objs = []
     procs = []
     for src in FC_SOURCES:
         obj = os.path.join(LIB, src.replace(".hip", ".o"))
-        cmd = [HIPCC] + COMMON + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [HIPCC] + COMMON + FILE_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
         print("+", " ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd)))
         objs.append(obj)
