@@ -112,7 +112,9 @@ constexpr int kRing = 16;  // weight tiles in flight per wavefront
 // scalar arguments to a wavefront in registers when it starts; everything else is read from
 // the argument segment as usual, ~0.5 us later, when the prologue has long begun (measured:
 // 12.55 -> 12.28 us per launch at 14336 x 4096, B = 1).
-template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS>
+// XREGS: 16-byte pieces of a float row a thread holds between the two passes of the fused
+// prologue (4, 8 or 16: rows up to 4096, 8192, 16384 deep); REG_ROWS * XREGS stays at 16 or less.
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS, int XREGS>
 __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(
     const int8_t* early_filter, const float* early_input_f32, int early_depth, int early_slabs,
     int early_out_depth, int batch0, int bt, int ksplit, PackedArgs p) {
@@ -142,7 +144,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(
   // activation tiles are therefore fetched into registers first (kXRegs float4 per row per
   // thread for up to REG_ROWS rows, or kQRegs 16-byte chunks of int8), without branches;
   // larger ones are staged completely before the weights are requested.
-  constexpr int kXRegs = 4, kQRegs = 4 * REG_ROWS;
+  constexpr int kXRegs = XREGS, kQRegs = 4 * REG_ROWS;
   const int padded = slabs * kSlabDepth;
   const int vector_end = depth - (depth % 8);
   float4 xr[REG_ROWS][kXRegs];
@@ -451,11 +453,11 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(
   }
 }
 
-template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS>
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS, int XREGS = 4>
 hipError_t LaunchSized(const PackedArgs& p, int batch0, int bt, hipStream_t stream) {
   const int qstride = p.slabs * kSlabDepth + kQPad;
   const size_t lds = SharedBytes(bt, qstride);
-  auto kernel = FcInt8PackedGemvKernel<EPI, FUSED, VARIANT, REG_ROWS>;
+  auto kernel = FcInt8PackedGemvKernel<EPI, FUSED, VARIANT, REG_ROWS, XREGS>;
   if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
   // How many wavefronts share one channel group's depth. What the memory system rewards is
@@ -484,8 +486,20 @@ hipError_t LaunchOne(const PackedArgs& p, int batch0, int bt, hipStream_t stream
     if (row_bytes <= 16 * kThreads * 8) return LaunchSized<EPI, false, VARIANT, 2>(p, batch0, bt, stream);
     return LaunchSized<EPI, false, VARIANT, 4>(p, batch0, bt, stream);
   }
-  if (bt <= 1) return LaunchSized<EPI, FUSED, VARIANT, 1>(p, batch0, bt, stream);
-  if (bt <= 2) return LaunchSized<EPI, FUSED, VARIANT, 2>(p, batch0, bt, stream);
+  // Deep rows stay in registers through the prologue too, as long as rows x depth fits 16
+  // pieces per thread: a row that does not is read twice, with the weight loads behind the
+  // first pass instead of under it (2048 x 16384, B = 1: 15.6 us that way, 11.8 us from
+  // registers).
+  const int depth = p.a.depth;
+  if (bt <= 1) {
+    if (depth > 8192 && depth <= 16384) return LaunchSized<EPI, FUSED, VARIANT, 1, 16>(p, batch0, bt, stream);
+    if (depth > 4096 && depth <= 8192) return LaunchSized<EPI, FUSED, VARIANT, 1, 8>(p, batch0, bt, stream);
+    return LaunchSized<EPI, FUSED, VARIANT, 1>(p, batch0, bt, stream);
+  }
+  if (bt <= 2) {
+    if (depth > 4096 && depth <= 8192) return LaunchSized<EPI, FUSED, VARIANT, 2, 8>(p, batch0, bt, stream);
+    return LaunchSized<EPI, FUSED, VARIANT, 2>(p, batch0, bt, stream);
+  }
   return LaunchSized<EPI, FUSED, VARIANT, 4>(p, batch0, bt, stream);
 }
 

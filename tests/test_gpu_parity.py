@@ -291,6 +291,19 @@ def test_hybrid_variants(fc, B, K, N, asym, per_channel, activation, packed):
     assert _bits_equal(y, want)
 
 
+@pytest.mark.parametrize("B,K,N", [(1, 16384, 40), (1, 8192, 48), (2, 8192, 24), (1, 10000, 33),
+                                   (1, 4100, 20), (2, 16384, 16), (3, 8192, 16), (1, 20000, 8)])
+@pytest.mark.parametrize("asym", [True, False])
+def test_hybrid_deep_rows(fc, B, K, N, asym):
+    """Rows deeper than 4096: one row up to 16384 deep and two rows up to 8192 stay in registers
+    through the fused prologue (their own kernel variants); the rest are read twice."""
+    c = wl.hybrid_fc(B, K, N, seed=21 + B + K)
+    op = fc.FullyConnectedHybrid(c["w"], c["pcs"], asymmetric_quantize_inputs=asym)
+    y = _hybrid_call(op, _cuda(c["x"]), "fused").cpu().numpy()
+    want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"], 1.0, None, asym, 0)
+    assert _bits_equal(y, want)
+
+
 def test_hybrid_dot_reference_kats_through_hip(fc):
     """tflite/kernels/internal/tensor_utils_test.cc:1214-1231 (per-channel + offsets), exact."""
     from tests.test_oracle_kat import _mv_data
