@@ -350,8 +350,9 @@ int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
  *     this kernel (16 channels x one block per 512-byte tile, sign-extended to int8, then the
  *     scales as float32); made once, like the other re-tilings.
  *   lrtfc_fc_blockwise_int4_gemm_workspace_bytes: device scratch for the quantized rows in
- *     both their forms (256-byte aligned).
- *   lrtfc_fc_blockwise_int4_gemm: row quantizer launch, row re-tiling launch, GEMM launch. */
+ *     the kernel's tile order, their scaling factors and zero points (256-byte aligned).
+ *   lrtfc_fc_blockwise_int4_gemm: row quantizer launch (it writes the tile order itself),
+ *     GEMM launch. */
 size_t lrtfc_gemm_int4_blockwise_bytes(int out_depth, int depth);
 int lrtfc_pack_int4_blockwise_gemm(const uint8_t* packed_filter, const uint16_t* scales_f16,
                                    int out_depth, int depth, int blocksize, uint8_t* gemm_filter,

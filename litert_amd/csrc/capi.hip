@@ -770,7 +770,9 @@ int lrtfc_pack_int4_blockwise_gemm(const uint8_t* packed_filter, const uint16_t*
 
 size_t lrtfc_fc_blockwise_int4_gemm_workspace_bytes(int batches, int depth) {
   if (batches <= 0 || depth <= 0) return 0;
-  return WorkspaceBytes(batches, depth) + lrtfc::AlignUp256(lrtfc::TiledRowsBytes(batches, depth));
+  // Tiled int8 rows (the batch padded to whole tiles), scaling factors, zero points.
+  return lrtfc::AlignUp256(lrtfc::TiledRowsBytes(batches, depth)) +
+         2 * lrtfc::AlignUp256(static_cast<size_t>(batches) * 4);
 }
 
 int lrtfc_fc_blockwise_int4_gemm(const float* input, const uint8_t* gemm_filter,
@@ -790,14 +792,17 @@ int lrtfc_fc_blockwise_int4_gemm(const float* input, const uint8_t* gemm_filter,
                 "workspace must be 256-byte aligned");
   LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(gemm_filter) & 15) == 0,
                 "re-tiled filter must be 16-byte aligned");
-  const Workspace w = SplitWorkspace(workspace, batches, depth);
-  void* tiled = static_cast<char*>(workspace) + WorkspaceBytes(batches, depth);
-  // EvalBlockwise4Bit always quantizes asymmetrically (fully_connected.cc:1044-1047).
-  int rc = lrtfc_batch_quantize_floats(input, batches, depth, w.q, w.sf, w.zp,
-                                       /*do_asymmetric=*/1, quant_variant, stream);
-  if (rc != LRTFC_OK) return rc;
-  return FromHip(lrtfc::LaunchFcInt4BlockwiseGemm(w.q, w.sf, w.zp, gemm_filter, kfsum, bias,
-                                                  output, batches, depth, out_depth, tiled,
+  LRTFC_REQUIRE(quant_variant >= LRTFC_QUANT_PORTABLE && quant_variant <= LRTFC_QUANT_NEON_LEGACY,
+                "unknown quantizer variant %d", quant_variant);
+  char* p = static_cast<char*>(workspace);
+  void* tiled = p;
+  p += lrtfc::AlignUp256(lrtfc::TiledRowsBytes(batches, depth));
+  float* scaling_factors = reinterpret_cast<float*>(p);
+  p += lrtfc::AlignUp256(static_cast<size_t>(batches) * 4);
+  int32_t* zero_points = reinterpret_cast<int32_t*>(p);
+  return FromHip(lrtfc::LaunchFcInt4BlockwiseGemm(input, quant_variant, scaling_factors,
+                                                  zero_points, gemm_filter, kfsum, bias, output,
+                                                  batches, depth, out_depth, tiled,
                                                   AsStream(stream)),
                  "blockwise int4 GEMM");
 }

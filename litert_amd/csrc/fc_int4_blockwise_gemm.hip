@@ -17,12 +17,13 @@
 //     int8 -- the A operand of the MFMA as one 8-byte load per lane; after all tiles, the block
 //     scales as float32, 16 per (t, b), so that a lane reads the scales of its four output
 //     channels in one 16-byte load.
-//   activations `tile16x32`: the same with batch rows in place of channels (B operand), made
-//     from the row-major int8 rows of the standalone quantizer.
+//   activations `tile16x32`: the same with batch rows in place of channels (B operand),
+//     written in that order by the row quantizer itself.
 // No LDS: a wavefront owns CT x RT tiles (16 to 32 channels x 16 to 64 rows, by batch size)
 // and requests the operands of the next blocks while it works on the current one (a ring of
 // kStages blocks in registers); both operands are re-read by other wavefronts from L2.
 #include "kernels.h"
+#include "quantize_device.h"
 
 namespace lrtfc {
 namespace {
@@ -84,23 +85,33 @@ __global__ __launch_bounds__(kThreads) void PackInt4BlockwiseGemmKernel(
   }
 }
 
-// Row-major int8 rows [batches, depth] -> tile16x32 (rows past the batch are zero).
-__global__ __launch_bounds__(kThreads) void TileQuantizedRowsKernel(
-    const int8_t* __restrict__ rows, int batches, int depth, int row_tiles, int nb,
-    uint2* __restrict__ dst) {
-  const int64_t slot = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (slot >= static_cast<int64_t>(row_tiles) * nb * 64) return;
-  const int lane = static_cast<int>(slot & 63);
-  const int64_t tb = slot >> 6;
-  const int b = static_cast<int>(tb % nb);
-  const int t = static_cast<int>(tb / nb);
-  const int m = t * kTile + (lane & 15);
-  uint2 v = make_uint2(0, 0);
-  if (m < batches) {
-    v = *reinterpret_cast<const uint2*>(rows + static_cast<size_t>(m) * depth + b * kBlock +
-                                        8 * (lane >> 4));
+// Element k of batch row m within its row tile of the tile16x32 layout, as a byte offset
+// from the tile row's base.
+struct Tile16x32Placement {
+  int row_in_tile;
+  __device__ __forceinline__ size_t operator()(int k) const {
+    return (static_cast<size_t>(k >> 5) * 64 + ((k & 31) >> 3) * 16 + row_in_tile) * 8 + (k & 7);
   }
-  dst[slot] = v;
+};
+
+// BatchQuantizeFloats of float rows [batches, depth] straight into tile16x32: one workgroup
+// per row of the padded batch (rows past the batch are zero).
+template <int VARIANT>
+__global__ __launch_bounds__(kQuantizeThreads) void QuantizeRowsTiledKernel(
+    const float* __restrict__ input, int batches, int depth, int8_t* __restrict__ tiled,
+    float* __restrict__ scaling_factors, int32_t* __restrict__ zero_points) {
+  const int m = blockIdx.x;
+  int8_t* tile_row = tiled + static_cast<size_t>(m / kTile) * kTile * depth;
+  const Tile16x32Placement place{m % kTile};
+  if (m < batches) {
+    // EvalBlockwise4Bit always quantizes asymmetrically (fully_connected.cc:1044-1047).
+    QuantizeRow<VARIANT>(input + static_cast<size_t>(m) * depth, depth, tile_row,
+                         scaling_factors + m, zero_points + m, /*do_asymmetric=*/1, place);
+  } else {
+    for (int k = threadIdx.x * 8; k < depth; k += kQuantizeThreads * 8) {
+      *reinterpret_cast<uint2*>(tile_row + place(k)) = make_uint2(0, 0);
+    }
+  }
 }
 
 struct GemmArgs {
@@ -272,8 +283,8 @@ size_t TiledRowsBytes(int batches, int depth) {
   return row_tiles * kTile * static_cast<size_t>(depth);
 }
 
-hipError_t LaunchFcInt4BlockwiseGemm(const int8_t* quantized_rows, const float* scaling_factors,
-                                     const int32_t* zero_points, const uint8_t* gemm_filter,
+hipError_t LaunchFcInt4BlockwiseGemm(const float* input, int variant, float* scaling_factors,
+                                     int32_t* zero_points, const uint8_t* gemm_filter,
                                      const float* kfsum, const float* bias, float* output,
                                      int batches, int depth, int out_depth, void* tiled_rows,
                                      hipStream_t stream) {
@@ -282,11 +293,22 @@ hipError_t LaunchFcInt4BlockwiseGemm(const int8_t* quantized_rows, const float* 
   const int row_tiles = (batches + kTile - 1) / kTile;
   const int channel_tiles = (out_depth + kTile - 1) / kTile;
   {
-    const int64_t slots = static_cast<int64_t>(row_tiles) * nb * 64;
-    const unsigned grid = static_cast<unsigned>((slots + kThreads - 1) / kThreads);
-    hipLaunchKernelGGL(TileQuantizedRowsKernel, dim3(grid), dim3(kThreads), 0, stream,
-                       quantized_rows, batches, depth, row_tiles, nb,
-                       static_cast<uint2*>(tiled_rows));
+    const dim3 grid(row_tiles * kTile), block(kQuantizeThreads);
+    int8_t* tiled = static_cast<int8_t*>(tiled_rows);
+    switch (variant) {
+      case LRTFC_QUANT_NEON_V8:
+        hipLaunchKernelGGL(QuantizeRowsTiledKernel<LRTFC_QUANT_NEON_V8>, grid, block, 0, stream,
+                           input, batches, depth, tiled, scaling_factors, zero_points);
+        break;
+      case LRTFC_QUANT_NEON_LEGACY:
+        hipLaunchKernelGGL(QuantizeRowsTiledKernel<LRTFC_QUANT_NEON_LEGACY>, grid, block, 0,
+                           stream, input, batches, depth, tiled, scaling_factors, zero_points);
+        break;
+      default:
+        hipLaunchKernelGGL(QuantizeRowsTiledKernel<LRTFC_QUANT_PORTABLE>, grid, block, 0, stream,
+                           input, batches, depth, tiled, scaling_factors, zero_points);
+        break;
+    }
     if (hipError_t err = hipGetLastError()) return err;
   }
   GemmArgs a;

@@ -157,16 +157,17 @@ hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const 
 // Blockwise-int4 FULLY_CONNECTED for prefill batches: matrix-core GEMM with one float32
 // accumulator per output walking the blocks in order (block size 32). The filter is re-tiled by
 // LaunchPackInt4BlockwiseGemm (GemmInt4BlockwiseBytes bytes: int8 tiles, then float32 scales);
-// the rows arrive quantized (row-major int8 + scaling factors + zero points) and are re-tiled
-// into `tiled_rows` (TiledRowsBytes bytes) by the launch itself.
+// the float rows are quantized (BatchQuantizeFloats, asymmetric, `variant`) straight into
+// `tiled_rows` (TiledRowsBytes bytes), their scaling factors and zero points into the two
+// arrays of `batches` entries, by a launch ahead of the GEMM's.
 size_t GemmInt4BlockwiseBytes(int out_depth, int depth);
 bool FcInt4BlockwiseGemmSupports(int depth, int blocksize);
 hipError_t LaunchPackInt4BlockwiseGemm(const uint8_t* filter, const uint16_t* scales_f16,
                                        int out_depth, int depth, uint8_t* packed,
                                        hipStream_t stream);
 size_t TiledRowsBytes(int batches, int depth);
-hipError_t LaunchFcInt4BlockwiseGemm(const int8_t* quantized_rows, const float* scaling_factors,
-                                     const int32_t* zero_points, const uint8_t* gemm_filter,
+hipError_t LaunchFcInt4BlockwiseGemm(const float* input, int variant, float* scaling_factors,
+                                     int32_t* zero_points, const uint8_t* gemm_filter,
                                      const float* kfsum, const float* bias, float* output,
                                      int batches, int depth, int out_depth, void* tiled_rows,
                                      hipStream_t stream);

@@ -212,13 +212,20 @@ __device__ __forceinline__ RowRange BlockMinMax(float mn, float mx) {
   return r;
 }
 
+// Where element i of a quantized row goes, as a byte offset from the row's base pointer.
+// A placement keeps aligned groups of four elements together, in order.
+struct RowMajorPlacement {
+  __device__ __forceinline__ size_t operator()(int i) const { return static_cast<size_t>(i); }
+};
+
 // One row through BatchQuantizeFloats by one workgroup of kQuantizeThreads threads: v[n_data]
-// -> q[n_data], *scaling_factor, *zero_point (may be null).
-template <int VARIANT>
+// -> q[place(0 .. n_data-1)], *scaling_factor, *zero_point (may be null).
+template <int VARIANT, typename PLACEMENT = RowMajorPlacement>
 __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_data,
                                             int8_t* __restrict__ q,
                                             float* __restrict__ scaling_factor,
-                                            int32_t* __restrict__ zero_point, int do_asymmetric) {
+                                            int32_t* __restrict__ zero_point, int do_asymmetric,
+                                            PLACEMENT place = PLACEMENT()) {
   const bool vec_ok = (n_data % 4 == 0) && ((reinterpret_cast<uintptr_t>(v) & 15) == 0) &&
                       ((reinterpret_cast<uintptr_t>(q) & 3) == 0);
 
@@ -257,7 +264,6 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   const int vector_end = n_data - (n_data % 8);
   if (vec_ok) {
     const float4* v4 = reinterpret_cast<const float4*>(v);
-    char4* q4 = reinterpret_cast<char4*>(q);
     for (int i = threadIdx.x; i < n_data / 4; i += kQuantizeThreads) {
       char4 o;
       if (all_zero) {
@@ -276,7 +282,7 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
           o.w = static_cast<char>(QuantizeSym<VARIANT>(t.w, inv, tail));
         }
       }
-      q4[i] = o;
+      *reinterpret_cast<char4*>(q + place(4 * i)) = o;
     }
   } else {
     for (int i = threadIdx.x; i < n_data; i += kQuantizeThreads) {
@@ -286,7 +292,7 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
         o = static_cast<int8_t>(do_asymmetric ? QuantizeAsym<VARIANT>(v[i], inv, zp, tail)
                                               : QuantizeSym<VARIANT>(v[i], inv, tail));
       }
-      q[i] = o;
+      q[place(i)] = o;
     }
   }
 }
