@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace lrtfc {
 
 constexpr int kWaveSize = 64;
@@ -95,6 +97,16 @@ __device__ __forceinline__ int32_t WaveSumI32(int32_t v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWaveSize);
   return v;
+}
+
+// f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{}): a loop whose
+// index is a compile-time constant in the body.
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void StaticFor(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    StaticFor<N, I + 1>(f);
+  }
 }
 
 // Float min / max over the 64 lanes; every lane receives the result (it is wave-uniform).

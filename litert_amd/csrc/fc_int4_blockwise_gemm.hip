@@ -15,13 +15,14 @@
 //   filter `tile16x32s`: for channel tile t (16 channels) and block b, 512 bytes: lane L's 8
 //     bytes are channel 16 t + L % 16, depths 32 b + 8 (L / 16) ... + 8, sign-extended to
 //     int8 -- the A operand of the MFMA as one 8-byte load per lane; after all tiles, the block
-//     scales as float32, 16 per (t, b), so that a lane reads the scales of its four output
-//     channels in one 16-byte load.
-//   activations `tile16x32`: the same with batch rows in place of channels (B operand),
-//     written in that order by the row quantizer itself.
+//     scales as float32, 16 per (t, b): a lane's 16-byte load is the scales of its four output
+//     channels for one block, and a wavefront fetches those of 16 blocks in one instruction.
+//   activations `tile16x64`: batch rows in place of channels (B operand), with the 8 bytes of
+//     blocks 2 p and 2 p + 1 side by side in a lane's 16 bytes; written in that order by the
+//     row quantizer itself.
 // No LDS: a wavefront owns CT x RT tiles (16 to 32 channels x 16 to 64 rows, by batch size)
-// and requests the operands of the next blocks while it works on the current one (a ring of
-// kStages blocks in registers); both operands are re-read by other wavefronts from L2.
+// and requests the operands of the next blocks while it works on the current ones (a ring of
+// pairs of blocks in registers); both operands are re-read by other wavefronts from L2.
 #include "kernels.h"
 #include "quantize_device.h"
 
@@ -35,6 +36,7 @@ constexpr int kTile = 16;     // channels / rows per MFMA tile
 // a workgroup is 2 x 2 wavefronts.
 
 using i64 = long;
+typedef long i64x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ int SignedNibble(uint32_t byte, int high) {
   const int n = high ? (byte >> 4) : (byte & 0xF);
@@ -85,24 +87,26 @@ __global__ __launch_bounds__(kThreads) void PackInt4BlockwiseGemmKernel(
   }
 }
 
-// Element k of batch row m within its row tile of the tile16x32 layout, as a byte offset
+// Element k of batch row m within its row tile of the tile16x64 layout, as a byte offset
 // from the tile row's base.
-struct Tile16x32Placement {
+struct Tile16x64Placement {
   int row_in_tile;
   __device__ __forceinline__ size_t operator()(int k) const {
-    return (static_cast<size_t>(k >> 5) * 64 + ((k & 31) >> 3) * 16 + row_in_tile) * 8 + (k & 7);
+    const size_t lane_slot = static_cast<size_t>(k >> 6) * 64 + ((k & 31) >> 3) * 16 + row_in_tile;
+    return (lane_slot * 2 + ((k >> 5) & 1)) * 8 + (k & 7);
   }
 };
 
-// BatchQuantizeFloats of float rows [batches, depth] straight into tile16x32: one workgroup
-// per row of the padded batch (rows past the batch are zero).
+// BatchQuantizeFloats of float rows [batches, depth] straight into tile16x64: one workgroup
+// per row of the padded batch (rows past the batch are zero). `tile_bytes`: one row tile.
 template <int VARIANT>
 __global__ __launch_bounds__(kQuantizeThreads) void QuantizeRowsTiledKernel(
-    const float* __restrict__ input, int batches, int depth, int8_t* __restrict__ tiled,
-    float* __restrict__ scaling_factors, int32_t* __restrict__ zero_points) {
+    const float* __restrict__ input, int batches, int depth, size_t tile_bytes,
+    int8_t* __restrict__ tiled, float* __restrict__ scaling_factors,
+    int32_t* __restrict__ zero_points) {
   const int m = blockIdx.x;
-  int8_t* tile_row = tiled + static_cast<size_t>(m / kTile) * kTile * depth;
-  const Tile16x32Placement place{m % kTile};
+  int8_t* tile_row = tiled + static_cast<size_t>(m / kTile) * tile_bytes;
+  const Tile16x64Placement place{m % kTile};
   if (m < batches) {
     // EvalBlockwise4Bit always quantizes asymmetrically (fully_connected.cc:1044-1047).
     QuantizeRow<VARIANT>(input + static_cast<size_t>(m) * depth, depth, tile_row,
@@ -117,7 +121,7 @@ __global__ __launch_bounds__(kQuantizeThreads) void QuantizeRowsTiledKernel(
 struct GemmArgs {
   const i64* filter;        // tile16x32s
   const float4* scales;     // float32 [tiles][nb][16] viewed as float4
-  const i64* activations;   // tile16x32
+  const i64x2* activations;  // tile16x64
   const float* scaling_factors;  // [batches]
   const int32_t* zero_points;    // [batches]
   const float* kfsum;            // [out_depth]
@@ -128,21 +132,28 @@ struct GemmArgs {
   int vector_store;              // rows of the output start on 16-byte boundaries
 };
 
+// One pair of consecutive blocks of a wavefront's operands.
 template <int CT, int RT>
 struct Stage {
-  i64 w[CT];      // channel tiles
-  float4 s[CT];   // their scales for this lane's four channels
-  i64 x[RT];      // row tiles
+  i64 w[2][CT];  // channel tiles of the two blocks
+  i64x2 x[RT];   // row tiles, both blocks
 };
 
+// Lane j of every 16 lanes to all 16 (row_newbcast:j).
+template <int J>
+__device__ __forceinline__ float RowBroadcast(float v) {
+  return DppMoveF32<0x150 + J>(v);
+}
+
 // WROWS: wavefronts of a workgroup along the batch rows (1 or 2); the others along the channels.
-template <int CT, int RT, int WROWS>
+// PAIRS: pairs of blocks in flight per wavefront. The count of outstanding vector loads a
+//   wavefront can wait on selectively is 63, so depth comes from few, wide loads: a row tile's
+//   two blocks in one 16-byte load, and the scales of 16 blocks in one load (lane = block
+//   16 g + lane % 16, its float4 = channels 4 (lane / 16) ... + 4), handed to the lanes of a
+//   block by a row broadcast.
+template <int CT, int RT, int WROWS, int PAIRS>
 __global__ __launch_bounds__(kThreads) void FcInt4BlockwiseGemmKernel(GemmArgs a) {
   constexpr int WCH = 4 / WROWS;
-  // Blocks in flight per wavefront: one or two tiles per block are bound by the filter stream
-  // and want many (16 rows: 33 us with 4, 27 us with 16); larger tiles are bound by their
-  // arithmetic and run best with 4.
-  constexpr int kStages = CT * RT <= 2 ? 16 : 4;
   const int lane = threadIdx.x & 63;
   // The wavefront index as a scalar: tile addresses then stay in scalar registers and every
   // load is "scalar base + lane offset".
@@ -159,31 +170,50 @@ __global__ __launch_bounds__(kThreads) void FcInt4BlockwiseGemmKernel(GemmArgs a
 #pragma unroll
   for (int j = 0; j < RT; ++j) rt[j] = min(rt0 + j, a.row_tiles - 1);
   const int nb = a.nb;
+  const int pairs = (nb + 1) / 2;
   const i64* wp[CT];
   const float4* sp[CT];
-  const i64* xp[RT];
+  const i64x2* xp[RT];
 #pragma unroll
   for (int j = 0; j < CT; ++j) {
     wp[j] = a.filter + static_cast<size_t>(ct[j]) * nb * 64 + lane;
     sp[j] = a.scales + static_cast<size_t>(ct[j]) * nb * 4 + (lane >> 4);
   }
 #pragma unroll
-  for (int j = 0; j < RT; ++j) xp[j] = a.activations + static_cast<size_t>(rt[j]) * nb * 64 + lane;
-  auto fetch = [&](int b) {
-    const int bb = min(b, nb - 1);  // past the end: a hot line, result unused
+  for (int j = 0; j < RT; ++j) {
+    xp[j] = a.activations + static_cast<size_t>(rt[j]) * pairs * 64 + lane;
+  }
+  auto fetch = [&](int p) {
+    const int pp = min(p, pairs - 1);  // past the end: a hot line, result unused
     Stage<CT, RT> st;
 #pragma unroll
-    for (int j = 0; j < CT; ++j) {
-      st.w[j] = wp[j][static_cast<size_t>(bb) * 64];
-      st.s[j] = sp[j][static_cast<size_t>(bb) * 4];
+    for (int h = 0; h < 2; ++h) {
+      const int bb = min(2 * pp + h, nb - 1);
+#pragma unroll
+      for (int j = 0; j < CT; ++j) {
+        st.w[h][j] = wp[j][static_cast<size_t>(bb) * 64];
+      }
     }
 #pragma unroll
-    for (int j = 0; j < RT; ++j) st.x[j] = xp[j][static_cast<size_t>(bb) * 64];
+    for (int j = 0; j < RT; ++j) st.x[j] = xp[j][static_cast<size_t>(pp) * 64];
     return st;
   };
-  Stage<CT, RT> ring[kStages];
+  // Scale groups (16 blocks = 8 pairs) held per wavefront: the current one and as many ahead
+  // as the ring of pairs reaches, so that a group is always requested before its blocks'
+  // weights; a power of two, group g in slot g % kGroups.
+  constexpr int kGroups = PAIRS > 8 ? 4 : 2;
+  static_assert((kGroups - 1) * 8 >= PAIRS, "scale groups must lead the ring");
+  float4 sg[kGroups][CT];
+  auto fetch_scales = [&](int g, float4 (&dst)[CT]) {
+    const int bb = min(16 * g + (lane & 15), nb - 1);
 #pragma unroll
-  for (int s = 0; s < kStages; ++s) ring[s] = fetch(s);
+    for (int j = 0; j < CT; ++j) dst[j] = sp[j][static_cast<size_t>(bb) * 4];
+  };
+#pragma unroll
+  for (int g = 0; g + 1 < kGroups; ++g) fetch_scales(g, sg[g]);
+  Stage<CT, RT> ring[PAIRS];
+#pragma unroll
+  for (int s = 0; s < PAIRS; ++s) ring[s] = fetch(s);
 
   // out[cj][rj][i]: channel 16 ct[cj] + 4 (lane / 16) + i, batch row 16 rt[rj] + lane % 16.
   float out[CT][RT][4];
@@ -195,28 +225,43 @@ __global__ __launch_bounds__(kThreads) void FcInt4BlockwiseGemmKernel(GemmArgs a
       for (int i = 0; i < 4; ++i) out[cj][rj][i] = 0.0f;
 
   const i32x4 zero = {0, 0, 0, 0};
-  for (int base = 0; base < nb; base += kStages) {
-#pragma unroll
-    for (int s = 0; s < kStages; ++s) {
+  // One trip covers whole turns of the ring and of the scale slots, so that ring slots,
+  // scale slots and broadcast lanes are compile-time constants.
+  constexpr int kTrip = PAIRS > 8 * kGroups ? PAIRS : 8 * kGroups;
+  static_assert(kTrip % PAIRS == 0 && kTrip % (8 * kGroups) == 0, "trip");
+  for (int base = 0; base < pairs; base += kTrip) {
+    StaticFor<kTrip>([&](auto u_const) {
+      constexpr int u = decltype(u_const)::value;
+      constexpr int s = u % PAIRS;
+      constexpr int cur = (u / 8) % kGroups;  // slot of this pair's scale group
+      if constexpr (u % 8 == 0) {
+        // A new group of 16 blocks starts: the slot of the one before it takes the farthest.
+        fetch_scales((base + u) / 8 + kGroups - 1, sg[(cur + kGroups - 1) % kGroups]);
+      }
       const Stage<CT, RT> st = ring[s];
-      ring[s] = fetch(base + kStages + s);
-      if (base + s < nb) {
+      ring[s] = fetch(base + u + PAIRS);
+      StaticFor<2>([&](auto h_const) {
+        constexpr int h = decltype(h_const)::value;
+        if (2 * (base + u) + h < nb) {
 #pragma unroll
-        for (int cj = 0; cj < CT; ++cj) {
-          const float sc[4] = {st.s[cj].x, st.s[cj].y, st.s[cj].z, st.s[cj].w};
+          for (int cj = 0; cj < CT; ++cj) {
+            constexpr int j = (2 * u + h) % 16;  // this block within its scale group
+            const float sc[4] = {RowBroadcast<j>(sg[cur][cj].x), RowBroadcast<j>(sg[cur][cj].y),
+                                 RowBroadcast<j>(sg[cur][cj].z), RowBroadcast<j>(sg[cur][cj].w)};
 #pragma unroll
-          for (int rj = 0; rj < RT; ++rj) {
-            const i32x4 acc =
-                __builtin_amdgcn_mfma_i32_16x16x32_i8(st.w[cj], st.x[rj], zero, 0, 0, 0);
+            for (int rj = 0; rj < RT; ++rj) {
+              const i32x4 acc =
+                  __builtin_amdgcn_mfma_i32_16x16x32_i8(st.w[h][cj], st.x[rj][h], zero, 0, 0, 0);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              out[cj][rj][i] =
-                  __fadd_rn(out[cj][rj][i], __fmul_rn(static_cast<float>(acc[i]), sc[i]));
+              for (int i = 0; i < 4; ++i) {
+                out[cj][rj][i] =
+                    __fadd_rn(out[cj][rj][i], __fmul_rn(static_cast<float>(acc[i]), sc[i]));
+              }
             }
           }
         }
-      }
-    }
+      });
+    });
   }
 
   // fully_connected.cc:1078-1082: zero-point term, row scale, bias.
@@ -278,9 +323,15 @@ hipError_t LaunchPackInt4BlockwiseGemm(const uint8_t* filter, const uint16_t* sc
   return hipGetLastError();
 }
 
+// One row tile: 16 rows x the depth padded to whole pairs of blocks.
+static size_t RowTileBytes(int depth) {
+  return static_cast<size_t>(kTile) * ((static_cast<size_t>(depth) + 2 * kBlock - 1) /
+                                       (2 * kBlock) * (2 * kBlock));
+}
+
 size_t TiledRowsBytes(int batches, int depth) {
   const size_t row_tiles = (static_cast<size_t>(batches) + kTile - 1) / kTile;
-  return row_tiles * kTile * static_cast<size_t>(depth);
+  return row_tiles * RowTileBytes(depth);
 }
 
 hipError_t LaunchFcInt4BlockwiseGemm(const float* input, int variant, float* scaling_factors,
@@ -295,18 +346,19 @@ hipError_t LaunchFcInt4BlockwiseGemm(const float* input, int variant, float* sca
   {
     const dim3 grid(row_tiles * kTile), block(kQuantizeThreads);
     int8_t* tiled = static_cast<int8_t*>(tiled_rows);
+    const size_t tile_bytes = RowTileBytes(depth);
     switch (variant) {
       case LRTFC_QUANT_NEON_V8:
         hipLaunchKernelGGL(QuantizeRowsTiledKernel<LRTFC_QUANT_NEON_V8>, grid, block, 0, stream,
-                           input, batches, depth, tiled, scaling_factors, zero_points);
+                           input, batches, depth, tile_bytes, tiled, scaling_factors, zero_points);
         break;
       case LRTFC_QUANT_NEON_LEGACY:
         hipLaunchKernelGGL(QuantizeRowsTiledKernel<LRTFC_QUANT_NEON_LEGACY>, grid, block, 0,
-                           stream, input, batches, depth, tiled, scaling_factors, zero_points);
+                           stream, input, batches, depth, tile_bytes, tiled, scaling_factors, zero_points);
         break;
       default:
         hipLaunchKernelGGL(QuantizeRowsTiledKernel<LRTFC_QUANT_PORTABLE>, grid, block, 0, stream,
-                           input, batches, depth, tiled, scaling_factors, zero_points);
+                           input, batches, depth, tile_bytes, tiled, scaling_factors, zero_points);
         break;
     }
     if (hipError_t err = hipGetLastError()) return err;
@@ -315,7 +367,7 @@ hipError_t LaunchFcInt4BlockwiseGemm(const float* input, int variant, float* sca
   a.filter = reinterpret_cast<const i64*>(gemm_filter);
   a.scales = reinterpret_cast<const float4*>(gemm_filter +
                                              static_cast<size_t>(channel_tiles) * nb * 512);
-  a.activations = static_cast<const i64*>(tiled_rows);
+  a.activations = static_cast<const i64x2*>(tiled_rows);
   a.scaling_factors = scaling_factors;
   a.zero_points = zero_points;
   a.kfsum = kfsum;
@@ -328,21 +380,29 @@ hipError_t LaunchFcInt4BlockwiseGemm(const float* input, int variant, float* sca
   a.row_tiles = row_tiles;
   a.vector_store = (out_depth % 4 == 0) && (reinterpret_cast<uintptr_t>(output) % 16 == 0);
   // Tiles per wavefront (channels x rows), the four wavefronts of a workgroup side by side
-  // along the channels. Measured at 14336 x 4096: up to 64 rows the filter stream decides and
-  // one channel tile per wavefront spreads it over the most wavefronts; beyond, 2 x 4 tiles
-  // re-read the least (2048 rows: 584 us against 767 us with 2 x 2).
-  const int CT = row_tiles <= 4 ? 1 : 2;
+  // along the channels. Measured at 14336 x 4096: up to 128 rows one channel tile per
+  // wavefront spreads the filter stream over the most wavefronts (128 rows: 42 us against 51 us
+  // with two; 256 rows: level); beyond, 2 x 4 tiles re-read the least.
+  const int CT = row_tiles <= 8 ? 1 : 2;
   const int RT = row_tiles <= 1 ? 1 : row_tiles <= 2 ? 2 : 4;
   const dim3 grid((channel_tiles + 4 * CT - 1) / (4 * CT), (row_tiles + RT - 1) / RT);
   if (grid.y > 65535) return hipErrorInvalidValue;
+  // Pairs in flight: small tiles are bound by the filter stream and want many (16 rows: 19.5 us
+  // with 16 blocks in flight, 17.1 us with 32); the 2 x 4 form is bound by its arithmetic and
+  // runs best with one pair and 124 registers, four wavefronts per SIMD (2048 rows: 443 us
+  // against 462 us with two pairs and two wavefronts per SIMD).
   if (CT == 2) {
-    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<2, 4, 1>), grid, dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<2, 4, 1, 1>), grid, dim3(kThreads), 0,
+                       stream, a);
   } else if (RT == 4) {
-    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 4, 1>), grid, dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 4, 1, 4>), grid, dim3(kThreads), 0,
+                       stream, a);
   } else if (RT == 2) {
-    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 2, 1>), grid, dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 2, 1, 8>), grid, dim3(kThreads), 0,
+                       stream, a);
   } else {
-    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 1, 1>), grid, dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 1, 1, 16>), grid, dim3(kThreads), 0,
+                       stream, a);
   }
   return hipGetLastError();
 }

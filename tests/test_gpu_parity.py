@@ -452,11 +452,14 @@ def test_blockwise_int4_wavefronts_spanning_channel_groups(fc, B):
 @pytest.mark.parametrize("B,K,N,bias", [(16, 64, 8, False), (33, 128, 20, True), (64, 256, 70, False),
                                         (100, 2048, 264, True), (17, 4096, 130, False),
                                         (128, 1024, 64, True), (65, 96, 5, True), (1, 64, 4, False),
-                                        (250, 32, 33, False)])
+                                        (250, 32, 33, False), (16, 1184, 40, True),
+                                        (32, 2080, 24, False), (140, 1056, 48, True),
+                                        (300, 4128, 36, False)])
 def test_blockwise_int4_gemm_matches_oracle(fc, B, K, N, bias):
     """Prefill form (matrix-core GEMM, one float accumulator per output walking the blocks in
     order): bit-identical to the oracle, edges in every direction (rows and channels that do
-    not fill their tiles, one block, odd channel counts with scalar stores)."""
+    not fill their tiles, one block, odd block counts that end inside a pair and inside a group
+    of 16 scales, odd channel counts with scalar stores) in each of the kernel's tile forms."""
     c = wl.blockwise_int4_fc(B, K, N, seed=11 + B + K + N, lo=-8, hi=7)
     b = np.random.default_rng(B).standard_normal(N).astype(np.float32) if bias else None
     op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], K, 32, b)
