@@ -149,10 +149,10 @@ int lrtfc_fc_int8(const int8_t* input, const int8_t* filter, const int32_t* bias
                   int32_t output_offset, int32_t act_min, int32_t act_max, void* stream);
 
 /* lrtfc_fc_int8 on a filter packed by lrtfc_pack_int8_filter, for every batch size: up to
- * 32 rows one matrix-core GEMV kernel whose cost does not grow with the batch up to 16 rows
- * (17..32 rows take two passes over the filter); above that an int8 MFMA GEMM that streams
- * the filter once (any batch count and out_depth; depth a multiple of 16, input and filter
- * 16-byte aligned -- other shapes keep the GEMV in tiles of 16 rows). Same arithmetic
+ * 16 rows one matrix-core GEMV kernel whose cost barely grows with the batch; above that an
+ * int8 MFMA GEMM that streams the filter once (any batch count and out_depth; depth a
+ * multiple of 16, input and filter 16-byte aligned -- other shapes keep the GEMV, one pass
+ * over the filter per 16 rows). Same arithmetic
  * contract as lrtfc_fc_int8 with filter_offset == 0; filter_row_sums (of the unpacked
  * filter) is required when input_offset != 0. */
 int lrtfc_fc_int8_packed(const int8_t* input, const int8_t* packed_filter, const int32_t* bias,

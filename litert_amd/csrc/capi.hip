@@ -46,8 +46,9 @@ int RequireInit() {
 // Batches from this size on go to the MFMA GEMM when its tiling fits.
 constexpr int kGemmMinBatches = 128;
 // On the re-tiled filter: up to this many rows the GEMV (16 rows per pass over the filter)
-// wins; beyond it the GEMM, which streams the filter once.
-constexpr int kPackedGemmMinBatches = 32;
+// wins; beyond it the GEMM, which streams the filter once (14336 x 4096 hybrid: 16 rows
+// 19 us on the GEMV; 24 and 32 rows 27 us on the GEMM against 32 and 34 us in two passes).
+constexpr int kPackedGemmMinBatches = 16;
 
 // Workspace layout for the hybrid paths (kernels.h).
 using Workspace = lrtfc::ActivationWorkspace;

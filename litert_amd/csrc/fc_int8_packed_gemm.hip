@@ -16,6 +16,9 @@
 // to 80 bytes so that the 16-byte operand reads are conflict-free) and every wavefront reads
 // its eight operands from there. Per step and wavefront: 4 global loads, 8 LDS reads, 16
 // MFMAs (512 matrix-core cycles), one barrier placed between the two halves of the MFMAs.
+// Launches that this 128 x 256 tile would cut into fewer workgroups than half the chip's CUs
+// (batches of a few dozen to a few hundred rows) run the same kernel with 64 rows x 128
+// channels per workgroup (32 channels per wavefront).
 //
 // int32 accumulation is exact, so tiling cannot change the accumulator; bit-exactness rests
 // on the epilogues, which are the ones of the GEMV kernels (fc_epilogues.h).
@@ -32,13 +35,8 @@ using i32x16 = int __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-constexpr int BM = 128;                       // batch rows per workgroup
-constexpr int kWaveTiles = 2;                 // 32-channel MFMA tiles per wavefront
-constexpr int BN = kWaves * kWaveTiles * 32;  // 256 output channels per workgroup
 constexpr int kStep = 64;                     // depth per step = one slab of the packed filter
 constexpr int kXStride = kStep + 16;          // padded LDS row
-constexpr int kStageBytes = BM * kXStride;    // 10240
-constexpr int kBatchTiles = BM / 32;          // 4
 constexpr int kSub = kStep / 32;              // MFMA depth sub-steps per step
 constexpr int kRing = 4;                      // weight register ring, in steps (even)
 constexpr int kGroupM = 4;                    // M-tiles per rasterization group
@@ -50,8 +48,15 @@ __device__ __forceinline__ void ForEachConst(std::integer_sequence<int, Is...>, 
   (f(std::integral_constant<int, Is>{}), ...);
 }
 
-template <Int8Epilogue EPI>
+// BM: batch rows per workgroup (128, or 64 for launches the large tile would leave with few
+// workgroups); kWaveTiles: 32-channel MFMA tiles per wavefront (2 or 1).
+template <Int8Epilogue EPI, int BM, int kWaveTiles>
 __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args a) {
+  constexpr int BN = kWaves * kWaveTiles * 32;  // output channels per workgroup
+  constexpr int kStageBytes = BM * kXStride;
+  constexpr int kBatchTiles = BM / 32;
+  constexpr int kXChunks = BM / 64;  // 16-byte chunks of activations a thread stages per step
+  static_assert(BM % 64 == 0 && BN <= kThreads, "tile shape");
   __shared__ __align__(16) int8_t smem[2 * kStageBytes];
   __shared__ i32x4 chan_params[BN];  // per output channel of the tile, for the epilogue
   const int M = a.batches, N = a.out_depth, K = a.depth;
@@ -105,18 +110,18 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
     const int ct = min(n0 / 16 + (wave * kWaveTiles + i) * 2 + ((lane & 31) >> 4), ctiles - 1);
     wp[i] = a.filter + static_cast<size_t>(ct) * slabs * 1024 + (lane & 15) * 16 + (lane >> 5) * 256;
   }
-  // Activation staging: two 16-byte chunks per thread and step, rows tid / 4 and 64 + tid / 4.
+  // Activation staging: 16-byte chunks per thread and step, rows tid / 4 (and 64 + tid / 4).
   const int ld_chunk = tid & 3;
-  const int8_t* xp[2];
+  const int8_t* xp[kXChunks];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < kXChunks; ++i) {
     const int row = min(m0 + (tid >> 2) + 64 * i, M - 1);
     xp[i] = a.input + static_cast<size_t>(row) * K;
   }
   const int st_off = (tid >> 2) * kXStride + ld_chunk * 16;
 
   i32x4 wring[kRing][kWaveTiles][kSub];
-  i32x4 xr[2][2];  // two sets: rows are requested two steps before they are staged
+  i32x4 xr[2][kXChunks];  // two sets: rows are requested two steps before they are staged
   auto load_w = [&](int step, auto slot) {
     const int s = min(step, slabs - 1);
 #pragma unroll
@@ -133,13 +138,13 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
     // into the row: whatever it reads meets zero padding in the packed filter or is unused.
     const int k = min(min(step, slabs - 1) * kStep + ld_chunk * 16, K - 16);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kXChunks; ++i) {
       xr[decltype(set)::value][i] = *reinterpret_cast<const i32x4*>(xp[i] + k);
     }
   };
   auto store_x = [&](int stage, auto set) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kXChunks; ++i) {
       *reinterpret_cast<i32x4*>(smem + stage * kStageBytes + st_off + i * 64 * kXStride) =
           xr[decltype(set)::value][i];
     }
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
   asm volatile("" ::: "memory");
   ForEachConst(std::make_integer_sequence<int, kRing - 1>{}, [&](auto u) { load_w(u, u); });
   asm volatile("" ::: "memory");
-  chan_params[tid] = chan_p;
+  if (tid < BN) chan_params[tid] = chan_p;
   __syncthreads();
   i32x4 fa[kBatchTiles][kSub];
 #pragma unroll
@@ -328,6 +333,23 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
   }
 }
 
+template <int BM, int kWaveTiles>
+hipError_t LaunchShape(const FcInt8Args& a, Int8Epilogue epilogue, int grid, hipStream_t stream) {
+  if (epilogue == Int8Epilogue::kRequantize) {
+    hipLaunchKernelGGL((FcInt8PackedGemmKernel<Int8Epilogue::kRequantize, BM, kWaveTiles>),
+                       dim3(grid), dim3(kThreads), 0, stream, a);
+  } else if (epilogue == Int8Epilogue::kHybrid) {
+    hipLaunchKernelGGL((FcInt8PackedGemmKernel<Int8Epilogue::kHybrid, BM, kWaveTiles>),
+                       dim3(grid), dim3(kThreads), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((FcInt8PackedGemmKernel<Int8Epilogue::kHybrid4Bit, BM, kWaveTiles>),
+                       dim3(grid), dim3(kThreads), 0, stream, a);
+  }
+  return hipGetLastError();
+}
+
+constexpr int kMinLargeTiles = 128;
+
 }  // namespace
 
 bool FcInt8PackedGemmSupports(const FcInt8Args& a) {
@@ -338,18 +360,12 @@ bool FcInt8PackedGemmSupports(const FcInt8Args& a) {
 
 hipError_t LaunchFcInt8PackedGemm(const FcInt8Args& a, Int8Epilogue epilogue, hipStream_t stream) {
   if (!FcInt8PackedGemmSupports(a)) return hipErrorNotSupported;
-  const int grid = ((a.batches + BM - 1) / BM) * ((a.out_depth + BN - 1) / BN);
-  if (epilogue == Int8Epilogue::kRequantize) {
-    hipLaunchKernelGGL(FcInt8PackedGemmKernel<Int8Epilogue::kRequantize>, dim3(grid),
-                       dim3(kThreads), 0, stream, a);
-  } else if (epilogue == Int8Epilogue::kHybrid) {
-    hipLaunchKernelGGL(FcInt8PackedGemmKernel<Int8Epilogue::kHybrid>, dim3(grid), dim3(kThreads),
-                       0, stream, a);
-  } else {
-    hipLaunchKernelGGL(FcInt8PackedGemmKernel<Int8Epilogue::kHybrid4Bit>, dim3(grid),
-                       dim3(kThreads), 0, stream, a);
-  }
-  return hipGetLastError();
+  // 128 x 256 tiles move the fewest bytes per MFMA; a launch they would cut into fewer
+  // workgroups than half the chip's CUs takes 64 x 128 tiles instead (four times as many).
+  const int large = ((a.batches + 127) / 128) * ((a.out_depth + 255) / 256);
+  if (large >= kMinLargeTiles) return LaunchShape<128, 2>(a, epilogue, large, stream);
+  return LaunchShape<64, 1>(a, epilogue, ((a.batches + 63) / 64) * ((a.out_depth + 127) / 128),
+                            stream);
 }
 
 }  // namespace lrtfc

@@ -142,7 +142,7 @@ class FullyConnectedInt8:
         capi.check(lib.lrtfc_row_sums_int8(_ptr(self.filter), self.out_depth, self.depth,
                                            _ptr(self.row_sums), _stream()))
         # packed: every batch size runs on a re-tiled copy of the filter (matrix-core GEMV up
-        # to 32 rows, MFMA GEMM above); otherwise the row-major kernels.
+        # to 16 rows, MFMA GEMM above); otherwise the row-major kernels.
         self.packed_filter = None
         if packed and self.filter_offset == 0 and self.depth > 0:
             self.packed_filter = _pack_int8(self.filter)

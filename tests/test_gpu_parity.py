@@ -152,22 +152,26 @@ def test_int8_prefill_gemm_bit_exact(fc, activation):
 
 @pytest.mark.parametrize("B,K,N", [(33, 64, 20), (128, 256, 256), (130, 272, 48), (200, 1040, 300),
                                    (64, 16, 4), (257, 192, 513), (40, 4096, 70), (300, 80, 257),
-                                   (129, 128, 30), (96, 2048, 64)])
+                                   (129, 128, 30), (96, 2048, 64), (1030, 48, 4100),
+                                   (2050, 80, 2049)])
 @pytest.mark.parametrize("activation", ["none", "relu6"])
 def test_int8_packed_gemm_ragged_shapes_bit_exact(fc, B, K, N, activation):
-    """More than 32 rows on the re-tiled filter take the MFMA GEMM: batch and channel counts
-    off the 128 x 256 tile, depths that end inside a 64-deep slab or give an odd slab count,
-    channel counts that rule out vector stores."""
+    """More than 16 rows on the re-tiled filter take the MFMA GEMM: batch and channel counts
+    off the tile (64 x 128 for the small launches, 128 x 256 for the last two), depths that
+    end inside a 64-deep slab or give an odd slab count, channel counts that rule out vector
+    stores."""
     c = wl.int8_fc(B, K, N, in_zp=(-3 if N % 2 else 0), seed=300 + B + K + N)
     y, want = _run_int8(fc, c, activation, bias=(N % 3 != 0))
     assert np.array_equal(y, want)
 
 
-@pytest.mark.parametrize("B,K,N", [(33, 64, 20), (128, 256, 256), (130, 272, 48), (65, 1040, 301)])
+@pytest.mark.parametrize("B,K,N", [(33, 64, 20), (128, 256, 256), (130, 272, 48), (65, 1040, 301),
+                                   (1025, 96, 4096)])
 @pytest.mark.parametrize("asym", [True, False])
 @pytest.mark.parametrize("per_channel", [True, False])
 def test_hybrid_packed_gemm_matches_oracle(fc, B, K, N, asym, per_channel):
-    """Hybrid rows beyond 32 run the same GEMM with the float epilogue."""
+    """Hybrid rows beyond 16 run the same GEMM with the float epilogue (the last shape in its
+    128 x 256 tile form)."""
     c = wl.hybrid_fc(B, K, N, seed=17 + B + K)
     bias = np.random.default_rng(3).standard_normal(N).astype(np.float32)
     pcs = c["pcs"] if per_channel else None
