@@ -458,7 +458,8 @@ def test_blockwise_int4_wavefronts_spanning_channel_groups(fc, B):
                                         (128, 1024, 64, True), (65, 96, 5, True), (1, 64, 4, False),
                                         (250, 32, 33, False), (16, 1184, 40, True),
                                         (32, 2080, 24, False), (140, 1056, 48, True),
-                                        (300, 4128, 36, False)])
+                                        (300, 4128, 36, False), (8, 32, 20, True), (40, 96, 24, False),
+                                        (20, 544, 16, True)])
 def test_blockwise_int4_gemm_matches_oracle(fc, B, K, N, bias):
     """Prefill form (matrix-core GEMM, one float accumulator per output walking the blocks in
     order): bit-identical to the oracle, edges in every direction (rows and channels that do
