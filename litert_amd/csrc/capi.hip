@@ -307,7 +307,7 @@ int lrtfc_fc_int8_preferred_layout(int batches, int depth, int out_depth, int32_
   a.depth = depth;
   a.out_depth = out_depth;
   a.filter_offset = filter_offset;
-  (void)batches;  // the re-tiled form serves every batch size (GEMV up to 32 rows, GEMM above)
+  (void)batches;  // the re-tiled form serves every batch size (GEMV up to 16 rows, GEMM above)
   return lrtfc::FcInt8PackedGemvSupports(a) ? LRTFC_LAYOUT_PACKED : LRTFC_LAYOUT_ROW_MAJOR;
 }
 

@@ -354,7 +354,8 @@ hipError_t LaunchFcInt4BlockwiseGemm(const float* input, int variant, float* sca
         break;
       case LRTFC_QUANT_NEON_LEGACY:
         hipLaunchKernelGGL(QuantizeRowsTiledKernel<LRTFC_QUANT_NEON_LEGACY>, grid, block, 0,
-                           stream, input, batches, depth, tile_bytes, tiled, scaling_factors, zero_points);
+                           stream, input, batches, depth, tile_bytes, tiled, scaling_factors,
+                           zero_points);
         break;
       default:
         hipLaunchKernelGGL(QuantizeRowsTiledKernel<LRTFC_QUANT_PORTABLE>, grid, block, 0, stream,
