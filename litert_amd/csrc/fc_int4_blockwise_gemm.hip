@@ -142,7 +142,9 @@ struct Stage {
 // Lane j of every 16 lanes to all 16 (row_newbcast:j).
 template <int J>
 __device__ __forceinline__ float RowBroadcast(float v) {
-  return DppMoveF32<0x150 + J>(v);
+  // Every lane has a source lane, so no previous value is kept: the move can then merge into
+  // the multiply that uses it.
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x150 + J, 0xF, 0xF, true));
 }
 
 // WROWS: wavefronts of a workgroup along the batch rows (1 or 2); the others along the channels.
