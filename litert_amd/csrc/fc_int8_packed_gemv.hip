@@ -14,12 +14,14 @@
 // depth, so a wavefront's load instruction reads 1 KiB of consecutive bytes and a
 // wavefront's whole share is one contiguous run.
 //
-// Each wavefront owns one 16-channel group over the whole depth and streams its
-// contiguous run through a ring of 16 outstanding 1 KiB loads, refilling a slot as soon
-// as the matrix core has consumed it; four wavefronts (four groups) form a workgroup and
-// share the staged activation rows. Short filters, which would leave most CUs without a
-// wavefront, split the depth over 2 or 4 wavefronts of the workgroup instead and add
-// their int32 partial tiles through LDS (exact: integer adds). The activation rows are
+// A wavefront streams a contiguous run of one 16-channel group's tiles through a ring of 16
+// outstanding 1 KiB loads, refilling a slot as soon as the matrix core has consumed it; four
+// wavefronts form a workgroup and share the staged activation rows. A group's depth is
+// shared out over 1, 2 or 4 wavefronts of the workgroup (int32 partial tiles added through
+// LDS: exact), chosen so that a wavefront's share stays about two rings long and the launch
+// has around a thousand wavefronts or more: shorter shares give more wavefronts per SIMD to
+// cover the prologue and the tail, longer ones amortize them better (14336 x 4096: two
+// wavefronts per group, 448 workgroups). The activation rows are
 // requested before the first weight load and staged in LDS while the ring fills. In the
 // hybrid form the staging step *is* the BatchQuantizeFloats of the op: the workgroup
 // reduces min/max of each float row, derives scale and zero point, and writes the
