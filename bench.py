@@ -211,9 +211,22 @@ def main():
                     algorithmic_bytes_per_launch=hybrid_bytes(b_dom),
                     avg_launch_us=per_b[b_dom]["op_us_cold"])
 
+    # Between decode and prefill (not a BASELINE configuration): config 2's filters against 16
+    # rows (row quantizer + GEMV) and 32 to 512 rows (row quantizer + MFMA GEMM, 64 x 128 tiles
+    # up to 256 rows).
+    between = {}
+    gen = torch.Generator(device="cuda").manual_seed(99)
+    for rows in (16, 32, 64, 128, 512):
+        xm = torch.randn((rows, K_IN), device="cuda", generator=gen)
+        ym = torch.empty((rows, N_OUT), dtype=torch.float32, device="cuda")
+        us = per_launch_us([(lambda o: lambda: o(xm, out=ym))(op) for op in ops])
+        between["us_%d_rows" % rows] = round(us, 1)
+        between["tops_%d_rows" % rows] = round(2.0 * rows * K_IN * N_OUT / us / 1e6, 1)
+
     also = {"config2_hybrid_per_batch": per_b, "config2_fused_vs_split": forms,
             "config2_step_ms_hot": round(ms_hot, 5),
-            "config2_step_gbps_hot": round(step_bytes / (ms_hot * 1e-3) / 1e9, 1)}
+            "config2_step_gbps_hot": round(step_bytes / (ms_hot * 1e-3) / 1e9, 1),
+            "next_hybrid_between_decode_and_prefill_14336x4096": between}
 
     if not args.skip_extras:
         also.update(extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_launch_us))
@@ -346,8 +359,8 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         frac_of_hbm_peak_cold=round(b3 / o_cold / 1e3 / HBM_PEAK_GBPS, 4), algorithmic_bytes=b3,
         kernel="FcInt4PackedKernel<fused quantize> on the re-tiled filter")
     # Prefill batches on the blockwise int4 path (not a BASELINE configuration): config 3's filter
-    # against 2048 and 128 rows through the matrix-core GEMM (row quantizer + row re-tiling +
-    # GEMM launches), and what the decode kernel needs for the same rows in passes of four.
+    # against 2048 and 128 rows through the matrix-core GEMM (row quantizer + GEMM launches),
+    # and what the decode kernel needs for the same rows in passes of four.
     op3 = fc.FullyConnectedBlockwiseInt4(c3["packed"], c3["scales"], 4096, 32)
     entry = {}
     for rows in (128, 2048):
