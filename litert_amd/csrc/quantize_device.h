@@ -232,7 +232,23 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   // Pass 1: range of the row. Starting from 0 gives min(0, min v) / max(0, max v),
   // which is also what max(|min|, |max|) needs for the symmetric case.
   float mn = 0.0f, mx = 0.0f;
-  if (vec_ok) {
+  // Rows of up to kRowRegs * kQuantizeThreads * 4 values stay in registers between the two
+  // passes instead of being read again.
+  constexpr int kRowRegs = 4;
+  const bool in_regs = vec_ok && n_data / 4 <= kRowRegs * kQuantizeThreads;
+  float4 held[kRowRegs];
+  if (in_regs) {
+    const float4* v4 = reinterpret_cast<const float4*>(v);
+#pragma unroll
+    for (int j = 0; j < kRowRegs; ++j) {
+      const int i = threadIdx.x + j * kQuantizeThreads;
+      // Past the end: zeros, which the range (it always includes 0) does not notice.
+      const float4 t = i < n_data / 4 ? v4[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      held[j] = t;
+      mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
+      mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
+    }
+  } else if (vec_ok) {
     const float4* v4 = reinterpret_cast<const float4*>(v);
     for (int i = threadIdx.x; i < n_data / 4; i += kQuantizeThreads) {
       const float4 t = v4[i];
@@ -262,28 +278,35 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   // Pass 2: elementwise. The NEON builds process 8 floats per step and finish
   // the remaining n_data % 8 with a scalar expression that rounds differently.
   const int vector_end = n_data - (n_data % 8);
-  if (vec_ok) {
-    const float4* v4 = reinterpret_cast<const float4*>(v);
-    for (int i = threadIdx.x; i < n_data / 4; i += kQuantizeThreads) {
-      char4 o;
-      if (all_zero) {
-        o = make_char4(0, 0, 0, 0);
+  // Elements 4 i .. 4 i + 3 of the row, given as t.
+  auto emit4 = [&](int i, const float4& t) {
+    char4 o;
+    if (all_zero) {
+      o = make_char4(0, 0, 0, 0);
+    } else {
+      const bool tail = 4 * i >= vector_end;
+      if (do_asymmetric) {
+        const int32_t packed = QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, tail);
+        o = make_char4(static_cast<char>(packed), static_cast<char>(packed >> 8),
+                       static_cast<char>(packed >> 16), static_cast<char>(packed >> 24));
       } else {
-        const float4 t = v4[i];
-        const bool tail = 4 * i >= vector_end;
-        if (do_asymmetric) {
-          const int32_t packed = QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, tail);
-          o = make_char4(static_cast<char>(packed), static_cast<char>(packed >> 8),
-                         static_cast<char>(packed >> 16), static_cast<char>(packed >> 24));
-        } else {
-          o.x = static_cast<char>(QuantizeSym<VARIANT>(t.x, inv, tail));
-          o.y = static_cast<char>(QuantizeSym<VARIANT>(t.y, inv, tail));
-          o.z = static_cast<char>(QuantizeSym<VARIANT>(t.z, inv, tail));
-          o.w = static_cast<char>(QuantizeSym<VARIANT>(t.w, inv, tail));
-        }
+        o.x = static_cast<char>(QuantizeSym<VARIANT>(t.x, inv, tail));
+        o.y = static_cast<char>(QuantizeSym<VARIANT>(t.y, inv, tail));
+        o.z = static_cast<char>(QuantizeSym<VARIANT>(t.z, inv, tail));
+        o.w = static_cast<char>(QuantizeSym<VARIANT>(t.w, inv, tail));
       }
-      *reinterpret_cast<char4*>(q + place(4 * i)) = o;
     }
+    *reinterpret_cast<char4*>(q + place(4 * i)) = o;
+  };
+  if (in_regs) {
+#pragma unroll
+    for (int j = 0; j < kRowRegs; ++j) {
+      const int i = threadIdx.x + j * kQuantizeThreads;
+      if (i < n_data / 4) emit4(i, held[j]);
+    }
+  } else if (vec_ok) {
+    const float4* v4 = reinterpret_cast<const float4*>(v);
+    for (int i = threadIdx.x; i < n_data / 4; i += kQuantizeThreads) emit4(i, v4[i]);
   } else {
     for (int i = threadIdx.x; i < n_data; i += kQuantizeThreads) {
       int8_t o = 0;
