@@ -40,6 +40,9 @@ typedef enum LrtFcActivation {
   LRTFC_ACT_RELU = 1,
   LRTFC_ACT_RELU_N1_TO_1 = 2,
   LRTFC_ACT_RELU6 = 3,
+  /* 4 (tanh) and 6 (sigmoid) go through Eigen in the reference and are not offered. */
+  LRTFC_ACT_SIGN_BIT = 5, /* float outputs only: 1.0f where the sign bit is set, else 0.0f
+                             (tflite/kernels/internal/portable_tensor_utils.cc:65-71) */
 } LrtFcActivation;
 
 /* Which build of the reference's activation quantizer to reproduce bit for bit
@@ -172,7 +175,8 @@ int lrtfc_batch_quantize_floats(const float* values, int n_batch, int n_data, in
  * MatrixBatchVectorMultiplyAccumulate (per-channel / offset form,
  * tflite/kernels/internal/reference/portable_tensor_utils.cc:165-206) together
  * with the bias initialisation and ApplyActivationToVector of EvalHybridDense
- * (tflite/kernels/fully_connected.cc:780-786, 854-856).
+ * (tflite/kernels/fully_connected.cc:780-786, 854-856), but not its early exit for a whole-zero
+ * input (:789-795), which belongs to the entry points that take the float rows.
  *   per_channel_scales NULL: per-tensor, filter_scale is folded into the batch
  *   scaling factor as the reference does (:838-843). bias may be NULL.
  *   zero_points NULL means symmetric activations (all zero). */
@@ -199,13 +203,26 @@ size_t lrtfc_activation_workspace_bytes(int batches, int depth);
 
 /* EvalHybridDense end to end (tflite/kernels/fully_connected.cc:763-858):
  * quantizes `input` per row into `workspace`, then runs lrtfc_fc_hybrid_int8.
- * The reference's all-zero-input early exit (:789-795) needs no special case:
- * an all-zero row quantizes to zeros and contributes nothing. */
+ * The reference's all-zero-input early exit (:789-795: output = activation(bias), product
+ * skipped) is reproduced, down to a bias element of -0.0f staying -0.0f. */
 int lrtfc_fc_hybrid(const float* input, const int8_t* filter, const float* per_channel_scales,
                     float filter_scale, const int32_t* filter_row_sums, const float* bias,
                     float* output, int batches, int depth, int out_depth,
                     int asymmetric_quantize_inputs, int activation, int quant_variant,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* lrtfc_fc_hybrid on a packed filter (lrtfc_pack_int8_filter) with the row quantizer as a
+ * launch of its own: the form for batch sizes where quantizing every row in every workgroup
+ * (lrtfc_fc_hybrid_packed) costs more than a second launch. Replaces EvalHybridDense,
+ * tflite/kernels/fully_connected.cc:763-858, all-zero-input early exit included; workspace as
+ * for lrtfc_fc_hybrid. Bit-identical results. */
+int lrtfc_fc_hybrid_packed_workspace(const float* input, const int8_t* packed_filter,
+                                     const float* per_channel_scales, float filter_scale,
+                                     const int32_t* filter_row_sums, const float* bias,
+                                     float* output, int batches, int depth, int out_depth,
+                                     int asymmetric_quantize_inputs, int activation,
+                                     int quant_variant, void* workspace, size_t workspace_bytes,
+                                     void* stream);
 
 /* EvalHybridDense as ONE kernel on a packed filter: each workgroup quantizes the float
  * rows itself (BatchQuantizeFloats semantics, same three variants) while its weight loads

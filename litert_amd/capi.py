@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "liblitert_amd_fc.so")
 
 OK, INVALID_ARGUMENT, NO_DEVICE, HIP_ERROR, UNSUPPORTED = range(5)
 ACT_NONE, ACT_RELU, ACT_RELU_N1_TO_1, ACT_RELU6 = range(4)
+ACT_SIGN_BIT = 5
 QUANT_PORTABLE, QUANT_NEON_V8, QUANT_NEON_LEGACY = range(3)
 OUT_FLOAT32, OUT_FLOAT16 = range(2)
 
@@ -49,6 +50,8 @@ SYMBOLS = [
     ("lrtfc_activation_workspace_bytes", _sz, [_i, _i]),
     ("lrtfc_fc_hybrid", _i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz,
                              _vp]),
+    ("lrtfc_fc_hybrid_packed_workspace", _i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i,
+                                              _i, _i, _vp, _sz, _vp]),
     ("lrtfc_fc_blockwise_int4", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz,
                                      _vp]),
     ("lrtfc_packed_int4_blockwise_bytes", _sz, [_i, _i]),

@@ -43,6 +43,12 @@ int RequireInit() {
     if (!(cond)) return Fail(LRTFC_INVALID_ARGUMENT, __VA_ARGS__); \
   } while (0)
 
+// Fused activations of the float-output paths: the clamps and the sign bit.
+bool FloatActivationOk(int activation) {
+  return (activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6) ||
+         activation == LRTFC_ACT_SIGN_BIT;
+}
+
 // Batches from this size on go to the MFMA GEMM when its tiling fits.
 constexpr int kGemmMinBatches = 128;
 // On the re-tiled filter: up to this many rows the GEMV (16 rows per pass over the filter)
@@ -383,8 +389,8 @@ int lrtfc_fc_hybrid_packed(const float* input, const int8_t* packed_filter,
   LRTFC_REQUIRE(input && packed_filter && output, "null pointer");
   LRTFC_REQUIRE(!asymmetric_quantize_inputs || filter_row_sums,
                 "filter_row_sums is required for asymmetric activation quantization");
-  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
-                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  LRTFC_REQUIRE(FloatActivationOk(activation),
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6/SignBit", activation);
   LRTFC_REQUIRE(quant_variant >= 0 && quant_variant <= LRTFC_QUANT_NEON_LEGACY,
                 "unknown quantizer variant");
   LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(packed_filter) & 15) == 0,
@@ -406,20 +412,21 @@ int lrtfc_fc_hybrid_packed(const float* input, const int8_t* packed_filter,
                  "packed hybrid GEMV");
 }
 
-int lrtfc_fc_hybrid_int8_packed(const int8_t* quantized_input, const float* scaling_factors,
-                                const int32_t* zero_points, const int8_t* packed_filter,
-                                const float* per_channel_scales, float filter_scale,
-                                const int32_t* filter_row_sums, const float* bias, float* output,
-                                int batches, int depth, int out_depth, int activation,
-                                void* stream) {
+namespace {
+int FcHybridInt8Packed(const int8_t* quantized_input, const float* scaling_factors,
+                       const int32_t* zero_points, const int8_t* packed_filter,
+                       const float* per_channel_scales, float filter_scale,
+                       const int32_t* filter_row_sums, const float* bias, float* output,
+                       int batches, int depth, int out_depth, int activation, int zero_input_exit,
+                       void* stream) {
   if (int rc = RequireInit()) return rc;
   LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
   if (batches == 0 || out_depth == 0) return LRTFC_OK;
   LRTFC_REQUIRE(quantized_input && scaling_factors && packed_filter && output, "null pointer");
   LRTFC_REQUIRE(!zero_points || filter_row_sums,
                 "filter_row_sums is required with activation zero points");
-  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
-                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  LRTFC_REQUIRE(FloatActivationOk(activation),
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6/SignBit", activation);
   LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(packed_filter) & 15) == 0,
                 "packed filter must be 16-byte aligned");
   lrtfc::FcInt8Args a{};
@@ -436,6 +443,7 @@ int lrtfc_fc_hybrid_int8_packed(const int8_t* quantized_input, const float* scal
   a.bias_f32 = bias;
   a.activation = activation;
   a.output_f32 = output;
+  a.zero_input_exit = zero_input_exit;
   if (batches > kPackedGemmMinBatches && lrtfc::FcInt8PackedGemmSupports(a)) {
     return FromHip(lrtfc::LaunchFcInt8PackedGemm(a, lrtfc::Int8Epilogue::kHybrid,
                                                  AsStream(stream)),
@@ -444,6 +452,43 @@ int lrtfc_fc_hybrid_int8_packed(const int8_t* quantized_input, const float* scal
   return FromHip(lrtfc::LaunchFcInt8PackedGemv(a, lrtfc::Int8Epilogue::kHybrid, nullptr, 0,
                                                LRTFC_QUANT_PORTABLE, AsStream(stream)),
                  "packed hybrid GEMV");
+}
+}  // namespace
+
+int lrtfc_fc_hybrid_int8_packed(const int8_t* quantized_input, const float* scaling_factors,
+                                const int32_t* zero_points, const int8_t* packed_filter,
+                                const float* per_channel_scales, float filter_scale,
+                                const int32_t* filter_row_sums, const float* bias, float* output,
+                                int batches, int depth, int out_depth, int activation,
+                                void* stream) {
+  return FcHybridInt8Packed(quantized_input, scaling_factors, zero_points, packed_filter,
+                            per_channel_scales, filter_scale, filter_row_sums, bias, output,
+                            batches, depth, out_depth, activation, /*zero_input_exit=*/0, stream);
+}
+
+int lrtfc_fc_hybrid_packed_workspace(const float* input, const int8_t* packed_filter,
+                                     const float* per_channel_scales, float filter_scale,
+                                     const int32_t* filter_row_sums, const float* bias,
+                                     float* output, int batches, int depth, int out_depth,
+                                     int asymmetric_quantize_inputs, int activation,
+                                     int quant_variant, void* workspace, size_t workspace_bytes,
+                                     void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(input && workspace, "null pointer");
+  LRTFC_REQUIRE(workspace_bytes >= WorkspaceBytes(batches, depth),
+                "workspace too small: %zu < %zu bytes", workspace_bytes,
+                WorkspaceBytes(batches, depth));
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
+                "workspace must be 256-byte aligned");
+  const Workspace w = SplitWorkspace(workspace, batches, depth);
+  int rc = lrtfc_batch_quantize_floats(input, batches, depth, w.q, w.sf, w.zp,
+                                       asymmetric_quantize_inputs, quant_variant, stream);
+  if (rc != LRTFC_OK) return rc;
+  return FcHybridInt8Packed(w.q, w.sf, asymmetric_quantize_inputs ? w.zp : nullptr, packed_filter,
+                            per_channel_scales, filter_scale, filter_row_sums, bias, output,
+                            batches, depth, out_depth, activation, /*zero_input_exit=*/1, stream);
 }
 
 int lrtfc_batch_quantize_floats(const float* values, int n_batch, int n_data, int8_t* quantized,
@@ -462,11 +507,13 @@ int lrtfc_batch_quantize_floats(const float* values, int n_batch, int n_data, in
                  "batch quantize");
 }
 
-int lrtfc_fc_hybrid_int8(const int8_t* quantized_input, const float* scaling_factors,
+namespace {
+int FcHybridInt8RowMajor(const int8_t* quantized_input, const float* scaling_factors,
                          const int32_t* zero_points, const int8_t* filter,
                          const float* per_channel_scales, float filter_scale,
                          const int32_t* filter_row_sums, const float* bias, float* output,
-                         int batches, int depth, int out_depth, int activation, void* stream) {
+                         int batches, int depth, int out_depth, int activation,
+                         int zero_input_exit, void* stream) {
   if (int rc = RequireInit()) return rc;
   LRTFC_REQUIRE(batches >= 0 && depth >= 0 && out_depth >= 0, "negative dimension");
   if (batches == 0 || out_depth == 0) return LRTFC_OK;
@@ -475,8 +522,8 @@ int lrtfc_fc_hybrid_int8(const int8_t* quantized_input, const float* scaling_fac
   LRTFC_REQUIRE(quantized_input && scaling_factors && filter, "null pointer");
   LRTFC_REQUIRE(!zero_points || filter_row_sums,
                 "filter_row_sums is required with activation zero points");
-  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
-                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  LRTFC_REQUIRE(FloatActivationOk(activation),
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6/SignBit", activation);
   lrtfc::FcInt8Args a{};
   a.input = quantized_input;
   a.filter = filter;
@@ -491,8 +538,21 @@ int lrtfc_fc_hybrid_int8(const int8_t* quantized_input, const float* scaling_fac
   a.bias_f32 = bias;
   a.activation = activation;
   a.output_f32 = output;
+  a.zero_input_exit = zero_input_exit;
   return FromHip(lrtfc::LaunchFcInt8Gemv(a, lrtfc::Int8Epilogue::kHybrid, AsStream(stream)),
                  "hybrid GEMV");
+}
+}  // namespace
+
+int lrtfc_fc_hybrid_int8(const int8_t* quantized_input, const float* scaling_factors,
+                         const int32_t* zero_points, const int8_t* filter,
+                         const float* per_channel_scales, float filter_scale,
+                         const int32_t* filter_row_sums, const float* bias, float* output,
+                         int batches, int depth, int out_depth, int activation, void* stream) {
+  return FcHybridInt8RowMajor(quantized_input, scaling_factors, zero_points, filter,
+                              per_channel_scales, filter_scale, filter_row_sums, bias, output,
+                              batches, depth, out_depth, activation, /*zero_input_exit=*/0,
+                              stream);
 }
 
 size_t lrtfc_activation_workspace_bytes(int batches, int depth) {
@@ -526,9 +586,9 @@ int lrtfc_fc_hybrid(const float* input, const int8_t* filter, const float* per_c
   if (rc != LRTFC_OK) return rc;
   // Symmetric quantization still writes zero points of 0, so the offset form of the
   // product applies to both modes, as in EvalHybridDense.
-  return lrtfc_fc_hybrid_int8(w.q, w.sf, w.zp, filter, per_channel_scales, filter_scale,
+  return FcHybridInt8RowMajor(w.q, w.sf, w.zp, filter, per_channel_scales, filter_scale,
                               filter_row_sums, bias, output, batches, depth, out_depth, activation,
-                              stream);
+                              /*zero_input_exit=*/1, stream);
 }
 
 int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
@@ -656,8 +716,8 @@ int lrtfc_fc_hybrid_int4_per_channel_packed(const float* input, const int8_t* pa
   LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
   if (batches == 0 || out_depth == 0) return LRTFC_OK;
   LRTFC_REQUIRE(input && packed_filter && output && workspace, "null pointer");
-  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
-                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  LRTFC_REQUIRE(FloatActivationOk(activation),
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6/SignBit", activation);
   LRTFC_REQUIRE(workspace_bytes >= WorkspaceBytes(batches, depth),
                 "workspace too small: %zu < %zu bytes", workspace_bytes,
                 WorkspaceBytes(batches, depth));
@@ -720,8 +780,8 @@ int lrtfc_fc_hybrid_int4_per_channel_nibbles(const float* input, const uint8_t* 
   LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
   if (batches == 0 || out_depth == 0) return LRTFC_OK;
   LRTFC_REQUIRE(input && retiled_filter && output && workspace, "null pointer");
-  LRTFC_REQUIRE(activation >= LRTFC_ACT_NONE && activation <= LRTFC_ACT_RELU6,
-                "activation %d is not one of None/Relu/ReluN1To1/Relu6", activation);
+  LRTFC_REQUIRE(FloatActivationOk(activation),
+                "activation %d is not one of None/Relu/ReluN1To1/Relu6/SignBit", activation);
   LRTFC_REQUIRE(lrtfc::FcInt4PerChannelGemvSupports(depth),
                 "depth %d is odd or too large for the nibble GEMV", depth);
   LRTFC_REQUIRE(workspace_bytes >= WorkspaceBytes(batches, depth),

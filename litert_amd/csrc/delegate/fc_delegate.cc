@@ -224,9 +224,12 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
     if (bias && bias->type != kTfLiteFloat32) return no("bias is not float32");
     if (filter.type == kTfLiteInt8) {
       if (!opt.claim_hybrid) return no("hybrid path disabled by option");
-      // The hybrid path accepts every fused activation; tanh/sigmoid/signbit go through
-      // Eigen in the reference and are left to the CPU.
-      if (!ClippingActivation(params->activation)) return no("activation not a clamp");
+      // The hybrid path accepts every fused activation (fully_connected.cc:748-753); tanh and
+      // sigmoid go through Eigen in the reference (no bit-level contract) and are left to the
+      // CPU. The sign bit is exact.
+      if (!ClippingActivation(params->activation) && params->activation != kTfLiteActSignBit) {
+        return no("activation is tanh or sigmoid");
+      }
       if (filter.quantization.type != kTfLiteAffineQuantization) return no("filter not affine");
       const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
       if (!fq || !fq->scale || fq->scale->size < 1) return no("filter has no scales");
@@ -258,12 +261,19 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
       // (fully_connected.cc:609-613) the builtin unpacks to int8 and runs the ordinary hybrid
       // kernels, which quantize differently: those shapes stay on the CPU.
       if (!opt.claim_int4_per_channel) return no("int4 per-channel path disabled by option");
-      if (!ClippingActivation(params->activation)) return no("activation not a clamp");
+      if (!ClippingActivation(params->activation) && params->activation != kTfLiteActSignBit) {
+        return no("activation is tanh or sigmoid");
+      }
       if (depth % 2 != 0 || out_depth < 4 || depth < 32) return no("shape outside 4-bit gate");
       const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
       if (!fq || !fq->scale || fq->scale->size < 1) return no("filter has no scales");
-      if (fq->scale->size > 1 && fq->scale->size != out_depth) {
+      if (fq->scale->size > 1 && (fq->quantized_dimension != 0 || fq->scale->size != out_depth)) {
         return no("per-channel scales do not match output channels");
+      }
+      // Both kernels of this path stage a whole activation row in LDS; rows too deep for that
+      // are declined here rather than failing at invoke.
+      if (lrtfc_fc_int8_preferred_layout(1, depth, out_depth, 0) != LRTFC_LAYOUT_PACKED) {
+        return no("depth beyond what the 4-bit path kernels stage in LDS");
       }
       return FcKind::kHybridInt4;
     }
@@ -1118,16 +1128,11 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                                    n.depth, n.out_depth, asym, n.params.activation,
                                                    variant, s));
         } else {
-          const ActivationScratch w = SplitScratch(scratch.get(), n.batches, n.depth);
-          RETURN_IF_FC(ctx, lrtfc_batch_quantize_floats(static_cast<const float*>(in_dev),
-                                                        n.batches, n.depth, w.q, w.sf, w.zp, asym,
-                                                        variant, s));
-          RETURN_IF_FC(ctx, lrtfc_fc_hybrid_int8_packed(w.q, w.sf, asym ? w.zp : nullptr,
-                                                        n.retiled_dev.as<int8_t>(), pcs,
-                                                        n.filter_scale, n.row_sums_dev.as<int32_t>(),
-                                                        bias_f32, static_cast<float*>(out_dev),
-                                                        n.batches, n.depth, n.out_depth,
-                                                        n.params.activation, s));
+          RETURN_IF_FC(ctx, lrtfc_fc_hybrid_packed_workspace(
+                                static_cast<const float*>(in_dev), n.retiled_dev.as<int8_t>(), pcs,
+                                n.filter_scale, n.row_sums_dev.as<int32_t>(), bias_f32,
+                                static_cast<float*>(out_dev), n.batches, n.depth, n.out_depth, asym,
+                                n.params.activation, variant, scratch.get(), scratch.bytes(), s));
         }
         break;
       }

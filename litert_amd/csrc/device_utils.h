@@ -56,14 +56,22 @@ __device__ __forceinline__ int32_t ClampI32(int32_t v, int32_t lo, int32_t hi) {
 // ---- float helpers (explicitly rounded: no FMA contraction) -----------------
 
 __device__ __forceinline__ float ApplyFloatActivation(float v, int activation) {
-  // tflite/kernels/internal/portable_tensor_utils.cc:41-62: max/min forms.
+  // tflite/kernels/internal/portable_tensor_utils.cc:41-71, written out as std::max(a, b) =
+  // (a < b) ? b : a and std::min(a, b) = (b < a) ? b : a, which also fixes what a -0.0f or a NaN
+  // turns into (std::max(0.0f, -0.0f) is +0.0f; std::max(-1.0f, -0.0f) is -0.0f).
   switch (activation) {
     case 1:
-      return fmaxf(0.0f, v);
-    case 2:
-      return fmaxf(-1.0f, fminf(v, 1.0f));
-    case 3:
-      return fmaxf(0.0f, fminf(v, 6.0f));
+      return (0.0f < v) ? v : 0.0f;
+    case 2: {
+      const float t = (1.0f < v) ? 1.0f : v;
+      return (-1.0f < t) ? t : -1.0f;
+    }
+    case 3: {
+      const float t = (6.0f < v) ? 6.0f : v;
+      return (0.0f < t) ? t : 0.0f;
+    }
+    case 5:  // kTfLiteActSignBit: std::signbit as a float
+      return (__float_as_uint(v) >> 31) ? 1.0f : 0.0f;
     default:
       return v;
   }

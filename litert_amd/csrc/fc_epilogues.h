@@ -28,6 +28,58 @@ __device__ __forceinline__ float HybridCore(int32_t dot, float batch_scale, floa
   return ApplyFloatActivation(out, activation);
 }
 
+// EvalHybridDense leaves the output at activation(bias) when the WHOLE input is zero and skips
+// the product (tflite/kernels/fully_connected.cc:789-795). Adding the zero product instead gives
+// the same bits except for a bias element of -0.0f (-0.0f + 0.0f is +0.0f). So the kernels add
+// the product as always and repair that one case lazily: a thread that meets a -0.0f bias with a
+// zero dot product scans the input; only a whole-zero input takes the scan to its end. A row
+// quantizes to all-zero values exactly when it was all zero (any other row has a value at the
+// far end of the int8 range), so the quantized rows can stand for the float ones.
+__device__ inline bool AllZeroInt8(const int8_t* p, size_t n) {
+  size_t i = 0;
+  if ((reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+    const i32x4* v = reinterpret_cast<const i32x4*>(p);
+    for (; i + 64 <= n; i += 64) {
+      const i32x4 t = (v[i / 16] | v[i / 16 + 1]) | (v[i / 16 + 2] | v[i / 16 + 3]);
+      if ((t.x | t.y | t.z | t.w) != 0) return false;
+    }
+  }
+  for (; i < n; ++i) {
+    if (p[i] != 0) return false;
+  }
+  return true;
+}
+
+__device__ inline bool AllZeroF32(const float* p, size_t n) {  // IsZeroVector: -0.0f counts as zero
+  const uint32_t* u = reinterpret_cast<const uint32_t*>(p);
+  size_t i = 0;
+  for (; i + 4 <= n; i += 4) {
+    if ((((u[i] | u[i + 1]) | (u[i + 2] | u[i + 3])) << 1) != 0) return false;
+  }
+  for (; i < n; ++i) {
+    if ((u[i] << 1) != 0) return false;
+  }
+  return true;
+}
+
+__device__ __forceinline__ bool IsNegativeZero(float v) {
+  return __float_as_uint(v) == 0x80000000u;
+}
+
+// HybridCore for kernels that run on already quantized rows (a.input), with the whole-zero-input
+// case above when the caller asked for EvalHybridDense semantics (a.zero_input_exit).
+__device__ __forceinline__ float HybridCoreZeroAware(const FcInt8Args& a, int32_t dot,
+                                                     float batch_scale, float channel_scale,
+                                                     int32_t batch_zero_point, int32_t row_sum,
+                                                     float base) {
+  if (a.zero_input_exit && dot == 0 && IsNegativeZero(base) &&
+      AllZeroInt8(a.input, static_cast<size_t>(a.batches) * a.depth)) {
+    return ApplyFloatActivation(base, a.activation);
+  }
+  return HybridCore(dot, batch_scale, channel_scale, batch_zero_point, row_sum, base,
+                    a.activation);
+}
+
 // Output value of the per-channel int4 hybrid path: ReferenceAssignBiasAndComputeOffsets and
 // ReferenceUnpack (tflite/kernels/internal/optimized/4bit/fully_connected_reference.cc:182-272)
 // followed by ApplyActivationToVector. `dot` is sum(w * q) over the depth with the signed
@@ -65,7 +117,7 @@ __device__ __forceinline__ void StoreHybrid(const FcInt8Args& a, int b, int n, i
   const int32_t row_sum = batch_zero_point != 0 ? a.filter_row_sums[n] : 0;
   const float base = a.bias_f32 ? a.bias_f32[n] : 0.0f;
   a.output_f32[static_cast<size_t>(b) * a.out_depth + n] =
-      HybridCore(dot, batch_scale, channel_scale, batch_zero_point, row_sum, base, a.activation);
+      HybridCoreZeroAware(a, dot, batch_scale, channel_scale, batch_zero_point, row_sum, base);
 }
 
 }  // namespace lrtfc

@@ -669,6 +669,19 @@ int MaxBatchTile(int depth) {
   return (FUSED && depth > kShallowDepth && depth <= kDeepDepth) ? 2 : 4;
 }
 
+// A workgroup may use 160 KB of LDS; the maps below keep 10 KB clear of that.
+constexpr size_t kLdsBudget = 150 * 1024;
+
+// Rows per launch: `want` (1, 2 or 4) cut down until the LDS map of that many rows fits.
+int FitBatchTile(int want, int padded, int ksplit) {
+  int bt = want > 2 ? 4 : want;
+  while (bt > 1 && (bt > 2 ? Int4Shared<4>::Bytes(padded, ksplit)
+                           : Int4Shared<2>::Bytes(padded, ksplit)) > kLdsBudget) {
+    bt = bt > 2 ? 2 : 1;
+  }
+  return bt;
+}
+
 template <bool FUSED>
 hipError_t LaunchTile(const Int4PackedArgs& a, int variant, int batch0, int bt,
                       hipStream_t stream) {
@@ -705,7 +718,7 @@ hipError_t LaunchPackInt4Blockwise(const uint8_t* filter, const uint16_t* scales
 bool FcInt4PackedSupports(int depth, int blocksize) {
   if (blocksize != kBlock || depth <= 0 || depth % kBlock != 0) return false;
   const int chunks = (depth / kBlock + kTileBlocks - 1) / kTileBlocks;
-  return Int4Shared<1>::Bytes(chunks * kTileBlocks * kBlock, kWaves) <= 150 * 1024;
+  return Int4Shared<1>::Bytes(chunks * kTileBlocks * kBlock, kWaves) <= kLdsBudget;
 }
 
 hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const float* input_f32,
@@ -726,15 +739,11 @@ hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const 
   a.out_depth = q.out_depth;
   a.chunks = (q.depth / kBlock + kTileBlocks - 1) / kTileBlocks;
   const int padded = a.chunks * kTileBlocks * kBlock;
+  const int tile = FitBatchTile(input_f32 ? MaxBatchTile<true>(q.depth) : MaxBatchTile<false>(q.depth),
+                                padded, ChooseKsplit(q.out_depth, a.chunks));
   int batch0 = 0;
   while (batch0 < q.batches) {
-    int bt = min(input_f32 ? MaxBatchTile<true>(q.depth) : MaxBatchTile<false>(q.depth),
-                 q.batches - batch0);
-    const int ksplit = ChooseKsplit(q.out_depth, a.chunks);
-    while (bt > 1 && (bt > 2 ? Int4Shared<4>::Bytes(padded, ksplit)
-                             : Int4Shared<2>::Bytes(padded, ksplit)) > 150 * 1024) {
-      bt = bt > 2 ? 2 : 1;
-    }
+    const int bt = min(tile, q.batches - batch0);
     const hipError_t err = input_f32 ? LaunchTile<true>(a, variant, batch0, bt, stream)
                                      : LaunchTile<false>(a, variant, batch0, bt, stream);
     if (err != hipSuccess) return err;
@@ -866,11 +875,14 @@ hipError_t LaunchGroupQuantizer(const void* table, const lrtfc_int4_group_launch
 hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_launch& l,
                                      int variant, hipStream_t stream) {
   if (l.count < 1 || l.grid_blocks < 1) return hipSuccess;
+  const int chunks = (l.depth / kBlock + kTileBlocks - 1) / kTileBlocks;
+  const int padded = chunks * kTileBlocks * kBlock;
   if (l.split_quantize) {
     if (hipError_t err = LaunchGroupQuantizer(table, l, variant, stream)) return err;
     const bool deep_rows = l.depth > kShallowDepth;
-    for (int batch0 = 0; batch0 < l.batches; batch0 += 4) {
-      const int bt = min(4, l.batches - batch0);
+    const int tile = FitBatchTile(4, padded, l.ksplit);
+    for (int batch0 = 0; batch0 < l.batches; batch0 += tile) {
+      const int bt = min(tile, l.batches - batch0);
       hipError_t err;
       if (deep_rows) {
         err = bt <= 1   ? LaunchGroupedOne<1, false, LRTFC_QUANT_PORTABLE, 8>(table, l, batch0, bt, stream)
@@ -886,7 +898,7 @@ hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_l
     return hipSuccess;
   }
   const bool deep = l.depth > kShallowDepth && l.depth <= kDeepDepth;
-  const int tile = MaxBatchTile<true>(l.depth);
+  const int tile = FitBatchTile(MaxBatchTile<true>(l.depth), padded, l.ksplit);
   for (int batch0 = 0; batch0 < l.batches; batch0 += tile) {  // more rows: one launch per tile
     const int bt = min(tile, l.batches - batch0);
     hipError_t err;

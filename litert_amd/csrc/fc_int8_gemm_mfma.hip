@@ -192,13 +192,10 @@ bool FcInt8GemmMfmaSupports(const FcInt8Args& a) {
 
 hipError_t LaunchFcInt8GemmMfma(const FcInt8Args& a, hipStream_t stream) {
   if (!FcInt8GemmMfmaSupports(a)) return hipErrorNotSupported;
-  static bool attribute_set = false;
   const int lds_bytes = 2 * kStageBytes;
-  if (!attribute_set) {
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(FcInt8GemmKernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (err != hipSuccess) return err;
-    attribute_set = true;
+  if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(FcInt8GemmKernel),
+                                        lds_bytes)) {
+    return err;
   }
   const int grid = (a.batches / BM) * (a.out_depth / BN);
   hipLaunchKernelGGL(FcInt8GemmKernel, dim3(grid), dim3(kThreads), lds_bytes, stream, a);

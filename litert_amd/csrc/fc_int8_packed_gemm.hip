@@ -307,8 +307,8 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
             v[r] = EPI == Int8Epilogue::kHybrid4Bit
                        ? Hybrid4BitCore(acc[i][j][4 * g + r], bscale, cscale[r], bzp, base[r],
                                         a.bias_f32 != nullptr, a.activation)
-                       : HybridCore(acc[i][j][4 * g + r], bscale, cscale[r], bzp, rsum[r],
-                                    base[r], a.activation);
+                       : HybridCoreZeroAware(a, acc[i][j][4 * g + r], bscale, cscale[r], bzp,
+                                             rsum[r], base[r]);
           }
           if (kFull || m < M) {
             float* dst = a.output_f32 + static_cast<size_t>(m) * N + c0;

@@ -445,12 +445,29 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(
       const float channel_scale = a.per_channel_scales ? ep_f0[i] : a.filter_scale;
       const float bias = a.bias_f32 ? ep_f1[i] : 0.0f;
       const int32_t row_sum = a.filter_row_sums ? ep_i0[i] : 0;
-      a.output_f32[static_cast<size_t>(b) * a.out_depth + n] =
-          EPI == Int8Epilogue::kHybrid4Bit
-              ? Hybrid4BitCore(acc[i], batch_scale, channel_scale, batch_zp, bias,
-                               a.bias_f32 != nullptr, a.activation)
-              : HybridCore(acc[i], batch_scale, channel_scale, batch_zp, row_sum, bias,
-                           a.activation);
+      float value;
+      if (EPI == Int8Epilogue::kHybrid4Bit) {
+        value = Hybrid4BitCore(acc[i], batch_scale, channel_scale, batch_zp, bias,
+                               a.bias_f32 != nullptr, a.activation);
+      } else if (FUSED) {
+        // Whole-zero input (fully_connected.cc:789-795): this launch knows its own rows from
+        // the prologue; rows of other launches of the same call are scanned, lazily.
+        bool zero_input = false;
+        if (sh.zero[col] != 0 && IsNegativeZero(bias)) {
+          zero_input = true;
+          for (int r = 0; r < bt; ++r) zero_input = zero_input && sh.zero[r] != 0;
+          if (zero_input && a.batches > bt) {
+            zero_input = AllZeroF32(p.input_f32, static_cast<size_t>(a.batches) * depth);
+          }
+        }
+        value = zero_input ? ApplyFloatActivation(bias, a.activation)
+                           : HybridCore(acc[i], batch_scale, channel_scale, batch_zp, row_sum,
+                                        bias, a.activation);
+      } else {
+        value = HybridCoreZeroAware(a, acc[i], batch_scale, channel_scale, batch_zp, row_sum,
+                                    bias);
+      }
+      a.output_f32[static_cast<size_t>(b) * a.out_depth + n] = value;
     }
   }
 }

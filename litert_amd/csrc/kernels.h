@@ -61,6 +61,9 @@ struct FcInt8Args {
   const float* bias_f32;
   int activation;
   float* output_f32;
+  // Non-zero: EvalHybridDense semantics for a whole-zero input (output = activation(bias), no
+  // product added; fully_connected.cc:789-795). Zero: MatrixBatchVectorMultiplyAccumulate as is.
+  int zero_input_exit;
 };
 
 // kHybrid4Bit: the float epilogue of the per-channel int4 hybrid path; a.zero_points then

@@ -15,7 +15,7 @@ import torch
 from . import capi
 
 _ACT = {"none": capi.ACT_NONE, "relu": capi.ACT_RELU, "relu_n1_to_1": capi.ACT_RELU_N1_TO_1,
-        "relu6": capi.ACT_RELU6}
+        "relu6": capi.ACT_RELU6, "sign_bit": capi.ACT_SIGN_BIT}
 
 
 def _act(a):
@@ -221,33 +221,20 @@ class FullyConnectedHybrid:
     # costs more than a separate quantization launch.
     FUSED_MAX_BATCHES = 4
 
-    def _split_buffers(self, batches, device):
-        key = (batches, str(device))
-        if getattr(self, "_split_key", None) != key:
-            self._split_q = torch.empty((batches, self.depth), dtype=torch.int8, device=device)
-            self._split_sf = torch.empty(batches, dtype=torch.float32, device=device)
-            self._split_zp = torch.zeros(batches, dtype=torch.int32, device=device)
-            self._split_key = key
-        return self._split_q, self._split_sf, self._split_zp
-
     def call_split(self, x, out=None):
         """Two launches on the packed filter: the standalone row quantizer, then the
-        matrix-core GEMV on its int8 output. Same results as the fused call."""
+        matrix-core GEMV (or GEMM) on its int8 output. Same results as the fused call."""
         if self.packed_filter is None:
             raise RuntimeError("call_split needs the packed filter (packed=True)")
         x = x.contiguous()
         batches = x.numel() // self.depth
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
-        q, sf, zp = self._split_buffers(batches, x.device)
-        lib = capi.load()
-        capi.check(lib.lrtfc_batch_quantize_floats(_ptr(x), batches, self.depth, _ptr(q), _ptr(sf),
-                                                   _ptr(zp), int(self.asymmetric), self.variant,
-                                                   _stream()))
-        capi.check(lib.lrtfc_fc_hybrid_int8_packed(
-            _ptr(q), _ptr(sf), _ptr(zp) if self.asymmetric else None, _ptr(self.packed_filter),
-            _ptr(self.pcs), self.filter_scale, _ptr(self.row_sums), _ptr(self.bias), _ptr(out),
-            batches, self.depth, self.out_depth, self.activation, _stream()))
+        ws = self._workspace(batches)
+        capi.check(capi.load().lrtfc_fc_hybrid_packed_workspace(
+            _ptr(x), _ptr(self.packed_filter), _ptr(self.pcs), self.filter_scale,
+            _ptr(self.row_sums), _ptr(self.bias), _ptr(out), batches, self.depth, self.out_depth,
+            int(self.asymmetric), self.activation, self.variant, _ptr(ws), ws.numel(), _stream()))
         return out
 
 

@@ -61,7 +61,7 @@ def test_claim_predicate_int8():
 
 
 def _float_node(h, B=2, K=64, N=8, filter_type=INT8, blockwise=False, bs=32, per_channel=True,
-                scale_type=FLOAT16, **kw):
+                scale_type=FLOAT16, quantized_dimension=0, **kw):
     x = h.tensor(FLOAT32, (B, K))
     if blockwise:
         w = h.tensor(INT4, (N, K), data=np.zeros(N * K // 2, np.uint8), const=True)
@@ -70,7 +70,7 @@ def _float_node(h, B=2, K=64, N=8, filter_type=INT8, blockwise=False, bs=32, per
     else:
         nbytes = N * K if filter_type == INT8 else N * K // 2
         w = h.tensor(filter_type, (N, K), data=np.zeros(nbytes, np.int8), const=True)
-        h.affine(w, np.full(N if per_channel else 1, 0.004))
+        h.affine(w, np.full(N if per_channel else 1, 0.004), quantized_dimension=quantized_dimension)
     y = h.tensor(FLOAT32, (B, N))
     return h.fc(x, w, None, y, **kw)
 
@@ -80,7 +80,11 @@ def test_claim_predicate_float_activations():
         assert h.classify(_float_node(h))[0] == "hybrid"
         assert h.classify(_float_node(h, per_channel=False, asymmetric=False))[0] == "hybrid"
         assert h.classify(_float_node(h, activation=3))[0] == "hybrid"
-        assert h.classify(_float_node(h, activation=6)) == (None, "activation not a clamp")
+        # the hybrid path takes every activation in the reference; the sign bit is exact and
+        # claimed, tanh (4) and sigmoid (6) go through Eigen there and stay on the CPU
+        assert h.classify(_float_node(h, activation=5))[0] == "hybrid"
+        assert h.classify(_float_node(h, activation=4)) == (None, "activation is tanh or sigmoid")
+        assert h.classify(_float_node(h, activation=6)) == (None, "activation is tanh or sigmoid")
         assert h.classify(_float_node(h, blockwise=True))[0] == "int4_blockwise"
         assert h.classify(_float_node(h, blockwise=True, K=128, bs=64))[0] == "int4_blockwise"
         # the builtin's 4-bit gate: N >= 4, K >= 32, K even, blocksize | K
@@ -93,7 +97,11 @@ def test_claim_predicate_float_activations():
         assert h.classify(_float_node(h, filter_type=INT4, per_channel=False))[0] == "int4_per_channel"
         assert h.classify(_float_node(h, filter_type=INT4, N=2)) == (None, "shape outside 4-bit gate")
         assert h.classify(_float_node(h, filter_type=INT4, K=16)) == (None, "shape outside 4-bit gate")
-        assert h.classify(_float_node(h, filter_type=INT4, activation=4)) == (None, "activation not a clamp")
+        assert h.classify(_float_node(h, filter_type=INT4, activation=4)) == (None, "activation is tanh or sigmoid")
+        assert h.classify(_float_node(h, filter_type=INT4, activation=5))[0] == "int4_per_channel"
+        # scales along the depth are not per-output-channel scales
+        assert h.classify(_float_node(h, filter_type=INT4, N=8, K=8 * 8, quantized_dimension=1)) == (
+            None, "per-channel scales do not match output channels")
 
 
 def test_bad_options_are_rejected_before_touching_the_device():

@@ -80,6 +80,34 @@ def test_hybrid_node_through_delegate(B):
         assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("B", [2, 8])  # fused prologue / quantizer launch of its own
+def test_hybrid_sign_bit_and_whole_zero_input_through_delegate(B):
+    """kTfLiteActSignBit on a hybrid node, and the builtin's early exit for a whole-zero input
+    (fully_connected.cc:789-795): a -0.0f bias element must come out with its sign bit set."""
+    c = wl.hybrid_fc(B, 512, 96)
+    bias = np.random.default_rng(1).standard_normal(96).astype(np.float32)
+    bias[::4] = -0.0
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (B, 512), data=c["x"])
+        w = h.tensor(INT8, (96, 512), data=c["w"], const=True)
+        h.affine(w, c["pcs"])
+        b = h.tensor(FLOAT32, (96,), data=bias, const=True)
+        y = h.tensor(FLOAT32, (B, 96))
+        h.fc(x, w, b, y, activation=5, asymmetric=True)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.plan()[0][0] == "delegate"
+        assert h.invoke() == OK, h.errors()
+        want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"], 1.0, bias, True, oracle.ACT_SIGN_BIT)
+        assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+        zeros = np.zeros((B, 512), np.float32)
+        h.write(x, zeros)
+        assert h.invoke() == OK, h.errors()
+        want = oracle.fc_hybrid(zeros, c["w"], c["pcs"], 1.0, bias, True, oracle.ACT_SIGN_BIT)
+        assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+        assert want[0, 0] == 1.0 and want[0, 1] == (1.0 if bias[1] < 0 else 0.0)
+
+
 @pytest.mark.parametrize("B,K,N", [(2, 2048, 512), (1, 16384, 40), (3, 8192, 24), (5, 1024, 16)])
 def test_blockwise_int4_node_through_delegate(B, K, N):
     """Shallow rows and up to two deep rows run the fused kernel on the re-tiled filter; three

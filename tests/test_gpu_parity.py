@@ -346,6 +346,47 @@ def test_hybrid_fused_quantizer_variants(fc, variant):
     assert _bits_equal(y, want)
 
 
+@pytest.mark.parametrize("activation", ["none", "relu", "relu_n1_to_1", "relu6", "sign_bit"])
+@pytest.mark.parametrize("packed", ["fused", "split", False])
+@pytest.mark.parametrize("B", [1, 3, 19])
+def test_hybrid_whole_zero_input_keeps_the_bias_bits(fc, activation, packed, B):
+    """tflite/kernels/fully_connected.cc:789-795: a whole-zero input (a -0.0f element counts as
+    zero) leaves activation(bias) in the output and skips the product. Adding a zero product
+    instead would turn a bias element of -0.0f into +0.0f, so the bias here holds -0.0f, +0.0f
+    and ordinary values. Then one row is made non-zero: the exit no longer applies and the zero
+    rows go through the product like any other (-0.0f + 0.0f = +0.0f)."""
+    K, N = 520, 70
+    c = wl.hybrid_fc(B, K, N, seed=31)
+    bias = np.random.default_rng(9).standard_normal(N).astype(np.float32)
+    bias[::3] = -0.0
+    bias[1::7] = 0.0
+    op = fc.FullyConnectedHybrid(c["w"], c["pcs"], bias=bias, activation=activation,
+                                 packed=bool(packed))
+    x = np.zeros((B, K), np.float32)
+    x[0, 5] = -0.0
+    y = _hybrid_call(op, _cuda(x), packed).cpu().numpy()
+    want = oracle.fc_hybrid(x, c["w"], c["pcs"], 1.0, bias, True, fc._act(activation))
+    assert _bits_equal(y, want)
+    if activation == "none":
+        assert _bits_equal(y, np.broadcast_to(bias, (B, N)).copy())
+    x[B - 1] = c["x"][B - 1]
+    y = _hybrid_call(op, _cuda(x), packed).cpu().numpy()
+    want = oracle.fc_hybrid(x, c["w"], c["pcs"], 1.0, bias, True, fc._act(activation))
+    assert _bits_equal(y, want)
+
+
+@pytest.mark.parametrize("packed", ["fused", "split", False])
+def test_hybrid_sign_bit_activation(fc, packed):
+    """kTfLiteActSignBit on the hybrid path (tensor_utils.h:58-77 ->
+    portable_tensor_utils.cc:65-71): 1.0f where the result's sign bit is set."""
+    c = wl.hybrid_fc(5, 1040, 33, seed=12)
+    op = fc.FullyConnectedHybrid(c["w"], c["pcs"], activation="sign_bit", packed=bool(packed))
+    y = _hybrid_call(op, _cuda(c["x"]), packed).cpu().numpy()
+    want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"], 1.0, None, True, oracle.ACT_SIGN_BIT)
+    assert _bits_equal(y, want)
+    assert set(np.unique(y)) == {0.0, 1.0}
+
+
 def test_hybrid_full_size_properties(fc):
     """Config 2 at full size (14336 x 4096, B = 8): row sums against numpy, a sample of
     output channels against the oracle, and batch-row independence (row b of a B=8 call
@@ -360,6 +401,11 @@ def test_hybrid_full_size_properties(fc):
     pick = np.random.default_rng(2).choice(14336, 256, replace=False)
     want = oracle.fc_hybrid(c["x"], c["w"][pick], c["pcs"][pick])
     assert _bits_equal(np.ascontiguousarray(y8[:, pick]), want)
+    # B = 4 at full width (the batch size at which the fused kernel keeps four rows in
+    # registers): every channel against the oracle.
+    y4 = op(x[:4]).cpu().numpy()
+    want4 = oracle.fc_hybrid(c["x"][:4], c["w"], c["pcs"])
+    assert _bits_equal(y4, want4)
 
 
 # ---- blockwise int4 -------------------------------------------------------------------------
@@ -407,7 +453,13 @@ def test_blockwise_int4_split_launch_matches_oracle(fc, B, K, N):
                                     (9, 2048, (24, 80)), (5, 16384, (8, 16)),
                                     # deep rows beyond two: quantized by the group's own launch
                                     (3, 8192, (24, 40, 8)), (4, 16384, (16, 264)), (9, 8192, (8, 72)),
-                                    (1, 64, tuple(range(4, 36))), (2, 64, tuple(range(3, 103)))])
+                                    (1, 64, tuple(range(4, 36))), (2, 64, tuple(range(3, 103))),
+                                    # 4096..8191 channels in all: two wavefronts share a channel
+                                    # group's depth and four deep rows no longer fit the LDS, so
+                                    # the launch falls back to two rows at a time
+                                    (4, 16384, (2048, 2056)), (3, 16384, (4100,)),
+                                    # deeper than the register forms: rows re-read, LDS-bound tile
+                                    (3, 32768, (16, 24)), (4, 32768, (8,))])
 def test_blockwise_int4_grouped_launch_matches_oracle(fc, B, K, Ns):
     """Several filters of one depth in one launch: every node against the oracle, with its
     own input and, for odd channel counts, its own bias; then again after re-binding to new
