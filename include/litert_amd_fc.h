@@ -211,6 +211,25 @@ int lrtfc_fc_hybrid(const float* input, const int8_t* filter, const float* per_c
                     int asymmetric_quantize_inputs, int activation, int quant_variant,
                     void* workspace, size_t workspace_bytes, void* stream);
 
+/* lrtfc_fc_hybrid without the workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc). It has
+ * no counterpart in the reference. The activation scratch is a static device array of
+ * LRTFC_STATIC_SCRATCH_BYTES that the library holds on every device it was initialised on
+ * (lrtfc_init looks its address up); the call allocates and frees nothing and enqueues the same
+ * two launches as lrtfc_fc_hybrid, with bit-identical results. Fails with
+ * LRTFC_INVALID_ARGUMENT when lrtfc_activation_workspace_bytes(batches, depth) exceeds
+ * LRTFC_STATIC_SCRATCH_BYTES (64 rows of depth 16384 fit). All calls on one device share the
+ * one array: calls that overlap on a device (different streams or threads) race; calls ordered
+ * on one stream do not. */
+#define LRTFC_STATIC_SCRATCH_BYTES (1024 * 1024 + 64 * 1024)
+size_t lrtfc_static_scratch_bytes(void);
+int lrtfc_fc_hybrid_static_scratch(const float* input, const int8_t* filter,
+                                   const float* per_channel_scales, float filter_scale,
+                                   const int32_t* filter_row_sums, const float* bias,
+                                   float* output, int batches, int depth, int out_depth,
+                                   int asymmetric_quantize_inputs, int activation,
+                                   int quant_variant, void* stream);
+
 /* lrtfc_fc_hybrid on a packed filter (lrtfc_pack_int8_filter) with the row quantizer as a
  * launch of its own: the form for batch sizes where quantizing every row in every workgroup
  * (lrtfc_fc_hybrid_packed) costs more than a second launch. Replaces EvalHybridDense,

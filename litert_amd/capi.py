@@ -52,6 +52,9 @@ SYMBOLS = [
                              _vp]),
     ("lrtfc_fc_hybrid_packed_workspace", _i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i,
                                               _i, _i, _vp, _sz, _vp]),
+    ("lrtfc_static_scratch_bytes", _sz, []),
+    ("lrtfc_fc_hybrid_static_scratch", _i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i,
+                                            _i, _vp]),
     ("lrtfc_fc_blockwise_int4", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz,
                                      _vp]),
     ("lrtfc_packed_int4_blockwise_bytes", _sz, [_i, _i]),

@@ -33,6 +33,16 @@ hipStream_t AsStream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 bool g_initialised = false;
 
+// Scratch of lrtfc_fc_hybrid_static_scratch, the entry point that allocates nothing: the
+// activation workspace (quantized rows, scaling factors, zero points) that lrtfc_fc_hybrid
+// takes as an argument lives in this array instead. Every device the library runs on holds
+// its own copy at its own address until the process ends; in host code the array's name is
+// only a handle for hipGetSymbolAddress, never a device address. lrtfc_init looks the address
+// up once per device and the entry point passes that pointer to the kernels.
+static __device__ __align__(256) unsigned char scratch[LRTFC_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+
 int RequireInit() {
   if (g_initialised) return LRTFC_OK;
   return Fail(LRTFC_NO_DEVICE, "lrtfc_init() has not succeeded: no gfx950 device selected");
@@ -115,6 +125,12 @@ int lrtfc_init(int device_ordinal) {
   }
   err = hipSetDevice(device_ordinal);
   if (err != hipSuccess) return FromHip(err, "hipSetDevice");
+  if (device_ordinal < kMaxDevices && g_scratch_ptr[device_ordinal] == nullptr) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return FromHip(err, "hipGetSymbolAddress(scratch)");
+    g_scratch_ptr[device_ordinal] = ptr;
+  }
   g_initialised = true;
   return LRTFC_OK;
 }
@@ -589,6 +605,35 @@ int lrtfc_fc_hybrid(const float* input, const int8_t* filter, const float* per_c
   return FcHybridInt8RowMajor(w.q, w.sf, w.zp, filter, per_channel_scales, filter_scale,
                               filter_row_sums, bias, output, batches, depth, out_depth, activation,
                               /*zero_input_exit=*/1, stream);
+}
+
+size_t lrtfc_static_scratch_bytes(void) { return LRTFC_STATIC_SCRATCH_BYTES; }
+
+int lrtfc_fc_hybrid_static_scratch(const float* input, const int8_t* filter,
+                                   const float* per_channel_scales, float filter_scale,
+                                   const int32_t* filter_row_sums, const float* bias,
+                                   float* output, int batches, int depth, int out_depth,
+                                   int asymmetric_quantize_inputs, int activation,
+                                   int quant_variant, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth >= 0 && out_depth >= 0, "negative dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(WorkspaceBytes(batches, depth) <= LRTFC_STATIC_SCRATCH_BYTES,
+                "%d rows of depth %d need %zu bytes of activation scratch; the static scratch "
+                "holds %d (use lrtfc_fc_hybrid with a workspace of the caller's)",
+                batches, depth, WorkspaceBytes(batches, depth), LRTFC_STATIC_SCRATCH_BYTES);
+  int device = -1;
+  if (hipError_t err = hipGetDevice(&device)) return FromHip(err, "hipGetDevice");
+  void* ptr = (device >= 0 && device < kMaxDevices) ? g_scratch_ptr[device] : nullptr;
+  if (ptr == nullptr) {
+    return Fail(LRTFC_NO_DEVICE,
+                "lrtfc_init() has not run for device %d: its scratch address is unknown", device);
+  }
+  // Same two launches as lrtfc_fc_hybrid; the quantizer rewrites every byte the product reads,
+  // so what the previous call left in the array does not matter.
+  return lrtfc_fc_hybrid(input, filter, per_channel_scales, filter_scale, filter_row_sums, bias,
+                         output, batches, depth, out_depth, asymmetric_quantize_inputs, activation,
+                         quant_variant, ptr, LRTFC_STATIC_SCRATCH_BYTES, stream);
 }
 
 int lrtfc_fc_blockwise_int4_quantized(const int8_t* quantized_input,
