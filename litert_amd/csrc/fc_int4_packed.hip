@@ -14,7 +14,7 @@
 // A wavefront owns 8 channels over the whole depth. All loads of its first two tiles go
 // out first (a ring that is refilled tile by tile for deeper filters); the activation
 // rows are quantized (BatchQuantizeFloats, always asymmetric on this path) and staged in
-// LDS, de-interleaved into even-k / odd-k bytes to line up with low / high nibbles,
+// LDS, split into planes of high and low nibbles that line up with the filter's dwords,
 // while the ring fills. The reference then adds float(block_sum) * scale over the blocks
 // of a row in block order in float32; that order is kept: the products of a tile are
 // parked in LDS and 8 x batch lanes walk them in order, tile after tile, each walk
@@ -92,36 +92,53 @@ struct Int4PackedArgs {
   int batches, depth, out_depth, chunks;
 };
 
-// Even-k bytes and odd-k bytes of eight consecutive int8 (lo = k0..k0+3, hi = k0+4..k0+7).
-__device__ __forceinline__ void Deinterleave(uint32_t lo, uint32_t hi, int32_t* even,
-                                             int32_t* odd) {
-  *even = static_cast<int32_t>((lo & 0xFFu) | ((lo >> 8) & 0xFF00u) | ((hi & 0xFFu) << 16) |
-                               ((hi << 8) & 0xFF000000u));
-  *odd = static_cast<int32_t>(((lo >> 8) & 0xFFu) | ((lo >> 16) & 0xFF00u) |
-                              ((hi << 8) & 0xFF0000u) | (hi & 0xFF000000u));
+// Nibble planes of eight consecutive int8 activations (lo = q0..q3, hi = q4..q7 as packed
+// bytes): `high` holds (q >> 4) & 15 and `low` holds q & 15 of element i in bits 4i .. 4i + 3,
+// the order in which a dword of the filter holds its eight weights. With q = 16 * qh + ql
+// (qh signed, ql unsigned) a block's sum(w * q) is 16 * sdot8(w, qh) + udot8(w + 8, ql) -
+// 8 * sum(ql): eight 8-way dot products per 32 weights and no nibble unpacking at all.
+__device__ __forceinline__ uint32_t CompressNibbles(uint32_t t) {  // bytes 0x0n -> 16 bits
+  t = (t | (t >> 4)) & 0x00FF00FFu;
+  return (t | (t >> 8)) & 0xFFFFu;
+}
+__device__ __forceinline__ void NibblePlanes(uint32_t lo, uint32_t hi, int32_t* high,
+                                             int32_t* low) {
+  *low = static_cast<int32_t>(CompressNibbles(lo & 0x0F0F0F0Fu) |
+                              (CompressNibbles(hi & 0x0F0F0F0Fu) << 16));
+  *high = static_cast<int32_t>(CompressNibbles((lo >> 4) & 0x0F0F0F0Fu) |
+                               (CompressNibbles((hi >> 4) & 0x0F0F0F0Fu) << 16));
+}
+__device__ __forceinline__ int32_t SDot8(int32_t a, int32_t b, int32_t acc) {
+  return __builtin_amdgcn_sdot8(a, b, acc, false);
+}
+__device__ __forceinline__ uint32_t UDot8(uint32_t a, uint32_t b, uint32_t acc) {
+  return __builtin_amdgcn_udot8(a, b, acc, false);
 }
 
-// LDS map: [BT][padded depth] de-interleaved activations; per wavefront [8 * BT][kPStride]
+// LDS map: [BT][padded depth] activations as nibble planes (per block of 32: four dwords of
+// high nibbles, then four of low nibbles); per wavefront [8 * BT][kPStride]
 // parked products; per-row quantization state.
 template <int BT>
 struct Int4Shared {
   int32_t* q;   // dwords: per row padded_depth / 4
-  float* p;     // [kWaves][8 * BT][kPStride]
+  float* p;     // [waves][8 * BT][kPStride]
   float* sf;    // [BT]
   float* inv;   // [BT]
   int32_t* zp;  // [BT]
   int32_t* zero;
-  float* mm;    // [BT][kWaves][2]
-  float* kb;    // [kWaves][2][64]: kfsum and bias of the channels a wavefront covers
-  float* ob;    // [kWaves][64 * BT]: finished outputs of those channels
+  float* mm;    // [BT][waves][2]
+  float* kb;    // [waves][2][64]: kfsum and bias of the channels a wavefront covers
+  float* ob;    // [waves][64 * BT]: finished outputs of those channels
   // Floats of parked products: one tile per wavefront when a wavefront owns a channel group
   // alone; every tile of the group when `ksplit` wavefronts share it (the ordered walk then
   // needs them all).
   __host__ __device__ static size_t ProductFloats(int chunks, int ksplit) {
+    constexpr int waves = kWaves;
     const size_t tile = static_cast<size_t>(8) * BT * kPStride;
-    return ksplit == 1 ? kWaves * tile : (kWaves / ksplit) * static_cast<size_t>(chunks) * tile;
+    return ksplit == 1 ? waves * tile : (waves / ksplit) * static_cast<size_t>(chunks) * tile;
   }
   __device__ Int4Shared(int8_t* base, int padded, int chunks, int ksplit) {
+    constexpr int waves = kWaves;
     q = reinterpret_cast<int32_t*>(base);
     size_t off = static_cast<size_t>(BT) * padded;
     p = reinterpret_cast<float*>(base + off);
@@ -131,13 +148,14 @@ struct Int4Shared {
     zp = reinterpret_cast<int32_t*>(inv + 8);
     zero = zp + 8;
     mm = reinterpret_cast<float*>(zero + 8);
-    kb = mm + BT * kWaves * 2;
-    ob = kb + kWaves * 2 * 64;
+    kb = mm + BT * waves * 2;
+    ob = kb + waves * 2 * 64;
   }
   static size_t Bytes(int padded, int ksplit) {
+    constexpr int waves = kWaves;
     const int chunks = padded / (kTileBlocks * kBlock);
     return static_cast<size_t>(BT) * padded + ProductFloats(chunks, ksplit) * 4 + 4 * 8 * 4 +
-           BT * kWaves * 2 * 4 + kWaves * 2 * 64 * 4 + kWaves * 64 * BT * 4;
+           BT * waves * 2 * 4 + waves * 2 * 64 * 4 + waves * 64 * BT * 4;
   }
 };
 
@@ -147,9 +165,25 @@ struct Int4Shared {
 // gpw: consecutive channel groups one wavefront works through (ksplit == 1 only). Their
 // tiles are one contiguous stretch of the filter, so the ring of loads runs on across group
 // boundaries and the prologue (the row quantizer) is paid once for all of them.
-template <int BT, bool FUSED, int VARIANT, int GPT>
+// ALL > 0: a wavefront has at most ALL tiles (ksplit == 1, gpw * chunks <= ALL) and requests
+// every one of them before it does anything else: no refills, one memory round trip per
+// wavefront, and straight-line code whose waits for each tile are exact.
+template <int N, class F>
+__device__ __forceinline__ void StaticFor(F&& f) {
+  if constexpr (N > 0) {
+    StaticFor<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+// PRE of them go out ahead of the prologue, the rest behind it: a compute unit accepts only
+// some tens of KiB of outstanding loads, and a wavefront whose load issue blocks cannot do its
+// share of the row quantizer (14336 x 4096, one row: two tiles per wavefront, one ahead, 8.3 us;
+// both ahead 9.0 us; four tiles per wavefront all ahead 9.9 us; the refilled ring of two 8.5 us).
+template <int BT, bool FUSED, int VARIANT, int GPT, int ALL = 0, int PRE = 0>
 __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int block, int batch0,
                                                  int bt, int ksplit, int gpw, int8_t* smem) {
+
   // Every tensor is in global memory. Pointers that a kernel read from a table in memory
   // carry no address space, and accesses through them would go the flat path, whose waits
   // cannot leave a ring of loads in flight; so the address space is stated here.
@@ -249,10 +283,10 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
               hi |= static_cast<uint32_t>(static_cast<uint8_t>(x[g * 8 + 4 + t])) << (8 * t);
             }
           }
-          int32_t even, odd;
-          Deinterleave(lo, hi, &even, &odd);
-          sh.q[b * (padded / 4) + 2 * g] = even;
-          sh.q[b * (padded / 4) + 2 * g + 1] = odd;
+          int32_t high, low;
+          NibblePlanes(lo, hi, &high, &low);
+          sh.q[b * (padded / 4) + (g >> 2) * 8 + (g & 3)] = high;
+          sh.q[b * (padded / 4) + (g >> 2) * 8 + 4 + (g & 3)] = low;
         }
       }
     }
@@ -262,17 +296,22 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
   // tile is requested after the prologue's arithmetic, which then overlaps the time load issue
   // spends blocked on a full memory pipeline (measured: 15.4 -> 14.2 us at four rows); with one
   // row the prologue is too short for that to pay (9.0 -> 9.5 us), so both go out at once.
-  i32x4 ring[kRingTiles][kPlanes];
+  constexpr int kRing = ALL > 0 ? ALL : kRingTiles;
+  i32x4 ring[kRing][kPlanes];
   auto request_tile = [&](int t) {
     const int lin = min(kpart + t * ksplit, max(ntiles, 1) - 1);
+    // The plane of scales goes first: loads return in issue order, so the rows of a tile can
+    // then be worked through as they arrive instead of after the whole tile.
 #pragma unroll
-    for (int j = 0; j < kPlanes; ++j) {
+    for (int jj = 0; jj < kPlanes; ++jj) {
+      const int j = (jj + kTileRows) % kPlanes;
       ring[t][j] =
           __builtin_nontemporal_load(tbase + static_cast<size_t>(lin) * kTileVecs + j * 64);
     }
   };
-  request_tile(0);
-  if (BT == 1) request_tile(1);
+  constexpr int kPre = ALL > 0 ? PRE : (BT == 1 ? kRing : 1);
+#pragma unroll
+  for (int t = 0; t < kPre; ++t) request_tile(t);
   // Chain lanes: lane = row * BT + batch.
   const int chain_row = lane / BT;
   const int chain_b = lane - chain_row * BT;
@@ -330,14 +369,17 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
           for (int j = 0; j < kGroupsPerThread; ++j) {
             const int g = j * kThreads + tid;
             if (g < padded / 8) {
-              int32_t even = 0, odd = 0;
+              int32_t high = 0, low = 0;
               if (g < groups8) {
                 const float4 lo = xr[b][j][0], hi = xr[b][j][1];
                 const bool tail = g * 8 >= vector_end;
-                even = QuantizePack4<VARIANT>(lo.x, lo.z, hi.x, hi.z, qp, tail);
-                odd = QuantizePack4<VARIANT>(lo.y, lo.w, hi.y, hi.w, qp, tail);
+                NibblePlanes(
+                    static_cast<uint32_t>(QuantizePack4<VARIANT>(lo.x, lo.y, lo.z, lo.w, qp, tail)),
+                    static_cast<uint32_t>(QuantizePack4<VARIANT>(hi.x, hi.y, hi.z, hi.w, qp, tail)),
+                    &high, &low);
               }
-              *reinterpret_cast<i32x2*>(sh.q + b * (padded / 4) + 2 * g) = i32x2{even, odd};
+              sh.q[b * (padded / 4) + (g >> 2) * 8 + (g & 3)] = high;
+              sh.q[b * (padded / 4) + (g >> 2) * 8 + 4 + (g & 3)] = low;
             }
           }
         }
@@ -357,8 +399,11 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
               v[t] = QuantizeElement<VARIANT>(x[g * 8 + t], qp, true, g * 8 + t >= vector_end);
             }
           }
-          sh.q[b * (padded / 4) + 2 * g] = PackBytes(v[0], v[2], v[4], v[6]);
-          sh.q[b * (padded / 4) + 2 * g + 1] = PackBytes(v[1], v[3], v[5], v[7]);
+          int32_t high, low;
+          NibblePlanes(static_cast<uint32_t>(PackBytes(v[0], v[1], v[2], v[3])),
+                       static_cast<uint32_t>(PackBytes(v[4], v[5], v[6], v[7])), &high, &low);
+          sh.q[b * (padded / 4) + (g >> 2) * 8 + (g & 3)] = high;
+          sh.q[b * (padded / 4) + (g >> 2) * 8 + 4 + (g & 3)] = low;
         }
       }
     }
@@ -370,12 +415,13 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
         for (int j = 0; j < kGroupsPerThread; ++j) {
           const int g = j * kThreads + tid;
           if (g < padded / 8) {
-            int32_t even = 0, odd = 0;
+            int32_t high = 0, low = 0;
             if (g < groups8) {
-              Deinterleave(static_cast<uint32_t>(qr[b][j].x), static_cast<uint32_t>(qr[b][j].y),
-                           &even, &odd);
+              NibblePlanes(static_cast<uint32_t>(qr[b][j].x), static_cast<uint32_t>(qr[b][j].y),
+                           &high, &low);
             }
-            *reinterpret_cast<i32x2*>(sh.q + b * (padded / 4) + 2 * g) = i32x2{even, odd};
+            sh.q[b * (padded / 4) + (g >> 2) * 8 + (g & 3)] = high;
+            sh.q[b * (padded / 4) + (g >> 2) * 8 + 4 + (g & 3)] = low;
           }
         }
       }
@@ -383,7 +429,8 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
   }
   __syncthreads();
 
-  if (BT > 1) request_tile(1);
+#pragma unroll
+  for (int t = kPre; t < kRing; ++t) request_tile(t);
 
   float* kb = sh.kb + wave * 2 * 64;
   kb[lane] = kfsum_raw;
@@ -441,25 +488,20 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
     constexpr bool REFILL = decltype(refill_tag)::value;
     float* pw = ksplit == 1 ? sh.p + static_cast<size_t>(wave) * kTileFloats
                             : pgroup + static_cast<size_t>(c) * kTileFloats;
-    // This block's activations (8 dwords per batch row) and 8 * sum(q).
-    i32x4 qe[BT], qo[BT];
-    int32_t qsum8[BT];
+    // This block's activations (four dwords of high nibbles, four of low ones, per batch row)
+    // and -8 * sum(low nibbles), the seed of the unsigned dot product.
+    i32x4 qh[BT], ql[BT];
+    uint32_t seed[BT];
     const int blk = c * kTileBlocks + lane;
 #pragma unroll
     for (int b = 0; b < BT; ++b) {
       const i32x4* qp = reinterpret_cast<const i32x4*>(sh.q + b * (padded / 4) + blk * 8);
-      qe[b] = qp[0];
-      qo[b] = qp[1];
-      int32_t s = 0;
-      s = Dot4(qe[b].x, 0x01010101, s);
-      s = Dot4(qe[b].y, 0x01010101, s);
-      s = Dot4(qe[b].z, 0x01010101, s);
-      s = Dot4(qe[b].w, 0x01010101, s);
-      s = Dot4(qo[b].x, 0x01010101, s);
-      s = Dot4(qo[b].y, 0x01010101, s);
-      s = Dot4(qo[b].z, 0x01010101, s);
-      s = Dot4(qo[b].w, 0x01010101, s);
-      qsum8[b] = 8 * s;
+      qh[b] = qp[0];
+      ql[b] = qp[1];
+      uint32_t t = 0;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) t = UDot8(static_cast<uint32_t>(ql[b][d]), 0x11111111u, t);
+      seed[b] = 0u - 8u * t;
     }
     const i32x4 sc = ring[SLOT][kTileRows];
 #pragma unroll
@@ -467,24 +509,20 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
       const uint32_t pair = static_cast<uint32_t>(sc[j >> 1]);
       const float scale =
           HalfBitsToFloatFast(static_cast<uint16_t>((j & 1) ? (pair >> 16) : (pair & 0xFFFF)));
-      const i32x4 wv = ring[SLOT][j];
-      uint32_t lo[4], hi[4];
+      const i32x4 wv = ring[SLOT][j];  // nibbles stored as w + 8
+      int32_t ws[4];                   // the same weights as signed nibbles
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        lo[d] = static_cast<uint32_t>(wv[d]) & 0x0F0F0F0Fu;
-        hi[d] = (static_cast<uint32_t>(wv[d]) >> 4) & 0x0F0F0F0Fu;
-      }
+      for (int d = 0; d < 4; ++d) ws[d] = wv[d] ^ static_cast<int32_t>(0x88888888u);
 #pragma unroll
       for (int b = 0; b < BT; ++b) {
-        int32_t acc = -qsum8[b];
-        acc = Dot4(lo[0], qe[b].x, acc);
-        acc = Dot4(hi[0], qe[b].y, acc);
-        acc = Dot4(lo[1], qe[b].z, acc);
-        acc = Dot4(hi[1], qe[b].w, acc);
-        acc = Dot4(lo[2], qo[b].x, acc);
-        acc = Dot4(hi[2], qo[b].y, acc);
-        acc = Dot4(lo[3], qo[b].z, acc);
-        acc = Dot4(hi[3], qo[b].w, acc);
+        int32_t sd = 0;
+        uint32_t ud = seed[b];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          sd = SDot8(ws[d], qh[b][d], sd);
+          ud = UDot8(static_cast<uint32_t>(wv[d]), static_cast<uint32_t>(ql[b][d]), ud);
+        }
+        const int32_t acc = (sd << 4) + static_cast<int32_t>(ud);
         pw[(j * BT + b) * kPStride + lane] = __fmul_rn(static_cast<float>(acc), scale);
       }
     }
@@ -493,7 +531,10 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
       const LRTFC_GLOBAL i32x4* src =
           next < ntiles ? tbase + static_cast<size_t>(next) * kTileVecs : g_packed;
 #pragma unroll
-      for (int j = 0; j < kPlanes; ++j) ring[SLOT][j] = __builtin_nontemporal_load(src + j * 64);
+      for (int jj = 0; jj < kPlanes; ++jj) {
+        const int j = (jj + kTileRows) % kPlanes;
+        ring[SLOT][j] = __builtin_nontemporal_load(src + j * 64);
+      }
     }
     // Ordered float32 accumulation over this tile's blocks (same wavefront wrote them).
     if (ksplit == 1 && chain_lane) walk_tile(pw, c);
@@ -517,15 +558,24 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
   using Slot0 = std::integral_constant<int, 0>;
   using Slot1 = std::integral_constant<int, 1>;
   int lin = kpart;
-  for (; lin + ksplit < ntiles; lin += kRingTiles * ksplit) {
-    process(Slot0{}, std::true_type{}, lin, c);
-    LRTFC_INT4_ADVANCE();
-    process(Slot1{}, std::true_type{}, lin + ksplit, c);
-    LRTFC_INT4_ADVANCE();
-  }
-  if (lin < ntiles) {
-    process(Slot0{}, std::false_type{}, lin, c);
-    LRTFC_INT4_ADVANCE();
+  if constexpr (ALL > 0) {
+    StaticFor<ALL>([&](auto t) {
+      if (decltype(t)::value < ntiles) {
+        process(t, std::false_type{}, decltype(t)::value, c);
+        LRTFC_INT4_ADVANCE();
+      }
+    });
+  } else {
+    for (; lin + ksplit < ntiles; lin += kRingTiles * ksplit) {
+      process(Slot0{}, std::true_type{}, lin, c);
+      LRTFC_INT4_ADVANCE();
+      process(Slot1{}, std::true_type{}, lin + ksplit, c);
+      LRTFC_INT4_ADVANCE();
+    }
+    if (lin < ntiles) {
+      process(Slot0{}, std::false_type{}, lin, c);
+      LRTFC_INT4_ADVANCE();
+    }
   }
 #undef LRTFC_INT4_ADVANCE
   if (ksplit > 1) {
@@ -551,11 +601,24 @@ __device__ __forceinline__ void FcInt4PackedBody(const Int4PackedArgs& a, int bl
   }
 }
 
-template <int BT, bool FUSED, int VARIANT, int GPT>
-__global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(Int4PackedArgs a, int batch0,
-                                                               int bt, int ksplit, int gpw) {
+// The leading scalar arguments repeat what the first loads need (filter and row addresses,
+// shapes): the library is built with kernel-argument preloading, which hands the leading scalar
+// arguments to a wavefront in registers when it starts; the rest of the argument block is read
+// from memory as usual while the first loads are already under way.
+template <int BT, bool FUSED, int VARIANT, int GPT, int ALL, int PRE>
+__global__ __launch_bounds__(kThreads) void FcInt4PackedKernel(
+    const uint8_t* early_packed, const float* early_input_f32, const int8_t* early_input_q,
+    int early_depth, int early_out_depth, int early_chunks, int batch0, int bt, int ksplit,
+    int gpw, Int4PackedArgs rest) {
   extern __shared__ __align__(16) int8_t smem[];
-  FcInt4PackedBody<BT, FUSED, VARIANT, GPT>(a, blockIdx.x, batch0, bt, ksplit, gpw, smem);
+  Int4PackedArgs a = rest;
+  a.packed = early_packed;
+  a.input_f32 = early_input_f32;
+  a.input_q = early_input_q;
+  a.depth = early_depth;
+  a.out_depth = early_out_depth;
+  a.chunks = early_chunks;
+  FcInt4PackedBody<BT, FUSED, VARIANT, GPT, ALL, PRE>(a, blockIdx.x, batch0, bt, ksplit, gpw, smem);
 }
 
 // Several filters of the same depth in one launch (nodes of a graph that do not depend on
@@ -627,19 +690,39 @@ int ChooseGroupsPerWave(int total_groups, int chunks, int ksplit) {
   return gpw;
 }
 
-template <int BT, bool FUSED, int VARIANT, int GPT>
-hipError_t LaunchOne(const Int4PackedArgs& a, int batch0, int bt, hipStream_t stream) {
+template <int BT, bool FUSED, int VARIANT, int GPT, int ALL, int PRE>
+hipError_t LaunchSized(const Int4PackedArgs& a, int batch0, int bt, int ksplit, int gpw,
+                       hipStream_t stream) {
   const int padded = a.chunks * kTileBlocks * kBlock;
-  const int ksplit = ChooseKsplit(a.out_depth, a.chunks);
   const size_t lds = Int4Shared<BT>::Bytes(padded, ksplit);
-  auto kernel = FcInt4PackedKernel<BT, FUSED, VARIANT, GPT>;
+  auto kernel = FcInt4PackedKernel<BT, FUSED, VARIANT, GPT, ALL, PRE>;
   if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   const int groups = (a.out_depth + kTileRows - 1) / kTileRows;
-  const int gpw = ChooseGroupsPerWave(groups, a.chunks, ksplit);
   const int groups_per_wg = kWaves / ksplit * gpw;
   const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, batch0, bt, ksplit, gpw);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a.packed, a.input_f32,
+                     a.input_q, a.depth, a.out_depth, a.chunks, batch0, bt, ksplit, gpw, a);
   return hipGetLastError();
+}
+
+// A single node of up to two batch rows whose wavefronts can be given at most two tiles each
+// (depth up to 4096) runs the straight-line form: first tile ahead of the prologue, second
+// behind it.
+constexpr int kStraightTiles = 2;
+
+template <int BT, bool FUSED, int VARIANT, int GPT>
+hipError_t LaunchOne(const Int4PackedArgs& a, int batch0, int bt, hipStream_t stream) {
+  const int ksplit = ChooseKsplit(a.out_depth, a.chunks);
+  const int groups = (a.out_depth + kTileRows - 1) / kTileRows;
+  int gpw = ChooseGroupsPerWave(groups, a.chunks, ksplit);
+  if constexpr (BT <= 2) {
+    if (ksplit == 1 && a.chunks <= kStraightTiles) {
+      gpw = min(gpw, kStraightTiles / a.chunks);
+      return LaunchSized<BT, FUSED, VARIANT, GPT, kStraightTiles, 1>(a, batch0, bt, ksplit, gpw,
+                                                                     stream);
+    }
+  }
+  return LaunchSized<BT, FUSED, VARIANT, GPT, 0, 0>(a, batch0, bt, ksplit, gpw, stream);
 }
 
 template <int BT, bool FUSED, int GPT>
