@@ -208,6 +208,9 @@ def main():
                     kernel="FcInt8PackedGemvKernel<hybrid, fused quantize> (config 2, B=1, cold)",
                     achieved=round(achieved, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
                     frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=measured_traffic(),
+                    traffic_source="profiles/hybrid_gemv_fused_B1_hbm_traffic.txt (rocprofv3 --pmc "
+                                   "FETCH_SIZE / WRITE_SIZE of `bench.py --traffic-probe`; a committed "
+                                   "counter summary, not measured in this run)",
                     algorithmic_bytes_per_launch=hybrid_bytes(b_dom),
                     avg_launch_us=per_b[b_dom]["op_us_cold"])
 
@@ -570,19 +573,17 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         del all_groups, decoder_groups
         res.update(fc_nodes=len(nodes), weight_bytes=chain_bytes)
         out["config5_gemma2b_fc_chain_B%d" % b] = res
-    try:
-        out["config5_through_delegate_B1"] = delegate_chain(torch, wl)
-    except Exception as e:  # the stand-in interpreter is test infrastructure; report, don't fail
-        out["config5_through_delegate_B1"] = {"error": repr(e)}
+    for b in (1, 4):
+        out["config5_through_delegate_B%d" % b] = delegate_chain(torch, wl, b)
     return out
 
 
 def delegate_chain(torch, wl, b=1, invokes=20):
-    """Config 5 end to end through the delegate plugin, driven by the stand-in interpreter of
-    the tests: 126 FULLY_CONNECTED nodes, host tensors in, host tensors out. Wall-clock time of
+    """Config 5 end to end through the delegate plugin, driven by the stand-in interpreter
+    (litert_amd/standin_host): 126 FULLY_CONNECTED nodes, host tensors in, host tensors out. Wall-clock time of
     Invoke(), i.e. including the upload of every node's input, the download of every node's
     output (all 126 are graph outputs here) and the final synchronization."""
-    from tests.fake_host import FakeHost, FLOAT32, FLOAT16, INT4, OK
+    from litert_amd.standin_host import FakeHost, FLOAT32, FLOAT16, INT4, OK
     rng = np.random.default_rng(5)
     with FakeHost() as h:
         for layer in range(wl.GEMMA2B_LAYERS):

@@ -40,7 +40,10 @@ def lib():
     global _LIB
     if _LIB is None:
         path = os.path.join(_HERE, "liboracle.so")
-        if not os.path.exists(path):
+        if os.environ.get("LITERT_AMD_SANITIZED") == "1":
+            # the build of `make -C oracle san` (tests/test_sanitizers.py runs under it)
+            path = os.path.join(_HERE, "_san", "liboracle_san.so")
+        elif not os.path.exists(path):
             build()
         L = C.CDLL(path)
         L.orc_quantize_multiplier.argtypes = [C.c_double, _i32p, _intp]

@@ -275,15 +275,18 @@ float orc_half_to_float(uint16_t h) {
 }
 
 void orc_unpack_int4(const int8_t* src, int num_elements, int8_t* dst) {
+  // The reference shifts the signed byte left (`byte << 4`, undefined for negative values before
+  // C++20, though every compiler it is built with gives the two's-complement result); the same
+  // value is formed here from the unsigned byte.
+  auto low = [](int8_t byte) {
+    return static_cast<int8_t>(static_cast<int8_t>(static_cast<uint8_t>(byte) << 4) >> 4);
+  };
   for (int i = 0; i < num_elements / 2; ++i) {
     const int8_t byte = src[i];
-    dst[2 * i] = static_cast<int8_t>(static_cast<int8_t>(byte << 4) >> 4);
+    dst[2 * i] = low(byte);
     dst[2 * i + 1] = static_cast<int8_t>(byte >> 4);
   }
-  if (num_elements % 2 != 0) {
-    const int8_t byte = src[num_elements / 2];
-    dst[num_elements - 1] = static_cast<int8_t>(static_cast<int8_t>(byte << 4) >> 4);
-  }
+  if (num_elements % 2 != 0) dst[num_elements - 1] = low(src[num_elements / 2]);
 }
 
 int orc_fc_prepare_per_channel(float input_scale, const float* filter_scales, int num_channels,
