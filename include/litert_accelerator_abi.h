@@ -64,6 +64,26 @@ typedef struct LiteRtEnvironmentT* LiteRtEnvironment;
 typedef struct LiteRtOptionsT* LiteRtOptions;
 typedef struct LiteRtDelegateWrapperT* LiteRtDelegateWrapper;
 typedef struct LiteRtMetricsT* LiteRtMetrics;
+
+/* litert/c/litert_any.h:24-62: the value of one metric. */
+typedef enum {
+  kLiteRtAnyTypeNone = 0,
+  kLiteRtAnyTypeBool = 1,
+  kLiteRtAnyTypeInt = 2,
+  kLiteRtAnyTypeReal = 3,
+  kLiteRtAnyTypeString = 8,
+  kLiteRtAnyTypeVoidPtr = 9,
+} LiteRtAnyType;
+typedef struct {
+  LiteRtAnyType type;
+  union {
+    bool bool_value;
+    int64_t int_value;
+    double real_value;
+    const char* str_value;
+    const void* ptr_value;
+  };
+} LiteRtAny;
 typedef struct TfLiteOpaqueDelegate TfLiteOpaqueDelegate;
 
 /* litert_custom_tensor_buffer_handlers_def.h: this plugin registers no buffer types, so the

@@ -292,6 +292,27 @@ int lrtfc_fc_blockwise_int4_packed_quantized(const int8_t* quantized_input,
                                              const float* bias, float* output, int batches,
                                              int depth, int out_depth, void* stream);
 
+/* ---- BATCH_MATMUL, float x int8 (hybrid) -----------------------------------------------
+ * Replaces batch_matmul::EvalHybrid, tflite/kernels/batch_matmul.cc:454-520, with the kernel it
+ * runs (tflite/kernels/internal/reference/batch_matmul.h:111-210): every row of the float
+ * operand is quantized as in the hybrid FULLY_CONNECTED, and output batch b is
+ * rows(b) x weights(b)^T, where the zero-point correction goes through float as the reference
+ * kernel's does (:199-200), so results match it bit for bit also beyond 2^24. No bias, no
+ * activation (the op has neither).
+ *   lhs: [lhs_batches, rows, depth] float32. packed_weights: weight_matrices matrices of
+ *   [units, depth] int8 -- the op's RHS with its last two dimensions swapped unless adj_y --
+ *   each re-tiled by lrtfc_pack_int8_filter and stored lrtfc_packed_int8_filter_bytes(units,
+ *   depth) bytes apart; row_sums: [weight_matrices, units] from lrtfc_row_sums_int8 per matrix.
+ *   Broadcasting: lhs_batches == weight_matrices, or either of them 1. output:
+ *   [max(lhs_batches, weight_matrices), rows, units]. workspace:
+ *   lrtfc_activation_workspace_bytes(lhs_batches * rows, depth), 256-byte aligned. */
+int lrtfc_batch_matmul_hybrid_packed(const float* lhs, int lhs_batches, int rows, int depth,
+                                     const int8_t* packed_weights, int weight_matrices, int units,
+                                     const float* per_channel_scales, float filter_scale,
+                                     const int32_t* row_sums, float* output,
+                                     int asymmetric_quantize_inputs, int quant_variant,
+                                     void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- Per-channel int4 hybrid FULLY_CONNECTED ------------------------------------------
  * Replaces EvalHybridDense4Bit (tflite/kernels/fully_connected.cc:1088-1178) in the
  * arithmetic of its reference kernels

@@ -434,7 +434,7 @@ int FcHybridInt8Packed(const int8_t* quantized_input, const float* scaling_facto
                        const float* per_channel_scales, float filter_scale,
                        const int32_t* filter_row_sums, const float* bias, float* output,
                        int batches, int depth, int out_depth, int activation, int zero_input_exit,
-                       void* stream) {
+                       void* stream, int batch_matmul = 0) {
   if (int rc = RequireInit()) return rc;
   LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
   if (batches == 0 || out_depth == 0) return LRTFC_OK;
@@ -460,6 +460,7 @@ int FcHybridInt8Packed(const int8_t* quantized_input, const float* scaling_facto
   a.activation = activation;
   a.output_f32 = output;
   a.zero_input_exit = zero_input_exit;
+  a.batch_matmul = batch_matmul;
   if (batches > kPackedGemmMinBatches && lrtfc::FcInt8PackedGemmSupports(a)) {
     return FromHip(lrtfc::LaunchFcInt8PackedGemm(a, lrtfc::Int8Epilogue::kHybrid,
                                                  AsStream(stream)),
@@ -505,6 +506,56 @@ int lrtfc_fc_hybrid_packed_workspace(const float* input, const int8_t* packed_fi
   return FcHybridInt8Packed(w.q, w.sf, asymmetric_quantize_inputs ? w.zp : nullptr, packed_filter,
                             per_channel_scales, filter_scale, filter_row_sums, bias, output,
                             batches, depth, out_depth, activation, /*zero_input_exit=*/1, stream);
+}
+
+int lrtfc_batch_matmul_hybrid_packed(const float* lhs, int lhs_batches, int rows, int depth,
+                                     const int8_t* packed_weights, int weight_matrices, int units,
+                                     const float* per_channel_scales, float filter_scale,
+                                     const int32_t* row_sums, float* output,
+                                     int asymmetric_quantize_inputs, int quant_variant,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(lhs_batches >= 0 && rows >= 0 && depth > 0 && weight_matrices >= 0 && units >= 0,
+                "bad dimension");
+  LRTFC_REQUIRE(lhs_batches == weight_matrices || lhs_batches == 1 || weight_matrices == 1,
+                "%d input batches against %d weight matrices: only equal counts, or one side "
+                "broadcast, are supported", lhs_batches, weight_matrices);
+  const int out_batches = lhs_batches > weight_matrices ? lhs_batches : weight_matrices;
+  if (out_batches == 0 || lhs_batches == 0 || weight_matrices == 0 || rows == 0 || units == 0) {
+    return LRTFC_OK;
+  }
+  const int64_t quant_rows = static_cast<int64_t>(lhs_batches) * rows;
+  LRTFC_REQUIRE(quant_rows <= 0x7fffffff, "too many rows");
+  LRTFC_REQUIRE(lhs && packed_weights && row_sums && output && workspace, "null pointer");
+  LRTFC_REQUIRE(workspace_bytes >= WorkspaceBytes(static_cast<int>(quant_rows), depth),
+                "workspace too small: %zu < %zu bytes", workspace_bytes,
+                WorkspaceBytes(static_cast<int>(quant_rows), depth));
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
+                "workspace must be 256-byte aligned");
+  // BatchQuantizeFloats over every row of the float operand (batch_matmul.cc:472-497); symmetric
+  // quantization leaves the offsets at zero (:487-489).
+  const Workspace w = SplitWorkspace(workspace, static_cast<int>(quant_rows), depth);
+  int rc = lrtfc_batch_quantize_floats(lhs, static_cast<int>(quant_rows), depth, w.q, w.sf, w.zp,
+                                       asymmetric_quantize_inputs, quant_variant, stream);
+  if (rc != LRTFC_OK) return rc;
+  const int32_t* zp = asymmetric_quantize_inputs ? w.zp : nullptr;
+  if (weight_matrices == 1) {  // one weight matrix for every row: a single product
+    return FcHybridInt8Packed(w.q, w.sf, zp, packed_weights, per_channel_scales, filter_scale,
+                              row_sums, nullptr, output, static_cast<int>(quant_rows), depth, units,
+                              LRTFC_ACT_NONE, 0, stream, /*batch_matmul=*/1);
+  }
+  const size_t matrix_bytes = lrtfc::PackedInt8FilterBytes(units, depth);
+  for (int b = 0; b < out_batches; ++b) {
+    const size_t row0 = lhs_batches == 1 ? 0 : static_cast<size_t>(b) * rows;
+    rc = FcHybridInt8Packed(w.q + row0 * depth, w.sf + row0, zp ? zp + row0 : nullptr,
+                            packed_weights + static_cast<size_t>(b) * matrix_bytes,
+                            per_channel_scales, filter_scale,
+                            row_sums + static_cast<size_t>(b) * units, nullptr,
+                            output + static_cast<size_t>(b) * rows * units, rows, depth, units,
+                            LRTFC_ACT_NONE, 0, stream, /*batch_matmul=*/1);
+    if (rc != LRTFC_OK) return rc;
+  }
+  return LRTFC_OK;
 }
 
 int lrtfc_batch_quantize_floats(const float* values, int n_batch, int n_data, int8_t* quantized,

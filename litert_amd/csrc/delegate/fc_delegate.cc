@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <chrono>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -27,6 +28,7 @@
 #include <tuple>
 #include <vector>
 
+#include "litert_amd_delegate.h"
 #include "litert_amd_fc.h"
 #include "tflite_abi.h"
 
@@ -53,10 +55,24 @@ struct RegisteredBuffer {
   size_t bytes = 0;
 };
 
+// What a metrics collection (litert_amd_start_metrics .. litert_amd_stop_metrics) adds up over
+// the partition invokes between the two calls.
+struct MetricsState {
+  bool on = false;
+  int detail_level = 0;
+  int64_t invokes = 0;        // partition invokes
+  int64_t nodes = 0;          // FULLY_CONNECTED / EMBEDDING_LOOKUP nodes those invokes ran
+  int64_t uploaded = 0;       // bytes copied host -> device
+  int64_t downloaded = 0;     // bytes copied device -> host
+  double host_us = 0.0;       // wall time inside the partitions' invoke callbacks
+  double device_us = 0.0;     // first enqueued copy to last finished one, per invoke, by HIP events
+};
+
 struct DelegateState {
   Options options;
   TfLiteDelegate delegate;
   std::vector<RegisteredBuffer> buffers;
+  MetricsState metrics;
 };
 
 // The registered memory behind a tensor that carries one of this delegate's handles, or
@@ -429,6 +445,7 @@ struct PartitionKernel {
   hipStream_t stream = nullptr;  // streams[0]: uploads, downloads, prepare-time work
   DeviceBuffer workspace[kMaxStreams];
   hipEvent_t upload_done = nullptr;
+  hipEvent_t metrics_begin = nullptr, metrics_end = nullptr;  // timing events, made on first use
   hipEvent_t lane_done[kMaxStreams] = {};
   std::vector<hipEvent_t> node_done;  // per node; only the signalling ones are created
   bool lane_used[kMaxStreams] = {};
@@ -450,6 +467,8 @@ struct PartitionKernel {
       if (e) (void)hipEventDestroy(e);
     }
     if (upload_done) (void)hipEventDestroy(upload_done);
+    if (metrics_begin) (void)hipEventDestroy(metrics_begin);
+    if (metrics_end) (void)hipEventDestroy(metrics_end);
     for (int i = 0; i < kMaxStreams; ++i) {
       if (lane_done[i]) (void)hipEventDestroy(lane_done[i]);
       if (streams[i]) (void)hipStreamDestroy(streams[i]);
@@ -1008,6 +1027,16 @@ TfLiteStatus KernelPrepare(TfLiteContext* ctx, TfLiteNode* node) {
 TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   auto* k = static_cast<PartitionKernel*>(node->user_data);
   RETURN_IF_HIP(ctx, hipSetDevice(k->state->options.device));
+  MetricsState& metrics = k->state->metrics;
+  const bool measure = metrics.on;
+  const auto host_begin = std::chrono::steady_clock::now();
+  if (measure) {
+    if (!k->metrics_begin) {
+      RETURN_IF_HIP(ctx, hipEventCreate(&k->metrics_begin));
+      RETURN_IF_HIP(ctx, hipEventCreate(&k->metrics_end));
+    }
+    RETURN_IF_HIP(ctx, hipEventRecord(k->metrics_begin, k->stream));
+  }
   // Tensor data pointers may move between invokes: read them from the context each time.
   // An input that carries a buffer handle of this delegate is already in device memory: it is
   // copied device to device behind the (single) host upload of the others.
@@ -1237,9 +1266,19 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                       k->arena.as<uint8_t>() + k->download_offset,
                                       k->download_bytes, hipMemcpyDeviceToHost, s));
   }
+  if (measure) RETURN_IF_HIP(ctx, hipEventRecord(k->metrics_end, s));
   // The runtime reads the outputs as soon as invoke returns; a consumer of a registered
   // buffer (another partition, the application's own kernels) may start right away too.
   RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+  if (measure) {
+    float ms = 0.0f;
+    RETURN_IF_HIP(ctx, hipEventElapsedTime(&ms, k->metrics_begin, k->metrics_end));
+    metrics.device_us += 1e3 * ms;
+    metrics.invokes += 1;
+    metrics.nodes += static_cast<int64_t>(k->nodes.size());
+    if (host_inputs) metrics.uploaded += static_cast<int64_t>(k->upload_bytes);
+    if (host_outputs) metrics.downloaded += static_cast<int64_t>(k->download_bytes);
+  }
   // A lookup outside the table fails the invoke, with the builtin's message
   // (tflite/kernels/embedding_lookup.cc:280-286, 365-371).
   for (const FcNode& n : k->nodes) {
@@ -1257,6 +1296,10 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     if (tensor.bytes == 0 || BoundBuffer(k->state, tensor)) continue;
     std::memcpy(tensor.data.raw,
                 k->download_stage.get() + (k->arena_offset[t] - k->download_offset), tensor.bytes);
+  }
+  if (measure) {
+    metrics.host_us += std::chrono::duration<double, std::micro>(
+                           std::chrono::steady_clock::now() - host_begin).count();
   }
   return kTfLiteOk;
 }
@@ -1467,6 +1510,32 @@ TfLiteBufferHandle litert_amd_register_device_buffer(TfLiteDelegate* delegate, v
   }
   state->buffers.push_back(RegisteredBuffer{device_memory, bytes});
   return static_cast<TfLiteBufferHandle>(state->buffers.size() - 1);
+}
+
+// Metrics of the partitions this delegate runs, for the LiteRT accelerator table's
+// start_metrics_collection / stop_metrics_collection
+// (litert/c/internal/litert_accelerator_def.h:57-62) and for applications that hold the
+// TfLiteDelegate itself. start clears the counters and switches collection on (detail_level
+// is recorded; every level collects the same counters today); stop switches it off and copies
+// the totals out. Both return 0, or 1 for a delegate that is not one of this library's.
+int litert_amd_start_metrics(TfLiteDelegate* delegate, int detail_level) {
+  if (!delegate || !delegate->data_) return 1;
+  auto* state = static_cast<DelegateState*>(delegate->data_);
+  if (&state->delegate != delegate || detail_level < 0) return 1;
+  state->metrics = MetricsState{};
+  state->metrics.on = true;
+  state->metrics.detail_level = detail_level;
+  return 0;
+}
+
+int litert_amd_stop_metrics(TfLiteDelegate* delegate, litert_amd_metrics* out) {
+  if (!delegate || !delegate->data_ || !out) return 1;
+  auto* state = static_cast<DelegateState*>(delegate->data_);
+  if (&state->delegate != delegate || !state->metrics.on) return 1;
+  const MetricsState& m = state->metrics;
+  *out = litert_amd_metrics{m.invokes, m.nodes, m.uploaded, m.downloaded, m.host_us, m.device_us};
+  state->metrics.on = false;
+  return 0;
 }
 
 // Test and tooling hook: the claim predicate on its own (no device needed). Returns

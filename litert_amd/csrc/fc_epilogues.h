@@ -66,12 +66,32 @@ __device__ __forceinline__ bool IsNegativeZero(float v) {
   return __float_as_uint(v) == 0x80000000u;
 }
 
+// Output value of the hybrid BATCH_MATMUL kernel, reference/batch_matmul.h:190-206: the
+// zero-point correction `total -= row_sum * batch_offset` runs through float (batch_offset is a
+// float there: int32 -> float, float product, float subtraction, truncation back to int32),
+// then `out += scale * total` onto a zero-filled output. Differs from HybridCore as soon as a
+// dot product or a correction exceeds 2^24.
+__device__ __forceinline__ float HybridBatchMatMulCore(int32_t dot, float batch_scale,
+                                                       float channel_scale,
+                                                       int32_t batch_zero_point, int32_t row_sum) {
+  const float corrected = __fsub_rn(
+      static_cast<float>(dot),
+      __fmul_rn(static_cast<float>(row_sum), static_cast<float>(batch_zero_point)));
+  const int32_t total = static_cast<int32_t>(corrected);
+  const float scale = __fmul_rn(batch_scale, channel_scale);
+  return __fadd_rn(0.0f, __fmul_rn(scale, static_cast<float>(total)));
+}
+
 // HybridCore for kernels that run on already quantized rows (a.input), with the whole-zero-input
-// case above when the caller asked for EvalHybridDense semantics (a.zero_input_exit).
+// case above when the caller asked for EvalHybridDense semantics (a.zero_input_exit), or the
+// BATCH_MATMUL arithmetic (a.batch_matmul).
 __device__ __forceinline__ float HybridCoreZeroAware(const FcInt8Args& a, int32_t dot,
                                                      float batch_scale, float channel_scale,
                                                      int32_t batch_zero_point, int32_t row_sum,
                                                      float base) {
+  if (a.batch_matmul) {
+    return HybridBatchMatMulCore(dot, batch_scale, channel_scale, batch_zero_point, row_sum);
+  }
   if (a.zero_input_exit && dot == 0 && IsNegativeZero(base) &&
       AllZeroInt8(a.input, static_cast<size_t>(a.batches) * a.depth)) {
     return ApplyFloatActivation(base, a.activation);

@@ -64,6 +64,9 @@ struct FcInt8Args {
   // Non-zero: EvalHybridDense semantics for a whole-zero input (output = activation(bias), no
   // product added; fully_connected.cc:789-795). Zero: MatrixBatchVectorMultiplyAccumulate as is.
   int zero_input_exit;
+  // Non-zero: the arithmetic of the hybrid BATCH_MATMUL kernel (reference/batch_matmul.h:
+  // 190-206) instead of MatrixBatchVectorMultiplyAccumulate's; no bias, no activation.
+  int batch_matmul;
 };
 
 // kHybrid4Bit: the float epilogue of the per-channel int4 hybrid path; a.zero_points then

@@ -88,6 +88,9 @@ def lib():
         L.orc_matrix_batch_vector_multiply_accumulate_sse.argtypes = [
             _i8p, C.c_int, C.c_int, _i8p, _f32p, C.c_int, _f32p, _f32p, _i32p, _i32p]
         L.orc_matrix_batch_vector_multiply_accumulate_sse.restype = None
+        L.orc_batch_matmul_hybrid.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, _i8p, C.c_int,
+                                              C.c_int, _f32p, C.c_float, C.c_int, C.c_int, _intp,
+                                              _intp, C.c_int, _f32p]
         L.orc_fc_blockwise_int4.argtypes = [_f32p, C.c_int, C.c_int, _u8p, C.c_int, _u16p,
                                             C.c_int, _f32p, C.c_int, _f32p]
         L.orc_fc_hybrid_int4_per_channel.argtypes = [_f32p, C.c_int, C.c_int, _u8p, C.c_int, _f32p,
@@ -332,6 +335,46 @@ def fc_hybrid(x, w, per_channel_scales=None, filter_scale=1.0, bias=None, asymme
     if rc:
         raise ValueError("activation not restated in the oracle")
     return (y, q, sf, zp) if return_quant else y
+
+
+# ---- BATCH_MATMUL hybrid ------------------------------------------------------
+
+def batch_matmul_broadcast(lhs_shape, rhs_shape, adj_y=False):
+    """Shapes and batch pairing of BATCH_MATMUL (tflite/kernels/batch_matmul.cc:356-391 and
+    reference/batch_matmul.h:120-146): returns (rows, depth, units, output shape, lhs batch
+    index per output batch, rhs batch index per output batch). adj_x is not supported."""
+    rank = max(len(lhs_shape), len(rhs_shape))
+    le = (1,) * (rank - len(lhs_shape)) + tuple(lhs_shape)
+    re = (1,) * (rank - len(rhs_shape)) + tuple(rhs_shape)
+    rows, depth = le[-2], le[-1]
+    units = re[-2] if adj_y else re[-1]
+    assert (re[-1] if adj_y else re[-2]) == depth
+    lb, rb = le[:-2], re[:-2]
+    ob = []
+    for a, b in zip(lb, rb):
+        assert a == b or a == 1 or b == 1
+        ob.append(max(a, b))
+    li = np.arange(int(np.prod(lb, dtype=np.int64))).reshape(lb) if lb else np.zeros((), np.int64)
+    ri = np.arange(int(np.prod(rb, dtype=np.int64))).reshape(rb) if rb else np.zeros((), np.int64)
+    li = np.broadcast_to(li, ob).ravel().astype(np.int32)
+    ri = np.broadcast_to(ri, ob).ravel().astype(np.int32)
+    return rows, depth, units, tuple(ob) + (rows, units), li, ri
+
+
+def batch_matmul_hybrid(lhs, rhs, per_channel_scales=None, filter_scale=1.0, asymmetric=True,
+                        adj_y=False, variant=QUANT_PORTABLE):
+    """lhs float32 [..., M, K]; rhs int8 [..., K, N] (adj_y: [..., N, K]); float32 [..., M, N]."""
+    lhs = _c(lhs, np.float32)
+    rhs = _c(rhs, np.int8)
+    rows, depth, units, out_shape, li, ri = batch_matmul_broadcast(lhs.shape, rhs.shape, adj_y)
+    w = rhs if adj_y else np.ascontiguousarray(np.swapaxes(rhs, -1, -2))  # the op's transposition
+    pcs = _c(per_channel_scales, np.float32)
+    out = np.empty(out_shape, np.float32)
+    lib().orc_batch_matmul_hybrid(
+        _p(lhs, _f32p), lhs.size // (rows * depth), rows, depth, _p(w, _i8p),
+        w.size // (units * depth), units, _p(pcs, _f32p), filter_scale, int(asymmetric), variant,
+        _p(li, _intp), _p(ri, _intp), li.size, _p(out, _f32p))
+    return out
 
 
 # ---- blockwise int4 ---------------------------------------------------------

@@ -570,6 +570,61 @@ int orc_fc_hybrid(const float* input, int batches, int depth, const int8_t* filt
                               quant_variant, output, q_out, sf_out, zp_out, row_sums.data(), 1);
 }
 
+// tflite/kernels/batch_matmul.cc:454-520 (EvalHybrid) over
+// tflite/kernels/internal/reference/batch_matmul.h:111-210 (the hybrid BatchMatMul kernel, which
+// both registrations run). The op has already put the int8 operand into [matrix][unit][depth]
+// order (its RHS transposed unless adj_y) and flattened the float operand to rows of `depth`
+// values; broadcasting arrives here resolved: output batch b multiplies the `rows` rows of float
+// batch lhs_batch_index[b] with weight matrix rhs_batch_index[b].
+// Note the zero-point correction: `total -= row_sum * batch_offset` with a FLOAT batch_offset
+// (batch_matmul.h:199-200), i.e. int32 total -> float, float product, float subtraction, and
+// truncation back to int32; and the final `out += scale * total` onto a zero-filled output.
+void orc_batch_matmul_hybrid(const float* lhs, int lhs_batches, int rows, int depth,
+                             const int8_t* weights, int weight_matrices, int units,
+                             const float* per_channel_scales, float filter_scale,
+                             int asymmetric_quantize_inputs, int quant_variant,
+                             const int* lhs_batch_index, const int* rhs_batch_index,
+                             int out_batches, float* output) {
+  const int quant_rows = lhs_batches * rows;  // num_batches_to_quantize, batch_matmul.cc:472-475
+  std::vector<int8_t> q(static_cast<size_t>(quant_rows) * depth);
+  std::vector<float> sf(quant_rows);
+  std::vector<int32_t> offsets(quant_rows, 0);  // memset to 0 when symmetric, :487-489
+  orc_batch_quantize_floats(lhs, quant_rows, depth, q.data(), sf.data(), offsets.data(),
+                            asymmetric_quantize_inputs, quant_variant);
+  if (!asymmetric_quantize_inputs) std::fill(offsets.begin(), offsets.end(), 0);
+  if (!per_channel_scales) {
+    for (int b = 0; b < quant_rows; ++b) sf[b] *= filter_scale;  // :508-513
+  }
+  // ReductionSumVector over every weight matrix, batch_matmul.h:148-163.
+  std::vector<int32_t> row_sums(static_cast<size_t>(weight_matrices) * units);
+  for (size_t r = 0; r < row_sums.size(); ++r) {
+    int32_t sum = 0;
+    for (int k = 0; k < depth; ++k) sum += weights[r * depth + k];
+    row_sums[r] = sum;
+  }
+  std::fill_n(output, static_cast<size_t>(out_batches) * rows * units, 0.0f);  // :520
+  for (int b = 0; b < out_batches; ++b) {
+    const int8_t* w = weights + static_cast<size_t>(rhs_batch_index[b]) * units * depth;
+    const int32_t* wsum = row_sums.data() + static_cast<size_t>(rhs_batch_index[b]) * units;
+    const size_t row0 = static_cast<size_t>(lhs_batch_index[b]) * rows;
+    float* out = output + static_cast<size_t>(b) * rows * units;
+    for (int j = 0; j < rows; ++j) {
+      const float batch_scaling_factor = sf[row0 + j];
+      const float batch_offset = static_cast<float>(offsets[row0 + j]);
+      const int8_t* x = q.data() + (row0 + j) * depth;
+      for (int i = 0; i < units; ++i) {
+        int32_t total = 0;
+        for (int k = 0; k < depth; ++k) total += w[static_cast<size_t>(i) * depth + k] * x[k];
+        const int32_t row_sum = wsum[i];
+        total -= row_sum * batch_offset;  // the reference's mixed int/float compound assignment
+        float scale = batch_scaling_factor;
+        if (per_channel_scales) scale *= per_channel_scales[i];
+        out[static_cast<size_t>(units) * j + i] += scale * total;
+      }
+    }
+  }
+}
+
 void orc_fc_blockwise_int4(const float* input, int batches, int depth,
                            const uint8_t* packed_filter, int out_depth,
                            const uint16_t* scales_f16, int blocksize, const float* bias,

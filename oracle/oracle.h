@@ -184,6 +184,22 @@ int orc_fc_hybrid_cached(const float* input, int batches, int depth, const int8_
 
 /* ---- blockwise int4 weights -------------------------------------------- */
 
+/* BATCH_MATMUL, float x int8 (hybrid): tflite/kernels/batch_matmul.cc:454-520 over the
+ * kernel of tflite/kernels/internal/reference/batch_matmul.h:111-210. lhs: lhs_batches x rows
+ * x depth floats; weights: weight_matrices x units x depth int8 (the op's RHS after its
+ * transposition); per_channel_scales [units] or NULL (then filter_scale); output batch b =
+ * lhs batch lhs_batch_index[b] x weight matrix rhs_batch_index[b], [out_batches, rows, units].
+ * The reference's own vectors for it (batch_matmul_test.cc:504-985) are tolerance-class; at
+ * the bit level it is pinned by reduction to orc_fc_hybrid wherever the float detour of its
+ * zero-point correction is exact, and by a numpy float32 replay of that detour where it is
+ * not (tests/test_oracle_batch_matmul.py). */
+void orc_batch_matmul_hybrid(const float* lhs, int lhs_batches, int rows, int depth,
+                             const int8_t* weights, int weight_matrices, int units,
+                             const float* per_channel_scales, float filter_scale,
+                             int asymmetric_quantize_inputs, int quant_variant,
+                             const int* lhs_batch_index, const int* rhs_batch_index,
+                             int out_batches, float* output);
+
 /* tflite/kernels/fully_connected.cc:1014-1086 (EvalBlockwise4Bit), float ops
  * in source order and uncontracted. packed_filter holds out_depth rows of
  * ceil_even(depth)/2 bytes, low nibble = even k. scales_f16 [out_depth,

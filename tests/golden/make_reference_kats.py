@@ -110,6 +110,51 @@ def embedding_lookup_cases():
     return cases
 
 
+def batch_matmul_hybrid_cases():
+    """tflite/kernels/batch_matmul_test.cc:504-985: float inputs, weights quantized per tensor
+    by the harness (SetSignedWeights -> QuantizeTensor), expected float outputs with the
+    tolerance each test states."""
+    b = "tflite/kernels/batch_matmul_test.cc"
+    w3 = [1, 1, 1, 2, 2, 2, 3, 3, 3, 4, 4, 4, 5, 5, 5, 6, 6, 6, 7, 7, 7, 8, 8, 8, 9, 9, 9, 10, 10, 10]
+    w9 = [v for r in range(10) for v in [r + 1] * 3 + [r + 17] * 3 + [r + 26] * 3]
+    w_two = ([v for r in range(10) for v in (r + 1, r - 3, r + 1)] +
+             [v for r in range(10) for v in (r + 1,) * 3])
+    w10 = [1] * 5 + [2] * 5 + [3] * 5 + [1] * 5 + [2] * 5 + [3] * 5
+    x_small = [1, 2, 3, 4, 5, 6, 7, 8, -9, -10, 1, 2, 3, 4, 5, 6, 7, -8, 9, -10]
+    x_big = [11, 12, 13, 14, 15, 16, 17, 18, -19, -20, 11, 12, 13, 14, 15, 16, 17, -18, 19, -20]
+    big_want = [23, 23, 23, 295, 295, 295, 448, 448, 448, 57, 57, 57, 361, 361, 361, 532, 532, 532,
+                193, 193, 193, 1425, 1425, 1425, 2118, 2118, 2118,
+                247, 247, 247, 1511, 1511, 1511, 2222, 2222, 2222]
+    cases = []
+
+    def add(source, lhs_shape, rhs_shape, weights, x, want, tol, asym=True, adj_y=False):
+        q, scale = kh.symmetric_quantize_tensor(weights)
+        cases.append(dict(source=source, lhs_shape=lhs_shape, rhs_shape=rhs_shape,
+                          rhs=q.reshape(rhs_shape).tolist(), filter_scale=float(scale),
+                          lhs=np.asarray(x, np.float32).reshape(lhs_shape).tolist(),
+                          asymmetric_quantize_inputs=asym, adj_y=adj_y, expected=want,
+                          max_abs_err=tol))
+
+    add(b + ":504-533", [2, 10], [10, 3], w3, x_big, [193] * 3 + [247] * 3, 3.0)
+    add(b + ":535-565", [1, 2, 2, 3], [3, 10], w10, [11, 12, 13] * 4, [73] * 40, 0.64)
+    add(b + ":567-592", [2, 3], [3, 10], w10, [11, 12, 13] * 2, [73] * 20, 0.64)
+    add(b + ":600-631", [6, 3], [3, 8], [1] * 8 + [2] * 8 + [3] * 8, [11, 12, 13] * 6, [74] * 48, 0.15)
+    add(b + ":663-698", [6, 3], [8, 3], [1, 2, 3] * 8, [11, 12, 13] * 6, [74] * 48, 0.15,
+        adj_y=True)
+    add(b + ":729-758", [2, 2, 10], [10, 3], w3, x_small + x_big,
+        [23] * 3 + [57] * 3 + [193] * 3 + [247] * 3, 3.0)
+    add(b + ":760-798", [2, 2, 10], [10, 9], w9, x_small + x_big, big_want, 10.0)
+    add(b + ":800-846", [2, 10], [2, 10, 3], w_two, x_small,
+        [23, -45, 23, 57, -19, 57, 23, 23, 23, 57, 57, 57], 1.5)
+    add(b + ":848-878", [2, 10], [10, 3], w3, x_big, [193] * 3 + [247] * 3, 1.5, asym=False)
+    add(b + ":880-910", [2, 2, 10], [10, 3], w3, x_small + x_big,
+        [23] * 3 + [57] * 3 + [193] * 3 + [247] * 3, 1.5, asym=False)
+    add(b + ":912-951", [2, 2, 10], [10, 9], w9, x_small + x_big, big_want, 10.0, asym=False)
+    add(b + ":953-985", [2, 10], [2, 10, 3], w_two, x_small,
+        [23, -45, 23, 57, -19, 57, 23, 23, 23, 57, 57, 57], 1.5, asym=False)
+    return cases
+
+
 def main():
     t = "tflite/kernels/fully_connected_test.cc"
     fc = []
@@ -191,6 +236,7 @@ def main():
     out = dict(embedding_lookup=lookups, fully_connected_int8=fc, batch_quantize_floats=quantize,
                quantize_multiplier=multiplier, multiply_by_quantized_multiplier=mbqm,
                hybrid_dot_per_channel=hybrid_dot,
+               batch_matmul_hybrid=batch_matmul_hybrid_cases(),
                unpack_int4=[dict(source=u + ":2110-2119", packed=[0x38, 0xBE], count=4,
                                  expected=[-8, 3, -2, -5]),
                             dict(source=u + ":2121-2130", packed=[0x21, 0x43], count=3,

@@ -54,3 +54,17 @@ def pack_int4(values_i8):
     lo = v[0::2].astype(np.uint8) & 0xF
     hi = v[1::2].astype(np.uint8) & 0xF
     return (lo | (hi << 4)).astype(np.uint8)
+
+
+def symmetric_quantize_tensor(values):
+    """SingleOpModel::QuantizeTensor (tflite/kernels/test_util.h:1407-1430): the whole tensor
+    through SymmetricQuantizeFloats (reference/portable_tensor_utils.cc:41-71). Returns
+    (int8 values, float32 scale)."""
+    v = np.asarray(values, dtype=np.float32)
+    rng = f32(np.max(np.abs(v))) if v.size else f32(0)
+    if rng == 0:
+        return np.zeros(v.shape, np.int8), f32(1)
+    scale = f32(rng / f32(127))
+    inv = f32(f32(127) / rng)
+    q = np.clip(_round_half_away((v * inv).astype(np.float32)), -127, 127).astype(np.int8)
+    return q, scale

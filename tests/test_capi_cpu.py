@@ -20,6 +20,18 @@ def _header_symbols():
     return sorted(set(re.findall(r"\b(lrtfc_[a-z0-9_]+)\s*\(", text)))
 
 
+def test_delegate_plugin_exports_every_declared_symbol():
+    """include/litert_amd_delegate.h and the plugin entry points of include/tflite_abi.h."""
+    text = open(os.path.join(ROOT, "include", "litert_amd_delegate.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(litert_amd_[a-z0-9_]+)\s*\(", text)))
+    assert len(declared) == 10
+    lib = C.CDLL(os.path.join(ROOT, "litert_amd", "lib", "liblitert_amd_delegate.so"))
+    for name in declared + ["tflite_plugin_create_delegate", "tflite_plugin_destroy_delegate",
+                            "LiteRtAcceleratorImpl"]:
+        assert hasattr(lib, name), name
+
+
 def test_library_exports_every_declared_symbol():
     lib = capi.load()
     declared = _header_symbols()

@@ -45,7 +45,10 @@ class AcceleratorDef(C.Structure):
                 ("is_jit", C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_bool))),
                 ("create_delegate", C.CFUNCTYPE(C.c_int, C.POINTER(RuntimeContext), C.c_void_p,
                                                 C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p))),
-                ("start_metrics_collection", C.c_void_p), ("stop_metrics_collection", C.c_void_p),
+                ("start_metrics_collection", C.CFUNCTYPE(C.c_int, C.POINTER(RuntimeContext),
+                                                         C.c_void_p, C.c_int)),
+                ("stop_metrics_collection", C.CFUNCTYPE(C.c_int, C.POINTER(RuntimeContext),
+                                                        C.c_void_p, C.c_void_p)),
                 ("buffer_handlers", BufferHandlers)]
 
 
@@ -65,7 +68,8 @@ def test_layout_constants_of_the_reference():
 def test_exported_table_is_what_the_runtime_accepts():
     _, d = _impl()
     assert (d.abi_header.struct_size, d.abi_header.major_version) == (200, 1)
-    for f in ("get_name", "get_version", "get_hardware_support", "is_jit", "create_delegate"):
+    for f in ("get_name", "get_version", "get_hardware_support", "is_jit", "create_delegate",
+              "start_metrics_collection", "stop_metrics_collection"):
         assert C.cast(getattr(d, f), C.c_void_p).value, f
     assert d.buffer_handlers.num_supported_buffer_types < 16  # registration_helper.cc:48-49
     name = C.c_char_p()
@@ -129,3 +133,70 @@ def test_create_delegate_hands_a_working_delegate_to_the_runtime():
     prepare = C.cast(rec["delegate"] + 8, C.POINTER(C.c_void_p))[0]
     assert prepare
     rec["deleter"](rec["delegate"])  # what the runtime does when the wrapper dies
+
+
+def test_metrics_callbacks_reject_what_they_cannot_unwrap():
+    """start/stop_metrics_collection (litert_accelerator_def.h:57-62) reach the delegate through
+    the runtime context's unwrap_delegate; without one, or with a wrapper it refuses, they fail
+    with kLiteRtStatusErrorInvalidArgument and touch nothing."""
+    lib, d = _impl()
+    assert d.start_metrics_collection(None, 0x1, 0) == 1
+    ctx = _context({})  # no unwrap_delegate in this table
+    assert d.start_metrics_collection(C.byref(ctx), 0x1, 0) == 1
+    ctx.unwrap_delegate = UNWRAP(lambda wrapper, out: 1)
+    assert d.start_metrics_collection(C.byref(ctx), 0x1, 0) == 1
+    lib.litert_amd_metrics_object_new.restype = C.c_void_p
+    lib.litert_amd_metrics_object_free.argtypes = [C.c_void_p]
+    m = lib.litert_amd_metrics_object_new()
+    assert d.stop_metrics_collection(C.byref(ctx), 0x1, m) == 1
+    assert d.stop_metrics_collection(C.byref(ctx), 0x1, None) == 1
+    lib.litert_amd_metrics_object_free(m)
+
+
+@pytest.mark.gpu
+def test_metrics_collection_reports_what_the_partitions_did():
+    torch = pytest.importorskip("torch")
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a gfx950 device; none visible")
+    import numpy as np
+    from litert_amd import workloads as wl
+    from tests.fake_host import FakeHost, FLOAT32, INT8, OK
+    lib, d = _impl()
+    lib.litert_amd_metrics_object_new.restype = C.c_void_p
+    lib.litert_amd_metrics_object_free.argtypes = [C.c_void_p]
+    lib.litert_amd_metrics_object_size.argtypes = [C.c_void_p]
+    lib.litert_amd_metrics_object_name.argtypes = [C.c_void_p, C.c_int]
+    lib.litert_amd_metrics_object_name.restype = C.c_char_p
+    lib.litert_amd_metrics_object_value.argtypes = [C.c_void_p, C.c_int]
+    lib.litert_amd_metrics_object_value.restype = C.c_double
+    c = wl.hybrid_fc(2, 512, 64)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (2, 512), data=c["x"])
+        w = h.tensor(INT8, (64, 512), data=c["w"], const=True)
+        h.affine(w, c["pcs"])
+        y = h.tensor(FLOAT32, (2, 64))
+        h.fc(x, w, None, y)
+        assert h.load_delegate() == 0 and h.modify_graph_with_delegate() == OK, h.errors()
+        assert h.allocate_tensors() == OK, h.errors()
+        delegate = h.L.fh_delegate(h.h)
+
+        def unwrap(wrapper, out):
+            out[0] = delegate if wrapper == 0xABC0 else None
+            return 0 if wrapper == 0xABC0 else 1
+        ctx = _context({})
+        ctx.unwrap_delegate = UNWRAP(unwrap)
+        m = lib.litert_amd_metrics_object_new()
+        assert d.stop_metrics_collection(C.byref(ctx), 0xABC0, m) == 1  # nothing was started
+        assert h.invoke() == OK  # before the collection: not counted
+        assert d.start_metrics_collection(C.byref(ctx), 0xABC0, 0) == 0
+        for _ in range(3):
+            assert h.invoke() == OK, h.errors()
+        assert d.stop_metrics_collection(C.byref(ctx), 0xABC0, m) == 0
+        got = {lib.litert_amd_metrics_object_name(m, i).decode(): lib.litert_amd_metrics_object_value(m, i)
+               for i in range(lib.litert_amd_metrics_object_size(m))}
+        lib.litert_amd_metrics_object_free(m)
+        assert got["litert_amd.partition_invokes"] == 3 and got["litert_amd.nodes_run"] == 3
+        assert got["litert_amd.bytes_uploaded"] == 3 * c["x"].nbytes
+        assert got["litert_amd.bytes_downloaded"] == 3 * 2 * 64 * 4
+        assert 0 < got["litert_amd.device_time_us"] <= got["litert_amd.host_time_us"]
+        assert h.invoke() == OK  # collection is off again
