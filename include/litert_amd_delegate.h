@@ -51,7 +51,8 @@ int litert_amd_stop_metrics(TfLiteDelegate* delegate, litert_amd_metrics* out);
 
 /* Tooling hooks (no device needed for the first): the node-claim predicate on its own —
  * returns 0 = declined, 1 = int8, 2 = hybrid, 3 = int4 blockwise, 4 = int4 per-channel hybrid,
- * 5 = EMBEDDING_LOOKUP, `reason` (may be NULL) receiving why a node was declined — and a text
+ * 5 = EMBEDDING_LOOKUP, 6 = hybrid BATCH_MATMUL, `reason` (may be NULL) receiving why a node was
+ * declined — and a text
  * account of how a prepared partition (the user_data of its delegate-kernel node) will run;
  * returns the number of grouped launches, -1 on bad arguments. */
 int litert_amd_classify_node(const TfLiteContext* ctx, const TfLiteNode* node,

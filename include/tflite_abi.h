@@ -299,10 +299,17 @@ typedef struct { /* builtin_op_data.h:191-211 */
   TfLiteType quantized_bias_type;
 } TfLiteFullyConnectedParams;
 
-enum { /* builtin_ops.h:39,81 */
+typedef struct { /* builtin_op_data.h:246-253 */
+  bool adj_x;
+  bool adj_y;
+  bool asymmetric_quantize_inputs;
+} TfLiteBatchMatMulParams;
+
+enum { /* builtin_ops.h:37,39,81,156 */
   kTfLiteBuiltinEmbeddingLookup = 7,
   kTfLiteBuiltinFullyConnected = 9,
   kTfLiteBuiltinDelegate = 51,
+  kTfLiteBuiltinBatchMatmul = 126,
 };
 
 #ifdef __cplusplus
@@ -321,7 +328,8 @@ extern "C" {
  *   device          GPU ordinal (default 0)
  *   quant_variant   portable | neon_v8 | neon_legacy: which build of the reference's
  *                   activation quantizer to reproduce (default portable)
- *   claim           comma list out of int8,hybrid,int4_blockwise (default: all) */
+ *   claim           comma list out of int8,hybrid,int4_blockwise,int4_per_channel,
+ *                   embedding_lookup,batch_matmul (default: all) */
 TfLiteDelegate* tflite_plugin_create_delegate(const char* const* options_keys,
                                               const char* const* options_values,
                                               size_t num_options,

@@ -45,6 +45,7 @@ struct Options {
   bool claim_int4_blockwise = true;
   bool claim_int4_per_channel = true;
   bool claim_embedding_lookup = true;
+  bool claim_batch_matmul = true;
 };
 
 // Device memory the application registered for a tensor (litert_amd_register_device_buffer);
@@ -86,7 +87,9 @@ const RegisteredBuffer* BoundBuffer(const DelegateState* state, const TfLiteTens
   return b.device ? &b : nullptr;
 }
 
-enum class FcKind { kNone, kInt8, kHybrid, kInt4Blockwise, kHybridInt4, kEmbeddingLookup };
+enum class FcKind {
+  kNone, kInt8, kHybrid, kInt4Blockwise, kHybridInt4, kEmbeddingLookup, kBatchMatMul
+};
 
 int64_t NumElements(const TfLiteIntArray* dims) {
   int64_t n = 1;
@@ -174,6 +177,81 @@ FcKind ClassifyEmbeddingLookup(const TfLiteContext* ctx, const TfLiteNode* node,
   return FcKind::kEmbeddingLookup;
 }
 
+// Shape facts of a BATCH_MATMUL node with a float left operand and a constant int8 right one:
+// the op extends both shapes to a common rank and broadcasts the batch dimensions
+// (tflite/kernels/batch_matmul.cc:356-391); this delegate takes the forms in which the batch
+// dimensions are equal or all 1 on one side.
+struct BatchMatMulShape {
+  int lhs_batches = 1, matrices = 1, rows = 0, depth = 0, units = 0;
+};
+bool BatchMatMulGeometry(const TfLiteTensor& lhs, const TfLiteTensor& rhs, bool adj_y,
+                         BatchMatMulShape* out, const char** why) {
+  const int lr = lhs.dims->size, rr = rhs.dims->size;
+  if (lr < 2 || lr > 5 || rr < 2 || rr > 5) return *why = "operand rank outside 2..5", false;
+  BatchMatMulShape g;
+  g.rows = lhs.dims->data[lr - 2];
+  g.depth = lhs.dims->data[lr - 1];
+  g.units = adj_y ? rhs.dims->data[rr - 2] : rhs.dims->data[rr - 1];
+  if ((adj_y ? rhs.dims->data[rr - 1] : rhs.dims->data[rr - 2]) != g.depth) {
+    return *why = "accumulation depths differ", false;
+  }
+  const int rank = std::max(lr, rr);
+  bool equal = true;
+  for (int i = 0; i < rank - 2; ++i) {
+    const int l = i - (rank - lr) >= 0 ? lhs.dims->data[i - (rank - lr)] : 1;
+    const int r = i - (rank - rr) >= 0 ? rhs.dims->data[i - (rank - rr)] : 1;
+    g.lhs_batches *= l;
+    g.matrices *= r;
+    equal = equal && l == r;
+  }
+  if (!equal && g.lhs_batches != 1 && g.matrices != 1) {
+    return *why = "batch dimensions broadcast on both sides", false;
+  }
+  if (g.depth <= 0) return *why = "empty depth", false;
+  *out = g;
+  return true;
+}
+
+// BATCH_MATMUL in its hybrid form (batch_matmul.cc:363-374: float32 x int8): the right operand
+// a constant int8 tensor with affine quantization, one scale or one per output unit.
+FcKind ClassifyBatchMatMul(const TfLiteContext* ctx, const TfLiteNode* node, const Options& opt,
+                           std::string* why_not) {
+  auto no = [&](const char* reason) {
+    if (why_not) *why_not = reason;
+    return FcKind::kNone;
+  };
+  if (!opt.claim_batch_matmul) return no("batch matmul disabled by option");
+  if (!node->builtin_data) return no("no builtin data");
+  if (node->inputs->size != 2 || node->outputs->size != 1) return no("needs 2 inputs, 1 output");
+  const auto* params = static_cast<const TfLiteBatchMatMulParams*>(node->builtin_data);
+  const TfLiteTensor& lhs = ctx->tensors[node->inputs->data[0]];
+  const TfLiteTensor& rhs = ctx->tensors[node->inputs->data[1]];
+  const TfLiteTensor& output = ctx->tensors[node->outputs->data[0]];
+  if (lhs.type != kTfLiteFloat32 || rhs.type != kTfLiteInt8 || output.type != kTfLiteFloat32) {
+    return no("not the float32 x int8 form");
+  }
+  if (params->adj_x) return no("adj_x is left to the CPU kernels");
+  if (!lhs.dims || !rhs.dims) return no("operand has no shape");
+  if (!IsConstant(rhs)) return no("right operand is not a constant tensor");
+  if (rhs.quantization.type != kTfLiteAffineQuantization) return no("right operand not affine");
+  BatchMatMulShape g;
+  const char* why = "";
+  if (!BatchMatMulGeometry(lhs, rhs, params->adj_y, &g, &why)) return no(why);
+  const auto* q = static_cast<const TfLiteAffineQuantization*>(rhs.quantization.params);
+  if (!q || !q->scale || q->scale->size < 1) return no("right operand has no scales");
+  if (q->scale->size > 1) {
+    // EvalHybrid indexes the scales by output unit (batch_matmul.h:201-203).
+    const int units_dim = params->adj_y ? rhs.dims->size - 2 : rhs.dims->size - 1;
+    if (q->quantized_dimension != units_dim || q->scale->size != g.units) {
+      return no("per-channel scales do not run along the output units");
+    }
+  }
+  if (lrtfc_fc_int8_preferred_layout(1, g.depth, g.units, 0) != LRTFC_LAYOUT_PACKED) {
+    return no("depth beyond what the kernels stage in LDS");
+  }
+  return FcKind::kBatchMatMul;
+}
+
 // The node-claim predicate: the same tensor / quantization-parameter / fused-activation
 // combinations the builtin kernel accepts for these three paths
 // (tflite/kernels/fully_connected.cc:254-308, 440-761), nothing else.
@@ -186,6 +264,9 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
   };
   if (registration->builtin_code == kTfLiteBuiltinEmbeddingLookup) {
     return ClassifyEmbeddingLookup(ctx, node, opt, why_not);
+  }
+  if (registration->builtin_code == kTfLiteBuiltinBatchMatmul) {
+    return ClassifyBatchMatMul(ctx, node, opt, why_not);
   }
   if (registration->builtin_code != kTfLiteBuiltinFullyConnected) return no("not FULLY_CONNECTED");
   if (registration->version > kMaxFcVersion) return no("op version newer than 14");
@@ -391,6 +472,11 @@ struct FcNode {
   // in pcs_dev; status_slot = the node's place in PartitionKernel::lookup_status.
   int table_rows = 0, value_bits = 0, status_slot = -1;
   bool out_f16 = false;
+  // BATCH_MATMUL nodes: input = the float operand, filter = the int8 one; batches = rows of one
+  // matrix product, out_depth = output units; retiled_dev holds `matrices` re-tiled weight
+  // matrices one after another, row_sums_dev their row sums.
+  int lhs_batches = 1, matrices = 1;
+  bool adj_y = false;
   // Scheduling inside the partition: the stream the node runs on, the node that produces its
   // input (-1: the input is uploaded from the host), and whether a node on another stream
   // waits for this one.
@@ -537,11 +623,16 @@ void* KernelInit(TfLiteContext* ctx, const char* buffer, size_t /*length*/) {
     n.kind = kind;
     n.input = node->inputs->data[0];
     n.filter = node->inputs->data[1];
-    n.bias = (kind != FcKind::kEmbeddingLookup && node->inputs->size == 3)
+    n.bias = (kind != FcKind::kEmbeddingLookup && kind != FcKind::kBatchMatMul &&
+              node->inputs->size == 3)
                  ? node->inputs->data[2]
                  : kTfLiteOptionalTensor;
     n.output = node->outputs->data[0];
-    if (kind != FcKind::kEmbeddingLookup) {
+    if (kind == FcKind::kBatchMatMul) {
+      const auto* bp = static_cast<const TfLiteBatchMatMulParams*>(node->builtin_data);
+      n.adj_y = bp->adj_y;
+      n.params.asymmetric_quantize_inputs = bp->asymmetric_quantize_inputs;
+    } else if (kind != FcKind::kEmbeddingLookup) {
       n.params = *static_cast<const TfLiteFullyConnectedParams*>(node->builtin_data);
     }
     if (!produced.count(n.input)) {
@@ -659,8 +750,79 @@ TfLiteStatus PrepareLookupNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n
   return kTfLiteOk;
 }
 
+// BATCH_MATMUL: the constant int8 operand is put into [matrix][unit][depth] order on the host
+// (the op transposes it once as well, batch_matmul.cc:776-782), uploaded, reduced to row sums
+// and re-tiled matrix by matrix.
+TfLiteStatus PrepareBatchMatMulNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
+  const TfLiteTensor& lhs = ctx->tensors[n->input];
+  const TfLiteTensor& rhs = ctx->tensors[n->filter];
+  const TfLiteTensor& output = ctx->tensors[n->output];
+  BatchMatMulShape g;
+  const char* why = "";
+  if (!BatchMatMulGeometry(lhs, rhs, n->adj_y, &g, &why)) {
+    ctx->ReportError(ctx, "litert_amd delegate: node %d: %s", n->node_index, why);
+    return kTfLiteError;
+  }
+  n->lhs_batches = g.lhs_batches;
+  n->matrices = g.matrices;
+  n->batches = g.rows;
+  n->depth = g.depth;
+  n->out_depth = g.units;
+  const int64_t out_batches = std::max(g.lhs_batches, g.matrices);
+  if (NumElements(output.dims) != out_batches * g.rows * g.units) {
+    ctx->ReportError(ctx, "litert_amd delegate: node %d output shape does not hold %lld x %d x %d values",
+                     n->node_index, static_cast<long long>(out_batches), g.rows, g.units);
+    return kTfLiteError;
+  }
+  const auto* q = static_cast<const TfLiteAffineQuantization*>(rhs.quantization.params);
+  n->per_channel = q->scale->size > 1;
+  n->filter_scale = rhs.params.scale;
+  n->use_retiled = true;
+  n->split_quantize = true;  // rows are always quantized by a launch of their own
+  hipStream_t s = k->stream;
+  if (n->uploaded_filter == rhs.data.raw && n->have_retiled) return kTfLiteOk;
+  const size_t matrix = static_cast<size_t>(g.units) * g.depth;
+  const size_t total = matrix * g.matrices;
+  if (total == 0) return kTfLiteOk;
+  std::vector<int8_t> ordered;
+  const int8_t* src = reinterpret_cast<const int8_t*>(rhs.data.raw);
+  if (!n->adj_y) {  // [.., depth, units] -> [.., units, depth]
+    ordered.resize(total);
+    for (int m = 0; m < g.matrices; ++m) {
+      for (int d = 0; d < g.depth; ++d) {
+        for (int u = 0; u < g.units; ++u) {
+          ordered[m * matrix + static_cast<size_t>(u) * g.depth + d] =
+              src[m * matrix + static_cast<size_t>(d) * g.units + u];
+        }
+      }
+    }
+    src = ordered.data();
+  }
+  RETURN_IF_HIP(ctx, n->filter_dev.Upload(src, total, s));
+  RETURN_IF_HIP(ctx, hipStreamSynchronize(s));  // `ordered` is a local
+  const size_t packed_bytes = lrtfc_packed_int8_filter_bytes(g.units, g.depth);
+  RETURN_IF_HIP(ctx, n->retiled_dev.Ensure(packed_bytes * g.matrices));
+  RETURN_IF_HIP(ctx, n->row_sums_dev.Ensure(static_cast<size_t>(g.matrices) * g.units * 4));
+  for (int m = 0; m < g.matrices; ++m) {
+    const int8_t* w = n->filter_dev.as<int8_t>() + m * matrix;
+    RETURN_IF_FC(ctx, lrtfc_row_sums_int8(w, g.units, g.depth,
+                                          n->row_sums_dev.as<int32_t>() + static_cast<size_t>(m) * g.units, s));
+    RETURN_IF_FC(ctx, lrtfc_pack_int8_filter(w, g.units, g.depth,
+                                             n->retiled_dev.as<int8_t>() + m * packed_bytes, s));
+  }
+  if (n->per_channel) {
+    RETURN_IF_HIP(ctx, n->pcs_dev.Upload(q->scale->data, static_cast<size_t>(g.units) * 4, s));
+  }
+  RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+  n->filter_dev.Release();  // only the re-tiled matrices are kept
+  n->have_retiled = true;
+  n->uploaded_filter = rhs.data.raw;
+  return kTfLiteOk;
+}
+
 TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
   if (n->kind == FcKind::kEmbeddingLookup) return PrepareLookupNode(ctx, k, n);
+  if (n->kind == FcKind::kBatchMatMul) return PrepareBatchMatMulNode(ctx, k, n);
   const TfLiteTensor& input = ctx->tensors[n->input];
   const TfLiteTensor& filter = ctx->tensors[n->filter];
   const TfLiteTensor* bias = n->bias == kTfLiteOptionalTensor ? nullptr : &ctx->tensors[n->bias];
@@ -978,6 +1140,11 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
                              lrtfc_fc_blockwise_int4_gemm_workspace_bytes(n.batches, n.depth)));
       continue;
     }
+    if (n.kind == FcKind::kBatchMatMul) {
+      RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(lrtfc_activation_workspace_bytes(
+                             n.lhs_batches * n.batches, n.depth)));
+      continue;
+    }
     if (n.kind == FcKind::kHybridInt4 ||
         (n.kind != FcKind::kInt8 && (!n.use_retiled || n.split_quantize))) {
       RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(
@@ -1212,6 +1379,15 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                 n.batches, n.depth, n.out_depth, s));
         }
         break;
+      case FcKind::kBatchMatMul:
+        RETURN_IF_FC(ctx, lrtfc_batch_matmul_hybrid_packed(
+                              static_cast<const float*>(in_dev), n.lhs_batches, n.batches, n.depth,
+                              n.retiled_dev.as<int8_t>(), n.matrices, n.out_depth,
+                              n.per_channel ? n.pcs_dev.as<float>() : nullptr, n.filter_scale,
+                              n.row_sums_dev.as<int32_t>(), static_cast<float*>(out_dev),
+                              n.params.asymmetric_quantize_inputs, variant, scratch.get(),
+                              scratch.bytes(), s));
+        break;
       case FcKind::kEmbeddingLookup: {
         int32_t* status = k->lookup_status_dev + 3 * n.status_slot;
         const int out_type = n.out_f16 ? LRTFC_OUT_FLOAT16 : LRTFC_OUT_FLOAT32;
@@ -1426,6 +1602,7 @@ bool ParseOptions(const char* const* keys, const char* const* values, size_t n, 
     } else if (key == "claim") {
       opt->claim_int8 = opt->claim_hybrid = opt->claim_int4_blockwise = false;
       opt->claim_int4_per_channel = opt->claim_embedding_lookup = false;
+      opt->claim_batch_matmul = false;
       size_t pos = 0;
       while (pos <= val.size()) {
         const size_t comma = val.find(',', pos);
@@ -1440,9 +1617,11 @@ bool ParseOptions(const char* const* keys, const char* const* values, size_t n, 
           opt->claim_int4_per_channel = true;
         } else if (item == "embedding_lookup") {
           opt->claim_embedding_lookup = true;
+        } else if (item == "batch_matmul") {
+          opt->claim_batch_matmul = true;
         } else if (!item.empty()) {
-          *error = "claim accepts int8, hybrid, int4_blockwise, int4_per_channel, embedding_lookup; got '" +
-                   item + "'";
+          *error = "claim accepts int8, hybrid, int4_blockwise, int4_per_channel, embedding_lookup, "
+                   "batch_matmul; got '" + item + "'";
           return false;
         }
         if (comma == std::string::npos) break;
@@ -1540,7 +1719,7 @@ int litert_amd_stop_metrics(TfLiteDelegate* delegate, litert_amd_metrics* out) {
 
 // Test and tooling hook: the claim predicate on its own (no device needed). Returns
 // 0 = declined, 1 = int8, 2 = hybrid, 3 = int4 blockwise, 4 = int4 per-channel hybrid,
-// 5 = EMBEDDING_LOOKUP from a quantized table; `reason` (may be NULL)
+// 5 = EMBEDDING_LOOKUP from a quantized table, 6 = hybrid BATCH_MATMUL; `reason` (may be NULL)
 // receives why a node was declined.
 int litert_amd_classify_node(const TfLiteContext* ctx, const TfLiteNode* node,
                              const TfLiteRegistration* registration, char* reason,

@@ -22,7 +22,7 @@ FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, INT16 = 1, 2, 3, 9, 10, 18, 7
 MMAP_RO, ARENA_RW = 1, 2
 OK, ERROR, DELEGATE_ERROR = 0, 1, 2
 KIND = {0: None, 1: "int8", 2: "hybrid", 3: "int4_blockwise", 4: "int4_per_channel",
-        5: "embedding_lookup"}
+        5: "embedding_lookup", 6: "batch_matmul"}
 
 _NP = {FLOAT32: np.float32, INT32: np.int32, UINT8: np.uint8, INT8: np.int8, FLOAT16: np.float16,
        INT16: np.int16, INT4: np.uint8}
@@ -46,6 +46,7 @@ def lib():
         L.fh_add_fc_node.argtypes = [C.c_void_p] + [C.c_int] * 10
         L.fh_add_other_node.argtypes = [C.c_void_p] + [C.c_int] * 3
         L.fh_add_embedding_lookup_node.argtypes = [C.c_void_p] + [C.c_int] * 3
+        L.fh_add_batch_matmul_node.argtypes = [C.c_void_p] + [C.c_int] * 6
         L.fh_mark_graph_output.argtypes = [C.c_void_p, C.c_int]
         L.fh_set_cpu_callback.argtypes = [C.c_void_p, CPU_CB]
         L.fh_load_delegate.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p),
@@ -147,6 +148,10 @@ class FakeHost:
 
     def embedding_lookup(self, lookup, value, out):
         return self.L.fh_add_embedding_lookup_node(self.h, lookup, value, out)
+
+    def batch_matmul(self, lhs, rhs, out, adj_x=False, adj_y=False, asymmetric=True):
+        return self.L.fh_add_batch_matmul_node(self.h, lhs, rhs, out, int(adj_x), int(adj_y),
+                                               int(asymmetric))
 
     def mark_output(self, tensor):
         self.L.fh_mark_graph_output(self.h, tensor)

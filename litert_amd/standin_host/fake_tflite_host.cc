@@ -35,6 +35,7 @@ struct NodeRec {
   TfLiteNode node{};
   TfLiteRegistration reg{};
   TfLiteFullyConnectedParams fc{};
+  TfLiteBatchMatMulParams bmm{};
   bool is_delegate_kernel = false;
   std::vector<int> replaced;  // original node indices, for delegate kernels
   TfLiteDelegateParams dparams{};
@@ -316,6 +317,24 @@ int fh_add_fc_node(void* hp, int input, int filter, int bias, int three_inputs, 
   rec->node.builtin_data = &rec->fc;
   rec->reg.builtin_code = kTfLiteBuiltinFullyConnected;
   rec->reg.version = version;
+  h->nodes.push_back(std::move(rec));
+  h->plan.push_back(static_cast<int>(h->nodes.size()) - 1);
+  return static_cast<int>(h->nodes.size()) - 1;
+}
+
+// BATCH_MATMUL (builtin code 126, TfLiteBatchMatMulParams).
+int fh_add_batch_matmul_node(void* hp, int lhs, int rhs, int output, int adj_x, int adj_y,
+                             int asymmetric_quantize_inputs) {
+  auto* h = static_cast<Host*>(hp);
+  auto rec = std::make_unique<NodeRec>();
+  rec->node.inputs = MakeIntArray({lhs, rhs});
+  rec->node.outputs = MakeIntArray({output});
+  rec->bmm.adj_x = adj_x != 0;
+  rec->bmm.adj_y = adj_y != 0;
+  rec->bmm.asymmetric_quantize_inputs = asymmetric_quantize_inputs != 0;
+  rec->node.builtin_data = &rec->bmm;
+  rec->reg.builtin_code = kTfLiteBuiltinBatchMatmul;
+  rec->reg.version = 4;
   h->nodes.push_back(std::move(rec));
   h->plan.push_back(static_cast<int>(h->nodes.size()) - 1);
   return static_cast<int>(h->nodes.size()) - 1;

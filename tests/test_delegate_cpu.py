@@ -104,6 +104,33 @@ def test_claim_predicate_float_activations():
             None, "per-channel scales do not match output channels")
 
 
+def _bmm_node(h, lhs_shape=(2, 5, 64), rhs_shape=(64, 8), lhs_type=FLOAT32, const=True,
+              scales=None, qdim=0, **kw):
+    x = h.tensor(lhs_type, lhs_shape)
+    w = h.tensor(INT8, rhs_shape, data=np.zeros(rhs_shape, np.int8), const=const)
+    h.affine(w, [0.004] if scales is None else scales, quantized_dimension=qdim)
+    y = h.tensor(FLOAT32, (2, 5, 8))
+    return h.batch_matmul(x, w, y, **kw)
+
+
+def test_claim_predicate_batch_matmul():
+    """The hybrid form of BATCH_MATMUL (tflite/kernels/batch_matmul.cc:363-374): float32 left
+    operand, constant int8 right operand; adj_x and two-sided broadcasting stay on the CPU."""
+    with FakeHost() as h:
+        assert h.classify(_bmm_node(h))[0] == "batch_matmul"
+        assert h.classify(_bmm_node(h, rhs_shape=(8, 64), adj_y=True))[0] == "batch_matmul"
+        assert h.classify(_bmm_node(h, rhs_shape=(2, 64, 8)))[0] == "batch_matmul"
+        assert h.classify(_bmm_node(h, scales=np.full(8, 0.01), qdim=1))[0] == "batch_matmul"
+        assert h.classify(_bmm_node(h, scales=np.full(8, 0.01), qdim=0)) == (
+            None, "per-channel scales do not run along the output units")
+        assert h.classify(_bmm_node(h, adj_x=True)) == (None, "adj_x is left to the CPU kernels")
+        assert h.classify(_bmm_node(h, const=False)) == (None, "right operand is not a constant tensor")
+        assert h.classify(_bmm_node(h, lhs_type=INT8)) == (None, "not the float32 x int8 form")
+        assert h.classify(_bmm_node(h, rhs_shape=(32, 8))) == (None, "accumulation depths differ")
+        assert h.classify(_bmm_node(h, lhs_shape=(2, 1, 5, 64), rhs_shape=(1, 3, 64, 8))) == (
+            None, "batch dimensions broadcast on both sides")
+
+
 def test_bad_options_are_rejected_before_touching_the_device():
     with FakeHost() as h:
         assert h.load_delegate({"no_such_option": "1"}) == 1
@@ -168,4 +195,4 @@ def test_claim_predicate_embedding_lookup():
         assert h.classify(_lookup_node(h, blockwise=False, zero_point=3))[1] == "non-zero table zero point"
         assert h.classify(_lookup_node(h, blockwise=False, cols=7, rows=2))[1] == "odd row length"
         assert h.load_delegate({"claim": "int8,lookup"}) == 1
-        assert "embedding_lookup; got 'lookup'" in h.errors()
+        assert "batch_matmul; got 'lookup'" in h.errors()

@@ -86,3 +86,42 @@ def test_rejects_partial_broadcasting(bmm):
     op = bmm.BatchMatMulHybrid(rhs)
     with pytest.raises(ValueError):
         op(torch.zeros((1, 3, 2, 16), device="cuda"))
+
+
+@pytest.mark.parametrize("lhs_shape,rhs_shape,adj_y,asym", [
+    ((3, 40), (40, 7), False, True), ((2, 3, 5, 64), (2, 3, 9, 64), True, False),
+    ((4, 48), (5, 48, 6), False, True), ((2, 20, 512), (512, 130), False, True)])
+def test_node_through_the_delegate(lhs_shape, rhs_shape, adj_y, asym):
+    """A BATCH_MATMUL node claimed by the plugin, then a FULLY_CONNECTED node fed by it in the
+    same partition."""
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a gfx950 device; none visible")
+    from tests.fake_host import FakeHost, FLOAT32, INT8, OK
+    rng = np.random.default_rng(11)
+    lhs = rng.standard_normal(lhs_shape).astype(np.float32)
+    rhs = rng.integers(-127, 128, rhs_shape).astype(np.int8)
+    units = rhs_shape[-2] if adj_y else rhs_shape[-1]
+    pcs = rng.uniform(2e-3, 8e-3, units).astype(np.float32)
+    want = oracle.batch_matmul_hybrid(lhs, rhs, pcs, 1.0, asym, adj_y)
+    w2 = rng.integers(-127, 128, (12, units)).astype(np.int8)
+    pcs2 = rng.uniform(2e-3, 8e-3, 12).astype(np.float32)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, lhs_shape, data=lhs)
+        w = h.tensor(INT8, rhs_shape, data=rhs, const=True)
+        h.affine(w, pcs, quantized_dimension=len(rhs_shape) - (2 if adj_y else 1))
+        y = h.tensor(FLOAT32, want.shape)
+        node = h.batch_matmul(x, w, y, adj_y=adj_y, asymmetric=asym)
+        f = h.tensor(INT8, w2.shape, data=w2, const=True)
+        h.affine(f, pcs2)
+        z = h.tensor(FLOAT32, (want.size // units, 12))
+        fc_node = h.fc(y, f, None, z)
+        h.mark_output(y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK, h.errors()
+        assert h.plan()[0][:2] == ("delegate", [node, fc_node])
+        assert h.allocate_tensors() == OK, h.errors()
+        assert h.invoke() == OK, h.errors()
+        got = h.read(y)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        want2 = oracle.fc_hybrid(want.reshape(-1, units), w2, pcs2)
+        assert np.array_equal(h.read(z).view(np.uint32), want2.view(np.uint32))
