@@ -34,8 +34,10 @@ __device__ __forceinline__ float HybridCore(int32_t dot, float batch_scale, floa
 // the product as always and repair that one case lazily: a thread that meets a -0.0f bias with a
 // zero dot product scans the input; only a whole-zero input takes the scan to its end. A row
 // quantizes to all-zero values exactly when it was all zero (any other row has a value at the
-// far end of the int8 range), so the quantized rows can stand for the float ones.
-__device__ inline bool AllZeroInt8(const int8_t* p, size_t n) {
+// far end of the int8 range), so the quantized rows can stand for the float ones. The scans are
+// real function calls: inlined into an unrolled epilogue their loops keep it from unrolling, and
+// the accumulator tiles then land in scratch memory.
+__device__ __attribute__((noinline)) bool AllZeroInt8(const int8_t* p, size_t n) {
   size_t i = 0;
   if ((reinterpret_cast<uintptr_t>(p) & 15) == 0) {
     const i32x4* v = reinterpret_cast<const i32x4*>(p);
@@ -50,7 +52,8 @@ __device__ inline bool AllZeroInt8(const int8_t* p, size_t n) {
   return true;
 }
 
-__device__ inline bool AllZeroF32(const float* p, size_t n) {  // IsZeroVector: -0.0f counts as zero
+// IsZeroVector: -0.0f counts as zero.
+__device__ __attribute__((noinline)) bool AllZeroF32(const float* p, size_t n) {
   const uint32_t* u = reinterpret_cast<const uint32_t*>(p);
   size_t i = 0;
   for (; i + 4 <= n; i += 4) {
@@ -98,6 +101,44 @@ __device__ __forceinline__ float HybridCoreZeroAware(const FcInt8Args& a, int32_
   }
   return HybridCore(dot, batch_scale, channel_scale, batch_zero_point, row_sum, base,
                     a.activation);
+}
+
+// The same choice without a branch or a loop, for epilogues that must unroll completely (an
+// accumulator tile indexed inside a loop that did not unroll lands in scratch memory): the
+// caller has settled `zero_input` for the whole workgroup beforehand. Adding -0.0f instead of the
+// zero product leaves every bias value as it is, -0.0f included, which is what the early exit
+// amounts to.
+__device__ __forceinline__ float HybridCoreSelect(int32_t dot, float batch_scale,
+                                                  float channel_scale, int32_t batch_zero_point,
+                                                  int32_t row_sum, float base, int activation,
+                                                  bool batch_matmul, bool zero_input) {
+  const float scale = __fmul_rn(batch_scale, channel_scale);
+  const float as_bmm =
+      HybridBatchMatMulCore(dot, batch_scale, channel_scale, batch_zero_point, row_sum);
+  const int32_t corrected = dot - row_sum * batch_zero_point;
+  const float term = zero_input ? -0.0f : __fmul_rn(static_cast<float>(corrected), scale);
+  const float as_fc = ApplyFloatActivation(__fadd_rn(base, term), activation);
+  return batch_matmul ? as_bmm : as_fc;
+}
+
+// Whole-input zero test by a whole workgroup (every thread must call it): threads scan
+// interleaved 16-byte pieces and meet after every round, so a non-zero input ends the scan
+// after the first round.
+__device__ inline bool WorkgroupAllZeroInt8(const int8_t* p, size_t n) {
+  const bool vec = (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+  const size_t pieces = vec ? n / 16 : 0;
+  for (size_t base = 0; base < pieces; base += blockDim.x) {
+    const size_t i = base + threadIdx.x;
+    int nonzero = 0;
+    if (i < pieces) {
+      const i32x4 t = reinterpret_cast<const i32x4*>(p)[i];
+      nonzero = (t.x | t.y | t.z | t.w) != 0;
+    }
+    if (__syncthreads_or(nonzero)) return false;
+  }
+  int nonzero = 0;
+  for (size_t i = pieces * 16 + threadIdx.x; i < n; i += blockDim.x) nonzero |= p[i] != 0;
+  return !__syncthreads_or(nonzero);
 }
 
 // Output value of the per-channel int4 hybrid path: ReferenceAssignBiasAndComputeOffsets and

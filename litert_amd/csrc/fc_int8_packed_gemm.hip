@@ -99,6 +99,17 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
     }
     chan_p = p;
   }
+  // EvalHybridDense's early exit for a whole-zero input (fully_connected.cc:789-795) matters only
+  // where a bias element is -0.0f: a workgroup that stages such a channel settles the question
+  // here, once, outside the loops that must unroll.
+  bool zero_input = false;
+  if (EPI == Int8Epilogue::kHybrid && a.zero_input_exit) {
+    const bool mine = tid < BN && n0 + tid < N && a.bias_f32 != nullptr &&
+                      IsNegativeZero(__int_as_float(chan_p[1]));
+    if (__syncthreads_or(mine)) {
+      zero_input = WorkgroupAllZeroInt8(a.input, static_cast<size_t>(M) * K);
+    }
+  }
 
   // Weight operands of this wavefront: lane L addresses channel L % 32 of MFMA tile i (tile
   // index clamped at the last 16-channel tile: duplicates are computed and never stored) and
@@ -307,8 +318,8 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
             v[r] = EPI == Int8Epilogue::kHybrid4Bit
                        ? Hybrid4BitCore(acc[i][j][4 * g + r], bscale, cscale[r], bzp, base[r],
                                         a.bias_f32 != nullptr, a.activation)
-                       : HybridCoreZeroAware(a, acc[i][j][4 * g + r], bscale, cscale[r], bzp,
-                                             rsum[r], base[r]);
+                       : HybridCoreSelect(acc[i][j][4 * g + r], bscale, cscale[r], bzp, rsum[r],
+                                          base[r], a.activation, a.batch_matmul != 0, zero_input);
           }
           if (kFull || m < M) {
             float* dst = a.output_f32 + static_cast<size_t>(m) * N + c0;
