@@ -58,6 +58,13 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--traffic-probe-int4", action="store_true",
                     help="launch only what the int4 grouped kernel's counter runs need, then exit")
+    ap.add_argument("--traffic-probe-int4-single", action="store_true",
+                    help="launch only config 3's single-node int4 kernel (cold, 12 times) and the "
+                         "64 MiB device copy (3 times), for a rocprofv3 counter or kernel-trace run")
+    ap.add_argument("--gemm-probe", action="store_true",
+                    help="launch only config 4's int8 GEMM: 10 times on the seeded operands, then 10 "
+                         "times on constant operands (a second kernel name is not involved: the "
+                         "two sets are told apart by launch order), for a rocprofv3 counter run")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch only the dominant kernel (cold, 12 times) and a 64 MiB device "
                          "copy (3 times), for a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run")
@@ -87,6 +94,12 @@ def main():
         return
     if args.traffic_probe_int4:
         traffic_probe_int4(torch, fc, wl)
+        return
+    if args.gemm_probe:
+        gemm_probe(torch, fc, wl)
+        return
+    if args.traffic_probe_int4_single:
+        traffic_probe_int4_single(torch, fc, wl)
         return
 
     def timed_replays(graphs, reps):
@@ -202,6 +215,16 @@ def main():
         split_us = per_launch_us([(lambda o: lambda: o.call_split(xs[b], out=outs[b]))(op)
                                   for op in ops])
         forms[b] = dict(fused_us_cold=round(fused_us, 3), split_us_cold=round(split_us, 3))
+    # What the memory system alone needs for a launch of this size: a kernel that only streams
+    # the same bytes (the re-tiled filter of each weight copy) with the GEMV's access pattern.
+    def stream_floor(buffers, nbytes):
+        sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+        fns = [(lambda t: lambda: capi.check(lib.lrtfc_stream_read_probe(p(t), nbytes, p(sink),
+                                                                          stream())))(t)
+               for t in buffers]
+        return per_launch_us(fns)
+
+    floor2_us = stream_floor([op.packed_filter for op in ops], N_OUT * K_IN)
     b_dom = 1
     achieved = hybrid_bytes(b_dom) / per_b[b_dom]["op_us_cold"] / 1e3
     roofline = dict(bound="hbm",
@@ -211,8 +234,14 @@ def main():
                     traffic_source="profiles/hybrid_gemv_fused_B1_hbm_traffic.txt (rocprofv3 --pmc "
                                    "FETCH_SIZE / WRITE_SIZE of `bench.py --traffic-probe`; a committed "
                                    "counter summary, not measured in this run)",
+                    traffic_commit=measured_traffic("library built from commit"),
                     algorithmic_bytes_per_launch=hybrid_bytes(b_dom),
-                    avg_launch_us=per_b[b_dom]["op_us_cold"])
+                    avg_launch_us=per_b[b_dom]["op_us_cold"],
+                    stream_only_us=round(floor2_us, 3),
+                    stream_only_note="a launch that only reads the same 58.7 MB filter (same "
+                                     "access pattern, cold): the memory system's own time for "
+                                     "this size, %.1f%% of peak" % (N_OUT * K_IN / floor2_us / 1e3 /
+                                                                  HBM_PEAK_GBPS * 100))
 
     # Between decode and prefill (not a BASELINE configuration): config 2's filters against 16
     # rows (row quantizer + GEMV) and 32 to 512 rows (row quantizer + MFMA GEMM, 64 x 128 tiles
@@ -276,6 +305,45 @@ def traffic_probe(torch, fc, wl):
                       "copy_bytes": 64 << 20, "algorithmic_bytes": hybrid_bytes(1)}))
 
 
+def gemm_probe(torch, fc, wl):
+    """Counter-run launches for config 4's kernel alone (FcInt8PackedGemmKernel, requantizing
+    epilogue, RELU6): ten launches on the seeded U[-128,127] operands, then ten on constant
+    operands (x = 3, w = 5)."""
+    c4 = wl.prefill_int8_fc()
+    y4 = torch.empty((2048, 4096), dtype=torch.int8, device="cuda")
+    for w, x in ((c4["w"], torch.from_numpy(c4["x"]).cuda()),
+                 (np.full_like(c4["w"], 5), torch.full((2048, 4096), 3, dtype=torch.int8, device="cuda"))):
+        op = fc.FullyConnectedInt8(w, c4["bias"], float(c4["in_scale"]), c4["in_zp"], c4["w_scale"],
+                                   float(c4["out_scale"]), c4["out_zp"], activation="relu6")
+        torch.cuda.synchronize()
+        for _ in range(10):
+            op(x, out=y4)
+        torch.cuda.synchronize()
+    print(json.dumps({"probe": "gemm", "launches_seeded": 10, "launches_constant": 10,
+                      "ops_per_launch": 2 * 2048 * 4096 * 4096}))
+
+
+def traffic_probe_int4_single(torch, fc, wl):
+    """Counter-run launches for config 3's kernel alone: the fused blockwise-int4 GEMV of
+    14336 x 4096 at B = 1 on rotating copies of the filter, plus the calibrating 64 MiB copy."""
+    c3 = wl.blockwise_int4_fc(1)
+    ops3 = [fc.FullyConnectedBlockwiseInt4(np.roll(c3["packed"], i, axis=0),
+                                           np.roll(c3["scales"], i, axis=0), 4096, 32)
+            for i in range(8)]
+    x = torch.from_numpy(c3["x"]).cuda()
+    y = torch.empty((1, 14336), dtype=torch.float32, device="cuda")
+    src = torch.ones(64 << 20, dtype=torch.int8, device="cuda")
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for i in range(12):
+        ops3[i % len(ops3)](x, out=y)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": "traffic-int4-single", "int4_launches": 12, "copy_launches": 3,
+                      "copy_bytes": 64 << 20, "algorithmic_bytes": int4_bytes(1, 14336, 4096)}))
+
+
 def traffic_probe_int4(torch, fc, wl):
     """Counter-run launches for the grouped int4 kernel: config 5's 108 nodes of depth 2048 in
     ONE launch (B = 1), four times, plus the 64 MiB copy that calibrates the counters."""
@@ -304,14 +372,16 @@ def traffic_probe_int4(torch, fc, wl):
                       "copy_launches": 3, "copy_bytes": 64 << 20, "algorithmic_bytes": total}))
 
 
-def measured_traffic():
+def measured_traffic(field="traffic_bytes_per_launch:"):
     """HBM bytes per launch of the dominant kernel, from the committed counter summary
-    (two rocprofv3 --pmc runs of `bench.py --traffic-probe`); None when it is absent."""
+    (two rocprofv3 --pmc runs of `bench.py --traffic-probe`); None when it is absent.
+    field "library built from commit" returns the commit the summary was taken at."""
     path = os.path.join(ROOT, "profiles", "hybrid_gemv_fused_B1_hbm_traffic.txt")
     try:
         for ln in open(path):
-            if ln.startswith("traffic_bytes_per_launch:"):
-                return int(ln.split(":")[1].split()[0])
+            if ln.startswith(field):
+                tail = ln[len(field):].split()
+                return int(tail[0]) if field.endswith(":") else tail[0]
     except OSError:
         pass
     return None
@@ -355,7 +425,12 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
     o_hot = per_launch_us([lambda: ops3[0](x3, out=y3)] * len(ops3))
     k_cold = per_launch_us([int4_kernel_only(op) for op in ops3])
     b3 = int4_bytes(1, 14336, 4096)
+    sink3 = torch.zeros(1, dtype=torch.int32, device="cuda")
+    floor3 = per_launch_us([(lambda o: lambda: capi.check(lib.lrtfc_stream_read_probe(
+        p(o.retiled), o.retiled.numel(), p(sink3), stream())))(op) for op in ops3])
     out["config3_int4_gemv_14336x4096_B1"] = dict(
+        stream_only_us=round(floor3, 3),
+        stream_only_frac_of_hbm_peak=round(ops3[0].retiled.numel() / floor3 / 1e3 / HBM_PEAK_GBPS, 4),
         op_us_cold=round(o_cold, 3), op_us_hot=round(o_hot, 3),
         prequantized_kernel_us_cold=round(k_cold, 3),
         op_gbps_cold=round(b3 / o_cold / 1e3, 1), op_gbps_hot=round(b3 / o_hot / 1e3, 1),

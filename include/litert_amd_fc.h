@@ -452,6 +452,14 @@ int lrtfc_embedding_lookup_hybrid(const int32_t* lookup, int count, const void* 
                                   const float* row_scales, int out_type, void* output,
                                   int32_t* status, void* stream);
 
+/* ---- measurement aid ------------------------------------------------------------------------
+ * No counterpart in the reference: a launch that does nothing but read `bytes` bytes (whole
+ * 16-byte pieces; src 16-byte aligned) from device memory with the decode kernels' access
+ * pattern. The benchmark times it on the same bytes as a GEMV to show what the memory system
+ * alone needs for a launch of that size. `sink` (device int32, may be NULL) is practically
+ * never written. */
+int lrtfc_stream_read_probe(const void* src, size_t bytes, int32_t* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -187,6 +187,9 @@ hipError_t LaunchEmbeddingLookup(const int32_t* lookup, int count, const void* t
                                  int blocksize, const float* row_scales, float scale, int out_f16,
                                  void* output, int32_t* status, hipStream_t stream);
 
+// Measurement aid: a launch that only reads `bytes` bytes (whole 16-byte pieces) from `src`.
+hipError_t LaunchStreamRead(const void* src, size_t bytes, int32_t* sink, hipStream_t stream);
+
 }  // namespace lrtfc
 
 #endif  // LITERT_AMD_CSRC_KERNELS_H_
