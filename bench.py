@@ -65,6 +65,10 @@ def main():
                     help="launch only config 4's int8 GEMM: 10 times on the seeded operands, then 10 "
                          "times on constant operands (a second kernel name is not involved: the "
                          "two sets are told apart by launch order), for a rocprofv3 counter run")
+    ap.add_argument("--sustain", type=float, default=0.0,
+                    help="with --gemm-probe: afterwards keep launching the GEMM for this many seconds "
+                         "on the seeded operands, then as long on the constant ones, printing a "
+                         "time-stamped line at each switch (for power / clock sampling from outside)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch only the dominant kernel (cold, 12 times) and a 64 MiB device "
                          "copy (3 times), for a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run")
@@ -96,7 +100,7 @@ def main():
         traffic_probe_int4(torch, fc, wl)
         return
     if args.gemm_probe:
-        gemm_probe(torch, fc, wl)
+        gemm_probe(torch, fc, wl, args.sustain)
         return
     if args.traffic_probe_int4_single:
         traffic_probe_int4_single(torch, fc, wl)
@@ -305,22 +309,43 @@ def traffic_probe(torch, fc, wl):
                       "copy_bytes": 64 << 20, "algorithmic_bytes": hybrid_bytes(1)}))
 
 
-def gemm_probe(torch, fc, wl):
+def gemm_probe(torch, fc, wl, sustain=0.0):
     """Counter-run launches for config 4's kernel alone (FcInt8PackedGemmKernel, requantizing
     epilogue, RELU6): ten launches on the seeded U[-128,127] operands, then ten on constant
-    operands (x = 3, w = 5)."""
+    operands (x = 3, w = 5). With `sustain` seconds, each set is then launched back to back for
+    that long, so that a sampler outside the process can read the power and clocks the part
+    settles at."""
     c4 = wl.prefill_int8_fc()
     y4 = torch.empty((2048, 4096), dtype=torch.int8, device="cuda")
-    for w, x in ((c4["w"], torch.from_numpy(c4["x"]).cuda()),
-                 (np.full_like(c4["w"], 5), torch.full((2048, 4096), 3, dtype=torch.int8, device="cuda"))):
+    sets = []
+    for name, w, x in (("seeded", c4["w"], torch.from_numpy(c4["x"]).cuda()),
+                       ("constant", np.full_like(c4["w"], 5),
+                        torch.full((2048, 4096), 3, dtype=torch.int8, device="cuda"))):
         op = fc.FullyConnectedInt8(w, c4["bias"], float(c4["in_scale"]), c4["in_zp"], c4["w_scale"],
                                    float(c4["out_scale"]), c4["out_zp"], activation="relu6")
         torch.cuda.synchronize()
         for _ in range(10):
             op(x, out=y4)
         torch.cuda.synchronize()
+        sets.append((name, op, x))
     print(json.dumps({"probe": "gemm", "launches_seeded": 10, "launches_constant": 10,
-                      "ops_per_launch": 2 * 2048 * 4096 * 4096}))
+                      "ops_per_launch": 2 * 2048 * 4096 * 4096}), flush=True)
+    for name, op, x in sets if sustain > 0 else []:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(50):
+                op(x, out=y4)
+        t0 = time.time()
+        print(json.dumps({"sustain": name, "begin_unix": round(t0, 3)}), flush=True)
+        launches = 0
+        while time.time() - t0 < sustain:
+            for _ in range(20):
+                g.replay()
+            torch.cuda.synchronize()
+            launches += 1000
+        t1 = time.time()
+        print(json.dumps({"sustain": name, "end_unix": round(t1, 3), "launches": launches,
+                          "us_per_launch": round((t1 - t0) / launches * 1e6, 2)}), flush=True)
 
 
 def traffic_probe_int4_single(torch, fc, wl):
@@ -505,15 +530,33 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
     x4 = dev(c4["x"])
     y4 = torch.empty((2048, 4096), dtype=torch.int8, device="cuda")
     ops_per_call = 2.0 * 2048 * 4096 * 4096
-    for act in ("none", "relu6"):
-        op4 = fc.FullyConnectedInt8(c4["w"], c4["bias"], float(c4["in_scale"]), c4["in_zp"],
-                                    c4["w_scale"], float(c4["out_scale"]), c4["out_zp"],
-                                    activation=act)
-        us = per_launch_us([lambda: op4(x4, out=y4)] * 4)
+    # The two activations are timed in alternation, replay by replay, so that clock drift over
+    # the run lands on both alike; median and minimum over the replays are reported.
+    ops4 = {act: fc.FullyConnectedInt8(c4["w"], c4["bias"], float(c4["in_scale"]), c4["in_zp"],
+                                       c4["w_scale"], float(c4["out_scale"]), c4["out_zp"],
+                                       activation=act) for act in ("none", "relu6")}
+    graphs4 = {act: many([(lambda o: lambda: o(x4, out=y4))(op)] * 4) for act, op in ops4.items()}
+    samples4 = {act: [] for act in ops4}
+    for g, _ in graphs4.values():
+        g.replay()
+    torch.cuda.synchronize()
+    for _ in range(25):
+        for act, (g, n) in graphs4.items():
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            samples4[act].append(e0.elapsed_time(e1) * 1e3 / n)
+    for act, samples in samples4.items():
+        samples.sort()
+        us, us_min = samples[len(samples) // 2], samples[0]
         tops = ops_per_call / us / 1e6
         out["config4_int8_gemm_2048x4096x4096_" + act] = dict(
-            us=round(us, 2), tops=round(tops, 1),
-            frac_of_int8_mfma_peak=round(tops / INT8_MFMA_PEAK_TOPS, 4))
+            us=round(us, 2), us_min=round(us_min, 2), tops=round(tops, 1),
+            frac_of_int8_mfma_peak=round(tops / INT8_MFMA_PEAK_TOPS, 4),
+            timing="median (us) and minimum (us_min) of 25 graph replays, alternating with the other activation")
+    del graphs4
     # The same launch on constant operands (every x = 3, every w = 5). The kernel executes the same
     # instructions in the same number of cycles; only the switching activity differs. The gap
     # to the seeded U[-128,127] operands above is the clock the part sustains under that

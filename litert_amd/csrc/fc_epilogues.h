@@ -16,6 +16,31 @@ __device__ __forceinline__ int8_t RequantizeCore(int32_t acc, int32_t multiplier
   return static_cast<int8_t>(ClampI32(v, act_min, act_max));
 }
 
+// The same value as RequantizeCore for the common case, in half the instructions: a right
+// shift by right_shift = 1..31 bits, multiplier != INT32_MIN, |acc| < 2^30 and act_lo <= act_hi
+// (the caller checks all four). SaturatingRoundingDoublingHighMul cannot saturate then and is
+// floor((acc * multiplier + 2^30) / 2^31); RoundingDivideByPOT of r, nearest with ties away from
+// zero, is (r + 2^(right_shift - 1) - (r < 0)) >> right_shift, a sum that stays below 2^31
+// because |r| <= |acc|. half = 2^(right_shift - 1).
+__device__ __forceinline__ int32_t RequantizeShort(int32_t acc, int32_t multiplier,
+                                                   int right_shift, int32_t half,
+                                                   int32_t output_offset, int32_t act_lo,
+                                                   int32_t act_hi) {
+  const int64_t t = static_cast<int64_t>(acc) * multiplier + (1ll << 30);
+  const int32_t r = static_cast<int32_t>(t >> 31);
+  const int32_t v = ((r + half + (r >> 31)) >> right_shift) + output_offset;
+  int32_t out;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(out) : "v"(v), "v"(act_lo), "v"(act_hi));
+  return out;
+}
+
+// The low bytes of four values as one dword, first value lowest.
+__device__ __forceinline__ int32_t PackLowBytes(int32_t q0, int32_t q1, int32_t q2, int32_t q3) {
+  const uint32_t lo = __builtin_amdgcn_perm(q1, q0, 0x0c0c0400u);
+  const uint32_t hi = __builtin_amdgcn_perm(q3, q2, 0x0c0c0400u);
+  return static_cast<int32_t>(__builtin_amdgcn_perm(hi, lo, 0x05040100u));
+}
+
 // Hybrid output value: reference/portable_tensor_utils.cc:186-203 after the bias
 // initialisation of fully_connected.cc:780-786, then ApplyActivationToVector.
 // channel_scale is the per-channel scale, or the per-tensor filter scale.

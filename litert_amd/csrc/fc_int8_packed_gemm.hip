@@ -10,12 +10,14 @@
 // bytes of half L / 32) is gathered from two such tiles by per-lane addresses; each quarter
 // of the wavefront still reads 256 consecutive bytes, so the load is as efficient as a
 // contiguous one. Each wavefront owns 64 output channels and loads their operands straight
-// from global memory into registers, three depth steps ahead -- the weights never touch
-// LDS, because no other wavefront of the workgroup needs them. Only the activation rows are
-// shared: the workgroup stages 128 rows x 64 depth per step in LDS (two buffers, rows padded
-// to 80 bytes so that the 16-byte operand reads are conflict-free) and every wavefront reads
-// its eight operands from there. Per step and wavefront: 4 global loads, 8 LDS reads, 16
-// MFMAs (512 matrix-core cycles), one barrier placed between the two halves of the MFMAs.
+// from global memory into registers, two depth steps ahead -- the weights never touch LDS,
+// because no other wavefront of the workgroup needs them. Only the activation rows are
+// shared: the workgroup stages 128 rows x 128 depth per step in LDS (two buffers, rows padded
+// to 144 bytes so that the 16-byte operand reads are conflict-free; 128 bytes of a row are one
+// whole cache line) and every wavefront reads its sixteen operands from there. Per step and
+// wavefront: 12 global loads, 16 LDS reads, 4 LDS writes, 32 MFMAs (1024 matrix-core cycles)
+// and one barrier, all dealt out singly between the MFMAs: a wavefront is alone on its SIMD,
+// so whatever holds up its instruction stream idles the matrix pipe.
 // Launches that this 128 x 256 tile would cut into fewer workgroups than half the chip's CUs
 // (batches of a few dozen to a few hundred rows) run the same kernel with 64 rows x 128
 // channels per workgroup (32 channels per wavefront).
@@ -35,10 +37,10 @@ using i32x16 = int __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-constexpr int kStep = 64;                     // depth per step = one slab of the packed filter
+constexpr int kSlab = 64;                     // depth of one tile of the packed filter
+constexpr int kStep = 128;                    // depth per step: two slabs, one cache line of a row
 constexpr int kXStride = kStep + 16;          // padded LDS row
 constexpr int kSub = kStep / 32;              // MFMA depth sub-steps per step
-constexpr int kRing = 4;                      // weight register ring, in steps (even)
 constexpr int kGroupM = 4;                    // M-tiles per rasterization group
 
 // f(std::integral_constant<int, 0>{}), f(<1>), ... : a loop whose index is a constant in
@@ -55,12 +57,13 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
   constexpr int BN = kWaves * kWaveTiles * 32;  // output channels per workgroup
   constexpr int kStageBytes = BM * kXStride;
   constexpr int kBatchTiles = BM / 32;
-  constexpr int kXChunks = BM / 64;  // 16-byte chunks of activations a thread stages per step
+  constexpr int kXChunks = BM / 32;  // 16-byte chunks of activations a thread stages per step
   static_assert(BM % 64 == 0 && BN <= kThreads, "tile shape");
   __shared__ __align__(16) int8_t smem[2 * kStageBytes];
   __shared__ i32x4 chan_params[BN];  // per output channel of the tile, for the epilogue
   const int M = a.batches, N = a.out_depth, K = a.depth;
-  const int slabs = (K + kStep - 1) / kStep;
+  const int slabs = (K + kSlab - 1) / kSlab;
+  const int steps = (slabs + 1) / 2;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int total = tiles_m * tiles_n;
 
@@ -81,9 +84,10 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   // Per-channel epilogue inputs, one channel per thread, fetched now so that their latency
-  // hides behind the main loop: {multiplier, shift, bias + input_offset * row_sum, -} or
-  // {channel scale, bias, row sum, -}.
+  // hides behind the main loop: {multiplier, shift, bias + input_offset * row_sum, rounding
+  // term of the right shift} or {channel scale, bias, row sum, -}.
   i32x4 chan_p;
+  bool plain_channel = true;  // this thread's channel allows the short requantization
   {
     const int n = min(n0 + tid, N - 1);
     i32x4 p = {0, 0, 0, 0};
@@ -92,6 +96,9 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
       p[1] = a.per_channel ? a.shifts[n] : a.shifts[0];
       p[2] = a.bias_i32 ? a.bias_i32[n] : 0;
       if (a.input_offset != 0) p[2] += a.input_offset * a.filter_row_sums[n];
+      p[3] = (p[1] < 0 && p[1] >= -31) ? (1 << (-p[1] - 1)) : 0;
+      plain_channel = p[1] <= -1 && p[1] >= -31 && p[0] != INT32_MIN &&
+                      p[2] > -(1 << 29) && p[2] < (1 << 29);
     } else {
       p[0] = __float_as_int(a.per_channel_scales ? a.per_channel_scales[n] : a.filter_scale);
       p[1] = __float_as_int(a.bias_f32 ? a.bias_f32[n] : 0.0f);
@@ -121,52 +128,59 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
     const int ct = min(n0 / 16 + (wave * kWaveTiles + i) * 2 + ((lane & 31) >> 4), ctiles - 1);
     wp[i] = a.filter + static_cast<size_t>(ct) * slabs * 1024 + (lane & 15) * 16 + (lane >> 5) * 256;
   }
-  // Activation staging: 16-byte chunks per thread and step, rows tid / 4 (and 64 + tid / 4).
-  const int ld_chunk = tid & 3;
+  // Activation staging: 16-byte chunks per thread and step, chunk tid % 8 of rows tid / 8 + 32 p
+  // (eight consecutive lanes read one whole 128-byte line of a row).
+  const int ld_chunk = tid & 7;
   const int8_t* xp[kXChunks];
 #pragma unroll
-  for (int i = 0; i < kXChunks; ++i) {
-    const int row = min(m0 + (tid >> 2) + 64 * i, M - 1);
-    xp[i] = a.input + static_cast<size_t>(row) * K;
+  for (int p = 0; p < kXChunks; ++p) {
+    const int row = min(m0 + (tid >> 3) + 32 * p, M - 1);
+    xp[p] = a.input + static_cast<size_t>(row) * K;
   }
-  const int st_off = (tid >> 2) * kXStride + ld_chunk * 16;
+  const int st_off = (tid >> 3) * kXStride + ld_chunk * 16;
+  // An odd number of slabs leaves the second half of the last step without a filter tile: the
+  // weight addresses are clamped to the last tile and the rows' half is staged as zeros.
+  const bool upper_chunk = ld_chunk >= 4;
+  const int half_step = (slabs & 1) ? steps - 1 : -1;
 
-  i32x4 wring[kRing][kWaveTiles][kSub];
-  i32x4 xr[2][kXChunks];  // two sets: rows are requested two steps before they are staged
-  auto load_w = [&](int step, auto slot) {
-    const int s = min(step, slabs - 1);
-#pragma unroll
-    for (int i = 0; i < kWaveTiles; ++i) {
-#pragma unroll
-      for (int h = 0; h < kSub; ++h) {
-        wring[decltype(slot)::value][i][h] =
-            *reinterpret_cast<const i32x4*>(wp[i] + static_cast<size_t>(s) * 1024 + h * 512);
-      }
-    }
+  // Weights: wring[step % 2] holds a step's operands; a piece is requested again, for two steps
+  // later, right after the last MFMA that reads it. Rows: xr[step % 2], requested three steps
+  // before their use, staged two steps before it, read into fa during the step before it.
+  i32x4 wring[2][kWaveTiles][kSub];
+  i32x4 xr[2][kXChunks];
+  auto load_w_piece = [&](int step, auto slot, auto tile, auto sub) {
+    constexpr int i = decltype(tile)::value, h = decltype(sub)::value;
+    const int slab = min(2 * step + h / 2, slabs - 1);
+    wring[decltype(slot)::value][i][h] = *reinterpret_cast<const i32x4*>(
+        wp[i] + static_cast<size_t>(slab) * 1024 + (h & 1) * 512);
   };
-  auto load_x = [&](int step, auto set) {
+  auto load_x_piece = [&](int step, auto set, auto piece) {
     // Past the end of a row (last partial slab, steps beyond the last) the address is clamped
-    // into the row: whatever it reads meets zero padding in the packed filter or is unused.
-    const int k = min(min(step, slabs - 1) * kStep + ld_chunk * 16, K - 16);
-#pragma unroll
-    for (int i = 0; i < kXChunks; ++i) {
-      xr[decltype(set)::value][i] = *reinterpret_cast<const i32x4*>(xp[i] + k);
-    }
+    // into the row: whatever it reads meets zero padding in the packed filter, is replaced by
+    // zeros when staged, or is never used.
+    const int k = min(min(step, steps - 1) * kStep + ld_chunk * 16, K - 16);
+    xr[decltype(set)::value][decltype(piece)::value] =
+        *reinterpret_cast<const i32x4*>(xp[decltype(piece)::value] + k);
   };
-  auto store_x = [&](int stage, auto set) {
-#pragma unroll
-    for (int i = 0; i < kXChunks; ++i) {
-      *reinterpret_cast<i32x4*>(smem + stage * kStageBytes + st_off + i * 64 * kXStride) =
-          xr[decltype(set)::value][i];
-    }
+  auto store_x_piece = [&](int step, auto set, auto piece) {
+    constexpr int p = decltype(piece)::value;
+    i32x4 v = xr[decltype(set)::value][p];
+    if (upper_chunk && step == half_step) v = i32x4{0, 0, 0, 0};
+    *reinterpret_cast<i32x4*>(smem + decltype(set)::value * kStageBytes + st_off +
+                              p * 32 * kXStride) = v;
   };
   // Operand of batch tile j, sub-step h: lane L reads row 32 j + L % 32, bytes
-  // 32 h + 16 * (L / 32) .. +16 of the staged 64.
+  // 32 h + 16 * (L / 32) .. +16 of the staged 128.
   const int frag_off = (lane & 31) * kXStride + (lane >> 5) * 16;
-  auto read_frag = [&](int stage, int j, int h) {
-    return *reinterpret_cast<const i32x4*>(smem + stage * kStageBytes + frag_off +
+  auto read_frag = [&](auto stage, int j, int h) {
+    return *reinterpret_cast<const i32x4*>(smem + decltype(stage)::value * kStageBytes + frag_off +
                                            j * 32 * kXStride + h * 32);
   };
+  using C0 = std::integral_constant<int, 0>;
+  using C1 = std::integral_constant<int, 1>;
+  constexpr auto kTiles = std::make_integer_sequence<int, kWaveTiles>{};
+  constexpr auto kSubs = std::make_integer_sequence<int, kSub>{};
+  constexpr auto kChunks = std::make_integer_sequence<int, kXChunks>{};
 
   i32x16 acc[kWaveTiles][kBatchTiles];
 #pragma unroll
@@ -178,86 +192,99 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
     }
   }
 
-  // Prologue: step 0 staged, steps 1 and 2 in registers, weights of steps 0 .. kRing - 2 in
-  // flight.
-  // (Same issue order as inside the loop: activation rows first, then weights.)
-  load_x(0, std::integral_constant<int, 0>{});
-  store_x(0, std::integral_constant<int, 0>{});
+  // Prologue: rows of steps 0 and 1 staged, those of step 2 requested, weights of steps 0 and 1
+  // requested, operands of step 0 read.
+  ForEachConst(kChunks, [&](auto p) { load_x_piece(0, C0{}, p); });
+  ForEachConst(kChunks, [&](auto p) { load_x_piece(1, C1{}, p); });
   asm volatile("" ::: "memory");
-  load_x(1, std::integral_constant<int, 1>{});
-  load_x(2, std::integral_constant<int, 0>{});
+  ForEachConst(kTiles, [&](auto i) { ForEachConst(kSubs, [&](auto h) { load_w_piece(0, C0{}, i, h); }); });
+  ForEachConst(kTiles, [&](auto i) { ForEachConst(kSubs, [&](auto h) { load_w_piece(1, C1{}, i, h); }); });
   asm volatile("" ::: "memory");
-  ForEachConst(std::make_integer_sequence<int, kRing - 1>{}, [&](auto u) { load_w(u, u); });
+  ForEachConst(kChunks, [&](auto p) { store_x_piece(0, C0{}, p); });
+  ForEachConst(kChunks, [&](auto p) { store_x_piece(1, C1{}, p); });
+  asm volatile("" ::: "memory");
+  ForEachConst(kChunks, [&](auto p) { load_x_piece(2, C0{}, p); });
   asm volatile("" ::: "memory");
   if (tid < BN) chan_params[tid] = chan_p;
-  __syncthreads();
+  // The short requantization (RequantizeShort) needs every channel of the tile to shift right by
+  // 1..31 bits and |accumulator + addend| < 2^30, which |addend| < 2^29 and a depth of at most
+  // 32768 guarantee; one channel outside that sends the whole workgroup down the general form.
+  const bool general_requantize =
+      __syncthreads_or(EPI == Int8Epilogue::kRequantize &&
+                       (!plain_channel || K > 32768 || a.act_min > a.act_max));
   i32x4 fa[kBatchTiles][kSub];
 #pragma unroll
   for (int j = 0; j < kBatchTiles; ++j) {
 #pragma unroll
-    for (int h = 0; h < kSub; ++h) fa[j][h] = read_frag(0, j, h);
+    for (int h = 0; h < kSub; ++h) fa[j][h] = read_frag(C0{}, j, h);
   }
 
+  // One depth step s (slot = s % 2). MFMA number m works on sub-step h = m / kHalf, channel tile
+  // i = (m % kHalf) / kBatchTiles, batch tile j = m % kBatchTiles; what follows it:
+  //   * after the first MFMA that frees an operand of the rows: the barrier that publishes the
+  //     rows of step s + 1 (staged at the end of step s - 1);
+  //   * after the last use of fa[j][h] (i = last tile): its LDS read for step s + 1;
+  //   * after the last use of weight piece (i, h) (j = last batch tile): its load for step s + 2;
+  //   * spread over the step: the loads of the rows of step s + 3;
+  //   * after the last MFMAs: the LDS writes of the rows of step s + 2, into the buffer whose
+  //     readers all passed this step's barrier.
+  // The scheduling fences keep exactly this order. Vector memory returns in issue order, which
+  // the waits the compiler derives from the registers respect.
+  constexpr int kHalf = kBatchTiles * kWaveTiles;
+  constexpr int kMfmas = kSub * kHalf;
+  constexpr int kFirstFree = (kWaveTiles - 1) * kBatchTiles;
   auto step_body = [&](int s, auto slot) {
     constexpr int kSlot = decltype(slot)::value;
-    constexpr int kNext = (kSlot + kRing - 1) % kRing;
-    const int next_stage = (s + 1) & 1;
-    constexpr int kXSet = (kSlot + 1) % 2;  // set of step s + 1, and then of step s + 3
-    store_x(next_stage, std::integral_constant<int, kXSet>{});  // rows requested two steps ago
-    // Vector memory returns in issue order and the next step's store_x waits for these rows,
-    // so they must be requested before the weights; the fences pin that order.
-    asm volatile("" ::: "memory");
-    load_x(s + 3, std::integral_constant<int, kXSet>{});
-    asm volatile("" ::: "memory");
-    load_w(s + kRing - 1, std::integral_constant<int, kNext>{});
-    asm volatile("" ::: "memory");
-    // The scheduling fences keep the instruction order written here: each group of LDS reads
-    // is followed by eight MFMAs that do not depend on it, which hides the read latency; left
-    // alone, the compiler moves every read next to its first use.
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < kBatchTiles; ++j) {
-#pragma unroll
-      for (int i = 0; i < kWaveTiles; ++i) {
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wring[kSlot][i][0], fa[j][0], acc[i][j], 0, 0, 0);
+    using Slot = std::integral_constant<int, kSlot>;
+    using Other = std::integral_constant<int, 1 - kSlot>;
+    ForEachConst(std::make_integer_sequence<int, kMfmas>{}, [&](auto index) {
+      constexpr int m = decltype(index)::value;
+      constexpr int h = m / kHalf, i = (m % kHalf) / kBatchTiles, j = m % kBatchTiles;
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wring[kSlot][i][h], fa[j][h], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (m == kFirstFree) {
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
       }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();  // step s + 1 is staged; the other buffer is free for step s + 2
-#pragma unroll
-    for (int j = 0; j < kBatchTiles; ++j) fa[j][0] = read_frag(next_stage, j, 0);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < kBatchTiles; ++j) {
-#pragma unroll
-      for (int i = 0; i < kWaveTiles; ++i) {
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wring[kSlot][i][1], fa[j][1], acc[i][j], 0, 0, 0);
+      if constexpr (i == kWaveTiles - 1) {
+        fa[j][h] = read_frag(Other{}, j, h);
+        __builtin_amdgcn_sched_barrier(0);
       }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < kBatchTiles; ++j) fa[j][1] = read_frag(next_stage, j, 1);
-    __builtin_amdgcn_sched_barrier(0);
+      if constexpr (j == kBatchTiles - 1) {
+        load_w_piece(s + 2, Slot{}, std::integral_constant<int, i>{}, std::integral_constant<int, h>{});
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (m % (kMfmas / kXChunks) == 1) {
+        load_x_piece(s + 3, Other{}, std::integral_constant<int, m / (kMfmas / kXChunks)>{});
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (m >= kMfmas - kXChunks) {
+        store_x_piece(s + 2, Slot{}, std::integral_constant<int, m - (kMfmas - kXChunks)>{});
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
   };
 
-  // Whole groups of kRing steps run without branches so that the ring slots stay fixed
-  // registers; the remainder repeats the first slots.
+  // Pairs of steps run without branches so that the two slots stay fixed registers.
   int s0 = 0;
-  for (; s0 + kRing <= slabs; s0 += kRing) {
-    ForEachConst(std::make_integer_sequence<int, kRing>{}, [&](auto u) { step_body(s0 + u, u); });
+  for (; s0 + 2 <= steps; s0 += 2) {
+    step_body(s0, C0{});
+    step_body(s0 + 1, C1{});
   }
-  ForEachConst(std::make_integer_sequence<int, kRing - 1>{}, [&](auto u) {
-    if (s0 + u < slabs) step_body(s0 + u, u);
-  });
+  if (s0 < steps) step_body(s0, C0{});
 
   // Epilogue. Register e of acc[i][j] holds channel 32 i + 8 * (e / 4) + 4 * (L / 32) + e % 4 of
   // the wavefront's 64 and batch row 32 j + L % 32 of the workgroup's 128: four groups (g) of
   // four consecutive channels per lane and tile.
   const int row_in_tile = lane & 31;
   const bool vec_ok = (N & 3) == 0;
+  // The clamp bounds in vector registers: v_med3_i32 takes at most one scalar operand.
+  int32_t act_lo = a.act_min, act_hi = a.act_max;
+  asm volatile("" : "+v"(act_lo), "+v"(act_hi));
   // Interior tiles (the common case) store whole dwords without any bounds test.
-  auto epilogue = [&](auto full_tag) {
+  auto epilogue = [&](auto full_tag, auto short_tag) {
   constexpr bool kFull = decltype(full_tag)::value;
+  constexpr bool kShort = decltype(short_tag)::value;
 #pragma unroll
   for (int i = 0; i < kWaveTiles; ++i) {
 #pragma unroll
@@ -265,13 +292,14 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
       const int c0 = n0 + (wave * kWaveTiles + i) * 32 + 8 * g + 4 * (lane >> 5);
       const int local = (wave * kWaveTiles + i) * 32 + 8 * g + 4 * (lane >> 5);
       if (EPI == Int8Epilogue::kRequantize) {
-        int32_t mult[4], shift[4], addend[4];
+        int32_t mult[4], shift[4], addend[4], half[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const i32x4 p = chan_params[local + r];
           mult[r] = p[0];
-          shift[r] = p[1];
+          shift[r] = kShort ? -p[1] : p[1];
           addend[r] = p[2];
+          half[r] = p[3];
         }
 #pragma unroll
         for (int j = 0; j < kBatchTiles; ++j) {
@@ -279,15 +307,15 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
           int32_t q[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            q[r] = RequantizeCore(acc[i][j][4 * g + r] + addend[r], mult[r], shift[r],
-                                  a.output_offset, a.act_min, a.act_max);
+            q[r] = kShort ? RequantizeShort(acc[i][j][4 * g + r] + addend[r], mult[r], shift[r],
+                                            half[r], a.output_offset, act_lo, act_hi)
+                          : RequantizeCore(acc[i][j][4 * g + r] + addend[r], mult[r], shift[r],
+                                           a.output_offset, a.act_min, a.act_max);
           }
           if (kFull || m < M) {
             int8_t* dst = a.output_i8 + static_cast<size_t>(m) * N + c0;
             if (kFull || (vec_ok && c0 + 3 < N)) {
-              *reinterpret_cast<int32_t*>(dst) =
-                  (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) |
-                  static_cast<int32_t>(static_cast<uint32_t>(q[3]) << 24);
+              *reinterpret_cast<int32_t*>(dst) = PackLowBytes(q[0], q[1], q[2], q[3]);
             } else {
 #pragma unroll
               for (int r = 0; r < 4; ++r) {
@@ -337,10 +365,17 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
     }
   }
   };
-  if (vec_ok && m0 + BM <= M && n0 + BN <= N) {
-    epilogue(std::true_type{});
+  const bool interior = vec_ok && m0 + BM <= M && n0 + BN <= N;
+  if (EPI == Int8Epilogue::kRequantize && !general_requantize) {
+    if (interior) {
+      epilogue(std::true_type{}, std::true_type{});
+    } else {
+      epilogue(std::false_type{}, std::true_type{});
+    }
+  } else if (interior) {
+    epilogue(std::true_type{}, std::false_type{});
   } else {
-    epilogue(std::false_type{});
+    epilogue(std::false_type{}, std::false_type{});
   }
 }
 

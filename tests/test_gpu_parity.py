@@ -165,6 +165,48 @@ def test_int8_packed_gemm_ragged_shapes_bit_exact(fc, B, K, N, activation):
     assert np.array_equal(y, want)
 
 
+@pytest.mark.parametrize("B,K,N", [(130, 272, 300), (1030, 48, 4100)])
+@pytest.mark.parametrize("case", ["zero_shift", "left_shift", "big_bias", "shift_31", "mixed"])
+def test_int8_packed_gemm_requantization_forms_bit_exact(fc, B, K, N, case):
+    """The GEMM epilogue has a short form of MultiplyByQuantizedMultiplier for tiles whose
+    channels all shift right by 1..31 bits with a small addend, and the general form for the
+    rest. Raw multipliers and shifts put single channels, or all of them, outside the short
+    form: a shift of zero, left shifts, a bias beyond 2^29, the multiplier INT32_MIN; the
+    tiles next to such a channel stay on the short form."""
+    c = wl.int8_fc(B, K, N, in_zp=-3, seed=900 + B + len(case))
+    rng = np.random.default_rng(len(case) + N)
+    mult = rng.integers(1 << 30, (1 << 31) - 1, N, dtype=np.int64).astype(np.int32)
+    shift = rng.integers(-13, -9, N).astype(np.int32)
+    bias = c["bias"].copy()
+    if case == "zero_shift":
+        shift[N // 2] = 0
+        mult[N // 2] = 1 << 20
+    elif case == "left_shift":
+        shift[:] = rng.integers(1, 4, N)
+        mult[:] = rng.integers(1 << 18, 1 << 21, N)
+    elif case == "big_bias":
+        bias[5] = (1 << 30) + 12345
+        bias[N - 1] = -(1 << 30) - 777
+        shift[5] = shift[N - 1] = -24
+    elif case == "shift_31":
+        shift[:] = rng.integers(-31, -27, N)
+        bias[:] = rng.integers(-(1 << 29) + 1, 1 << 29, N)
+    else:
+        shift[::97] = 0
+        mult[::97] = 1 << 20
+        shift[3::131] = 2
+        mult[3::131] = 1 << 18
+        mult[7] = np.iinfo(np.int32).min
+    op = fc.FullyConnectedInt8(c["w"], bias, float(c["in_scale"]), c["in_zp"], c["w_scale"],
+                               float(c["out_scale"]), c["out_zp"])
+    op.multipliers, op.shifts = _cuda(mult), _cuda(shift)
+    y = op(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_int8_per_channel(c["x"], c["w"], bias, mult, shift, -c["in_zp"], c["out_zp"],
+                                      -128, 127)
+    assert np.array_equal(y, want)
+    assert len(np.unique(y)) > 3
+
+
 @pytest.mark.parametrize("B,K,N", [(33, 64, 20), (128, 256, 256), (130, 272, 48), (65, 1040, 301),
                                    (1025, 96, 4096)])
 @pytest.mark.parametrize("asym", [True, False])
