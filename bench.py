@@ -287,6 +287,32 @@ def main():
     print(json.dumps(line))
 
 
+def mfma_rate(torch, seconds, random_operands):
+    """Sustained rate (TOPS) of the matrix cores alone on this part: lrtfc_mfma_rate_probe (256
+    workgroups x 4 wavefronts, register operands, no memory traffic) launched back to back for
+    about `seconds`, wall-clock timed around device synchronisations."""
+    import ctypes
+    from litert_amd import capi
+    lib = capi.load()
+    sink = torch.empty(256 * 256, dtype=torch.int32, device="cuda")
+    ops = ctypes.c_double(0.0)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch(n):
+        for _ in range(n):
+            capi.check(lib.lrtfc_mfma_rate_probe(256, 2000, int(random_operands), sink.data_ptr(),
+                                                 ctypes.byref(ops), stream))
+        torch.cuda.synchronize()
+
+    launch(2)
+    t0 = time.time()
+    launches = 0
+    while time.time() - t0 < seconds:
+        launch(20)   # 20 launches of about 0.8 ms
+        launches += 20
+    return ops.value * launches / (time.time() - t0) / 1e12
+
+
 def traffic_probe(torch, fc, wl):
     """The launches a counter run needs and nothing else: the fused hybrid kernel at B = 1
     on rotating weight copies (so every launch streams its filter from HBM) and a plain
@@ -330,6 +356,13 @@ def gemm_probe(torch, fc, wl, sustain=0.0):
         sets.append((name, op, x))
     print(json.dumps({"probe": "gemm", "launches_seeded": 10, "launches_constant": 10,
                       "ops_per_launch": 2 * 2048 * 4096 * 4096}), flush=True)
+    if sustain > 0:
+        for name, rnd in (("random", 1), ("constant", 0)):
+            t0 = time.time()
+            print(json.dumps({"sustain": "mfma_only_" + name, "begin_unix": round(t0, 3)}), flush=True)
+            tops = mfma_rate(torch, sustain, rnd)
+            print(json.dumps({"sustain": "mfma_only_" + name, "end_unix": round(time.time(), 3),
+                              "tops": round(tops, 1)}), flush=True)
     for name, op, x in sets if sustain > 0 else []:
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
@@ -535,7 +568,10 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
     ops4 = {act: fc.FullyConnectedInt8(c4["w"], c4["bias"], float(c4["in_scale"]), c4["in_zp"],
                                        c4["w_scale"], float(c4["out_scale"]), c4["out_zp"],
                                        activation=act) for act in ("none", "relu6")}
-    graphs4 = {act: many([(lambda o: lambda: o(x4, out=y4))(op)] * 4) for act, op in ops4.items()}
+    # 64 launches per replay (about 2.5 ms): long enough that the clock ramp after the idle gap
+    # between two replays does not colour the figure.
+    graphs4 = {act: (capture((lambda o: lambda: [o(x4, out=y4) for _ in range(64)])(op)), 64)
+               for act, op in ops4.items()}
     samples4 = {act: [] for act in ops4}
     for g, _ in graphs4.values():
         g.replay()
@@ -564,11 +600,21 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
     op4c = fc.FullyConnectedInt8(np.full_like(c4["w"], 5), c4["bias"], float(c4["in_scale"]),
                                  c4["in_zp"], c4["w_scale"], float(c4["out_scale"]), c4["out_zp"])
     x4c = torch.full_like(x4, 3)
-    us_c = per_launch_us([lambda: op4c(x4c, out=y4)] * 4)
+    us_c = per_launch_us([lambda: op4c(x4c, out=y4)] * 16)
     out["config4_int8_gemm_constant_operands"] = dict(
         us=round(us_c, 2), tops=round(ops_per_call / us_c / 1e6, 1),
         frac_of_int8_mfma_peak=round(ops_per_call / us_c / 1e6 / INT8_MFMA_PEAK_TOPS, 4),
         note="same kernel and launch, x = 3 and w = 5 everywhere: lower switching activity, higher sustained clock")
+    # The matrix cores alone (no operand traffic, one wavefront per SIMD as in the GEMM), 0.4 s
+    # each: what this part sustains under its power limit, against the nominal 5.0 POPS.
+    probe_random, probe_constant = mfma_rate(torch, 0.4, 1), mfma_rate(torch, 0.4, 0)
+    out["config4_matrix_cores_alone"] = dict(
+        tops_random_operands=round(probe_random, 1), tops_constant_operands=round(probe_constant, 1),
+        us_for_config4_random=round(ops_per_call / probe_random / 1e6, 2),
+        us_for_config4_constant=round(ops_per_call / probe_constant / 1e6, 2),
+        note="lrtfc_mfma_rate_probe: v_mfma_i32_32x32x32_i8 back to back on register operands, "
+             "256 workgroups x 4 wavefronts, sustained; the clock the part holds under this load "
+             "sets the figure, and the GEMM's operand traffic draws on the same power budget")
     # Yardstick (not this library): the vendor int8 GEMM through torch._int_mm on the same
     # operands, int32 output, no requantization.
     try:

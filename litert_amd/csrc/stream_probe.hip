@@ -1,12 +1,58 @@
-// Measurement aid, not part of the op: a kernel that only streams `bytes` bytes out of device
+// Measurement aids, not part of the op. First: a kernel that only streams `bytes` bytes out of device
 // memory, with the access pattern of the decode kernels (every wavefront walks its own
 // contiguous 32 KiB run through a ring of sixteen outstanding non-temporal 1 KiB loads) and
 // nothing else to do. Timed beside a GEMV on the same bytes it tells how much of that kernel's
 // time is the memory system's and how much is the kernel's own (prologue, epilogue, tail).
+//
+// Second: a kernel that only issues v_mfma_i32_32x32x32_i8 on register operands, one wavefront
+// per SIMD as in the prefill GEMM, eight independent accumulators so that the instructions go
+// back to back. Launched for a few hundred milliseconds it shows the int8 rate this part's
+// matrix cores sustain under its power limit, for operands that toggle like random data and
+// for constant ones: the ceiling of the GEMM's main loop, with no operand traffic at all.
 #include "kernels.h"
 
 namespace lrtfc {
 namespace {
+
+using i32x16 = int __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ uint32_t MixBits(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7feb352dU;
+  x ^= x >> 15;
+  x *= 0x846ca68bU;
+  x ^= x >> 16;
+  return x;
+}
+
+constexpr int kProbeAccumulators = 8;
+
+__global__ __launch_bounds__(256) void MfmaRateKernel(int iterations, int random_operands,
+                                                      int32_t* sink) {
+  const uint32_t id = blockIdx.x * 256 + threadIdx.x;
+  i32x4 a[4], b[4];
+  for (int i = 0; i < 4; ++i) {
+    for (int e = 0; e < 4; ++e) {
+      a[i][e] = random_operands ? static_cast<int>(MixBits(id * 64 + i * 8 + e)) : 0x05050505;
+      b[i][e] = random_operands ? static_cast<int>(MixBits(id * 64 + i * 8 + e + 4)) : 0x03030303;
+    }
+  }
+  i32x16 acc[kProbeAccumulators];
+  for (int i = 0; i < kProbeAccumulators; ++i) {
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0;
+  }
+  for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+    for (int i = 0; i < kProbeAccumulators; ++i) {
+      acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[(i + (i >> 2)) & 3], acc[i], 0, 0, 0);
+    }
+  }
+  int32_t r = 0;
+  for (int i = 0; i < kProbeAccumulators; ++i) {
+    for (int e = 0; e < 16; ++e) r ^= acc[i][e];
+  }
+  sink[id] = r;
+}
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWaveSize;
@@ -55,6 +101,18 @@ hipError_t LaunchStreamRead(const void* src, size_t bytes, int32_t* sink, hipStr
   hipLaunchKernelGGL(StreamReadKernel, dim3(grid), dim3(kThreads), 0, stream,
                      static_cast<const i32x4*>(src), vecs, sink);
   return hipGetLastError();
+}
+
+
+hipError_t LaunchMfmaRate(int workgroups, int iterations, int random_operands, int32_t* sink,
+                          hipStream_t stream) {
+  hipLaunchKernelGGL(MfmaRateKernel, dim3(workgroups), dim3(256), 0, stream, iterations,
+                     random_operands, sink);
+  return hipGetLastError();
+}
+
+double MfmaRateOpsPerLaunch(int workgroups, int iterations) {
+  return 65536.0 * kProbeAccumulators * iterations * 4.0 * workgroups;
 }
 
 }  // namespace lrtfc
