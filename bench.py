@@ -739,20 +739,26 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         out["config5_gemma2b_fc_chain_B%d" % b] = res
     for b in (1, 4):
         out["config5_through_delegate_B%d" % b] = delegate_chain(torch, wl, b)
+        out["config5_through_delegate_device_bound_B%d" % b] = delegate_chain(torch, wl, b, bound=True)
     return out
 
 
-def delegate_chain(torch, wl, b=1, invokes=20):
+def delegate_chain(torch, wl, b=1, invokes=20, bound=False):
     """Config 5 end to end through the delegate plugin, driven by the stand-in interpreter
-    (litert_amd/standin_host): 126 FULLY_CONNECTED nodes, host tensors in, host tensors out. Wall-clock time of
-    Invoke(), i.e. including the upload of every node's input, the download of every node's
-    output (all 126 are graph outputs here) and the final synchronization."""
+    (litert_amd/standin_host): 126 FULLY_CONNECTED nodes in one partition. Wall-clock time of
+    Invoke(), final synchronization included. With host tensors in and out (bound=False) that
+    includes the upload of every node's input and the download of every node's output (all 126
+    are graph outputs here); with bound=True every input and output is bound to registered
+    device memory through a buffer handle (litert_amd_register_device_buffer +
+    Interpreter::SetBufferHandle), as an application that keeps its activations in HBM does."""
     from litert_amd.standin_host import FakeHost, FLOAT32, FLOAT16, INT4, OK
     rng = np.random.default_rng(5)
     with FakeHost() as h:
+        io = []
         for layer in range(wl.GEMMA2B_LAYERS):
             for name, k, n in wl.GEMMA2B_LAYER_FCS:
-                x = h.tensor(FLOAT32, (b, k), data=rng.standard_normal((b, k)).astype(np.float32))
+                x_np = rng.standard_normal((b, k)).astype(np.float32)
+                x = h.tensor(FLOAT32, (b, k), data=x_np)
                 w = h.tensor(INT4, (n, k), const=True,
                              data=rng.integers(0, 256, (n, k // 2), dtype=np.uint8))
                 s_ = h.tensor(FLOAT16, (n, k // 32), const=True,
@@ -760,8 +766,20 @@ def delegate_chain(torch, wl, b=1, invokes=20):
                 h.blockwise(w, s_, 32)
                 y = h.tensor(FLOAT32, (b, n))
                 h.fc(x, w, None, y)
+                io.append((x, x_np, y, n))
         if h.load_delegate() != 0 or h.modify_graph_with_delegate() != OK or h.allocate_tensors() != OK:
             raise RuntimeError(h.errors())
+        keep = []
+        if bound:
+            for x, x_np, y, n in io:
+                xd = torch.from_numpy(x_np).cuda()
+                yd = torch.empty((b, n), dtype=torch.float32, device="cuda")
+                keep += [xd, yd]
+                for tensor, dev in ((x, xd), (y, yd)):
+                    handle = h.register_device_buffer(dev.data_ptr(), dev.numel() * 4)
+                    if handle < 0 or h.set_buffer_handle(tensor, handle) != OK:
+                        raise RuntimeError("binding a device buffer failed: " + h.errors())
+                h.set_data_is_stale(x)
         plan = h.plan()
         groups, _ = h.describe_partition(plan[0][2])
         for _ in range(3):
@@ -771,9 +789,11 @@ def delegate_chain(torch, wl, b=1, invokes=20):
         for _ in range(invokes):
             h.invoke()
         us = (time.perf_counter() - t0) / invokes * 1e6
+    note = ("every input and output bound to registered device memory (buffer handles): no copies, "
+            "the kernels work on the bound memory" if bound else
+            "host tensors in and out: 126 uploads + 126 downloads per invoke included")
     return {"invoke_wall_us": round(us, 1), "partitions": len(plan), "grouped_launches": groups,
-            "fc_nodes": wl.GEMMA2B_LAYERS * len(wl.GEMMA2B_LAYER_FCS),
-            "note": "host tensors in and out: 126 uploads + 126 downloads per invoke included"}
+            "fc_nodes": wl.GEMMA2B_LAYERS * len(wl.GEMMA2B_LAYER_FCS), "note": note}
 
 
 def cpu_baseline_leg(c):

@@ -511,7 +511,15 @@ struct PartitionKernel {
   std::map<int, size_t> arena_offset;  // tensor index -> byte offset in the arena
   size_t upload_bytes = 0, download_offset = 0, download_bytes = 0;
   PinnedBuffer upload_stage, download_stage;
+  // A boundary tensor (uploaded or downloaded) that carries a buffer handle of this delegate
+  // lives in the registered memory itself for as long as the binding lasts: the kernels read and
+  // write it there. `bindings` is the device address each boundary tensor had at the last
+  // invoke (uploads, then downloads; nullptr = not bound or not usable in place).
+  std::map<int, void*> alias;
+  std::vector<void*> bindings;
   void* Activation(int tensor) const {
+    auto bound = alias.find(tensor);
+    if (bound != alias.end()) return bound->second;
     auto it = arena_offset.find(tensor);
     return it == arena_offset.end() ? nullptr : arena.as<uint8_t>() + it->second;
   }
@@ -1016,6 +1024,8 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
   return kTfLiteOk;
 }
 
+TfLiteStatus BuildGroupTables(TfLiteContext* ctx, PartitionKernel* k);
+
 // After every node is prepared (shapes and kernel forms known): which nodes share a launch,
 // which stream each unit runs on, which nodes other streams wait for.
 TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
@@ -1151,7 +1161,14 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
                              lrtfc_activation_workspace_bytes(n.batches, n.depth)));
     }
   }
-  // Group tables: device addresses of every member's tensors (stable until the next prepare).
+  k->alias.clear();
+  k->bindings.clear();
+  return BuildGroupTables(ctx, k);
+}
+
+// Group tables: device addresses of every member's tensors (stable until the next prepare or
+// until a boundary tensor is bound to other memory).
+TfLiteStatus BuildGroupTables(TfLiteContext* ctx, PartitionKernel* k) {
   for (PartitionKernel::Group& g : k->groups) {
     std::vector<lrtfc_int4_group_node> nodes(g.members.size());
     const FcNode& head = k->nodes[g.members.front()];
@@ -1191,6 +1208,68 @@ TfLiteStatus KernelPrepare(TfLiteContext* ctx, TfLiteNode* node) {
   return kTfLiteOk;
 }
 
+// Which registered memory each boundary tensor is bound to now; on a change, the tensors are
+// re-pointed and the address tables of the grouped launches rebuilt (nothing of this partition
+// is in flight between two invokes). An output bound to memory that overlaps a bound input
+// would be written while that input is still being read, so such a binding fails the invoke.
+TfLiteStatus RefreshBindings(TfLiteContext* ctx, PartitionKernel* k) {
+  std::vector<void*> now;
+  now.reserve(k->uploads.size() + k->downloads.size());
+  auto bound_address = [&](int t, void** address) {
+    const TfLiteTensor& tensor = ctx->tensors[t];
+    const RegisteredBuffer* bound = tensor.bytes ? BoundBuffer(k->state, tensor) : nullptr;
+    *address = nullptr;
+    if (!bound) return kTfLiteOk;
+    if (bound->bytes < tensor.bytes) {
+      ctx->ReportError(ctx, "litert_amd delegate: buffer handle %d holds %zu bytes, tensor %d needs %zu",
+                       tensor.buffer_handle, bound->bytes, t, tensor.bytes);
+      return kTfLiteError;
+    }
+    if (reinterpret_cast<uintptr_t>(bound->device) % 16 != 0) {
+      ctx->ReportError(ctx, "litert_amd delegate: the memory behind buffer handle %d is not 16-byte aligned",
+                       tensor.buffer_handle);
+      return kTfLiteError;
+    }
+    *address = bound->device;
+    return kTfLiteOk;
+  };
+  for (int t : k->uploads) {
+    void* address = nullptr;
+    RETURN_IF_OK(bound_address(t, &address));
+    now.push_back(address);
+  }
+  for (int t : k->downloads) {
+    void* address = nullptr;
+    RETURN_IF_OK(bound_address(t, &address));
+    now.push_back(address);
+  }
+  if (now == k->bindings) return kTfLiteOk;
+  const size_t inputs = k->uploads.size();
+  for (size_t o = inputs; o < now.size(); ++o) {
+    if (!now[o]) continue;
+    const auto* out_begin = static_cast<const uint8_t*>(now[o]);
+    const auto* out_end = out_begin + ctx->tensors[k->downloads[o - inputs]].bytes;
+    for (size_t i = 0; i < inputs; ++i) {
+      if (!now[i]) continue;
+      const auto* in_begin = static_cast<const uint8_t*>(now[i]);
+      const auto* in_end = in_begin + ctx->tensors[k->uploads[i]].bytes;
+      if (out_begin < in_end && in_begin < out_end) {
+        ctx->ReportError(ctx, "litert_amd delegate: output tensor %d and input tensor %d are bound to overlapping device memory",
+                         k->downloads[o - inputs], k->uploads[i]);
+        return kTfLiteError;
+      }
+    }
+  }
+  k->alias.clear();
+  for (size_t i = 0; i < now.size(); ++i) {
+    if (now[i]) k->alias[i < inputs ? k->uploads[i] : k->downloads[i - inputs]] = now[i];
+  }
+  k->bindings = std::move(now);
+  RETURN_IF_OK(BuildGroupTables(ctx, k));
+  RETURN_IF_HIP(ctx, hipStreamSynchronize(k->stream));
+  return kTfLiteOk;
+}
+
 TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   auto* k = static_cast<PartitionKernel*>(node->user_data);
   RETURN_IF_HIP(ctx, hipSetDevice(k->state->options.device));
@@ -1205,30 +1284,21 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     RETURN_IF_HIP(ctx, hipEventRecord(k->metrics_begin, k->stream));
   }
   // Tensor data pointers may move between invokes: read them from the context each time.
-  // An input that carries a buffer handle of this delegate is already in device memory: it is
-  // copied device to device behind the (single) host upload of the others.
+  // A boundary tensor that carries a buffer handle of this delegate is already in device memory
+  // (an input) or is to stay there (an output): the kernels work on the registered memory
+  // itself. The bindings are compared with those of the last invoke; a change re-points the
+  // tensors and rebuilds the grouped launches' address tables.
+  RETURN_IF_OK(RefreshBindings(ctx, k));
   bool host_inputs = false;
   for (int t : k->uploads) {
     const TfLiteTensor& tensor = ctx->tensors[t];
-    if (tensor.bytes == 0 || BoundBuffer(k->state, tensor)) continue;
+    if (tensor.bytes == 0 || k->alias.count(t)) continue;
     std::memcpy(k->upload_stage.get() + k->arena_offset[t], tensor.data.raw, tensor.bytes);
     host_inputs = true;
   }
   if (host_inputs) {
     RETURN_IF_HIP(ctx, hipMemcpyAsync(k->arena.get(), k->upload_stage.get(), k->upload_bytes,
                                       hipMemcpyHostToDevice, k->stream));
-  }
-  for (int t : k->uploads) {
-    const TfLiteTensor& tensor = ctx->tensors[t];
-    const RegisteredBuffer* bound = tensor.bytes ? BoundBuffer(k->state, tensor) : nullptr;
-    if (!bound) continue;
-    if (bound->bytes < tensor.bytes) {
-      ctx->ReportError(ctx, "litert_amd delegate: buffer handle %d holds %zu bytes, tensor %d needs %zu",
-                       tensor.buffer_handle, bound->bytes, t, tensor.bytes);
-      return kTfLiteError;
-    }
-    RETURN_IF_HIP(ctx, hipMemcpyAsync(k->arena.as<uint8_t>() + k->arena_offset[t], bound->device,
-                                      tensor.bytes, hipMemcpyDeviceToDevice, k->stream));
   }
   bool multi = false;
   for (int i = 1; i < k->num_streams; ++i) multi = multi || k->lane_used[i];
@@ -1416,26 +1486,18 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     RETURN_IF_HIP(ctx, hipEventRecord(k->lane_done[i], k->streams[i]));
     RETURN_IF_HIP(ctx, hipStreamWaitEvent(s, k->lane_done[i], 0));
   }
-  // An output that carries a buffer handle of this delegate stays in device memory: it goes
-  // to the registered buffer and the host copy is marked stale (the runtime fetches it
-  // through CopyFromBufferHandle if a CPU node or the application asks: subgraph.cc:876-889).
+  // An output that carries a buffer handle of this delegate stays in device memory, where the
+  // kernels have written it, and the host copy is marked stale (the runtime fetches it through
+  // CopyFromBufferHandle if a CPU node or the application asks: subgraph.cc:876-889).
   bool host_outputs = false;
   for (int t : k->downloads) {
     TfLiteTensor& tensor = ctx->tensors[t];
     if (tensor.bytes == 0) continue;
-    const RegisteredBuffer* bound = BoundBuffer(k->state, tensor);
-    if (!bound) {
+    if (k->alias.count(t)) {
+      tensor.data_is_stale = true;
+    } else {
       host_outputs = true;
-      continue;
     }
-    if (bound->bytes < tensor.bytes) {
-      ctx->ReportError(ctx, "litert_amd delegate: buffer handle %d holds %zu bytes, tensor %d needs %zu",
-                       tensor.buffer_handle, bound->bytes, t, tensor.bytes);
-      return kTfLiteError;
-    }
-    RETURN_IF_HIP(ctx, hipMemcpyAsync(bound->device, k->arena.as<uint8_t>() + k->arena_offset[t],
-                                      tensor.bytes, hipMemcpyDeviceToDevice, s));
-    tensor.data_is_stale = true;
   }
   if (host_outputs) {
     RETURN_IF_HIP(ctx, hipMemcpyAsync(k->download_stage.get(),
@@ -1469,7 +1531,7 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   }
   for (int t : k->downloads) {
     TfLiteTensor& tensor = ctx->tensors[t];
-    if (tensor.bytes == 0 || BoundBuffer(k->state, tensor)) continue;
+    if (tensor.bytes == 0 || k->alias.count(t)) continue;
     std::memcpy(tensor.data.raw,
                 k->download_stage.get() + (k->arena_offset[t] - k->download_offset), tensor.bytes);
   }

@@ -145,3 +145,78 @@ def test_handles_are_freed_and_slots_reused():
         assert h.set_buffer_handle(y, 0) == OK
         assert h.invoke() != OK and "holds 8 bytes" in h.errors()
         assert h.register_device_buffer(None, 16) == -1
+
+
+def _int4_nodes(h, rng, shapes, b):
+    nodes = []
+    for k, n in shapes:
+        x_np = rng.standard_normal((b, k)).astype(np.float32)
+        packed = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+        scales = rng.uniform(5e-3, 2e-2, (n, k // 32)).astype(np.float16)
+        x = h.tensor(FLOAT32, (b, k), data=x_np)
+        w = h.tensor(INT4, (n, k), const=True, data=packed)
+        s = h.tensor(FLOAT16, (n, k // 32), const=True, data=scales)
+        h.blockwise(w, s, 32)
+        y = h.tensor(FLOAT32, (b, n))
+        h.fc(x, w, None, y)
+        nodes.append((x, y, x_np, packed, scales, n))
+    return nodes
+
+
+@pytest.mark.parametrize("b", [1, 4])
+def test_grouped_launch_works_in_place_on_bound_tensors_and_follows_rebinding(b):
+    """A partition of independent blockwise-int4 nodes runs as one grouped launch whose address
+    table names each member's tensors. Bound tensors are used where they are (no copy into the
+    partition's own memory): the table must name the registered memory, and name the new
+    memory after a tensor is bound to another buffer between two invokes."""
+    rng = np.random.default_rng(40 + b)
+    with FakeHost() as h:
+        nodes = _int4_nodes(h, rng, [(2048, 256), (2048, 512), (2048, 64)], b)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        plan = h.plan()
+        assert len(plan) == 1 and h.describe_partition(plan[0][2])[0] >= 1
+        want = [oracle.fc_blockwise_int4(x_np, packed, n, scales.view(np.uint16), 32)
+                for _, _, x_np, packed, scales, n in nodes]
+        x_dev = [torch.from_numpy(x_np).cuda() for _, _, x_np, _, _, _ in nodes]
+        y_dev = [torch.full((b, n), float("nan"), dtype=torch.float32, device="cuda")
+                 for *_, n in nodes]
+        for (x, y, *_), xd, yd in zip(nodes, x_dev, y_dev):
+            assert h.set_buffer_handle(x, h.register_device_buffer(xd.data_ptr(), xd.numel() * 4)) == OK
+            h.set_data_is_stale(x)
+            h.write(x, np.zeros_like(xd.cpu().numpy()))      # the host copy is not the input
+            assert h.set_buffer_handle(y, h.register_device_buffer(yd.data_ptr(), yd.numel() * 4)) == OK
+        assert h.invoke() == OK, h.errors()
+        for (x, y, *_), yd, w in zip(nodes, y_dev, want):
+            assert h.data_is_stale(y)
+            assert np.array_equal(_bits(yd.cpu().numpy()), _bits(w))
+        # the second node's output moves to other memory, its input too
+        y_new = torch.full_like(y_dev[1], float("nan"))
+        x_new_np = rng.standard_normal(x_dev[1].shape).astype(np.float32)
+        x_new = torch.from_numpy(x_new_np).cuda()
+        y_dev[1].fill_(float("nan"))
+        assert h.set_buffer_handle(nodes[1][1], h.register_device_buffer(y_new.data_ptr(), y_new.numel() * 4)) == OK
+        assert h.set_buffer_handle(nodes[1][0], h.register_device_buffer(x_new.data_ptr(), x_new.numel() * 4)) == OK
+        assert h.invoke() == OK, h.errors()
+        _, _, _, packed, scales, n = nodes[1]
+        assert np.array_equal(_bits(y_new.cpu().numpy()),
+                              _bits(oracle.fc_blockwise_int4(x_new_np, packed, n, scales.view(np.uint16), 32)))
+        assert torch.isnan(y_dev[1]).all()                    # the old memory is no longer written
+        assert np.array_equal(_bits(y_dev[0].cpu().numpy()), _bits(want[0]))
+        assert np.array_equal(_bits(y_dev[2].cpu().numpy()), _bits(want[2]))
+        # host tensors still work beside bound ones: read a stale output back through the runtime
+        assert h.ensure_readable(nodes[0][1]) == OK
+        assert np.array_equal(_bits(h.read(nodes[0][1])), _bits(want[0]))
+
+
+def test_output_bound_over_an_input_is_refused():
+    c = wl.hybrid_fc(2, 64, 64, seed=8)
+    with FakeHost() as h:
+        _, x, y = _hybrid_node(h, c)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        dev = torch.from_numpy(c["x"]).cuda()
+        assert h.set_buffer_handle(x, h.register_device_buffer(dev.data_ptr(), dev.numel() * 4)) == OK
+        h.set_data_is_stale(x)
+        assert h.set_buffer_handle(y, h.register_device_buffer(dev.data_ptr(), dev.numel() * 4)) == OK
+        assert h.invoke() != OK and "overlapping device memory" in h.errors()
