@@ -28,7 +28,9 @@ extern "C" {
  * device) and returns a buffer handle to bind to an input or output tensor with
  * Interpreter::SetBufferHandle (tflite/core/subgraph.h:1043-1057); kTfLiteNullBufferHandle on
  * failure. Counterpart of StatefulNnApiDelegate::RegisterNnapiMemory
- * (tflite/delegates/nnapi/nnapi_delegate.cc:6645-6660). */
+ * (tflite/delegates/nnapi/nnapi_delegate.cc:6645-6660). The kernels work on the registered
+ * memory itself: it must be 16-byte aligned and at least as large as the tensor bound to it, and
+ * an output must not be bound to memory that overlaps a bound input of the same partition. */
 TfLiteBufferHandle litert_amd_register_device_buffer(TfLiteDelegate* delegate,
                                                      void* device_memory, size_t bytes);
 
