@@ -1162,7 +1162,7 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
     }
   }
   k->alias.clear();
-  k->bindings.clear();
+  k->bindings.assign(k->uploads.size() + k->downloads.size(), nullptr);
   return BuildGroupTables(ctx, k);
 }
 
