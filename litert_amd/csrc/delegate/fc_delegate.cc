@@ -501,6 +501,10 @@ constexpr int kInt4PerChannelNibbleMaxBatches = 32;
 // of once per four rows.
 constexpr int kInt4BlockwiseGemmMinBatches = 16;
 
+// Up to this many bytes of host outputs per partition are written by the kernels directly into
+// page-locked host memory instead of being copied there afterwards.
+constexpr size_t kDirectOutputMaxBytes = 16 << 20;
+
 struct PartitionKernel {
   DelegateState* state = nullptr;
   std::vector<FcNode> nodes;
@@ -517,11 +521,22 @@ struct PartitionKernel {
   // invoke (uploads, then downloads; nullptr = not bound or not usable in place).
   std::map<int, void*> alias;
   std::vector<void*> bindings;
+  // Small sets of host outputs are written by the kernels straight into the page-locked
+  // download staging area (device-visible host memory), which saves the copy command behind the
+  // last kernel: direct_outputs, decided at prepare, holds when no node of the partition reads
+  // any of the downloaded tensors back.
+  bool direct_outputs = false;
+  uint8_t* download_stage_device = nullptr;  // the staging area as the device addresses it
   void* Activation(int tensor) const {
     auto bound = alias.find(tensor);
     if (bound != alias.end()) return bound->second;
     auto it = arena_offset.find(tensor);
-    return it == arena_offset.end() ? nullptr : arena.as<uint8_t>() + it->second;
+    if (it == arena_offset.end()) return nullptr;
+    if (direct_outputs && it->second >= download_offset &&
+        it->second < download_offset + download_bytes) {
+      return download_stage_device + (it->second - download_offset);
+    }
+    return arena.as<uint8_t>() + it->second;
   }
   // Three int32 per EMBEDDING_LOOKUP node, in page-locked host memory the lookup kernels write
   // straight into: {0 or 1, first offending position, the index found there}.
@@ -1051,6 +1066,25 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
     RETURN_IF_HIP(ctx, k->arena.Ensure(next));
     RETURN_IF_HIP(ctx, k->upload_stage.Ensure(k->upload_bytes));
     RETURN_IF_HIP(ctx, k->download_stage.Ensure(k->download_bytes));
+    // Outputs straight into host memory: worth it while the copy command's fixed cost matters
+    // more than PCIe write combining (decode-sized outputs), and only for tensors nobody in the
+    // partition reads (a reader would fetch them over PCIe, workgroup by workgroup).
+    k->direct_outputs = false;
+    k->download_stage_device = nullptr;
+    if (k->download_bytes > 0 && k->download_bytes <= kDirectOutputMaxBytes) {
+      bool read_back = false;
+      for (const FcNode& n : k->nodes) {
+        read_back = read_back || std::find(k->downloads.begin(), k->downloads.end(), n.input) !=
+                                     k->downloads.end();
+        read_back = read_back || n.depth == 0;  // such a node's output is cleared with a memset
+      }
+      void* device_view = nullptr;
+      if (!read_back &&
+          hipHostGetDevicePointer(&device_view, k->download_stage.get(), 0) == hipSuccess) {
+        k->direct_outputs = true;
+        k->download_stage_device = static_cast<uint8_t*>(device_view);
+      }
+    }
   }
   // Levels: a node without a producer inside the partition is at level 0, a consumer one
   // above its producer (an FC node has one activation input, so one producer at most).
@@ -1499,7 +1533,7 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
       host_outputs = true;
     }
   }
-  if (host_outputs) {
+  if (host_outputs && !k->direct_outputs) {
     RETURN_IF_HIP(ctx, hipMemcpyAsync(k->download_stage.get(),
                                       k->arena.as<uint8_t>() + k->download_offset,
                                       k->download_bytes, hipMemcpyDeviceToHost, s));

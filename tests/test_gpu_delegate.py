@@ -167,6 +167,37 @@ def test_chain_stays_on_device_and_splits_around_cpu_nodes():
         assert np.array_equal(h.read(y2), w2) and np.array_equal(h.read(y3), w3)
 
 
+def test_link_that_is_also_a_graph_output_is_copied_not_written_to_the_host():
+    """FC -> FC in one partition. Host outputs that no node of the partition reads are written by
+    the kernels straight into page-locked host memory; once the link tensor is a graph output as
+    well, the second node reads a downloaded tensor, so the partition keeps its outputs in device
+    memory and copies them out. Both forms give the oracle's bits, on repeated invokes with new
+    inputs."""
+    c1 = wl.int8_fc(3, 256, 128, seed=11)
+    c2 = wl.int8_fc(3, 128, 64, in_scale=float(c1["out_scale"]), in_zp=c1["out_zp"], seed=12)
+    for link_is_output in (False, True):
+        with FakeHost() as h:
+            n1, x, y1 = _add_int8_fc(h, c1, activation=3)
+            n2, _, y2 = _add_int8_fc(h, c2, x=y1)
+            if link_is_output:
+                h.mark_output(y1)
+            assert h.load_delegate() == 0 and h.modify_graph_with_delegate() == OK, h.errors()
+            plan = h.plan()
+            assert [(k, r) for k, r, _ in plan] == [("delegate", [n1, n2])]
+            _, outs = h.node_io(plan[0][2])
+            assert sorted(outs) == sorted([y1, y2] if link_is_output else [y2])
+            assert h.allocate_tensors() == OK, h.errors()
+            rng = np.random.default_rng(3)
+            for trial in range(3):
+                xin = c1["x"] if trial == 0 else rng.integers(-128, 128, c1["x"].shape).astype(np.int8)
+                h.write(x, xin)
+                assert h.invoke() == OK, h.errors()
+                w1 = _oracle_int8(c1, xin, activation=3)
+                assert np.array_equal(h.read(y2), _oracle_int8(c2, w1))
+                if link_is_output:
+                    assert np.array_equal(h.read(y1), w1)
+
+
 @pytest.mark.parametrize("streams", [1, 2, 4])
 def test_decoder_shaped_partition_on_several_streams(streams):
     """x -> up -> {a, b, c} (three consumers of one tensor, on different streams) plus two
