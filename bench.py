@@ -737,6 +737,7 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         del all_groups, decoder_groups
         res.update(fc_nodes=len(nodes), weight_bytes=chain_bytes)
         out["config5_gemma2b_fc_chain_B%d" % b] = res
+    out["single_node_through_delegate"] = single_node_invokes(wl)
     for b in (1, 4):
         out["config5_through_delegate_B%d" % b] = delegate_chain(torch, wl, b)
         out["config5_through_delegate_device_bound_B%d" % b] = delegate_chain(torch, wl, b, bound=True)
@@ -794,6 +795,65 @@ def delegate_chain(torch, wl, b=1, invokes=20, bound=False):
             "host tensors in and out: 126 uploads + 126 downloads per invoke included")
     return {"invoke_wall_us": round(us, 1), "partitions": len(plan), "grouped_launches": groups,
             "fc_nodes": wl.GEMMA2B_LAYERS * len(wl.GEMMA2B_LAYER_FCS), "note": note}
+
+
+def single_node_invokes(wl, invokes=200):
+    """Configs 1, 2 and 3 as ONE FULLY_CONNECTED node each through the delegate plugin with host
+    tensors in and out, driven by the stand-in interpreter: median wall-clock time of Invoke()
+    (gather into page-locked memory, one host-to-device copy, the kernel -- which writes its
+    output straight into page-locked host memory --, one stream synchronisation, scatter)."""
+    from litert_amd.standin_host import FakeHost, FLOAT32, FLOAT16, INT4, INT8, INT32, OK
+    rng = np.random.default_rng(6)
+
+    def timed(h):
+        if h.load_delegate() != 0 or h.modify_graph_with_delegate() != OK or h.allocate_tensors() != OK:
+            raise RuntimeError(h.errors())
+        if [kind for kind, _, _ in h.plan()] != ["delegate"]:
+            raise RuntimeError("the node was not claimed: " + h.errors())
+        for _ in range(20):
+            if h.invoke() != OK:
+                raise RuntimeError(h.errors())
+        samples = []
+        for _ in range(invokes):
+            t0 = time.perf_counter()
+            h.invoke()
+            samples.append((time.perf_counter() - t0) * 1e6)
+        samples.sort()
+        return round(samples[len(samples) // 2], 1)
+
+    out = {}
+    c1 = wl.int8_fc()
+    with FakeHost() as h:
+        x = h.tensor(INT8, c1["x"].shape, data=c1["x"])
+        h.affine(x, [c1["in_scale"]], [c1["in_zp"]])
+        w = h.tensor(INT8, c1["w"].shape, data=c1["w"], const=True)
+        h.affine(w, c1["w_scale"])
+        b = h.tensor(INT32, (c1["w"].shape[0],), data=c1["bias"], const=True)
+        y = h.tensor(INT8, (c1["x"].shape[0], c1["w"].shape[0]))
+        h.affine(y, [c1["out_scale"]], [c1["out_zp"]])
+        h.fc(x, w, b, y)
+        out["config1_int8_2048x2048_B1"] = timed(h)
+    for batch in (1, 4):
+        c2 = wl.hybrid_fc(batch)
+        with FakeHost() as h:
+            x = h.tensor(FLOAT32, c2["x"].shape, data=c2["x"])
+            w = h.tensor(INT8, c2["w"].shape, data=c2["w"], const=True)
+            h.affine(w, c2["pcs"])
+            y = h.tensor(FLOAT32, (batch, c2["w"].shape[0]))
+            h.fc(x, w, None, y, asymmetric=True)
+            out["config2_hybrid_14336x4096_B%d" % batch] = timed(h)
+    n, k = N_OUT, K_IN
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (1, k), data=rng.standard_normal((1, k)).astype(np.float32))
+        w = h.tensor(INT4, (n, k), const=True, data=rng.integers(0, 256, (n, k // 2), dtype=np.uint8))
+        s_ = h.tensor(FLOAT16, (n, k // 32), const=True,
+                      data=(rng.random((n, k // 32), dtype=np.float32) * 1.5e-2 + 5e-3).astype(np.float16))
+        h.blockwise(w, s_, 32)
+        y = h.tensor(FLOAT32, (1, n))
+        h.fc(x, w, None, y)
+        out["config3_int4_14336x4096_B1"] = timed(h)
+    out["unit"] = "us per Invoke(), median of %d, host tensors in and out" % invokes
+    return out
 
 
 def cpu_baseline_leg(c):
