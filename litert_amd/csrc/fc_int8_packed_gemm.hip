@@ -211,7 +211,7 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
   // 32768 guarantee; one channel outside that sends the whole workgroup down the general form.
   const bool general_requantize =
       __syncthreads_or(EPI == Int8Epilogue::kRequantize &&
-                       (!plain_channel || K > 32768 || a.act_min > a.act_max));
+                       ((tid < BN && !plain_channel) || K > 32768 || a.act_min > a.act_max));
   i32x4 fa[kBatchTiles][kSub];
 #pragma unroll
   for (int j = 0; j < kBatchTiles; ++j) {
