@@ -221,10 +221,13 @@ def main():
         forms[b] = dict(fused_us_cold=round(fused_us, 3), split_us_cold=round(split_us, 3))
     # What the memory system alone needs for a launch of this size: a kernel that only streams
     # the same bytes (the re-tiled filter of each weight copy) with the GEMV's access pattern.
+    from litert_amd import bench_probes as probes
+    plib = probes.load()
+
     def stream_floor(buffers, nbytes):
         sink = torch.zeros(1, dtype=torch.int32, device="cuda")
-        fns = [(lambda t: lambda: capi.check(lib.lrtfc_stream_read_probe(p(t), nbytes, p(sink),
-                                                                          stream())))(t)
+        fns = [(lambda t: lambda: probes.check(plib.lrtprobe_stream_read(p(t), nbytes, p(sink),
+                                                                           stream())))(t)
                for t in buffers]
         return per_launch_us(fns)
 
@@ -288,20 +291,20 @@ def main():
 
 
 def mfma_rate(torch, seconds, random_operands):
-    """Sustained rate (TOPS) of the matrix cores alone on this part: lrtfc_mfma_rate_probe (256
+    """Sustained rate (TOPS) of the matrix cores alone on this part: lrtprobe_mfma_rate (256
     workgroups x 4 wavefronts, register operands, no memory traffic) launched back to back for
     about `seconds`, wall-clock timed around device synchronisations."""
     import ctypes
-    from litert_amd import capi
-    lib = capi.load()
+    from litert_amd import bench_probes as probes
+    plib = probes.load()
     sink = torch.empty(256 * 256, dtype=torch.int32, device="cuda")
     ops = ctypes.c_double(0.0)
     stream = torch.cuda.current_stream().cuda_stream
 
     def launch(n):
         for _ in range(n):
-            capi.check(lib.lrtfc_mfma_rate_probe(256, 2000, int(random_operands), sink.data_ptr(),
-                                                 ctypes.byref(ops), stream))
+            probes.check(plib.lrtprobe_mfma_rate(256, 2000, int(random_operands), sink.data_ptr(),
+                                                  ctypes.byref(ops), stream))
         torch.cuda.synchronize()
 
     launch(2)
@@ -447,6 +450,8 @@ def measured_traffic(field="traffic_bytes_per_launch:"):
 
 def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_launch_us):
     """Configs 1, 3, 4 and 5 of the benchmark contract (reported under "also")."""
+    from litert_amd import bench_probes as probes
+    plib = probes.load()
     out = {}
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
@@ -484,7 +489,7 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
     k_cold = per_launch_us([int4_kernel_only(op) for op in ops3])
     b3 = int4_bytes(1, 14336, 4096)
     sink3 = torch.zeros(1, dtype=torch.int32, device="cuda")
-    floor3 = per_launch_us([(lambda o: lambda: capi.check(lib.lrtfc_stream_read_probe(
+    floor3 = per_launch_us([(lambda o: lambda: probes.check(plib.lrtprobe_stream_read(
         p(o.retiled), o.retiled.numel(), p(sink3), stream())))(op) for op in ops3])
     out["config3_int4_gemv_14336x4096_B1"] = dict(
         stream_only_us=round(floor3, 3),
@@ -612,7 +617,7 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         tops_random_operands=round(probe_random, 1), tops_constant_operands=round(probe_constant, 1),
         us_for_config4_random=round(ops_per_call / probe_random / 1e6, 2),
         us_for_config4_constant=round(ops_per_call / probe_constant / 1e6, 2),
-        note="lrtfc_mfma_rate_probe: v_mfma_i32_32x32x32_i8 back to back on register operands, "
+        note="lrtprobe_mfma_rate: v_mfma_i32_32x32x32_i8 back to back on register operands, "
              "256 workgroups x 4 wavefronts, sustained; the clock the part holds under this load "
              "sets the figure, and the GEMM's operand traffic draws on the same power budget")
     # Yardstick (not this library): the vendor int8 GEMM through torch._int_mm on the same

@@ -452,25 +452,6 @@ int lrtfc_embedding_lookup_hybrid(const int32_t* lookup, int count, const void* 
                                   const float* row_scales, int out_type, void* output,
                                   int32_t* status, void* stream);
 
-/* ---- measurement aid ------------------------------------------------------------------------
- * No counterpart in the reference: a launch that does nothing but read `bytes` bytes (whole
- * 16-byte pieces; src 16-byte aligned) from device memory with the decode kernels' access
- * pattern. The benchmark times it on the same bytes as a GEMV to show what the memory system
- * alone needs for a launch of that size. `sink` (device int32, may be NULL) is practically
- * never written. */
-int lrtfc_stream_read_probe(const void* src, size_t bytes, int32_t* sink, void* stream);
-
-/* No counterpart in the reference either: a launch of `workgroups` x 4 wavefronts (one per
- * SIMD of a CU, as in the prefill GEMM) that do nothing but issue 8 x `iterations`
- * v_mfma_i32_32x32x32_i8 each on register operands -- pseudo-random bit patterns
- * (random_operands != 0) or constants. Timed over some hundred milliseconds of back-to-back
- * launches it gives the int8 rate the matrix cores sustain on this part under its power limit,
- * without any operand traffic: the ceiling the GEMM's main loop is measured against. `sink`
- * (device) receives workgroups x 256 int32; *ops_per_launch (host, may be NULL) the integer
- * operations (2 per multiply-add) one launch performs. */
-int lrtfc_mfma_rate_probe(int workgroups, int iterations, int random_operands, int32_t* sink,
-                          double* ops_per_launch, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

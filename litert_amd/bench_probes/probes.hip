@@ -1,4 +1,6 @@
-// Measurement aids, not part of the op. First: a kernel that only streams `bytes` bytes out of device
+// Measurement aids of the benchmark, not part of the op and not part of the kernel library: this
+// file builds into its own shared library (liblitert_amd_bench_probes.so) with its own header
+// (bench_probes.h beside it). First: a kernel that only streams `bytes` bytes out of device
 // memory, with the access pattern of the decode kernels (every wavefront walks its own
 // contiguous 32 KiB run through a ring of sixteen outstanding non-temporal 1 KiB loads) and
 // nothing else to do. Timed beside a GEMV on the same bytes it tells how much of that kernel's
@@ -9,10 +11,18 @@
 // back to back. Launched for a few hundred milliseconds it shows the int8 rate this part's
 // matrix cores sustain under its power limit, for operands that toggle like random data and
 // for constant ones: the ceiling of the GEMM's main loop, with no operand traffic at all.
-#include "kernels.h"
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-namespace lrtfc {
+#include <cstdarg>
+#include <cstdio>
+
+#include "bench_probes.h"
+
 namespace {
+
+constexpr int kWaveSize = 64;
+using i32x4 = int __attribute__((ext_vector_type(4)));
 
 using i32x16 = int __attribute__((ext_vector_type(16)));
 
@@ -91,28 +101,65 @@ __global__ __launch_bounds__(kThreads) void StreamReadKernel(const i32x4* __rest
   if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5EED1234 && sink) sink[0] = 1;
 }
 
+thread_local char g_last_error[256] = "";
+
+int Fail(int status, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof g_last_error, fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+int FromHip(hipError_t err, const char* what) {
+  if (err == hipSuccess) return LRTPROBE_OK;
+  return Fail(LRTPROBE_HIP_ERROR, "%s: %s", what, hipGetErrorString(err));
+}
+
+// One launch may hold at most this many MFMAs per wavefront-slot of the chip: about 0.1 s on a
+// 256-CU part. Sustained measurements launch back to back instead of launching longer.
+constexpr double kMaxMfmaPerLaunch = 256.0 * 4 * 2.0e6;
+
 }  // namespace
 
-hipError_t LaunchStreamRead(const void* src, size_t bytes, int32_t* sink, hipStream_t stream) {
+extern "C" {
+
+const char* lrtprobe_last_error(void) { return g_last_error; }
+
+int lrtprobe_stream_read(const void* src, size_t bytes, int32_t* sink, void* stream) {
+  if (bytes < 16) return LRTPROBE_OK;
+  if (!src) return Fail(LRTPROBE_INVALID_ARGUMENT, "null pointer");
+  if ((reinterpret_cast<uintptr_t>(src) & 15) != 0) {
+    return Fail(LRTPROBE_INVALID_ARGUMENT, "src must be 16-byte aligned");
+  }
   const size_t vecs = bytes / 16;
-  if (vecs == 0) return hipSuccess;
   const size_t waves = (vecs + kRunVecs - 1) / kRunVecs;
   const unsigned grid = static_cast<unsigned>((waves + kWaves - 1) / kWaves);
-  hipLaunchKernelGGL(StreamReadKernel, dim3(grid), dim3(kThreads), 0, stream,
-                     static_cast<const i32x4*>(src), vecs, sink);
-  return hipGetLastError();
+  hipLaunchKernelGGL(StreamReadKernel, dim3(grid), dim3(kThreads), 0,
+                     reinterpret_cast<hipStream_t>(stream), static_cast<const i32x4*>(src), vecs,
+                     sink);
+  return FromHip(hipGetLastError(), "stream read probe");
 }
 
-
-hipError_t LaunchMfmaRate(int workgroups, int iterations, int random_operands, int32_t* sink,
-                          hipStream_t stream) {
-  hipLaunchKernelGGL(MfmaRateKernel, dim3(workgroups), dim3(256), 0, stream, iterations,
-                     random_operands, sink);
-  return hipGetLastError();
+int lrtprobe_mfma_rate(int workgroups, int iterations, int random_operands, int32_t* sink,
+                       double* ops_per_launch, void* stream) {
+  if (!sink) return Fail(LRTPROBE_INVALID_ARGUMENT, "null pointer");
+  if (workgroups < 1 || workgroups > 65536 || iterations < 1) {
+    return Fail(LRTPROBE_INVALID_ARGUMENT,
+                "workgroups %d (1..65536) or iterations %d (>= 1) out of range", workgroups,
+                iterations);
+  }
+  const double mfmas = 4.0 * kProbeAccumulators * static_cast<double>(iterations) * workgroups;
+  if (mfmas > kMaxMfmaPerLaunch) {
+    return Fail(LRTPROBE_INVALID_ARGUMENT,
+                "workgroups %d x iterations %d is more than one launch may hold (about 0.1 s of "
+                "matrix-core time); launch back to back for longer measurements",
+                workgroups, iterations);
+  }
+  if (ops_per_launch) *ops_per_launch = 65536.0 * mfmas;
+  hipLaunchKernelGGL(MfmaRateKernel, dim3(workgroups), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), iterations, random_operands, sink);
+  return FromHip(hipGetLastError(), "matrix-core rate probe");
 }
 
-double MfmaRateOpsPerLaunch(int workgroups, int iterations) {
-  return 65536.0 * kProbeAccumulators * iterations * 4.0 * workgroups;
-}
-
-}  // namespace lrtfc
+}  // extern "C"

@@ -28,7 +28,7 @@ COMMON += os.environ.get("LITERT_AMD_EXTRA_HIPCC_FLAGS", "").split()
 
 FC_SOURCES = ["capi.hip", "quantize.hip", "fc_int8_gemv.hip", "fc_int8_packed_gemv.hip", "fc_int8_packed_gemm.hip",
               "fc_int8_gemm_mfma.hip", "fc_int4_blockwise.hip", "fc_int4_packed.hip", "fc_int4_per_channel_gemv.hip",
-              "embedding_lookup.hip", "fc_int4_blockwise_gemm.hip", "stream_probe.hip"]
+              "embedding_lookup.hip", "fc_int4_blockwise_gemm.hip"]
 
 
 def _run(cmd):
@@ -74,8 +74,16 @@ def build_delegate():
     return out
 
 
+def build_bench_probes():
+    """The benchmark's measurement aids: a library of their own, not linked into the others."""
+    os.makedirs(LIB, exist_ok=True)
+    out = os.path.join(LIB, "liblitert_amd_bench_probes.so")
+    _run([HIPCC] + COMMON + ["-shared", "-o", out, os.path.join(HERE, "bench_probes", "probes.hip")])
+    return out
+
+
 def build_all():
-    outs = [build_fc()]
+    outs = [build_fc(), build_bench_probes()]
     d = build_delegate()
     if d:
         outs.append(d)
@@ -84,12 +92,14 @@ def build_all():
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", choices=["fc", "delegate"])
+    ap.add_argument("--only", choices=["fc", "delegate", "probes"])
     args = ap.parse_args()
     if args.only == "fc":
         build_fc()
     elif args.only == "delegate":
         build_delegate()
+    elif args.only == "probes":
+        build_bench_probes()
     else:
         build_all()
     sys.exit(0)

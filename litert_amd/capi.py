@@ -77,8 +77,6 @@ SYMBOLS = [
     ("lrtfc_fc_blockwise_int4_gemm", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
     ("lrtfc_embedding_lookup_blockwise_int4", _i, [_vp, _i, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_embedding_lookup_hybrid", _i, [_vp, _i, _vp, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp]),
-    ("lrtfc_stream_read_probe", _i, [_vp, _sz, _vp, _vp]),
-    ("lrtfc_mfma_rate_probe", _i, [_i, _i, _i, _vp, C.POINTER(C.c_double), _vp]),
     ("lrtfc_int4_group_table_bytes", _sz, []),
     ("lrtfc_int4_group_prepare", _i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_fc_blockwise_int4_packed_grouped", _i, [_vp, _vp, _i, _vp]),

@@ -1012,26 +1012,6 @@ int lrtfc_embedding_lookup_hybrid(const int32_t* lookup, int count, const void* 
                  "hybrid embedding lookup");
 }
 
-int lrtfc_stream_read_probe(const void* src, size_t bytes, int32_t* sink, void* stream) {
-  if (int rc = RequireInit()) return rc;
-  if (bytes < 16) return LRTFC_OK;
-  LRTFC_REQUIRE(src, "null pointer");
-  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(src) & 15) == 0, "src must be 16-byte aligned");
-  return FromHip(lrtfc::LaunchStreamRead(src, bytes, sink, AsStream(stream)), "stream read probe");
-}
-
-int lrtfc_mfma_rate_probe(int workgroups, int iterations, int random_operands, int32_t* sink,
-                          double* ops_per_launch, void* stream) {
-  if (int rc = RequireInit()) return rc;
-  LRTFC_REQUIRE(sink, "null pointer");
-  LRTFC_REQUIRE(workgroups >= 1 && workgroups <= 65536 && iterations >= 1,
-                "workgroups %d (1..65536) or iterations %d (>= 1) out of range", workgroups,
-                iterations);
-  if (ops_per_launch) *ops_per_launch = lrtfc::MfmaRateOpsPerLaunch(workgroups, iterations);
-  return FromHip(lrtfc::LaunchMfmaRate(workgroups, iterations, random_operands, sink,
-                                       AsStream(stream)), "matrix-core rate probe");
-}
-
 size_t lrtfc_int4_group_table_bytes(void) { return lrtfc::Int4GroupTableBytes(); }
 
 int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,

@@ -35,6 +35,7 @@
 namespace {
 
 constexpr int kMaxFcVersion = 14;  // tflite/core/kernels/register.cc:84-86
+constexpr int kMaxBatchMatMulVersion = 4;  // tflite/core/kernels/register.cc:327-329
 
 struct Options {
   int device = 0;
@@ -214,13 +215,15 @@ bool BatchMatMulGeometry(const TfLiteTensor& lhs, const TfLiteTensor& rhs, bool 
 
 // BATCH_MATMUL in its hybrid form (batch_matmul.cc:363-374: float32 x int8): the right operand
 // a constant int8 tensor with affine quantization, one scale or one per output unit.
-FcKind ClassifyBatchMatMul(const TfLiteContext* ctx, const TfLiteNode* node, const Options& opt,
+FcKind ClassifyBatchMatMul(const TfLiteContext* ctx, const TfLiteNode* node,
+                           const TfLiteRegistration* registration, const Options& opt,
                            std::string* why_not) {
   auto no = [&](const char* reason) {
     if (why_not) *why_not = reason;
     return FcKind::kNone;
   };
   if (!opt.claim_batch_matmul) return no("batch matmul disabled by option");
+  if (registration->version > kMaxBatchMatMulVersion) return no("op version newer than 4");
   if (!node->builtin_data) return no("no builtin data");
   if (node->inputs->size != 2 || node->outputs->size != 1) return no("needs 2 inputs, 1 output");
   const auto* params = static_cast<const TfLiteBatchMatMulParams*>(node->builtin_data);
@@ -266,7 +269,7 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
     return ClassifyEmbeddingLookup(ctx, node, opt, why_not);
   }
   if (registration->builtin_code == kTfLiteBuiltinBatchMatmul) {
-    return ClassifyBatchMatMul(ctx, node, opt, why_not);
+    return ClassifyBatchMatMul(ctx, node, registration, opt, why_not);
   }
   if (registration->builtin_code != kTfLiteBuiltinFullyConnected) return no("not FULLY_CONNECTED");
   if (registration->version > kMaxFcVersion) return no("op version newer than 14");
@@ -502,8 +505,27 @@ constexpr int kInt4PerChannelNibbleMaxBatches = 32;
 constexpr int kInt4BlockwiseGemmMinBatches = 16;
 
 // Up to this many bytes of host outputs per partition are written by the kernels directly into
-// page-locked host memory instead of being copied there afterwards.
+// page-locked host memory instead of being copied there afterwards. The invariant this rests on:
+// a kernel writes every element of its output exactly once and never reads it (no atomics, no
+// zero-fill-then-accumulate, no split-depth partial sums parked in the output); anything else
+// would run its read-modify-write over PCIe against host memory. It holds for the kernels the
+// node kinds below launch today; a new kind, or a kernel form that breaks it, must stay out of
+// the list and take the copy-out path.
 constexpr size_t kDirectOutputMaxBytes = 16 << 20;
+
+bool WritesOutputOnce(FcKind kind) {
+  switch (kind) {
+    case FcKind::kInt8:
+    case FcKind::kHybrid:
+    case FcKind::kInt4Blockwise:
+    case FcKind::kHybridInt4:
+    case FcKind::kEmbeddingLookup:
+    case FcKind::kBatchMatMul:
+      return true;
+    default:
+      return false;
+  }
+}
 
 struct PartitionKernel {
   DelegateState* state = nullptr;
@@ -1077,6 +1099,7 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
         read_back = read_back || std::find(k->downloads.begin(), k->downloads.end(), n.input) !=
                                      k->downloads.end();
         read_back = read_back || n.depth == 0;  // such a node's output is cleared with a memset
+        read_back = read_back || !WritesOutputOnce(n.kind);
       }
       void* device_view = nullptr;
       if (!read_back &&

@@ -57,9 +57,13 @@ __device__ __forceinline__ float HybridCore(int32_t dot, float batch_scale, floa
 // the product (tflite/kernels/fully_connected.cc:789-795). Adding the zero product instead gives
 // the same bits except for a bias element of -0.0f (-0.0f + 0.0f is +0.0f). So the kernels add
 // the product as always and repair that one case lazily: a thread that meets a -0.0f bias with a
-// zero dot product scans the input; only a whole-zero input takes the scan to its end. A row
-// quantizes to all-zero values exactly when it was all zero (any other row has a value at the
-// far end of the int8 range), so the quantized rows can stand for the float ones. The scans are
+// zero dot product scans the input; only a whole-zero input takes the scan to its end. A row of
+// finite values quantizes to all-zero values exactly when it was all zero (any other row has a
+// value at the far end of the int8 range), so the quantized rows can stand for the float ones.
+// Not so for NaN: the row's min/max (fminf/fmaxf) drop NaNs, so a row of only zeros and NaNs
+// quantizes to zeros and takes the exit here, while the reference's IsZeroVector (v != 0) counts
+// a NaN as non-zero and adds the product; the difference shows only in a -0.0f bias element.
+// The scans are
 // real function calls: inlined into an unrolled epilogue their loops keep it from unrolling, and
 // the accumulator tiles then land in scratch memory.
 __device__ __attribute__((noinline)) bool AllZeroInt8(const int8_t* p, size_t n) {

@@ -187,15 +187,6 @@ hipError_t LaunchEmbeddingLookup(const int32_t* lookup, int count, const void* t
                                  int blocksize, const float* row_scales, float scale, int out_f16,
                                  void* output, int32_t* status, hipStream_t stream);
 
-// Measurement aid: a launch that only reads `bytes` bytes (whole 16-byte pieces) from `src`.
-hipError_t LaunchStreamRead(const void* src, size_t bytes, int32_t* sink, hipStream_t stream);
-
-// Measurement aid: `workgroups` x 4 wavefronts that each issue 8 x `iterations`
-// v_mfma_i32_32x32x32_i8 on register operands; sink holds workgroups x 256 int32.
-hipError_t LaunchMfmaRate(int workgroups, int iterations, int random_operands, int32_t* sink,
-                          hipStream_t stream);
-double MfmaRateOpsPerLaunch(int workgroups, int iterations);
-
 }  // namespace lrtfc
 
 #endif  // LITERT_AMD_CSRC_KERNELS_H_

@@ -46,7 +46,7 @@ def lib():
         L.fh_add_fc_node.argtypes = [C.c_void_p] + [C.c_int] * 10
         L.fh_add_other_node.argtypes = [C.c_void_p] + [C.c_int] * 3
         L.fh_add_embedding_lookup_node.argtypes = [C.c_void_p] + [C.c_int] * 3
-        L.fh_add_batch_matmul_node.argtypes = [C.c_void_p] + [C.c_int] * 6
+        L.fh_add_batch_matmul_node.argtypes = [C.c_void_p] + [C.c_int] * 7
         L.fh_mark_graph_output.argtypes = [C.c_void_p, C.c_int]
         L.fh_set_cpu_callback.argtypes = [C.c_void_p, CPU_CB]
         L.fh_load_delegate.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p),
@@ -149,9 +149,9 @@ class FakeHost:
     def embedding_lookup(self, lookup, value, out):
         return self.L.fh_add_embedding_lookup_node(self.h, lookup, value, out)
 
-    def batch_matmul(self, lhs, rhs, out, adj_x=False, adj_y=False, asymmetric=True):
+    def batch_matmul(self, lhs, rhs, out, adj_x=False, adj_y=False, asymmetric=True, version=4):
         return self.L.fh_add_batch_matmul_node(self.h, lhs, rhs, out, int(adj_x), int(adj_y),
-                                               int(asymmetric))
+                                               int(asymmetric), version)
 
     def mark_output(self, tensor):
         self.L.fh_mark_graph_output(self.h, tensor)

@@ -324,7 +324,7 @@ int fh_add_fc_node(void* hp, int input, int filter, int bias, int three_inputs, 
 
 // BATCH_MATMUL (builtin code 126, TfLiteBatchMatMulParams).
 int fh_add_batch_matmul_node(void* hp, int lhs, int rhs, int output, int adj_x, int adj_y,
-                             int asymmetric_quantize_inputs) {
+                             int asymmetric_quantize_inputs, int version) {
   auto* h = static_cast<Host*>(hp);
   auto rec = std::make_unique<NodeRec>();
   rec->node.inputs = MakeIntArray({lhs, rhs});
@@ -334,7 +334,7 @@ int fh_add_batch_matmul_node(void* hp, int lhs, int rhs, int output, int adj_x, 
   rec->bmm.asymmetric_quantize_inputs = asymmetric_quantize_inputs != 0;
   rec->node.builtin_data = &rec->bmm;
   rec->reg.builtin_code = kTfLiteBuiltinBatchMatmul;
-  rec->reg.version = 4;
+  rec->reg.version = version;
   h->nodes.push_back(std::move(rec));
   h->plan.push_back(static_cast<int>(h->nodes.size()) - 1);
   return static_cast<int>(h->nodes.size()) - 1;

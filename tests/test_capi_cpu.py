@@ -32,6 +32,23 @@ def test_delegate_plugin_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
+def test_bench_probe_library_is_separate_and_exports_its_header():
+    """The measurement aids have their own header and library; the kernel library's header
+    declares none of them."""
+    from litert_amd import bench_probes as probes
+    text = open(os.path.join(ROOT, "litert_amd", "bench_probes", "bench_probes.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(lrtprobe_[a-z0-9_]+)\s*\(", text)))
+    assert declared == ["lrtprobe_last_error", "lrtprobe_mfma_rate", "lrtprobe_stream_read"]
+    lib = probes.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert not [n for n in _header_symbols() if "probe" in n]
+    fc_lib = capi.load()
+    assert not hasattr(fc_lib, "lrtfc_stream_read_probe")
+    assert not hasattr(fc_lib, "lrtfc_mfma_rate_probe")
+
+
 def test_library_exports_every_declared_symbol():
     lib = capi.load()
     declared = _header_symbols()

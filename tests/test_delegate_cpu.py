@@ -124,6 +124,9 @@ def test_claim_predicate_batch_matmul():
         assert h.classify(_bmm_node(h, scales=np.full(8, 0.01), qdim=0)) == (
             None, "per-channel scales do not run along the output units")
         assert h.classify(_bmm_node(h, adj_x=True)) == (None, "adj_x is left to the CPU kernels")
+        # register.cc:327-329 registers versions 1..4; a newer one may mean other arithmetic
+        assert h.classify(_bmm_node(h, version=4))[0] == "batch_matmul"
+        assert h.classify(_bmm_node(h, version=5)) == (None, "op version newer than 4")
         assert h.classify(_bmm_node(h, const=False)) == (None, "right operand is not a constant tensor")
         assert h.classify(_bmm_node(h, lhs_type=INT8)) == (None, "not the float32 x int8 form")
         assert h.classify(_bmm_node(h, rhs_shape=(32, 8))) == (None, "accumulation depths differ")

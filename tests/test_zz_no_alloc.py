@@ -41,12 +41,17 @@ def _both(lib, capi, c, bias, asym, activation):
     torch.cuda.synchronize()
     capi.check(lib.lrtfc_fc_hybrid(_p(x), _p(w), _p(pcs), 1.0, _p(rs), _p(b), _p(want), B, K, N,
                                    int(asym), activation, 0, _p(ws), need, None))
+    # Free device memory as the driver sees it (hipMemGetInfo): a hipMalloc inside the entry
+    # point would lower it, which torch's own allocator statistics cannot see.
+    torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]
     capi.check(lib.lrtfc_fc_hybrid_static_scratch(_p(x), _p(w), _p(pcs), 1.0, _p(rs), _p(b),
                                                   _p(got), B, K, N, int(asym), activation, 0,
                                                   None))
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     return got.cpu().numpy(), want.cpu().numpy()
 
 
