@@ -77,6 +77,20 @@ __device__ __forceinline__ float ApplyFloatActivation(float v, int activation) {
   }
 }
 
+// The same function without a branch, for epilogues whose few active lanes should not walk a
+// switch per value: every clamp is `t = (hi < v) ? hi : v; (lo < t) ? t : lo` with its bounds
+// (RELU: 0 and +infinity, whose upper test never holds, as in the form above), selected by
+// wave-uniform conditions.
+__device__ __forceinline__ float ApplyFloatActivationSelect(float v, int activation) {
+  const float lo = activation == 2 ? -1.0f : 0.0f;
+  const float hi = activation == 2 ? 1.0f : (activation == 3 ? 6.0f : __builtin_inff());
+  const float t = (hi < v) ? hi : v;
+  const float clamped = (lo < t) ? t : lo;
+  const float sign = (__float_as_uint(v) >> 31) ? 1.0f : 0.0f;
+  const bool clamps = activation >= 1 && activation <= 3;
+  return clamps ? clamped : (activation == 5 ? sign : v);
+}
+
 // IEEE binary16 -> binary32, exact for every finite pattern, subnormals included.
 __device__ __forceinline__ float HalfBitsToFloat(uint16_t h) {
   const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;

@@ -26,6 +26,8 @@
 // hybrid form the staging step *is* the BatchQuantizeFloats of the op: the workgroup
 // reduces min/max of each float row, derives scale and zero point, and writes the
 // quantized row straight to LDS, so the op is a single kernel.
+#include <cstdlib>
+
 #include "fc_epilogues.h"
 #include "kernels.h"
 #include "quantize_device.h"
@@ -472,6 +474,471 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(
   }
 }
 
+// ---- the form for filters a launch can hold in its registers --------------------------------
+//
+// A decode launch of this size is a chain of latencies in front of a stream: the memory system
+// needs about 8 us for 58 MB however the loads are arranged, and every microsecond in which
+// loads that could have been in flight were not is added to that. A ring that is refilled as
+// it is consumed ties the stream to the consumer: a slot is requested again only after the
+// product that empties it, and nothing beyond the ring is requested until the activation rows
+// are quantized and staged. This form unties them. A wavefront's whole share of the depth (at
+// most TILES tiles of 1 KiB; the vector register file of the chip holds 128 MB, a filter of
+// this class fits) has a register of its own, so a request never waits for a product:
+//   * kAhead tiles are requested before anything waits for anything; the one barrier of the
+//     kernel (rows staged) follows, and from there on the wavefront alternates "request tile
+//     u" with "multiply tile u - kLag", in straight-line code whose waits the compiler counts
+//     exactly. A compute unit accepts only some tens of KiB of outstanding loads, so a
+//     wavefront spends most of its time blocked in load issue: whatever it has to compute
+//     must sit between two requests, not behind the last one.
+//   * The per-row work is given to single wavefronts: wavefront r of a workgroup (r < rows)
+//     reads row r into its registers, reduces it, derives the row's parameters and writes the
+//     quantized row to LDS on its own, with no workgroup-wide step. Its row loads must not
+//     queue behind the other wavefronts' weight requests (the vector memory path of a compute
+//     unit serves requests in order): it runs at raised priority until the row is requested,
+//     and the others hold their first request back for some hundred cycles.
+#ifndef LRT_V_LAG
+#define LRT_V_LAG 8
+#endif
+#ifndef LRT_V_AHEAD
+#define LRT_V_AHEAD 16
+#endif
+constexpr int kStreamLag = LRT_V_LAG;    // products trail the requests by this many tiles
+constexpr int kStreamAhead = LRT_V_AHEAD; // tiles requested before the barrier (wavefronts without a row)
+
+// Where `PackedArgs p` lies in the kernel's argument segment: behind three pointers and seven
+// ints, at its own alignment.
+struct UpfrontLeadingArgs {
+  const void* pointers[3];
+  int ints[7];
+};
+constexpr size_t kUpfrontPackedArgsOffset =
+    (sizeof(UpfrontLeadingArgs) + alignof(PackedArgs) - 1) / alignof(PackedArgs) * alignof(PackedArgs);
+static_assert(kUpfrontPackedArgsOffset == 56, "argument layout of FcInt8UpfrontGemvKernel");
+
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void FcInt8UpfrontGemvKernel(
+    const int8_t* early_filter, const float* early_input_f32, const int8_t* early_input_i8,
+    int early_depth, int early_slabs, int early_out_depth, int batch0, int bt, int ksplit_log2,
+    int per_part, PackedArgs p) {
+  extern __shared__ __align__(16) int8_t smem[];
+  const FcInt8Args& a = p.a;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWaveSize - 1);
+  const int ksplit = 1 << ksplit_log2;
+  // The wavefront's index as a scalar: everything derived from it (its channel group, its
+  // share of the depth, whether it has a row to quantize) is then uniform to the compiler,
+  // which keeps the branches scalar and the tile addresses in scalar registers.
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWaveSize);
+  const int col = lane & 15;
+  const int kgroup = lane >> 4;
+  const int slabs = early_slabs;
+  const int depth = early_depth;
+  // per_part = ceil(slabs / ksplit) <= TILES (the launcher's choice). A staged row is
+  // zero-filled up to the end of the last share, so that a share that runs past the depth
+  // multiplies its (clamped, re-read) tiles by zeros instead of branching.
+  const int staged = ksplit * per_part * kSlabDepth;
+  const int qstride = staged + kQPad;
+  const Shared sh = CarveShared(smem, bt, qstride);
+  const int tiles = (early_out_depth + kTileRows - 1) / kTileRows;
+  const int tile = ((blockIdx.x * kWaves) >> ksplit_log2) + (wave >> ksplit_log2);
+  const int part = wave & (ksplit - 1);
+  const int s0 = part * per_part;
+  const int8_t* group_base =
+      early_filter + static_cast<size_t>(min(tile, tiles - 1)) * slabs * 1024;  // uniform
+  // The argument segment beyond the leading (preloaded) arguments, as a pointer the compiler
+  // cannot see through: scalar loads through it stay where the code asks for them. Read in the
+  // ordinary way, the compiler moves every argument load to the kernel's entry, and the first
+  // weight request -- which needs the preloaded arguments only -- waits behind a fetch of the
+  // argument segment from memory.
+  using LateArgs = const __attribute__((address_space(4))) PackedArgs;
+  auto late_args = [&]() -> LateArgs* {
+    auto* segment = (const __attribute__((address_space(4))) char*)
+        __builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(segment));
+    return (LateArgs*)(segment + kUpfrontPackedArgsOffset);
+  };
+  i32x4 ring[TILES];
+  auto request = [&](int u) {
+    // Past the share or the depth: the share's last tile again (a hit in the nearest cache).
+    const int8_t* t =
+        group_base + static_cast<size_t>(min(s0 + min(u, per_part - 1), slabs - 1)) * 1024;
+    ring[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(t + lane * 16));
+    __builtin_amdgcn_sched_barrier(0);  // issue order = the order the products take them in
+  };
+
+  // Per-channel epilogue parameters, requested behind the first tiles (they are needed last).
+  // Unconditional loads: an absent array reads a valid dummy address.
+  int32_t ep_i0[4], ep_i1[4], ep_i2[4], ep_i3[4];
+  float ep_f0[4], ep_f1[4];
+  auto request_parameters = [&]() {
+    // Pointers from the argument segment, read HERE (see late_args).
+    const LateArgs* late = late_args();
+    const int out_depth = early_out_depth;
+    const int32_t* dummy_i = reinterpret_cast<const int32_t*>(early_filter);
+    const float* dummy_f = reinterpret_cast<const float*>(early_filter);
+    if (EPI == Int8Epilogue::kRequantize) {
+      const int32_t* multipliers = late->a.multipliers;
+      const int32_t* shifts = late->a.shifts;
+      const int32_t* bias = late->a.bias_i32;
+      const int32_t* row_sums = late->a.filter_row_sums;
+      const int per_channel = late->a.per_channel;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = min(min(tile, tiles - 1) * kTileRows + 4 * kgroup + i, out_depth - 1);
+        ep_i0[i] = multipliers[per_channel ? n : 0];
+        ep_i1[i] = shifts[per_channel ? n : 0];
+        ep_i2[i] = *(bias ? bias + n : dummy_i);
+        ep_i3[i] = *(row_sums ? row_sums + n : dummy_i);
+      }
+    } else {
+      const int32_t* row_sums = late->a.filter_row_sums;
+      const float* scales = late->a.per_channel_scales;
+      const float* bias = late->a.bias_f32;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = min(min(tile, tiles - 1) * kTileRows + 4 * kgroup + i, out_depth - 1);
+        ep_i0[i] = *(row_sums ? row_sums + n : dummy_i);
+        ep_f0[i] = *(scales ? scales + n : dummy_f);
+        ep_f1[i] = *(bias ? bias + n : dummy_f);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // The epilogue's scalar inputs, read from the argument segment where `stream` says (while the
+  // wavefront waits at the barrier anyway: a scalar load issued at the end of the kernel queues
+  // behind the whole chip's weight stream).
+  void* ep_out;
+  int ep_activation, ep_flags, ep_batches;
+  float ep_filter_scale;
+  int32_t ep_offsets0, ep_offsets1, ep_offsets2, ep_offsets3;
+  const float* ep_scaling_factors;
+  const int32_t* ep_zero_points;
+  auto fetch_epilogue_scalars = [&]() {
+    const LateArgs* late = late_args();
+    ep_out = EPI == Int8Epilogue::kRequantize ? static_cast<void*>(late->a.output_i8)
+                                              : static_cast<void*>(late->a.output_f32);
+    ep_activation = late->a.activation;
+    ep_flags = (late->a.bias_i32 ? 1 : 0) | (late->a.filter_row_sums ? 2 : 0) |
+               (late->a.per_channel_scales ? 4 : 0) | (late->a.bias_f32 ? 8 : 0) |
+               (late->a.zero_input_exit ? 32 : 0) | (late->a.batch_matmul ? 64 : 0);
+    ep_filter_scale = late->a.filter_scale;
+    ep_offsets0 = late->a.input_offset;
+    ep_offsets1 = late->a.output_offset;
+    ep_offsets2 = late->a.act_min;
+    ep_offsets3 = late->a.act_max;
+    ep_batches = late->a.batches;
+    ep_scaling_factors = late->a.scaling_factors;
+    ep_zero_points = late->a.zero_points;
+  };
+  const int8_t* qbase = sh.q + (col < bt ? col : 0) * qstride + kgroup * 16 + s0 * kSlabDepth;
+  const int8_t* pad_zero = sh.q + staged;  // the kQPad bytes behind row 0, cleared below
+  constexpr int kAccs = 4;
+  i32x4 acc4[kAccs];
+#pragma unroll
+  for (int i = 0; i < kAccs; ++i) acc4[i] = i32x4{0, 0, 0, 0};
+  // Products of tiles g .. g + 3: four activation operands per LDS wait.
+  auto multiply4 = [&](int g) {
+    i32x4 bq[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      // Past the share (which only happens when TILES is larger than the share) the operand
+      // is the 16 bytes of zeros behind row 0.
+      const int8_t* at = g + u < per_part ? qbase + (g + u) * kSlabDepth : pad_zero;
+      bq[u] = *reinterpret_cast<const i32x4*>(at);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      acc4[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ring[g + u], bq[u], acc4[u], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // Tiles [0, first) are requested; requests up to `ahead`, the barrier, then requests and
+  // products in alternation, the products kLag tiles behind.
+  auto stream = [&](auto first_c, auto ahead_c) {
+    constexpr int kFirst = decltype(first_c)::value;
+    constexpr int kAhead = decltype(ahead_c)::value < TILES ? decltype(ahead_c)::value : TILES;
+    constexpr int kLag = kStreamLag < kAhead ? kStreamLag : kAhead;
+    static_assert(kFirst <= kAhead && kAhead % 4 == 0 && kLag % 4 == 0 && TILES % 4 == 0, "");
+#pragma unroll
+    for (int u = kFirst; u < kAhead; ++u) request(u);
+    request_parameters();
+    if (tid < 4) *reinterpret_cast<int32_t*>(sh.q + staged + tid * 4) = 0;  // pad_zero
+    // What the epilogue reads from the argument segment is fetched here, while the wavefront
+    // waits at the barrier anyway: a scalar load issued at the end of the kernel queues behind
+    // the whole chip's weight stream and costs some hundred nanoseconds of every launch.
+    fetch_epilogue_scalars();
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < kAhead - kLag; g += 4) multiply4(g);
+#pragma unroll
+    for (int g = kAhead; g < TILES; g += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) request(g + u);
+      multiply4(g - kLag);
+    }
+#pragma unroll
+    for (int g = TILES - kLag; g < TILES; g += 4) multiply4(g);
+  };
+  using std::integral_constant;
+
+#ifndef LRT_V_SLEEP
+#define LRT_V_SLEEP 8
+#endif
+  if (FUSED) {
+    if (wave < bt) {
+      __builtin_amdgcn_s_setprio(3);
+      // This wavefront's row: 16 pieces of 16 bytes per lane (depth <= 4096).
+      constexpr int kPieces = 16;
+      constexpr int kEarly = EARLY ? (TILES < 8 ? TILES : 8) : 0;
+      const float* x = early_input_f32 + static_cast<size_t>(batch0 + wave) * depth;
+      float4 xr[kPieces];
+#pragma unroll
+      for (int j = 0; j < kPieces; ++j) {
+        const int i = (j * kWaveSize + lane) * 4;
+        xr[j] = *reinterpret_cast<const float4*>(x + min(i, depth - 4));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (EARLY) {
+        // Every wavefront of the workgroup has a row: some weights go out ahead of the row's
+        // arithmetic, or nothing would be in flight meanwhile.
+#pragma unroll
+        for (int u = 0; u < kEarly; ++u) request(u);
+      }
+      float mn = 0.0f, mx = 0.0f;
+#pragma unroll
+      for (int j = 0; j < kPieces; ++j) {
+        const float4 t = xr[j];  // past the row: a clamped duplicate, harmless for min/max
+        mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
+        mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
+      }
+      mn = WaveMinF32(mn);
+      mx = WaveMaxF32(mx);
+      const int asymmetric = late_args()->asymmetric;
+      RowQuantParams qp =
+          asymmetric ? AsymmetricRowParams<VARIANT>(mn, mx) : SymmetricRowParams(mn, mx);
+      if (lane == 0) {
+        sh.sf[wave] = qp.scale;
+        sh.zp[wave] = qp.zero_point;
+        sh.zero[wave] = qp.all_zero ? 1 : 0;
+      }
+      qp.inv = ElementwiseInv(qp);
+      const int vector_end = depth - (depth % 8);
+      int8_t* qrow = sh.q + wave * qstride;
+#pragma unroll
+      for (int j = 0; j < kPieces; ++j) {
+        const int i = (j * kWaveSize + lane) * 4;
+        const float4 t = xr[j];
+        int32_t packed = QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, i >= vector_end);
+        packed = i < depth ? packed : 0;
+        if (i < staged) *reinterpret_cast<int32_t*>(qrow + i) = packed;
+      }
+      // Zeros between 16 pieces' worth and the end of the last share (a few slabs at most).
+      for (int i = kPieces * kWaveSize * 4 + lane * 4; i < staged; i += kWaveSize * 4) {
+        *reinterpret_cast<int32_t*>(qrow + i) = 0;
+      }
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      stream(integral_constant<int, kEarly>{}, integral_constant<int, (kEarly > kStreamLag ? kEarly : kStreamLag)>{});
+    } else {
+      if (LRT_V_SLEEP) __builtin_amdgcn_s_sleep(LRT_V_SLEEP);
+      stream(integral_constant<int, 0>{}, integral_constant<int, kStreamAhead>{});
+    }
+  } else {
+    // Rows that arrive quantized: up to 16 rows of depth 4096, 16 bytes per thread and piece,
+    // requested ahead of the weights and written to LDS when they are there.
+    constexpr int kQRegs = 4;
+    constexpr int kFirst = TILES < 8 ? TILES : 8;
+    i32x4 qr[kQRegs];
+    const int chunks_per_row = staged / 16;
+#pragma unroll
+    for (int j = 0; j < kQRegs; ++j) {
+      const int c = j * kThreads + tid;
+      const int b = min(c / chunks_per_row, bt - 1);
+      const int i = (c % chunks_per_row) * 16;
+      qr[j] = *reinterpret_cast<const i32x4*>(
+          early_input_i8 + static_cast<size_t>(batch0 + b) * depth + min(i, depth - 16));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < kFirst; ++u) request(u);
+#pragma unroll
+    for (int j = 0; j < kQRegs; ++j) {
+      const int c = j * kThreads + tid;
+      const int b = c / chunks_per_row;
+      const int i = (c % chunks_per_row) * 16;
+      if (b < bt) {
+        *reinterpret_cast<i32x4*>(sh.q + b * qstride + i) = i < depth ? qr[j] : i32x4{0, 0, 0, 0};
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    stream(integral_constant<int, kFirst>{}, integral_constant<int, kStreamAhead>{});
+  }
+  i32x4 acc = (acc4[0] + acc4[1]) + (acc4[2] + acc4[3]);
+
+  if (ksplit > 1) {
+    sh.partial[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (part != 0) return;
+    for (int w = 1; w < ksplit; ++w) acc += sh.partial[(wave + w) * 64 + lane];
+  }
+
+  if (col >= bt || tile >= tiles) return;
+  const int b = batch0 + col;
+  const int out_depth = early_out_depth;
+  const int n0 = tile * kTileRows + 4 * kgroup;  // this lane's four channels: n0 .. n0 + 3
+  if (EPI == Int8Epilogue::kRequantize) {
+    int32_t q[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int32_t bias = (ep_flags & 1) ? ep_i2[i] : 0;
+      const int32_t row_sum = (ep_flags & 2) ? ep_i3[i] : 0;
+      q[i] = RequantizeCore(acc[i] + bias + ep_offsets0 * row_sum, ep_i0[i], ep_i1[i],
+                            ep_offsets1, ep_offsets2, ep_offsets3);
+    }
+    int8_t* out = static_cast<int8_t*>(ep_out) + static_cast<size_t>(b) * out_depth + n0;
+    if (n0 + 4 <= out_depth && (reinterpret_cast<uintptr_t>(out) & 3) == 0) {
+      *reinterpret_cast<int32_t*>(out) = PackLowBytes(q[0], q[1], q[2], q[3]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (n0 + i < out_depth) out[i] = static_cast<int8_t>(q[i]);
+      }
+    }
+    return;
+  }
+  // Float epilogues. The four values of a lane are computed side by side without branches (the
+  // tail of the slowest wavefront is the tail of the launch); the one rare case that needs a
+  // scan of the input, a whole-zero input meeting a -0.0f bias, takes a branch of its own.
+  const float batch_scale = FUSED ? sh.sf[col] : ep_scaling_factors[b];
+  const int32_t batch_zp = FUSED ? sh.zp[col] : (ep_zero_points ? ep_zero_points[b] : 0);
+  const bool row_zero = FUSED ? sh.zero[col] != 0 : true;
+  float value[4];
+  bool rare = false;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float channel_scale = (ep_flags & 4) ? ep_f0[i] : ep_filter_scale;
+    const float bias = (ep_flags & 8) ? ep_f1[i] : 0.0f;
+    const int32_t row_sum = (ep_flags & 2) ? ep_i0[i] : 0;
+    if (EPI == Int8Epilogue::kHybrid4Bit) {
+      // Hybrid4BitCore with the activation as selects.
+      const float val = __fmul_rn(static_cast<float>(batch_zp), batch_scale);
+      float out = __fmul_rn(val, channel_scale);
+      if (ep_flags & 8) out = __fadd_rn(out, bias);
+      const float term = __fmul_rn(static_cast<float>(acc[i] - batch_zp), batch_scale);
+      out = __fadd_rn(out, __fmul_rn(term, channel_scale));
+      value[i] = ApplyFloatActivationSelect(out, ep_activation);
+    } else {
+      const float scale = __fmul_rn(batch_scale, channel_scale);
+      const float as_bmm =
+          HybridBatchMatMulCore(acc[i], batch_scale, channel_scale, batch_zp, row_sum);
+      const int32_t corrected = acc[i] - row_sum * batch_zp;
+      const float as_fc = ApplyFloatActivationSelect(
+          __fadd_rn(bias, __fmul_rn(static_cast<float>(corrected), scale)), ep_activation);
+      value[i] = (!FUSED && (ep_flags & 64)) ? as_bmm : as_fc;
+      // Whole-zero input (fully_connected.cc:789-795): possible only where the dot product is
+      // zero under a -0.0f bias (fused: and this row quantized to zeros).
+      rare = rare || (IsNegativeZero(bias) && acc[i] == 0 && row_zero);
+    }
+  }
+  if (EPI != Int8Epilogue::kHybrid4Bit && rare && (FUSED || (ep_flags & 32)) &&
+      !(ep_flags & 64)) {
+    bool zero_input;
+    if (FUSED) {
+      // This launch knows its own rows from the prologue; rows of other launches of the same
+      // call are scanned.
+      zero_input = true;
+      for (int r = 0; r < bt; ++r) zero_input = zero_input && sh.zero[r] != 0;
+      if (zero_input && ep_batches > bt) {
+        zero_input = AllZeroF32(early_input_f32, static_cast<size_t>(ep_batches) * depth);
+      }
+    } else {
+      zero_input = AllZeroInt8(early_input_i8, static_cast<size_t>(ep_batches) * depth);
+    }
+    if (zero_input) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float bias = (ep_flags & 8) ? ep_f1[i] : 0.0f;
+        if (IsNegativeZero(bias) && acc[i] == 0) {
+          value[i] = ApplyFloatActivation(bias, ep_activation);
+        }
+      }
+    }
+  }
+  float* out = static_cast<float*>(ep_out) + static_cast<size_t>(b) * out_depth + n0;
+  if (n0 + 4 <= out_depth && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+    *reinterpret_cast<float4*>(out) = make_float4(value[0], value[1], value[2], value[3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (n0 + i < out_depth) out[i] = value[i];
+    }
+  }
+}
+
+// How many wavefronts share one channel group's depth (see LaunchSized below).
+int ChooseKsplit(int slabs, int tiles) {
+  int ksplit = 1;
+  while (ksplit < kWaves && slabs / (ksplit * 2) >= 2 * kRing) ksplit *= 2;
+  while (ksplit < kWaves && tiles * ksplit < 1024 && slabs / (ksplit * 2) >= 4) ksplit *= 2;
+  return ksplit;
+}
+
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY>
+hipError_t LaunchUpfrontSized(const PackedArgs& p, int batch0, int bt, int ksplit,
+                              hipStream_t stream) {
+  const int per_part = (p.slabs + ksplit - 1) / ksplit;
+  const int qstride = ksplit * per_part * kSlabDepth + kQPad;
+  const size_t lds = SharedBytes(bt, qstride);
+  auto kernel = FcInt8UpfrontGemvKernel<EPI, FUSED, VARIANT, TILES, EARLY>;
+  if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
+  const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
+  const int tiles_per_wg = kWaves / ksplit;
+  const int grid = (tiles + tiles_per_wg - 1) / tiles_per_wg;
+  int ksplit_log2 = 0;
+  while ((1 << ksplit_log2) < ksplit) ++ksplit_log2;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, p.a.filter, p.input_f32,
+                     p.a.input, p.a.depth, p.slabs, p.a.out_depth, batch0, bt, ksplit_log2,
+                     per_part, p);
+  return hipGetLastError();
+}
+
+// Whether the all-up-front form takes this launch; *launched tells. It needs a wavefront's share
+// of the depth to fit TILES tiles, and rows that fit the registers set aside for them.
+template <Int8Epilogue EPI, bool FUSED, int VARIANT>
+hipError_t TryLaunchUpfront(const PackedArgs& p, int batch0, int bt, hipStream_t stream,
+                            bool* launched) {
+  *launched = false;
+  const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
+  const int depth = p.a.depth;
+  int ksplit = ChooseKsplit(p.slabs, tiles);
+  while (ksplit < kWaves && (p.slabs + ksplit - 1) / ksplit > 32) ksplit *= 2;
+  const int per_part = (p.slabs + ksplit - 1) / ksplit;
+  if (per_part > 32) return hipSuccess;
+  if (FUSED) {
+    const bool vec_ok =
+        (depth % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.input_f32) & 15) == 0);
+    if (!vec_ok || depth > 4096 || depth < 4 || bt > kWaves) return hipSuccess;
+  } else {
+    const bool vec_ok = (depth % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a.input) & 15) == 0);
+    const int64_t chunks = static_cast<int64_t>(bt) * (ksplit * per_part * kSlabDepth / 16);
+    if (!vec_ok || chunks > 4 * kThreads) return hipSuccess;
+  }
+  *launched = true;
+  const bool early = FUSED && bt > 2;
+  if (per_part <= 8) {
+    return early ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, FUSED>(p, batch0, bt, ksplit, stream)
+                 : LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, false>(p, batch0, bt, ksplit, stream);
+  }
+  if (per_part <= 16) {
+    return early ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, FUSED>(p, batch0, bt, ksplit, stream)
+                 : LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, false>(p, batch0, bt, ksplit, stream);
+  }
+  return early ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 32, FUSED>(p, batch0, bt, ksplit, stream)
+               : LaunchUpfrontSized<EPI, FUSED, VARIANT, 32, false>(p, batch0, bt, ksplit, stream);
+}
+
 template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS, int XREGS = 4>
 hipError_t LaunchSized(const PackedArgs& p, int batch0, int bt, hipStream_t stream) {
   const int qstride = p.slabs * kSlabDepth + kQPad;
@@ -497,6 +964,12 @@ hipError_t LaunchSized(const PackedArgs& p, int batch0, int bt, hipStream_t stre
 
 template <Int8Epilogue EPI, bool FUSED, int VARIANT>
 hipError_t LaunchOne(const PackedArgs& p, int batch0, int bt, hipStream_t stream) {
+  static const bool use_upfront = getenv("LRT_GEMV_OLD") == nullptr;
+  if (use_upfront) {
+    bool launched = false;
+    hipError_t err = TryLaunchUpfront<EPI, FUSED, VARIANT>(p, batch0, bt, stream, &launched);
+    if (launched || err != hipSuccess) return err;
+  }
   if (!FUSED) {
     // Quantized rows that fit the registers are requested before the weights and need no
     // wait of their own: up to 16 rows of depth 4096.
