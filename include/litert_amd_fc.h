@@ -122,6 +122,13 @@ enum { LRTFC_LAYOUT_ROW_MAJOR = 0, LRTFC_LAYOUT_PACKED = 1 };
 int lrtfc_fc_int8_preferred_layout(int batches, int depth, int out_depth, int32_t filter_offset);
 int lrtfc_fc_blockwise_int4_preferred_layout(int depth, int blocksize);
 
+/* Up to how many batch rows lrtfc_fc_hybrid_packed should be handed float rows directly (one
+ * launch: the row quantizer runs inside the product kernel, one wavefront per row) rather than
+ * through lrtfc_fc_hybrid_packed_workspace (row quantizer launch, then the product). Both give
+ * the same bits; this is the faster choice per shape, where the reference has a single code path
+ * for every batch size (tflite/kernels/fully_connected.cc:847-851). Pure host function. */
+int lrtfc_fc_hybrid_fused_max_batches(int depth, int out_depth);
+
 /* Re-tiles a row-major int8 filter [out_depth, depth] for the matrix-core GEMV: tiles of
  * 16 output channels x 64 depth (1 KiB each, zero-padded at the edges), the 16 bytes of
  * lane L inside a tile being channel L % 16, depth 16 * (L / 16) .. +16; tiles of one

@@ -34,6 +34,7 @@ SYMBOLS = [
     ("lrtfc_blockwise_int4_kfsum", _i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     ("lrtfc_fc_int8_preferred_layout", _i, [_i, _i, _i, _i]),
     ("lrtfc_fc_blockwise_int4_preferred_layout", _i, [_i, _i]),
+    ("lrtfc_fc_hybrid_fused_max_batches", _i, [_i, _i]),
     ("lrtfc_packed_int8_filter_bytes", _sz, [_i, _i]),
     ("lrtfc_pack_int8_filter", _i, [_vp, _i, _i, _vp, _vp]),
     ("lrtfc_fc_int8_packed", _i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i32, _i32,

@@ -333,6 +333,11 @@ int lrtfc_fc_int8_preferred_layout(int batches, int depth, int out_depth, int32_
   return lrtfc::FcInt8PackedGemvSupports(a) ? LRTFC_LAYOUT_PACKED : LRTFC_LAYOUT_ROW_MAJOR;
 }
 
+int lrtfc_fc_hybrid_fused_max_batches(int depth, int out_depth) {
+  (void)out_depth;
+  return lrtfc::FcInt8PackedGemvFusedMaxRows(depth);
+}
+
 int lrtfc_fc_blockwise_int4_preferred_layout(int depth, int blocksize) {
   return lrtfc::FcInt4PackedSupports(depth, blocksize) ? LRTFC_LAYOUT_PACKED
                                                        : LRTFC_LAYOUT_ROW_MAJOR;

@@ -494,7 +494,6 @@ struct FcNode {
 
 // Rows above which the fused kernels' prologue (every workgroup quantizes every row) costs
 // more than a separate quantization launch; deep int4 rows fuse at most two batch rows.
-constexpr int kHybridFusedMaxBatches = 4;
 constexpr int kInt4FusedMaxDepth = 4096;
 constexpr int kInt4DeepFusedMaxBatches = 2;
 // Up to this many rows a per-channel int4 node streams its filter as nibbles (one pass per 16
@@ -945,7 +944,7 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
     n->filter_scale = filter.params.scale;
     n->use_retiled = weights > 0 && lrtfc_fc_int8_preferred_layout(1, n->depth, n->out_depth, 0) ==
                                         LRTFC_LAYOUT_PACKED;
-    n->split_quantize = n->batches > kHybridFusedMaxBatches;
+    n->split_quantize = n->batches > lrtfc_fc_hybrid_fused_max_batches(n->depth, n->out_depth);
     if (weights > 0 && !(n->use_retiled ? n->have_retiled : n->have_model_layout)) {
       if (!n->have_model_layout) {
         RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));

@@ -26,8 +26,6 @@
 // hybrid form the staging step *is* the BatchQuantizeFloats of the op: the workgroup
 // reduces min/max of each float row, derives scale and zero point, and writes the
 // quantized row straight to LDS, so the op is a single kernel.
-#include <cstdlib>
-
 #include "fc_epilogues.h"
 #include "kernels.h"
 #include "quantize_device.h"
@@ -81,12 +79,13 @@ struct Shared {
   float* mm;       // [16][kWaves][2]
 };
 
-__device__ __forceinline__ Shared CarveShared(int8_t* base, int bt, int qstride) {
+__device__ __forceinline__ Shared CarveShared(int8_t* base, int bt, int qstride,
+                                              int waves = kWaves) {
   Shared s;
   s.q = base;
   size_t off = (static_cast<size_t>(bt) * qstride + 15) & ~static_cast<size_t>(15);
   s.partial = reinterpret_cast<i32x4*>(base + off);
-  off += kWaves * 64 * sizeof(i32x4);
+  off += waves * 64 * sizeof(i32x4);
   s.sf = reinterpret_cast<float*>(base + off);
   off += 16 * 4;
   s.inv = reinterpret_cast<float*>(base + off);
@@ -99,9 +98,9 @@ __device__ __forceinline__ Shared CarveShared(int8_t* base, int bt, int qstride)
   return s;
 }
 
-size_t SharedBytes(int bt, int qstride) {
+size_t SharedBytes(int bt, int qstride, int waves = kWaves) {
   return ((static_cast<size_t>(bt) * qstride + 15) & ~static_cast<size_t>(15)) +
-         kWaves * 64 * sizeof(i32x4) + 4 * 16 * 4 + 16 * kWaves * 2 * 4;
+         waves * 64 * sizeof(i32x4) + 4 * 16 * 4 + 16 * waves * 2 * 4;
 }
 
 constexpr int kRing = 16;  // weight tiles in flight per wavefront
@@ -496,14 +495,11 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(
 //     queue behind the other wavefronts' weight requests (the vector memory path of a compute
 //     unit serves requests in order): it runs at raised priority until the row is requested,
 //     and the others hold their first request back for some hundred cycles.
-#ifndef LRT_V_LAG
-#define LRT_V_LAG 8
-#endif
-#ifndef LRT_V_AHEAD
-#define LRT_V_AHEAD 16
-#endif
-constexpr int kStreamLag = LRT_V_LAG;    // products trail the requests by this many tiles
-constexpr int kStreamAhead = LRT_V_AHEAD; // tiles requested before the barrier (wavefronts without a row)
+
+constexpr int kFusedRowMaxDepth = 4096;  // a wavefront holds its row in 16 x 16 bytes per lane
+constexpr int kFusedMaxRows = 8;          // one wavefront of eight per row
+constexpr int kStreamLag = 12;    // products trail the requests by this many tiles
+constexpr int kStreamAhead = 24;  // tiles requested before the barrier (wavefronts without a row)
 
 // Where `PackedArgs p` lies in the kernel's argument segment: behind three pointers and seven
 // ints, at its own alignment.
@@ -515,14 +511,14 @@ constexpr size_t kUpfrontPackedArgsOffset =
     (sizeof(UpfrontLeadingArgs) + alignof(PackedArgs) - 1) / alignof(PackedArgs) * alignof(PackedArgs);
 static_assert(kUpfrontPackedArgsOffset == 56, "argument layout of FcInt8UpfrontGemvKernel");
 
-template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY, int WAVES>
+__global__ __launch_bounds__(WAVES * kWaveSize)
+__attribute__((amdgpu_waves_per_eu(WAVES / 2, WAVES / 2)))
 void FcInt8UpfrontGemvKernel(
     const int8_t* early_filter, const float* early_input_f32, const int8_t* early_input_i8,
     int early_depth, int early_slabs, int early_out_depth, int batch0, int bt, int ksplit_log2,
     int per_part, PackedArgs p) {
   extern __shared__ __align__(16) int8_t smem[];
-  const FcInt8Args& a = p.a;
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
   const int ksplit = 1 << ksplit_log2;
@@ -539,9 +535,9 @@ void FcInt8UpfrontGemvKernel(
   // multiplies its (clamped, re-read) tiles by zeros instead of branching.
   const int staged = ksplit * per_part * kSlabDepth;
   const int qstride = staged + kQPad;
-  const Shared sh = CarveShared(smem, bt, qstride);
+  const Shared sh = CarveShared(smem, bt, qstride, WAVES);
   const int tiles = (early_out_depth + kTileRows - 1) / kTileRows;
-  const int tile = ((blockIdx.x * kWaves) >> ksplit_log2) + (wave >> ksplit_log2);
+  const int tile = ((blockIdx.x * WAVES) >> ksplit_log2) + (wave >> ksplit_log2);
   const int part = wave & (ksplit - 1);
   const int s0 = part * per_part;
   const int8_t* group_base =
@@ -567,6 +563,11 @@ void FcInt8UpfrontGemvKernel(
     __builtin_amdgcn_sched_barrier(0);  // issue order = the order the products take them in
   };
 
+  // The row parameters of this lane's batch column: read from LDS behind the barrier (fused) or
+  // requested with the per-channel parameters (rows that arrive quantized).
+  float lds_scale = 0.0f;
+  int32_t lds_zp = 0, lds_zero = 0;
+  bool ep_has_row_zero_points = false;
   // Per-channel epilogue parameters, requested behind the first tiles (they are needed last).
   // Unconditional loads: an absent array reads a valid dummy address.
   int32_t ep_i0[4], ep_i1[4], ep_i2[4], ep_i3[4];
@@ -595,6 +596,16 @@ void FcInt8UpfrontGemvKernel(
       const int32_t* row_sums = late->a.filter_row_sums;
       const float* scales = late->a.per_channel_scales;
       const float* bias = late->a.bias_f32;
+      if (!FUSED) {
+        // The rows' own parameters: a global load in the epilogue would queue behind the
+        // whole weight stream.
+        const float* row_scales = late->a.scaling_factors;
+        const int32_t* row_zero_points = late->a.zero_points;
+        const int row = batch0 + min(col, bt - 1);
+        lds_scale = row_scales[row];
+        lds_zp = *(row_zero_points ? row_zero_points + row : dummy_i);
+        ep_has_row_zero_points = row_zero_points != nullptr;
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int n = min(min(tile, tiles - 1) * kTileRows + 4 * kgroup + i, out_depth - 1);
@@ -613,8 +624,6 @@ void FcInt8UpfrontGemvKernel(
   int ep_activation, ep_flags, ep_batches;
   float ep_filter_scale;
   int32_t ep_offsets0, ep_offsets1, ep_offsets2, ep_offsets3;
-  const float* ep_scaling_factors;
-  const int32_t* ep_zero_points;
   auto fetch_epilogue_scalars = [&]() {
     const LateArgs* late = late_args();
     ep_out = EPI == Int8Epilogue::kRequantize ? static_cast<void*>(late->a.output_i8)
@@ -629,8 +638,6 @@ void FcInt8UpfrontGemvKernel(
     ep_offsets2 = late->a.act_min;
     ep_offsets3 = late->a.act_max;
     ep_batches = late->a.batches;
-    ep_scaling_factors = late->a.scaling_factors;
-    ep_zero_points = late->a.zero_points;
   };
   const int8_t* qbase = sh.q + (col < bt ? col : 0) * qstride + kgroup * 16 + s0 * kSlabDepth;
   const int8_t* pad_zero = sh.q + staged;  // the kQPad bytes behind row 0, cleared below
@@ -670,6 +677,11 @@ void FcInt8UpfrontGemvKernel(
     // the whole chip's weight stream and costs some hundred nanoseconds of every launch.
     fetch_epilogue_scalars();
     __syncthreads();
+    if (FUSED) {  // the row's parameters for the epilogue, while nothing waits for them
+      lds_scale = sh.sf[col < bt ? col : 0];
+      lds_zp = sh.zp[col < bt ? col : 0];
+      lds_zero = sh.zero[col < bt ? col : 0];
+    }
 #pragma unroll
     for (int g = 0; g < kAhead - kLag; g += 4) multiply4(g);
 #pragma unroll
@@ -683,15 +695,12 @@ void FcInt8UpfrontGemvKernel(
   };
   using std::integral_constant;
 
-#ifndef LRT_V_SLEEP
-#define LRT_V_SLEEP 8
-#endif
   if (FUSED) {
     if (wave < bt) {
       __builtin_amdgcn_s_setprio(3);
       // This wavefront's row: 16 pieces of 16 bytes per lane (depth <= 4096).
       constexpr int kPieces = 16;
-      constexpr int kEarly = EARLY ? (TILES < 8 ? TILES : 8) : 0;
+      constexpr int kEarly = EARLY ? (WAVES > 4 ? 4 : (TILES < 8 ? TILES : 8)) : 0;
       const float* x = early_input_f32 + static_cast<size_t>(batch0 + wave) * depth;
       float4 xr[kPieces];
 #pragma unroll
@@ -742,19 +751,21 @@ void FcInt8UpfrontGemvKernel(
       __builtin_amdgcn_sched_barrier(0);
       stream(integral_constant<int, kEarly>{}, integral_constant<int, (kEarly > kStreamLag ? kEarly : kStreamLag)>{});
     } else {
-      if (LRT_V_SLEEP) __builtin_amdgcn_s_sleep(LRT_V_SLEEP);
+      __builtin_amdgcn_s_sleep(8);  // 512 cycles: the rows' requests go first
       stream(integral_constant<int, 0>{}, integral_constant<int, kStreamAhead>{});
     }
   } else {
     // Rows that arrive quantized: up to 16 rows of depth 4096, 16 bytes per thread and piece,
     // requested ahead of the weights and written to LDS when they are there.
-    constexpr int kQRegs = 4;
+    // 16-byte pieces of quantized rows per thread: 4 rows of depth 4096, or 16 (EARLY, which
+    // has no other meaning for rows that arrive quantized).
+    constexpr int kQRegs = (EARLY ? 64 : 16) / WAVES;
     constexpr int kFirst = TILES < 8 ? TILES : 8;
     i32x4 qr[kQRegs];
     const int chunks_per_row = staged / 16;
 #pragma unroll
     for (int j = 0; j < kQRegs; ++j) {
-      const int c = j * kThreads + tid;
+      const int c = j * (WAVES * kWaveSize) + tid;
       const int b = min(c / chunks_per_row, bt - 1);
       const int i = (c % chunks_per_row) * 16;
       qr[j] = *reinterpret_cast<const i32x4*>(
@@ -765,7 +776,7 @@ void FcInt8UpfrontGemvKernel(
     for (int u = 0; u < kFirst; ++u) request(u);
 #pragma unroll
     for (int j = 0; j < kQRegs; ++j) {
-      const int c = j * kThreads + tid;
+      const int c = j * (WAVES * kWaveSize) + tid;
       const int b = c / chunks_per_row;
       const int i = (c % chunks_per_row) * 16;
       if (b < bt) {
@@ -811,9 +822,9 @@ void FcInt8UpfrontGemvKernel(
   // Float epilogues. The four values of a lane are computed side by side without branches (the
   // tail of the slowest wavefront is the tail of the launch); the one rare case that needs a
   // scan of the input, a whole-zero input meeting a -0.0f bias, takes a branch of its own.
-  const float batch_scale = FUSED ? sh.sf[col] : ep_scaling_factors[b];
-  const int32_t batch_zp = FUSED ? sh.zp[col] : (ep_zero_points ? ep_zero_points[b] : 0);
-  const bool row_zero = FUSED ? sh.zero[col] != 0 : true;
+  const float batch_scale = lds_scale;
+  const int32_t batch_zp = (FUSED || ep_has_row_zero_points) ? lds_zp : 0;
+  const bool row_zero = FUSED ? lds_zero != 0 : true;
   float value[4];
   bool rare = false;
 #pragma unroll
@@ -878,65 +889,84 @@ void FcInt8UpfrontGemvKernel(
 }
 
 // How many wavefronts share one channel group's depth (see LaunchSized below).
-int ChooseKsplit(int slabs, int tiles) {
+int ChooseKsplit(int slabs, int tiles, int waves = kWaves) {
   int ksplit = 1;
-  while (ksplit < kWaves && slabs / (ksplit * 2) >= 2 * kRing) ksplit *= 2;
-  while (ksplit < kWaves && tiles * ksplit < 1024 && slabs / (ksplit * 2) >= 4) ksplit *= 2;
+  while (ksplit < waves && slabs / (ksplit * 2) >= 2 * kRing) ksplit *= 2;
+  while (ksplit < waves && tiles * ksplit < 1024 && slabs / (ksplit * 2) >= 4) ksplit *= 2;
   return ksplit;
 }
 
-template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY>
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY, int WAVES = kWaves>
 hipError_t LaunchUpfrontSized(const PackedArgs& p, int batch0, int bt, int ksplit,
                               hipStream_t stream) {
   const int per_part = (p.slabs + ksplit - 1) / ksplit;
   const int qstride = ksplit * per_part * kSlabDepth + kQPad;
-  const size_t lds = SharedBytes(bt, qstride);
-  auto kernel = FcInt8UpfrontGemvKernel<EPI, FUSED, VARIANT, TILES, EARLY>;
+  const size_t lds = SharedBytes(bt, qstride, WAVES);
+  auto kernel = FcInt8UpfrontGemvKernel<EPI, FUSED, VARIANT, TILES, EARLY, WAVES>;
   if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
-  const int tiles_per_wg = kWaves / ksplit;
+  const int tiles_per_wg = WAVES / ksplit;
   const int grid = (tiles + tiles_per_wg - 1) / tiles_per_wg;
   int ksplit_log2 = 0;
   while ((1 << ksplit_log2) < ksplit) ++ksplit_log2;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, p.a.filter, p.input_f32,
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(WAVES * kWaveSize), lds, stream, p.a.filter, p.input_f32,
                      p.a.input, p.a.depth, p.slabs, p.a.out_depth, batch0, bt, ksplit_log2,
                      per_part, p);
   return hipGetLastError();
 }
 
-// Whether the all-up-front form takes this launch; *launched tells. It needs a wavefront's share
-// of the depth to fit TILES tiles, and rows that fit the registers set aside for them.
+// Whether the register-resident form takes this launch; *launched tells. It needs a wavefront's
+// share of the depth to fit its tile registers, and rows that fit the registers set aside for
+// them. Workgroups of four wavefronts with up to 32 tiles each serve one fused row and rows that
+// arrive quantized; two to eight fused rows take workgroups of eight wavefronts with up to 16
+// tiles each, so that the wavefronts that quantize (one per row) leave as many that only
+// stream (measured at 14336 x 4096, one launch, cold: 1 row 11.0 us narrow / 11.4 wide; 2 rows
+// 11.4 / 11.3; 4 rows 12.6 / 12.0; 8 rows 13.1 wide against 14.7 as row quantizer + product).
 template <Int8Epilogue EPI, bool FUSED, int VARIANT>
 hipError_t TryLaunchUpfront(const PackedArgs& p, int batch0, int bt, hipStream_t stream,
                             bool* launched) {
   *launched = false;
   const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
   const int depth = p.a.depth;
+  if (FUSED) {
+    const bool vec_ok =
+        (depth % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.input_f32) & 15) == 0);
+    if (!vec_ok || depth > kFusedRowMaxDepth || depth < 4 || bt > kFusedMaxRows) return hipSuccess;
+    if (bt > 1) {
+      int ksplit = 1;
+      while ((p.slabs + ksplit - 1) / ksplit > 16) ksplit *= 2;  // depth <= 4096: at most 4
+      const int per_part = (p.slabs + ksplit - 1) / ksplit;
+      *launched = true;
+      if (per_part <= 8) {
+        return bt > 4 ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, true, 8>(p, batch0, bt, ksplit, stream)
+                      : LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, false, 8>(p, batch0, bt, ksplit, stream);
+      }
+      return bt > 4 ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, true, 8>(p, batch0, bt, ksplit, stream)
+                    : LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, false, 8>(p, batch0, bt, ksplit, stream);
+    }
+  }
   int ksplit = ChooseKsplit(p.slabs, tiles);
   while (ksplit < kWaves && (p.slabs + ksplit - 1) / ksplit > 32) ksplit *= 2;
   const int per_part = (p.slabs + ksplit - 1) / ksplit;
   if (per_part > 32) return hipSuccess;
-  if (FUSED) {
-    const bool vec_ok =
-        (depth % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.input_f32) & 15) == 0);
-    if (!vec_ok || depth > 4096 || depth < 4 || bt > kWaves) return hipSuccess;
-  } else {
+  bool many_rows = false;
+  if (!FUSED) {
     const bool vec_ok = (depth % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a.input) & 15) == 0);
     const int64_t chunks = static_cast<int64_t>(bt) * (ksplit * per_part * kSlabDepth / 16);
-    if (!vec_ok || chunks > 4 * kThreads) return hipSuccess;
+    if (!vec_ok || chunks > 16 * kThreads) return hipSuccess;
+    many_rows = chunks > 4 * kThreads;
   }
   *launched = true;
-  const bool early = FUSED && bt > 2;
   if (per_part <= 8) {
-    return early ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, FUSED>(p, batch0, bt, ksplit, stream)
-                 : LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, false>(p, batch0, bt, ksplit, stream);
+    return many_rows ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, !FUSED>(p, batch0, bt, ksplit, stream)
+                     : LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, false>(p, batch0, bt, ksplit, stream);
   }
   if (per_part <= 16) {
-    return early ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, FUSED>(p, batch0, bt, ksplit, stream)
-                 : LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, false>(p, batch0, bt, ksplit, stream);
+    return many_rows ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, !FUSED>(p, batch0, bt, ksplit, stream)
+                     : LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, false>(p, batch0, bt, ksplit, stream);
   }
-  return early ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 32, FUSED>(p, batch0, bt, ksplit, stream)
-               : LaunchUpfrontSized<EPI, FUSED, VARIANT, 32, false>(p, batch0, bt, ksplit, stream);
+  return many_rows ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 32, !FUSED>(p, batch0, bt, ksplit, stream)
+                   : LaunchUpfrontSized<EPI, FUSED, VARIANT, 32, false>(p, batch0, bt, ksplit, stream);
 }
 
 template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS, int XREGS = 4>
@@ -964,8 +994,7 @@ hipError_t LaunchSized(const PackedArgs& p, int batch0, int bt, hipStream_t stre
 
 template <Int8Epilogue EPI, bool FUSED, int VARIANT>
 hipError_t LaunchOne(const PackedArgs& p, int batch0, int bt, hipStream_t stream) {
-  static const bool use_upfront = getenv("LRT_GEMV_OLD") == nullptr;
-  if (use_upfront) {
+  {
     bool launched = false;
     hipError_t err = TryLaunchUpfront<EPI, FUSED, VARIANT>(p, batch0, bt, stream, &launched);
     if (launched || err != hipSuccess) return err;
@@ -1026,6 +1055,12 @@ hipError_t LaunchPackInt8Filter(const int8_t* filter, int out_depth, int depth, 
   hipLaunchKernelGGL(PackInt8FilterKernel, dim3(grid), dim3(kThreads), 0, stream, filter,
                      out_depth, depth, slabs, chunks, packed);
   return hipGetLastError();
+}
+
+int FcInt8PackedGemvFusedMaxRows(int depth) {
+  // Eight rows where a wavefront can hold a whole row (the register-resident form: one wavefront
+  // of eight per row); four on deeper rows, which every wavefront of a workgroup quantizes.
+  return (depth % 4 == 0 && depth <= kFusedRowMaxDepth) ? kFusedMaxRows : 4;
 }
 
 bool FcInt8PackedGemvSupports(const FcInt8Args& a) {

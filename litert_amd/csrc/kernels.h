@@ -99,6 +99,8 @@ size_t PackedInt8FilterBytes(int out_depth, int depth);
 hipError_t LaunchPackInt8Filter(const int8_t* filter, int out_depth, int depth, int8_t* packed,
                                 hipStream_t stream);
 bool FcInt8PackedGemvSupports(const FcInt8Args& a);
+// Rows up to which the fused (quantize-in-kernel) form beats quantizer launch + product.
+int FcInt8PackedGemvFusedMaxRows(int depth);
 hipError_t LaunchFcInt8PackedGemv(const FcInt8Args& a, Int8Epilogue epilogue,
                                   const float* input_f32, int asymmetric, int variant,
                                   hipStream_t stream);

@@ -201,7 +201,7 @@ class FullyConnectedHybrid:
         batches = x.numel() // self.depth
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
-        if self.packed_filter is not None and batches > self.FUSED_MAX_BATCHES:
+        if self.packed_filter is not None and batches > self._fused_max():
             return self.call_split(x, out)
         if self.packed_filter is not None:
             capi.check(capi.load().lrtfc_fc_hybrid_packed(
@@ -217,9 +217,14 @@ class FullyConnectedHybrid:
         return out
 
 
-    # Above this many rows the fused kernel's prologue (every workgroup quantizes every row)
-    # costs more than a separate quantization launch.
-    FUSED_MAX_BATCHES = 4
+    # Above this many rows the fused kernel's prologue costs more than a separate quantization
+    # launch: None = what the library says for the shape (lrtfc_fc_hybrid_fused_max_batches).
+    FUSED_MAX_BATCHES = None
+
+    def _fused_max(self):
+        if self.FUSED_MAX_BATCHES is not None:
+            return self.FUSED_MAX_BATCHES
+        return capi.load().lrtfc_fc_hybrid_fused_max_batches(self.depth, self.out_depth)
 
     def call_split(self, x, out=None):
         """Two launches on the packed filter: the standalone row quantizer, then the
