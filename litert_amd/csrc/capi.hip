@@ -1,5 +1,6 @@
 // C-ABI layer of the gfx950 FULLY_CONNECTED kernels: argument checking, the
 // Prepare-time host math, and dispatch to the kernel launchers.
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -31,7 +32,11 @@ int FromHip(hipError_t err, const char* what) {
 
 hipStream_t AsStream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
-bool g_initialised = false;
+// Process-wide state, shared by every interpreter and thread that uses the library: whether a
+// gfx950 device has been found, and the per-device scratch addresses below. Written under
+// g_init_mutex by lrtfc_init, read without it by the compute entry points.
+std::atomic<bool> g_initialised{false};
+std::mutex g_init_mutex;
 
 // Scratch of lrtfc_fc_hybrid_static_scratch, the entry point that allocates nothing: the
 // activation workspace (quantized rows, scaling factors, zero points) that lrtfc_fc_hybrid
@@ -41,7 +46,7 @@ bool g_initialised = false;
 // up once per device and the entry point passes that pointer to the kernels.
 static __device__ __align__(256) unsigned char scratch[LRTFC_STATIC_SCRATCH_BYTES];
 constexpr int kMaxDevices = 64;
-void* g_scratch_ptr[kMaxDevices] = {};
+std::atomic<void*> g_scratch_ptr[kMaxDevices] = {};
 
 int RequireInit() {
   if (g_initialised) return LRTFC_OK;
@@ -104,6 +109,7 @@ int lrtfc_abi_version(void) { return LRTFC_ABI_VERSION; }
 const char* lrtfc_last_error(void) { return g_last_error; }
 
 int lrtfc_init(int device_ordinal) {
+  std::lock_guard<std::mutex> lock(g_init_mutex);
   int count = 0;
   hipError_t err = hipGetDeviceCount(&count);
   if (err != hipSuccess || count == 0) {
@@ -119,13 +125,13 @@ int lrtfc_init(int device_ordinal) {
   err = hipGetDeviceProperties(&prop, device_ordinal);
   if (err != hipSuccess) return FromHip(err, "hipGetDeviceProperties");
   if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
-    g_initialised = false;
+    // Another caller's successful init of a gfx950 device stands.
     return Fail(LRTFC_NO_DEVICE, "device %d is %s; this library is built for gfx950 only",
                 device_ordinal, prop.gcnArchName);
   }
   err = hipSetDevice(device_ordinal);
   if (err != hipSuccess) return FromHip(err, "hipSetDevice");
-  if (device_ordinal < kMaxDevices && g_scratch_ptr[device_ordinal] == nullptr) {
+  if (device_ordinal < kMaxDevices && g_scratch_ptr[device_ordinal].load() == nullptr) {
     void* ptr = nullptr;
     err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (err != hipSuccess) return FromHip(err, "hipGetSymbolAddress(scratch)");
@@ -680,7 +686,7 @@ int lrtfc_fc_hybrid_static_scratch(const float* input, const int8_t* filter,
                 batches, depth, WorkspaceBytes(batches, depth), LRTFC_STATIC_SCRATCH_BYTES);
   int device = -1;
   if (hipError_t err = hipGetDevice(&device)) return FromHip(err, "hipGetDevice");
-  void* ptr = (device >= 0 && device < kMaxDevices) ? g_scratch_ptr[device] : nullptr;
+  void* ptr = (device >= 0 && device < kMaxDevices) ? g_scratch_ptr[device].load() : nullptr;
   if (ptr == nullptr) {
     return Fail(LRTFC_NO_DEVICE,
                 "lrtfc_init() has not run for device %d: its scratch address is unknown", device);

@@ -357,18 +357,25 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
       return FcKind::kInt4Blockwise;
     }
     if (filter.type == kTfLiteInt4 && filter.quantization.type == kTfLiteAffineQuantization) {
-      // The builtin's optimized 4-bit path (EvalHybridDense4Bit); outside its gate
-      // (fully_connected.cc:609-613) the builtin unpacks to int8 and runs the ordinary hybrid
-      // kernels, which quantize differently: those shapes stay on the CPU.
+      // The builtin's optimized 4-bit path (EvalHybridDense4Bit) inside its gate, the ordinary
+      // hybrid kernels on the unpacked filter outside it.
       if (!opt.claim_int4_per_channel) return no("int4 per-channel path disabled by option");
       if (!ClippingActivation(params->activation) && params->activation != kTfLiteActSignBit) {
         return no("activation is tanh or sigmoid");
       }
-      if (depth % 2 != 0 || out_depth < 4 || depth < 32) return no("shape outside 4-bit gate");
       const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
       if (!fq || !fq->scale || fq->scale->size < 1) return no("filter has no scales");
       if (fq->scale->size > 1 && (fq->quantized_dimension != 0 || fq->scale->size != out_depth)) {
         return no("per-channel scales do not match output channels");
+      }
+      if (depth % 2 != 0 || out_depth < 4 || depth < 32) {
+        // Outside the gate of the 4-bit path (fully_connected.cc:609-613) the builtin unpacks the
+        // nibbles to int8 on every Eval and runs the ordinary hybrid kernels on them
+        // (EvalHybridDense, fully_connected.cc:805-814). Here: unpacked once at prepare, then the
+        // int8 hybrid path.
+        if (!opt.claim_hybrid) return no("hybrid path disabled by option");
+        if (depth == 0) return no("empty depth");
+        return FcKind::kHybrid;
       }
       // Both kernels of this path stage a whole activation row in LDS; rows too deep for that
       // are declined here rather than failing at invoke.
@@ -592,6 +599,8 @@ struct PartitionKernel {
     lrtfc_int4_group_launch launch{};
   };
   std::vector<Group> groups;
+  // What TfLiteRegistration::profiling_string reports for this partition (built at prepare).
+  std::string profile_text;
   ~PartitionKernel() {
     for (hipEvent_t e : node_done) {
       if (e) (void)hipEventDestroy(e);
@@ -947,7 +956,18 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
     n->split_quantize = n->batches > lrtfc_fc_hybrid_fused_max_batches(n->depth, n->out_depth);
     if (weights > 0 && !(n->use_retiled ? n->have_retiled : n->have_model_layout)) {
       if (!n->have_model_layout) {
-        RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
+        if (filter.type == kTfLiteInt4) {
+          // An Int4 filter outside the 4-bit gate: UnpackPackedIntToInt8 over the flat tensor
+          // (fully_connected.cc:805-814), once here instead of on every Eval.
+          DeviceBuffer packed;
+          RETURN_IF_HIP(ctx, packed.Upload(filter.data.raw, (weights + 1) / 2, s));
+          RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
+          RETURN_IF_FC(ctx, lrtfc_unpack_int4(packed.as<uint8_t>(), static_cast<int64_t>(weights),
+                                              n->filter_dev.as<int8_t>(), s));
+          RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+        } else {
+          RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
+        }
         RETURN_IF_HIP(ctx, n->row_sums_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
         RETURN_IF_FC(ctx, lrtfc_row_sums_int8(n->filter_dev.as<int8_t>(), n->out_depth, n->depth,
                                               n->row_sums_dev.as<int32_t>(), s));
@@ -1261,7 +1281,33 @@ TfLiteStatus KernelPrepare(TfLiteContext* ctx, TfLiteNode* node) {
   }
   RETURN_IF_OK(PlanSchedule(ctx, k));
   RETURN_IF_HIP(ctx, hipStreamSynchronize(k->stream));
+  // The profiler's summary groups executions by this text (tflite/core/c/common.h:1264-1270,
+  // profile_summarizer.cc:84-88): the node kinds of the partition with their counts, and how
+  // many launch units they form (a grouped launch of several nodes counts once; a unit may be
+  // a row quantizer launch followed by a product launch).
+  static const char* const kKindNames[] = {"none", "int8", "hybrid", "int4_blockwise",
+                                           "int4_per_channel", "embedding_lookup",
+                                           "batch_matmul"};
+  int per_kind[7] = {0, 0, 0, 0, 0, 0, 0};
+  int ungrouped = 0;
+  for (const FcNode& n : k->nodes) {
+    ++per_kind[static_cast<int>(n.kind)];
+    if (n.group < 0) ++ungrouped;
+  }
+  std::string text;
+  for (int kind = 1; kind < 7; ++kind) {
+    if (per_kind[kind] == 0) continue;
+    text += (text.empty() ? "" : " ") + std::string(kKindNames[kind]) + ":" +
+            std::to_string(per_kind[kind]);
+  }
+  text += " launches:" + std::to_string(k->groups.size() + ungrouped);
+  k->profile_text = text;
   return kTfLiteOk;
+}
+
+const char* KernelProfilingString(const TfLiteContext*, const TfLiteNode* node) {
+  const auto* k = node ? static_cast<const PartitionKernel*>(node->user_data) : nullptr;
+  return k ? k->profile_text.c_str() : nullptr;
 }
 
 // Which registered memory each boundary tensor is bound to now; on a change, the tensors are
@@ -1604,7 +1650,7 @@ TfLiteRegistration KernelRegistration() {
   r.free = KernelFree;
   r.prepare = KernelPrepare;
   r.invoke = KernelInvoke;
-  r.profiling_string = nullptr;
+  r.profiling_string = KernelProfilingString;
   r.builtin_code = kTfLiteBuiltinDelegate;
   r.custom_name = "LiteRtAmdFullyConnected";
   r.version = 1;

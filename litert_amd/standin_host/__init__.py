@@ -265,6 +265,13 @@ class FakeHost:
         n = lib.litert_amd_describe_partition(self.L.fh_node_user_data(self.h, node), buf, 4096)
         return n, buf.value.decode()
 
+    def profiling_string(self, node):
+        """TfLiteRegistration::profiling_string of the node, or None."""
+        self.L.fh_node_profiling_string.restype = C.c_char_p
+        self.L.fh_node_profiling_string.argtypes = [C.c_void_p, C.c_int]
+        text = self.L.fh_node_profiling_string(self.h, node)
+        return None if text is None else text.decode()
+
     def node_io(self, node):
         ins = [self.L.fh_node_input(self.h, node, i) for i in range(self.L.fh_node_num_inputs(self.h, node))]
         outs = [self.L.fh_node_output(self.h, node, i) for i in range(self.L.fh_node_num_outputs(self.h, node))]

@@ -522,6 +522,14 @@ int fh_tensor_has_delegate(void* hp, int tensor) {
   return static_cast<Host*>(hp)->tensors[tensor].delegate != nullptr;
 }
 void* fh_node_user_data(void* hp, int node) { return static_cast<Host*>(hp)->nodes[node]->node.user_data; }
+// What the node's registration reports to a profiler (profile_summarizer.cc:84-88 calls it
+// with the interpreter's context and the node); nullptr when the registration has none.
+const char* fh_node_profiling_string(void* hp, int node) {
+  auto* h = static_cast<Host*>(hp);
+  const auto& rec = h->nodes[node];
+  if (!rec->reg.profiling_string) return nullptr;
+  return rec->reg.profiling_string(&h->ctx, &rec->node);
+}
 int fh_replace_calls(void* hp) { return static_cast<Host*>(hp)->replace_calls; }
 const char* fh_errors(void* hp) { return static_cast<Host*>(hp)->errors.c_str(); }
 void fh_clear_errors(void* hp) { static_cast<Host*>(hp)->errors.clear(); }

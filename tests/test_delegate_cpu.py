@@ -95,8 +95,12 @@ def test_claim_predicate_float_activations():
         # per-channel int4 hybrid (EvalHybridDense4Bit): claimed inside the builtin's 4-bit gate
         assert h.classify(_float_node(h, filter_type=INT4))[0] == "int4_per_channel"
         assert h.classify(_float_node(h, filter_type=INT4, per_channel=False))[0] == "int4_per_channel"
-        assert h.classify(_float_node(h, filter_type=INT4, N=2)) == (None, "shape outside 4-bit gate")
-        assert h.classify(_float_node(h, filter_type=INT4, K=16)) == (None, "shape outside 4-bit gate")
+        # outside that gate the builtin unpacks the nibbles and runs the ordinary hybrid kernels
+        # (fully_connected.cc:805-814): claimed as a hybrid node
+        assert h.classify(_float_node(h, filter_type=INT4, N=2))[0] == "hybrid"
+        assert h.classify(_float_node(h, filter_type=INT4, K=16))[0] == "hybrid"
+        assert h.classify(_float_node(h, filter_type=INT4, K=16, activation=4)) == (
+            None, "activation is tanh or sigmoid")
         assert h.classify(_float_node(h, filter_type=INT4, activation=4)) == (None, "activation is tanh or sigmoid")
         assert h.classify(_float_node(h, filter_type=INT4, activation=5))[0] == "int4_per_channel"
         # scales along the depth are not per-output-channel scales

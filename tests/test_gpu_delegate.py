@@ -365,6 +365,76 @@ def test_int4_per_channel_hybrid_node_through_delegate(B, per_channel):
         assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
 
 
+def test_profiling_string_names_the_partition():
+    """TfLiteRegistration::profiling_string (tflite/core/c/common.h:1264-1270), which the
+    profiler's summary groups executions by (profile_summarizer.cc:84-88): the node kinds of the
+    partition with their counts, and its launch units."""
+    c8 = wl.int8_fc(1, 128, 64, seed=3)
+    ch = wl.hybrid_fc(2, 64, 32, seed=4)
+    with FakeHost() as h:
+        x = h.tensor(INT8, (1, 128), data=c8["x"])
+        h.affine(x, [c8["in_scale"]], [c8["in_zp"]])
+        w = h.tensor(INT8, (64, 128), data=c8["w"], const=True)
+        h.affine(w, c8["w_scale"])
+        b = h.tensor(INT32, (64,), data=c8["bias"], const=True)
+        y = h.tensor(INT8, (1, 64))
+        h.affine(y, [c8["out_scale"]], [c8["out_zp"]])
+        n0 = h.fc(x, w, b, y)
+        xs, ys = [], []
+        for i in range(2):
+            xf = h.tensor(FLOAT32, (2, 64), data=ch["x"])
+            wf = h.tensor(INT8, (32, 64), data=ch["w"], const=True)
+            h.affine(wf, ch["pcs"])
+            yf = h.tensor(FLOAT32, (2, 32))
+            h.fc(xf, wf, None, yf)
+        assert h.profiling_string(n0) is None      # a builtin node's own registration has none here
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        kind, replaced, node = h.plan()[0]
+        assert kind == "delegate" and len(replaced) == 3
+        assert h.profiling_string(node) == "int8:1 hybrid:2 launches:3"
+        assert h.invoke() == OK, h.errors()
+        assert h.profiling_string(node) == "int8:1 hybrid:2 launches:3"
+
+
+@pytest.mark.parametrize("B,N,K,per_channel,asymmetric", [
+    (1, 2, 64, True, True),      # fewer than 4 output channels
+    (3, 8, 16, False, True),     # depth below 32
+    (2, 5, 33, True, False),     # odd depth: nibbles packed over the flat tensor, rows not byte-aligned
+    (20, 3, 48, True, True),     # prefill-sized batch on a narrow filter
+])
+def test_int4_affine_filter_outside_the_4bit_gate_runs_the_int8_hybrid_path(B, N, K, per_channel,
+                                                                            asymmetric):
+    """fully_connected.cc:609-613 keeps such shapes off EvalHybridDense4Bit; EvalHybridDense then
+    unpacks the nibbles to int8 (:805-814) and runs the ordinary hybrid kernels. Oracle:
+    unpack_int4 followed by fc_hybrid, both pinned on their own."""
+    from tests import kat_harness as kh
+    rng = np.random.default_rng(50 + N + K)
+    x_np = rng.standard_normal((B, K)).astype(np.float32)
+    w_np = rng.integers(-8, 8, (N, K)).astype(np.int8)
+    packed = kh.pack_int4(w_np.ravel())
+    fs = rng.uniform(0.01, 0.1, N).astype(np.float32) if per_channel else np.array([0.05], np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (B, K), data=x_np)
+        w = h.tensor(INT4, (N, K), data=packed, const=True)
+        h.affine(w, fs)
+        b = h.tensor(FLOAT32, (N,), data=bias, const=True)
+        y = h.tensor(FLOAT32, (B, N))
+        node = h.fc(x, w, b, y, activation=3, asymmetric=asymmetric)
+        assert h.classify(node)[0] == "hybrid"
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.plan()[0][:2] == ("delegate", [node])
+        assert h.invoke() == OK, h.errors()
+        unpacked = oracle.unpack_int4(packed, N * K).reshape(N, K)
+        assert np.array_equal(unpacked, w_np)
+        want = oracle.fc_hybrid(x_np, unpacked, fs if per_channel else None,
+                                1.0 if per_channel else float(fs[0]), bias, asymmetric,
+                                oracle.ACT_RELU6)
+        assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+
+
 def test_int4_per_channel_node_switches_layout_with_the_batch():
     """Decode batches run on the filter kept as nibbles, prefill batches on its int8 expansion;
     a resize moves the node from one to the other and back (prepare runs after every resize)."""
