@@ -235,7 +235,7 @@ def main():
     b_dom = 1
     achieved = hybrid_bytes(b_dom) / per_b[b_dom]["op_us_cold"] / 1e3
     roofline = dict(bound="hbm",
-                    kernel="FcInt8PackedGemvKernel<hybrid, fused quantize> (config 2, B=1, cold)",
+                    kernel="FcInt8ResidentGemvKernel<hybrid, fused quantize> (config 2, B=1, cold)",
                     achieved=round(achieved, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
                     frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=measured_traffic(),
                     traffic_source="profiles/hybrid_gemv_fused_B1_hbm_traffic.txt (rocprofv3 --pmc "

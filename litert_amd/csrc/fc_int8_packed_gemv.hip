@@ -14,18 +14,18 @@
 // depth, so a wavefront's load instruction reads 1 KiB of consecutive bytes and a
 // wavefront's whole share is one contiguous run.
 //
-// A wavefront streams a contiguous run of one 16-channel group's tiles through a ring of 16
-// outstanding 1 KiB loads, refilling a slot as soon as the matrix core has consumed it; four
-// wavefronts form a workgroup and share the staged activation rows. A group's depth is
-// shared out over 1, 2 or 4 wavefronts of the workgroup (int32 partial tiles added through
-// LDS: exact), chosen so that a wavefront's share stays about two rings long and the launch
-// has around a thousand wavefronts or more: shorter shares give more wavefronts per SIMD to
-// cover the prologue and the tail, longer ones amortize them better (14336 x 4096: two
-// wavefronts per group, 448 workgroups). The activation rows are
-// requested before the first weight load and staged in LDS while the ring fills. In the
-// hybrid form the staging step *is* the BatchQuantizeFloats of the op: the workgroup
-// reduces min/max of each float row, derives scale and zero point, and writes the
-// quantized row straight to LDS, so the op is a single kernel.
+// Two kernels run on this layout. FcInt8ResidentGemvKernel (further down, with its own
+// account) takes the launches whose per-wavefront share of the depth fits the registers:
+// depth up to 8192 at decode widths, i.e. the BASELINE shapes. FcInt8PackedGemvKernel is the
+// general form for everything else: a wavefront streams a contiguous run of one 16-channel
+// group's tiles through a ring of 16 outstanding 1 KiB loads, refilling a slot as soon as the
+// matrix core has consumed it; four wavefronts form a workgroup and share the staged
+// activation rows. A group's depth is shared out over 1, 2 or 4 wavefronts of the workgroup
+// (int32 partial tiles added through LDS: exact). The activation rows are requested before the
+// first weight load and staged in LDS while the ring fills. In the hybrid form the staging
+// step *is* the BatchQuantizeFloats of the op: the workgroup reduces min/max of each float
+// row, derives scale and zero point, and writes the quantized row straight to LDS, so the op
+// is a single kernel.
 #include "fc_epilogues.h"
 #include "kernels.h"
 #include "quantize_device.h"
@@ -503,18 +503,18 @@ constexpr int kStreamAhead = 24;  // tiles requested before the barrier (wavefro
 
 // Where `PackedArgs p` lies in the kernel's argument segment: behind three pointers and seven
 // ints, at its own alignment.
-struct UpfrontLeadingArgs {
+struct ResidentLeadingArgs {
   const void* pointers[3];
   int ints[7];
 };
-constexpr size_t kUpfrontPackedArgsOffset =
-    (sizeof(UpfrontLeadingArgs) + alignof(PackedArgs) - 1) / alignof(PackedArgs) * alignof(PackedArgs);
-static_assert(kUpfrontPackedArgsOffset == 56, "argument layout of FcInt8UpfrontGemvKernel");
+constexpr size_t kResidentPackedArgsOffset =
+    (sizeof(ResidentLeadingArgs) + alignof(PackedArgs) - 1) / alignof(PackedArgs) * alignof(PackedArgs);
+static_assert(kResidentPackedArgsOffset == 56, "argument layout of FcInt8ResidentGemvKernel");
 
 template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY, int WAVES>
 __global__ __launch_bounds__(WAVES * kWaveSize)
 __attribute__((amdgpu_waves_per_eu(WAVES / 2, WAVES / 2)))
-void FcInt8UpfrontGemvKernel(
+void FcInt8ResidentGemvKernel(
     const int8_t* early_filter, const float* early_input_f32, const int8_t* early_input_i8,
     int early_depth, int early_slabs, int early_out_depth, int batch0, int bt, int ksplit_log2,
     int per_part, PackedArgs p) {
@@ -552,7 +552,7 @@ void FcInt8UpfrontGemvKernel(
     auto* segment = (const __attribute__((address_space(4))) char*)
         __builtin_amdgcn_kernarg_segment_ptr();
     asm volatile("" : "+s"(segment));
-    return (LateArgs*)(segment + kUpfrontPackedArgsOffset);
+    return (LateArgs*)(segment + kResidentPackedArgsOffset);
   };
   i32x4 ring[TILES];
   auto request = [&](int u) {
@@ -897,12 +897,12 @@ int ChooseKsplit(int slabs, int tiles, int waves = kWaves) {
 }
 
 template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY, int WAVES = kWaves>
-hipError_t LaunchUpfrontSized(const PackedArgs& p, int batch0, int bt, int ksplit,
+hipError_t LaunchResidentSized(const PackedArgs& p, int batch0, int bt, int ksplit,
                               hipStream_t stream) {
   const int per_part = (p.slabs + ksplit - 1) / ksplit;
   const int qstride = ksplit * per_part * kSlabDepth + kQPad;
   const size_t lds = SharedBytes(bt, qstride, WAVES);
-  auto kernel = FcInt8UpfrontGemvKernel<EPI, FUSED, VARIANT, TILES, EARLY, WAVES>;
+  auto kernel = FcInt8ResidentGemvKernel<EPI, FUSED, VARIANT, TILES, EARLY, WAVES>;
   if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
   const int tiles_per_wg = WAVES / ksplit;
@@ -923,7 +923,7 @@ hipError_t LaunchUpfrontSized(const PackedArgs& p, int batch0, int bt, int kspli
 // stream (measured at 14336 x 4096, one launch, cold: 1 row 11.0 us narrow / 11.4 wide; 2 rows
 // 11.4 / 11.3; 4 rows 12.6 / 12.0; 8 rows 13.1 wide against 14.7 as row quantizer + product).
 template <Int8Epilogue EPI, bool FUSED, int VARIANT>
-hipError_t TryLaunchUpfront(const PackedArgs& p, int batch0, int bt, hipStream_t stream,
+hipError_t TryLaunchResident(const PackedArgs& p, int batch0, int bt, hipStream_t stream,
                             bool* launched) {
   *launched = false;
   const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
@@ -938,11 +938,11 @@ hipError_t TryLaunchUpfront(const PackedArgs& p, int batch0, int bt, hipStream_t
       const int per_part = (p.slabs + ksplit - 1) / ksplit;
       *launched = true;
       if (per_part <= 8) {
-        return bt > 4 ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, true, 8>(p, batch0, bt, ksplit, stream)
-                      : LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, false, 8>(p, batch0, bt, ksplit, stream);
+        return bt > 4 ? LaunchResidentSized<EPI, FUSED, VARIANT, 8, true, 8>(p, batch0, bt, ksplit, stream)
+                      : LaunchResidentSized<EPI, FUSED, VARIANT, 8, false, 8>(p, batch0, bt, ksplit, stream);
       }
-      return bt > 4 ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, true, 8>(p, batch0, bt, ksplit, stream)
-                    : LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, false, 8>(p, batch0, bt, ksplit, stream);
+      return bt > 4 ? LaunchResidentSized<EPI, FUSED, VARIANT, 16, true, 8>(p, batch0, bt, ksplit, stream)
+                    : LaunchResidentSized<EPI, FUSED, VARIANT, 16, false, 8>(p, batch0, bt, ksplit, stream);
     }
   }
   int ksplit = ChooseKsplit(p.slabs, tiles);
@@ -958,15 +958,15 @@ hipError_t TryLaunchUpfront(const PackedArgs& p, int batch0, int bt, hipStream_t
   }
   *launched = true;
   if (per_part <= 8) {
-    return many_rows ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, !FUSED>(p, batch0, bt, ksplit, stream)
-                     : LaunchUpfrontSized<EPI, FUSED, VARIANT, 8, false>(p, batch0, bt, ksplit, stream);
+    return many_rows ? LaunchResidentSized<EPI, FUSED, VARIANT, 8, !FUSED>(p, batch0, bt, ksplit, stream)
+                     : LaunchResidentSized<EPI, FUSED, VARIANT, 8, false>(p, batch0, bt, ksplit, stream);
   }
   if (per_part <= 16) {
-    return many_rows ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, !FUSED>(p, batch0, bt, ksplit, stream)
-                     : LaunchUpfrontSized<EPI, FUSED, VARIANT, 16, false>(p, batch0, bt, ksplit, stream);
+    return many_rows ? LaunchResidentSized<EPI, FUSED, VARIANT, 16, !FUSED>(p, batch0, bt, ksplit, stream)
+                     : LaunchResidentSized<EPI, FUSED, VARIANT, 16, false>(p, batch0, bt, ksplit, stream);
   }
-  return many_rows ? LaunchUpfrontSized<EPI, FUSED, VARIANT, 32, !FUSED>(p, batch0, bt, ksplit, stream)
-                   : LaunchUpfrontSized<EPI, FUSED, VARIANT, 32, false>(p, batch0, bt, ksplit, stream);
+  return many_rows ? LaunchResidentSized<EPI, FUSED, VARIANT, 32, !FUSED>(p, batch0, bt, ksplit, stream)
+                   : LaunchResidentSized<EPI, FUSED, VARIANT, 32, false>(p, batch0, bt, ksplit, stream);
 }
 
 template <Int8Epilogue EPI, bool FUSED, int VARIANT, int REG_ROWS, int XREGS = 4>
@@ -996,7 +996,7 @@ template <Int8Epilogue EPI, bool FUSED, int VARIANT>
 hipError_t LaunchOne(const PackedArgs& p, int batch0, int bt, hipStream_t stream) {
   {
     bool launched = false;
-    hipError_t err = TryLaunchUpfront<EPI, FUSED, VARIANT>(p, batch0, bt, stream, &launched);
+    hipError_t err = TryLaunchResident<EPI, FUSED, VARIANT>(p, batch0, bt, stream, &launched);
     if (launched || err != hipSuccess) return err;
   }
   if (!FUSED) {
