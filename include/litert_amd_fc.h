@@ -427,6 +427,29 @@ int lrtfc_fc_blockwise_int4_gemm(const float* input, const uint8_t* gemm_filter,
                                  int batches, int depth, int out_depth, int quant_variant,
                                  void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same GEMM on a filter that stays 4 bits per weight in device memory, for batches between
+ * decode and prefill (5 to a few dozen rows), where the filter stream bounds the kernel and the
+ * int8 form above would double it: lrtfc_pack_int4_blockwise_gemm_nibbles re-tiles the model's
+ * nibbles and fp16 scales into lrtfc_gemm_int4_blockwise_nibble_bytes(out_depth, depth) bytes
+ * (16-byte aligned), and lrtfc_fc_blockwise_int4_gemm_nibbles takes that filter with the
+ * arguments, the workspace and the results -- bit for bit -- of lrtfc_fc_blockwise_int4_gemm.
+ * A wavefront expands each block's nibbles to the matrix cores' int8 operand itself. */
+enum { LRTFC_INT4_FORM_DECODE = 0, LRTFC_INT4_FORM_GEMM_NIBBLES = 1, LRTFC_INT4_FORM_GEMM_INT8 = 2 };
+/* Which of the three forms of the blockwise-int4 op runs a shape fastest (block size 32): the
+ * streaming kernel of lrtfc_fc_blockwise_int4_packed (up to four rows per pass over the filter),
+ * this nibble-resident GEMM, or the int8-expanded GEMM. All three give the same bits; a caller
+ * keeps the filter in the one layout its batch size asks for. Pure host function. */
+int lrtfc_fc_blockwise_int4_preferred_form(int batches, int depth, int out_depth);
+size_t lrtfc_gemm_int4_blockwise_nibble_bytes(int out_depth, int depth);
+int lrtfc_pack_int4_blockwise_gemm_nibbles(const uint8_t* packed_filter,
+                                           const uint16_t* scales_f16, int out_depth, int depth,
+                                           int blocksize, uint8_t* nibble_filter, void* stream);
+int lrtfc_fc_blockwise_int4_gemm_nibbles(const float* input, const uint8_t* nibble_filter,
+                                         const float* kfsum, const float* bias, float* output,
+                                         int batches, int depth, int out_depth,
+                                         int quant_variant, void* workspace,
+                                         size_t workspace_bytes, void* stream);
+
 /* ---- EMBEDDING_LOOKUP from quantized tables (the op that feeds a decoder's first
  * FULLY_CONNECTED nodes) ------------------------------------------------------------------ */
 

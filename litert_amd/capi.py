@@ -16,6 +16,7 @@ ACT_NONE, ACT_RELU, ACT_RELU_N1_TO_1, ACT_RELU6 = range(4)
 ACT_SIGN_BIT = 5
 QUANT_PORTABLE, QUANT_NEON_V8, QUANT_NEON_LEGACY = range(3)
 OUT_FLOAT32, OUT_FLOAT16 = range(2)
+INT4_FORM_DECODE, INT4_FORM_GEMM_NIBBLES, INT4_FORM_GEMM_INT8 = range(3)
 
 # Every symbol include/litert_amd_fc.h declares: (name, restype, argtypes).
 _vp, _i, _i32, _i64, _f, _d, _sz = (C.c_void_p, C.c_int, C.c_int32, C.c_int64, C.c_float,
@@ -76,6 +77,11 @@ SYMBOLS = [
     ("lrtfc_pack_int4_blockwise_gemm", _i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     ("lrtfc_fc_blockwise_int4_gemm_workspace_bytes", _sz, [_i, _i]),
     ("lrtfc_fc_blockwise_int4_gemm", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
+    ("lrtfc_fc_blockwise_int4_preferred_form", _i, [_i, _i, _i]),
+    ("lrtfc_gemm_int4_blockwise_nibble_bytes", _sz, [_i, _i]),
+    ("lrtfc_pack_int4_blockwise_gemm_nibbles", _i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    ("lrtfc_fc_blockwise_int4_gemm_nibbles", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz,
+                                                  _vp]),
     ("lrtfc_embedding_lookup_blockwise_int4", _i, [_vp, _i, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_embedding_lookup_hybrid", _i, [_vp, _i, _vp, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp]),
     ("lrtfc_int4_group_table_bytes", _sz, []),

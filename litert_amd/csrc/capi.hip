@@ -975,6 +975,75 @@ int lrtfc_fc_blockwise_int4_gemm(const float* input, const uint8_t* gemm_filter,
                  "blockwise int4 GEMM");
 }
 
+int lrtfc_fc_blockwise_int4_preferred_form(int batches, int depth, int out_depth) {
+  if (depth <= 0 || depth % 32 != 0 || !lrtfc::FcInt4PackedSupports(depth, 32)) {
+    return LRTFC_INT4_FORM_DECODE;
+  }
+  // Up to four rows the streaming kernel makes one pass over the filter. Beyond that the GEMMs
+  // stream it once for the whole batch: the nibble-resident one where the filter stream is the
+  // bound (up to 32 rows) and the filter is wide enough to give every SIMD a wavefront (one
+  // wavefront per 16 channels walks the whole depth: 14336 x 4096 takes 16.8 us at 5 to 16
+  // rows against 24 us in two passes of the streaming kernel and 21 us on the int8 copy), the
+  // int8-expanded one from 16 rows on otherwise.
+  const int channel_tiles = (out_depth + 15) / 16;
+  if (batches <= 4) return LRTFC_INT4_FORM_DECODE;
+  if (batches <= 32 && channel_tiles >= 512 && depth <= 8192) return LRTFC_INT4_FORM_GEMM_NIBBLES;
+  return batches >= 16 ? LRTFC_INT4_FORM_GEMM_INT8 : LRTFC_INT4_FORM_DECODE;
+}
+
+size_t lrtfc_gemm_int4_blockwise_nibble_bytes(int out_depth, int depth) {
+  if (out_depth <= 0 || depth <= 0) return 0;
+  return lrtfc::GemmInt4BlockwiseNibbleBytes(out_depth, depth);
+}
+
+int lrtfc_pack_int4_blockwise_gemm_nibbles(const uint8_t* packed_filter,
+                                           const uint16_t* scales_f16, int out_depth, int depth,
+                                           int blocksize, uint8_t* nibble_filter, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(out_depth >= 0 && depth >= 0, "negative dimension");
+  if (out_depth == 0 || depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(packed_filter && scales_f16 && nibble_filter, "null pointer");
+  LRTFC_REQUIRE(lrtfc::FcInt4BlockwiseGemmSupports(depth, blocksize),
+                "the int4 GEMM needs block size 32 and a depth that is a multiple of 32");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(nibble_filter) & 15) == 0,
+                "re-tiled filter must be 16-byte aligned");
+  return FromHip(lrtfc::LaunchPackInt4BlockwiseNibbles(packed_filter, scales_f16, out_depth,
+                                                       depth, nibble_filter, AsStream(stream)),
+                 "int4 nibble GEMM filter re-tiling");
+}
+
+int lrtfc_fc_blockwise_int4_gemm_nibbles(const float* input, const uint8_t* nibble_filter,
+                                 const float* kfsum, const float* bias, float* output,
+                                 int batches, int depth, int out_depth, int quant_variant,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(batches >= 0 && depth > 0 && out_depth >= 0, "bad dimension");
+  if (batches == 0 || out_depth == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(input && nibble_filter && kfsum && output && workspace, "null pointer");
+  LRTFC_REQUIRE(lrtfc::FcInt4BlockwiseGemmSupports(depth, 32), "depth %d is not a multiple of 32",
+                depth);
+  LRTFC_REQUIRE(workspace_bytes >= lrtfc_fc_blockwise_int4_gemm_workspace_bytes(batches, depth),
+                "workspace too small: %zu < %zu bytes", workspace_bytes,
+                lrtfc_fc_blockwise_int4_gemm_workspace_bytes(batches, depth));
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
+                "workspace must be 256-byte aligned");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(nibble_filter) & 15) == 0,
+                "re-tiled filter must be 16-byte aligned");
+  LRTFC_REQUIRE(quant_variant >= LRTFC_QUANT_PORTABLE && quant_variant <= LRTFC_QUANT_NEON_LEGACY,
+                "unknown quantizer variant %d", quant_variant);
+  char* p = static_cast<char*>(workspace);
+  void* tiled = p;
+  p += lrtfc::AlignUp256(lrtfc::TiledRowsBytes(batches, depth));
+  float* scaling_factors = reinterpret_cast<float*>(p);
+  p += lrtfc::AlignUp256(static_cast<size_t>(batches) * 4);
+  int32_t* zero_points = reinterpret_cast<int32_t*>(p);
+  return FromHip(lrtfc::LaunchFcInt4BlockwiseNibbleGemm(input, quant_variant, scaling_factors,
+                                                  zero_points, nibble_filter, kfsum, bias, output,
+                                                  batches, depth, out_depth, tiled,
+                                                  AsStream(stream)),
+                 "blockwise int4 GEMM (nibble layout)");
+}
+
 int lrtfc_embedding_lookup_blockwise_int4(const int32_t* lookup, int count, const uint8_t* table,
                                           int rows, int cols, const uint16_t* scales_f16,
                                           int blocksize, int out_type, void* output,

@@ -476,6 +476,9 @@ struct FcNode {
   // Blockwise-int4 nodes run prefill batches on the filter re-tiled for the matrix-core GEMM
   // (retiled_dev then holds that form) and decode batches on the streaming form.
   bool gemm_layout = false, have_gemm = false;
+  // ... and batches in between on the GEMM that keeps the filter at 4 bits per weight
+  // (gemm_layout is set too; retiled_dev then holds that form).
+  bool gemm_nibbles = false;
   bool split_quantize = false;  // quantize rows in a launch of their own, not in the prologue
   // EMBEDDING_LOOKUP nodes: input = the lookup vector, filter = the table (filter_dev), batches =
   // lookups, depth = out_depth = columns of a row; block scales in scales_dev or per-row scales
@@ -506,9 +509,6 @@ constexpr int kInt4DeepFusedMaxBatches = 2;
 // Up to this many rows a per-channel int4 node streams its filter as nibbles (one pass per 16
 // rows); above, the MFMA GEMM on the int8 expansion streams it once.
 constexpr int kInt4PerChannelNibbleMaxBatches = 32;
-// From this many rows on a blockwise-int4 node streams its filter once through the GEMM instead
-// of once per four rows.
-constexpr int kInt4BlockwiseGemmMinBatches = 16;
 
 // Up to this many bytes of host outputs per partition are written by the kernels directly into
 // page-locked host memory instead of being copied there afterwards. The invariant this rests on:
@@ -1021,7 +1021,13 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
     n->use_retiled = weights > 0 && lrtfc_fc_blockwise_int4_preferred_layout(
                                         n->depth, n->blocksize) == LRTFC_LAYOUT_PACKED;
     n->split_quantize = n->depth > kInt4FusedMaxDepth && n->batches > kInt4DeepFusedMaxBatches;
-    n->gemm_layout = n->use_retiled && n->batches >= kInt4BlockwiseGemmMinBatches;
+    const int form = n->use_retiled ? lrtfc_fc_blockwise_int4_preferred_form(
+                                          n->batches, n->depth, n->out_depth)
+                                    : LRTFC_INT4_FORM_DECODE;
+    const bool want_nibbles = form == LRTFC_INT4_FORM_GEMM_NIBBLES;
+    n->gemm_layout = form != LRTFC_INT4_FORM_DECODE;
+    if (n->gemm_layout && n->have_gemm && want_nibbles != n->gemm_nibbles) n->have_gemm = false;
+    n->gemm_nibbles = want_nibbles;
     if (n->gemm_layout) {
       if (!n->have_gemm) {
         DeviceBuffer nibbles, block_scales;
@@ -1034,12 +1040,19 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
                                                      n->depth, n->blocksize,
                                                      n->kfsum_dev.as<float>(), s));
         n->retiled_dev.Release();
-        RETURN_IF_HIP(ctx, n->retiled_dev.Ensure(
-                               lrtfc_gemm_int4_blockwise_bytes(n->out_depth, n->depth)));
-        RETURN_IF_FC(ctx, lrtfc_pack_int4_blockwise_gemm(nibbles.as<uint8_t>(),
-                                                         block_scales.as<uint16_t>(), n->out_depth,
-                                                         n->depth, n->blocksize,
-                                                         n->retiled_dev.as<uint8_t>(), s));
+        if (n->gemm_nibbles) {
+          RETURN_IF_HIP(ctx, n->retiled_dev.Ensure(
+                                 lrtfc_gemm_int4_blockwise_nibble_bytes(n->out_depth, n->depth)));
+          RETURN_IF_FC(ctx, lrtfc_pack_int4_blockwise_gemm_nibbles(
+                                nibbles.as<uint8_t>(), block_scales.as<uint16_t>(), n->out_depth,
+                                n->depth, n->blocksize, n->retiled_dev.as<uint8_t>(), s));
+        } else {
+          RETURN_IF_HIP(ctx, n->retiled_dev.Ensure(
+                                 lrtfc_gemm_int4_blockwise_bytes(n->out_depth, n->depth)));
+          RETURN_IF_FC(ctx, lrtfc_pack_int4_blockwise_gemm(
+                                nibbles.as<uint8_t>(), block_scales.as<uint16_t>(), n->out_depth,
+                                n->depth, n->blocksize, n->retiled_dev.as<uint8_t>(), s));
+        }
         RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
         n->filter_dev.Release();
         n->scales_dev.Release();
@@ -1520,7 +1533,13 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                               n.out_depth, n.params.activation, scratch.get(), scratch.bytes(), s));
         break;
       case FcKind::kInt4Blockwise:
-        if (n.gemm_layout) {
+        if (n.gemm_layout && n.gemm_nibbles) {
+          RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4_gemm_nibbles(
+                                static_cast<const float*>(in_dev), n.retiled_dev.as<uint8_t>(),
+                                n.kfsum_dev.as<float>(), bias_f32, static_cast<float*>(out_dev),
+                                n.batches, n.depth, n.out_depth, variant, scratch.get(),
+                                scratch.bytes(), s));
+        } else if (n.gemm_layout) {
           RETURN_IF_FC(ctx, lrtfc_fc_blockwise_int4_gemm(
                                 static_cast<const float*>(in_dev), n.retiled_dev.as<uint8_t>(),
                                 n.kfsum_dev.as<float>(), bias_f32, static_cast<float*>(out_dev),

@@ -300,6 +300,236 @@ __global__ __launch_bounds__(kThreads) void FcInt4BlockwiseGemmKernel(GemmArgs a
   }
 }
 
+
+// ---- the same product on a filter that stays 4 bits per weight --------------------------
+//
+// For batches between decode and prefill (5 to a few dozen rows) the filter stream bounds the
+// kernel above, and sign-extending the nibbles to int8 at prepare doubles that stream. Here
+// the filter stays packed (`tile16x128n`) and a wavefront expands a block's nibbles itself,
+// three vector operations per block and 16 channels: for channel tile t and quad q of blocks
+// (128 depth positions), 1 KiB: lane L's 16 bytes are four dwords, dword j for block 4 q + j,
+// channel 16 t + L % 16, depths 8 (L / 16) ... + 8 of that block; byte k of a dword holds
+// weight k of those eight in its low nibble and weight k + 4 in its high one (two's
+// complement, as in the model). `(d << 4) & 0xF0F0F0F0` and `d & 0xF0F0F0F0` are then the
+// eight weights as int8 values 16 w, in depth order: the A operand of v_mfma_i32_16x16x32_i8.
+// Every block sum comes out multiplied by 16, hence every product and every partial sum of an
+// output (scaling by a power of two commutes with each rounding; fp16 scales times integers
+// stay far from the float32 range limits), and the finished sum is multiplied by 1/16 once.
+// Behind the weight tiles lie the block scales as fp16: per channel tile and group of 16
+// blocks, 512 bytes, lane L's 8 bytes = block 16 g + L % 16, channels 4 (L / 16) ... + 4.
+// Activations: `tile16x64`, as above. One channel tile per wavefront (these batch sizes want
+// the filter stream spread over as many wavefronts as possible).
+
+
+__global__ __launch_bounds__(kThreads) void PackInt4BlockwiseNibblesKernel(
+    const uint8_t* __restrict__ filter, const uint16_t* __restrict__ scales_f16, int out_depth,
+    int depth, int tiles, int nb, int nq, int ng, uint8_t* __restrict__ dst) {
+  const int64_t slot = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t slots = static_cast<int64_t>(tiles) * nq * 64;  // 16-byte lane slots
+  if (slot < slots) {
+    const int lane = static_cast<int>(slot & 63);
+    const int64_t tq = slot >> 6;
+    const int q = static_cast<int>(tq % nq);
+    const int t = static_cast<int>(tq / nq);
+    const int n = t * kTile + (lane & 15);
+    uint32_t d[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int b = 4 * q + j;
+      if (n < out_depth && b < nb) {
+        // the slice's 8 weights lie in 4 consecutive bytes of the model's row: byte m holds
+        // weights 2 m (low nibble) and 2 m + 1 (high nibble)
+        const uint8_t* src = filter + static_cast<size_t>(n) * (depth / 2) + b * (kBlock / 2) +
+                             4 * (lane >> 4);
+        uint32_t w[8];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          w[2 * m] = src[m] & 0xFu;
+          w[2 * m + 1] = src[m] >> 4;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) d[j] |= (w[k] | (w[k + 4] << 4)) << (8 * k);
+      }
+    }
+    reinterpret_cast<uint4*>(dst)[slot] = make_uint4(d[0], d[1], d[2], d[3]);
+  }
+  // scales: one thread per (tile, group of 16 blocks, lane)
+  const int64_t scale_slots = static_cast<int64_t>(tiles) * ng * 64;
+  if (slot < scale_slots) {
+    const int lane = static_cast<int>(slot & 63);
+    const int64_t tg = slot >> 6;
+    const int g = static_cast<int>(tg % ng);
+    const int t = static_cast<int>(tg / ng);
+    const int b = 16 * g + (lane & 15);
+    uint16_t h[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = t * kTile + 4 * (lane >> 4) + i;
+      if (n < out_depth && b < nb) h[i] = scales_f16[static_cast<size_t>(n) * nb + b];
+    }
+    uint2* out = reinterpret_cast<uint2*>(dst + slots * 16);
+    out[slot] = make_uint2(h[0] | (static_cast<uint32_t>(h[1]) << 16),
+                           h[2] | (static_cast<uint32_t>(h[3]) << 16));
+  }
+}
+
+struct NibbleGemmArgs {
+  const i32x4* filter;      // tile16x128n
+  const uint2* scales;      // fp16 [tiles][ng][64 lanes][4]
+  const i64x2* activations;  // tile16x64
+  const float* scaling_factors;
+  const int32_t* zero_points;
+  const float* kfsum;
+  const float* bias;
+  float* output;
+  int batches, out_depth, nb;
+  int channel_tiles, row_tiles;
+  int vector_store;
+};
+
+// WQ: quads of weights in flight per wavefront; XQ: quads of activations in flight (they come
+// from L2 and cost 8 registers per row tile and quad, so this ring is shorter). Measured at
+// 14336 x 4096, 16 rows: 8 and 4 quads 16.9 us for quantizer + product; 16 weight quads 18.1 us
+// -- a wavefront is alone on its SIMD here (896 wavefronts), and what bounds it is its own
+// chain of about 15 vector operations per block, not the loads.
+template <int RT, int WQ, int XQ>
+__global__ __launch_bounds__(kThreads) void FcInt4NibbleGemmKernel(NibbleGemmArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int ct0 = blockIdx.x * 4 + wave;
+  const int rt0 = blockIdx.y * RT;
+  if (ct0 >= a.channel_tiles || rt0 >= a.row_tiles) return;
+  int rt[RT];
+#pragma unroll
+  for (int j = 0; j < RT; ++j) rt[j] = min(rt0 + j, a.row_tiles - 1);
+  const int nb = a.nb;
+  const int pairs = (nb + 1) / 2;
+  const int nq = (nb + 3) / 4;
+  const int ng = (nb + 15) / 16;
+  const i32x4* wp = a.filter + static_cast<size_t>(ct0) * nq * 64 + lane;
+  const uint2* sp = a.scales + static_cast<size_t>(ct0) * ng * 64 + lane;
+  const i64x2* xp[RT];
+#pragma unroll
+  for (int j = 0; j < RT; ++j) {
+    xp[j] = a.activations + static_cast<size_t>(rt[j]) * pairs * 64 + lane;
+  }
+  // Past the end: a hot line, result unused.
+  auto fetch_w = [&](int q) {
+    return __builtin_nontemporal_load(wp + static_cast<size_t>(min(q, nq - 1)) * 64);
+  };
+  struct XStage {
+    i64x2 x[RT][2];  // row tiles: blocks 0-1, blocks 2-3 of the quad
+  };
+  auto fetch_x = [&](int q) {
+    const int qq = min(q, nq - 1);
+    XStage st;
+#pragma unroll
+    for (int j = 0; j < RT; ++j) {
+      st.x[j][0] = xp[j][static_cast<size_t>(min(2 * qq, pairs - 1)) * 64];
+      st.x[j][1] = xp[j][static_cast<size_t>(min(2 * qq + 1, pairs - 1)) * 64];
+    }
+    return st;
+  };
+  // Scale groups (16 blocks = 4 quads): the current one and as many ahead as the weight ring
+  // reaches, so that a group is requested before its blocks' weights.
+  constexpr int kGroups = WQ / 4 + 1 <= 2 ? 2 : (WQ / 4 + 1 <= 4 ? 4 : 8);
+  static_assert((kGroups - 1) * 4 >= WQ, "scale groups must lead the weight ring");
+  uint2 sg[kGroups];
+  auto fetch_scales = [&](int g) { return sp[static_cast<size_t>(min(g, ng - 1)) * 64]; };
+#pragma unroll
+  for (int g = 0; g + 1 < kGroups; ++g) sg[g] = fetch_scales(g);
+  i32x4 wring[WQ];
+  XStage xring[XQ];
+#pragma unroll
+  for (int s = 0; s < WQ; ++s) wring[s] = fetch_w(s);
+#pragma unroll
+  for (int s = 0; s < XQ; ++s) xring[s] = fetch_x(s);
+
+  // out[rj][i]: channel 16 ct0 + 4 (lane / 16) + i, batch row 16 rt[rj] + lane % 16, times 16.
+  float out[RT][4];
+#pragma unroll
+  for (int rj = 0; rj < RT; ++rj)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[rj][i] = 0.0f;
+
+  const i32x4 zero = {0, 0, 0, 0};
+  constexpr int kTrip = WQ > 4 * kGroups ? WQ : 4 * kGroups;
+  static_assert(kTrip % WQ == 0 && kTrip % XQ == 0 && kTrip % (4 * kGroups) == 0, "trip");
+  float4 cur_scales = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  for (int base = 0; base < nq; base += kTrip) {
+    StaticFor<kTrip>([&](auto u_const) {
+      constexpr int u = decltype(u_const)::value;
+      constexpr int cur = (u / 4) % kGroups;
+      if constexpr (u % 4 == 0) {
+        // A new group of 16 blocks starts: its scales become float32, and the slot of the group
+        // before it takes the farthest one.
+        const uint2 raw = sg[cur];
+        cur_scales = make_float4(HalfBitsToFloatFast(static_cast<uint16_t>(raw.x & 0xFFFF)),
+                                 HalfBitsToFloatFast(static_cast<uint16_t>(raw.x >> 16)),
+                                 HalfBitsToFloatFast(static_cast<uint16_t>(raw.y & 0xFFFF)),
+                                 HalfBitsToFloatFast(static_cast<uint16_t>(raw.y >> 16)));
+        sg[(cur + kGroups - 1) % kGroups] = fetch_scales((base + u) / 4 + kGroups - 1);
+      }
+      const i32x4 w = wring[u % WQ];
+      wring[u % WQ] = fetch_w(base + u + WQ);
+      const XStage st = xring[u % XQ];
+      xring[u % XQ] = fetch_x(base + u + XQ);
+      StaticFor<4>([&](auto h_const) {
+        constexpr int h = decltype(h_const)::value;
+        if (4 * (base + u) + h < nb) {
+          constexpr int j = (4 * u + h) % 16;  // this block within its scale group
+          const float sc[4] = {RowBroadcast<j>(cur_scales.x), RowBroadcast<j>(cur_scales.y),
+                               RowBroadcast<j>(cur_scales.z), RowBroadcast<j>(cur_scales.w)};
+          const uint32_t d = static_cast<uint32_t>(w[h]);
+          const uint32_t lo = (d << 4) & 0xF0F0F0F0u;
+          const uint32_t hi = d & 0xF0F0F0F0u;
+          const i64 wa = static_cast<i64>(static_cast<uint64_t>(lo) |
+                                          (static_cast<uint64_t>(hi) << 32));
+#pragma unroll
+          for (int rj = 0; rj < RT; ++rj) {
+            const i32x4 acc =
+                __builtin_amdgcn_mfma_i32_16x16x32_i8(wa, st.x[rj][h >> 1][h & 1], zero, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              out[rj][i] = __fadd_rn(out[rj][i], __fmul_rn(static_cast<float>(acc[i]), sc[i]));
+            }
+          }
+        }
+      });
+    });
+  }
+
+  // fully_connected.cc:1078-1082: zero-point term, row scale, bias -- after taking the factor
+  // 16 back out (exact).
+#pragma unroll
+  for (int rj = 0; rj < RT; ++rj) {
+    if (rt0 + rj >= a.row_tiles) break;
+    const int m = rt[rj] * kTile + (lane & 15);
+    if (m >= a.batches) continue;
+    const float zp = static_cast<float>(a.zero_points[m]);
+    const float row_scale = a.scaling_factors[m];
+    const int n0 = ct0 * kTile + 4 * (lane >> 4);
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = min(n0 + i, a.out_depth - 1);
+      float v = __fsub_rn(__fmul_rn(out[rj][i], 0.0625f), __fmul_rn(zp, a.kfsum[n]));
+      v = __fmul_rn(v, row_scale);
+      if (a.bias) v = __fadd_rn(v, a.bias[n]);
+      o[i] = v;
+    }
+    float* dst = a.output + static_cast<size_t>(m) * a.out_depth + n0;
+    if (n0 + 3 < a.out_depth && a.vector_store) {
+      *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (n0 + i < a.out_depth) dst[i] = o[i];
+      }
+    }
+  }
+}
+
 }  // namespace
 
 size_t GemmInt4BlockwiseBytes(int out_depth, int depth) {
@@ -406,6 +636,90 @@ hipError_t LaunchFcInt4BlockwiseGemm(const float* input, int variant, float* sca
   } else {
     hipLaunchKernelGGL((FcInt4BlockwiseGemmKernel<1, 1, 1, 16>), grid, dim3(kThreads), 0,
                        stream, a);
+  }
+  return hipGetLastError();
+}
+
+size_t GemmInt4BlockwiseNibbleBytes(int out_depth, int depth) {
+  const size_t tiles = (static_cast<size_t>(out_depth) + kTile - 1) / kTile;
+  const size_t nb = static_cast<size_t>(depth) / kBlock;
+  return tiles * ((nb + 3) / 4 * 1024 + (nb + 15) / 16 * 512);
+}
+
+hipError_t LaunchPackInt4BlockwiseNibbles(const uint8_t* filter, const uint16_t* scales_f16,
+                                          int out_depth, int depth, uint8_t* packed,
+                                          hipStream_t stream) {
+  if (out_depth == 0 || depth == 0) return hipSuccess;
+  const int tiles = (out_depth + kTile - 1) / kTile;
+  const int nb = depth / kBlock;
+  const int nq = (nb + 3) / 4, ng = (nb + 15) / 16;
+  const int64_t slots = static_cast<int64_t>(tiles) * nq * 64;
+  const unsigned grid = static_cast<unsigned>((slots + kThreads - 1) / kThreads);
+  hipLaunchKernelGGL(PackInt4BlockwiseNibblesKernel, dim3(grid), dim3(kThreads), 0, stream,
+                     filter, scales_f16, out_depth, depth, tiles, nb, nq, ng, packed);
+  return hipGetLastError();
+}
+
+namespace {
+template <int VARIANT>
+void LaunchTiledQuantizer(const float* input, int batches, int depth, int row_tiles,
+                          void* tiled_rows, float* scaling_factors, int32_t* zero_points,
+                          hipStream_t stream) {
+  const dim3 grid(row_tiles * kTile), block(kQuantizeThreads);
+  hipLaunchKernelGGL(QuantizeRowsTiledKernel<VARIANT>, grid, block, 0, stream, input, batches,
+                     depth, RowTileBytes(depth), static_cast<int8_t*>(tiled_rows),
+                     scaling_factors, zero_points);
+}
+}  // namespace
+
+hipError_t LaunchFcInt4BlockwiseNibbleGemm(const float* input, int variant,
+                                           float* scaling_factors, int32_t* zero_points,
+                                           const uint8_t* nibble_filter, const float* kfsum,
+                                           const float* bias, float* output, int batches,
+                                           int depth, int out_depth, void* tiled_rows,
+                                           hipStream_t stream) {
+  if (batches == 0 || out_depth == 0) return hipSuccess;
+  const int nb = depth / kBlock;
+  const int row_tiles = (batches + kTile - 1) / kTile;
+  const int channel_tiles = (out_depth + kTile - 1) / kTile;
+  switch (variant) {
+    case LRTFC_QUANT_NEON_V8:
+      LaunchTiledQuantizer<LRTFC_QUANT_NEON_V8>(input, batches, depth, row_tiles, tiled_rows,
+                                                scaling_factors, zero_points, stream);
+      break;
+    case LRTFC_QUANT_NEON_LEGACY:
+      LaunchTiledQuantizer<LRTFC_QUANT_NEON_LEGACY>(input, batches, depth, row_tiles, tiled_rows,
+                                                    scaling_factors, zero_points, stream);
+      break;
+    default:
+      LaunchTiledQuantizer<LRTFC_QUANT_PORTABLE>(input, batches, depth, row_tiles, tiled_rows,
+                                                 scaling_factors, zero_points, stream);
+      break;
+  }
+  if (hipError_t err = hipGetLastError()) return err;
+  NibbleGemmArgs a;
+  a.filter = reinterpret_cast<const i32x4*>(nibble_filter);
+  a.scales = reinterpret_cast<const uint2*>(
+      nibble_filter + static_cast<size_t>(channel_tiles) * ((nb + 3) / 4) * 1024);
+  a.activations = static_cast<const i64x2*>(tiled_rows);
+  a.scaling_factors = scaling_factors;
+  a.zero_points = zero_points;
+  a.kfsum = kfsum;
+  a.bias = bias;
+  a.output = output;
+  a.batches = batches;
+  a.out_depth = out_depth;
+  a.nb = nb;
+  a.channel_tiles = channel_tiles;
+  a.row_tiles = row_tiles;
+  a.vector_store = (out_depth % 4 == 0) && (reinterpret_cast<uintptr_t>(output) % 16 == 0);
+  const int RT = row_tiles <= 1 ? 1 : 2;
+  const dim3 grid((channel_tiles + 3) / 4, (row_tiles + RT - 1) / RT);
+  if (grid.y > 65535) return hipErrorInvalidValue;
+  if (RT == 1) {
+    hipLaunchKernelGGL((FcInt4NibbleGemmKernel<1, 8, 4>), grid, dim3(kThreads), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((FcInt4NibbleGemmKernel<2, 8, 2>), grid, dim3(kThreads), 0, stream, a);
   }
   return hipGetLastError();
 }

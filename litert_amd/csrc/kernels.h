@@ -180,6 +180,19 @@ hipError_t LaunchFcInt4BlockwiseGemm(const float* input, int variant, float* sca
                                      int batches, int depth, int out_depth, void* tiled_rows,
                                      hipStream_t stream);
 
+// The same product on a filter kept at 4 bits per weight (`tile16x128n` + fp16 scales), for
+// batches between decode and prefill.
+size_t GemmInt4BlockwiseNibbleBytes(int out_depth, int depth);
+hipError_t LaunchPackInt4BlockwiseNibbles(const uint8_t* filter, const uint16_t* scales_f16,
+                                          int out_depth, int depth, uint8_t* packed,
+                                          hipStream_t stream);
+hipError_t LaunchFcInt4BlockwiseNibbleGemm(const float* input, int variant,
+                                           float* scaling_factors, int32_t* zero_points,
+                                           const uint8_t* nibble_filter, const float* kfsum,
+                                           const float* bias, float* output, int batches,
+                                           int depth, int out_depth, void* tiled_rows,
+                                           hipStream_t stream);
+
 // EMBEDDING_LOOKUP from an Int4 (value_bits 4) or Int8 (8) table to float32 / binary16 rows.
 // block_scales != nullptr: blockwise fp16 scales [rows, cols / blocksize]; otherwise row_scales
 // [rows] or `scale`. status: three device int32 {0 or 1, first offending position or -1, the

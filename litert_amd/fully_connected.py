@@ -272,6 +272,7 @@ class FullyConnectedBlockwiseInt4:
             _ptr(self.kfsum), _stream()))
         self._ws = None
         self._gemm_filter = None
+        self._nibble_filter = None
         self._gemm_ws = None
         # packed: one fused kernel on the re-tiled filter (block size 32 only); otherwise the
         # two-kernel form on the reference layout.
@@ -291,8 +292,8 @@ class FullyConnectedBlockwiseInt4:
             self._ws = torch.empty(need, dtype=torch.uint8, device="cuda")
         return self._ws
 
-    # From this many rows on the matrix-core GEMM streams the filter once for the whole batch;
-    # below, the decode kernel (one pass over the filter per four rows) is faster.
+    # From this many rows on a matrix-core GEMM streams the filter once for the whole batch,
+    # whatever the shape (lrtfc_fc_blockwise_int4_preferred_form picks the form per shape).
     GEMM_MIN_BATCHES = 16
 
     def call_gemm(self, x, out=None):
@@ -321,11 +322,42 @@ class FullyConnectedBlockwiseInt4:
             _stream()))
         return out
 
+    def call_gemm_nibbles(self, x, out=None):
+        """The same GEMM on the filter kept at 4 bits per weight (made on first use and kept):
+        the form for batches between decode and prefill. Same results as the other forms."""
+        if self.blocksize != 32 or self.depth % 32:
+            raise RuntimeError("call_gemm_nibbles needs block size 32")
+        lib = capi.load()
+        x = x.contiguous()
+        batches = x.numel() // self.depth
+        if out is None:
+            out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
+        if self._nibble_filter is None:
+            self._nibble_filter = torch.empty(
+                lib.lrtfc_gemm_int4_blockwise_nibble_bytes(self.out_depth, self.depth),
+                dtype=torch.uint8, device="cuda")
+            capi.check(lib.lrtfc_pack_int4_blockwise_gemm_nibbles(
+                _ptr(self.filter), _ptr(self.scales), self.out_depth, self.depth, 32,
+                _ptr(self._nibble_filter), _stream()))
+        need = lib.lrtfc_fc_blockwise_int4_gemm_workspace_bytes(batches, self.depth)
+        if self._gemm_ws is None or self._gemm_ws.numel() < need:
+            self._gemm_ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        capi.check(lib.lrtfc_fc_blockwise_int4_gemm_nibbles(
+            _ptr(x), _ptr(self._nibble_filter), _ptr(self.kfsum), _ptr(self.bias), _ptr(out),
+            batches, self.depth, self.out_depth, self.variant, _ptr(self._gemm_ws),
+            self._gemm_ws.numel(), _stream()))
+        return out
+
     def __call__(self, x, out=None):
         x = x.contiguous()
         batches = x.numel() // self.depth
-        if batches >= self.GEMM_MIN_BATCHES and self.blocksize == 32 and self.depth % 32 == 0:
-            return self.call_gemm(x, out)
+        if self.blocksize == 32 and self.depth % 32 == 0 and self.retiled is not None:
+            form = capi.load().lrtfc_fc_blockwise_int4_preferred_form(batches, self.depth,
+                                                                      self.out_depth)
+            if form == capi.INT4_FORM_GEMM_NIBBLES:
+                return self.call_gemm_nibbles(x, out)
+            if form == capi.INT4_FORM_GEMM_INT8:
+                return self.call_gemm(x, out)
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
         if (self.retiled is not None and self.depth > self.FUSED_MAX_DEPTH

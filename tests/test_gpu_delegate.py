@@ -108,10 +108,12 @@ def test_hybrid_sign_bit_and_whole_zero_input_through_delegate(B):
         assert want[0, 0] == 1.0 and want[0, 1] == (1.0 if bias[1] < 0 else 0.0)
 
 
-@pytest.mark.parametrize("B,K,N", [(2, 2048, 512), (1, 16384, 40), (3, 8192, 24), (5, 1024, 16)])
+@pytest.mark.parametrize("B,K,N", [(2, 2048, 512), (1, 16384, 40), (3, 8192, 24), (5, 1024, 16),
+                                   (8, 160, 8200), (20, 96, 8192)])
 def test_blockwise_int4_node_through_delegate(B, K, N):
     """Shallow rows and up to two deep rows run the fused kernel on the re-tiled filter; three
-    or more deep rows are quantized by a launch of their own first."""
+    or more deep rows are quantized by a launch of their own first; five to 32 rows on a wide
+    filter take the GEMM that keeps the filter at 4 bits per weight."""
     c = wl.blockwise_int4_fc(B, K, N, lo=-8, hi=7)
     bias = np.random.default_rng(2).standard_normal(N).astype(np.float32)
     with FakeHost() as h:

@@ -565,8 +565,43 @@ def test_blockwise_int4_gemm_matches_oracle(fc, B, K, N, bias):
     y = op.call_gemm(_cuda(c["x"])).cpu().numpy()
     want = oracle.fc_blockwise_int4(c["x"], c["packed"], N, c["scales"].view(np.uint16), 32, b)
     assert _bits_equal(y, want)
-    if B >= op.GEMM_MIN_BATCHES:  # the op picks this form by itself from 16 rows on
+    if B >= op.GEMM_MIN_BATCHES:  # the op picks a GEMM form by itself from 16 rows on
         assert _bits_equal(op(_cuda(c["x"])).cpu().numpy(), want)
+    # The same shapes on the filter kept at 4 bits per weight (quads of blocks, groups of 16
+    # scales, one or two row tiles per wavefront).
+    assert _bits_equal(op.call_gemm_nibbles(_cuda(c["x"])).cpu().numpy(), want)
+
+
+def test_blockwise_int4_nibble_gemm_full_width_and_dispatch(fc):
+    """The nibble-resident GEMM on config 3's filter at 5, 8 and 24 rows: what the op picks by
+    itself for this shape (lrtfc_fc_blockwise_int4_preferred_form), bit-identical to the decode
+    kernel on the same rows and, on a sample of channels, to the oracle; with the two NEON
+    quantizer flavours on the way."""
+    from litert_amd import capi
+    lib = capi.load()
+    assert lib.lrtfc_fc_blockwise_int4_preferred_form(4, 4096, 14336) == capi.INT4_FORM_DECODE
+    assert lib.lrtfc_fc_blockwise_int4_preferred_form(5, 4096, 14336) == capi.INT4_FORM_GEMM_NIBBLES
+    assert lib.lrtfc_fc_blockwise_int4_preferred_form(32, 4096, 14336) == capi.INT4_FORM_GEMM_NIBBLES
+    assert lib.lrtfc_fc_blockwise_int4_preferred_form(33, 4096, 14336) == capi.INT4_FORM_GEMM_INT8
+    assert lib.lrtfc_fc_blockwise_int4_preferred_form(8, 16384, 2048) == capi.INT4_FORM_DECODE
+    assert lib.lrtfc_fc_blockwise_int4_preferred_form(16, 16384, 2048) == capi.INT4_FORM_GEMM_INT8
+    c = wl.blockwise_int4_fc(4)
+    sample = np.arange(0, 14336, 449)
+    for rows, variant in ((5, 0), (8, 1), (24, 2)):
+        x = np.random.default_rng(rows).standard_normal((rows, 4096)).astype(np.float32)
+        x[0, :4] = [-125.0, 130.0, 2.5, -2.5]
+        op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], 4096, 32,
+                                            quant_variant=variant)
+        xd = _cuda(x)
+        got = op(xd).cpu().numpy()
+        assert op._nibble_filter is not None and op._gemm_filter is None
+        decode = torch.cat([fc.FullyConnectedBlockwiseInt4.__call__(op, xd[i:i + 4])
+                            for i in range(0, rows, 4)]).cpu().numpy()
+        assert _bits_equal(got, decode)
+        want = oracle.fc_blockwise_int4(x, c["packed"][sample], sample.size,
+                                        c["scales"][sample].view(np.uint16), 32,
+                                        variant=variant)
+        assert _bits_equal(got[:, sample], want)
 
 
 def test_blockwise_int4_gemm_full_width_agrees_with_decode_kernel(fc):
