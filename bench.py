@@ -805,8 +805,9 @@ def delegate_chain(torch, wl, b=1, invokes=20, bound=False):
 def single_node_invokes(wl, invokes=200):
     """Configs 1, 2 and 3 as ONE FULLY_CONNECTED node each through the delegate plugin with host
     tensors in and out, driven by the stand-in interpreter: median wall-clock time of Invoke()
-    (gather into page-locked memory, one host-to-device copy, the kernel -- which writes its
-    output straight into page-locked host memory --, one stream synchronisation, scatter)."""
+    (gather into page-locked memory, the kernel -- which reads its input rows from that memory and
+    writes its output straight into page-locked host memory --, one stream synchronisation,
+    scatter), and the same invoke split into those phases by the delegate's metrics collection."""
     from litert_amd.standin_host import FakeHost, FLOAT32, FLOAT16, INT4, INT8, INT32, OK
     rng = np.random.default_rng(6)
 
@@ -824,7 +825,17 @@ def single_node_invokes(wl, invokes=200):
             h.invoke()
             samples.append((time.perf_counter() - t0) * 1e6)
         samples.sort()
-        return round(samples[len(samples) // 2], 1)
+        # The same invoke split by phase, from the delegate's own clocks (its metrics collection
+        # adds two event records and their read-back, so the phases sum to more than the median).
+        if h.start_metrics() != 0:
+            raise RuntimeError("metrics collection did not start")
+        for _ in range(invokes):
+            h.invoke()
+        m = h.stop_metrics()
+        phases = {p: round(m["host_%s_us" % p] / m["invokes"], 1)
+                  for p in ("gather", "enqueue", "wait", "scatter")}
+        phases["device_span_us"] = round(m["device_time_us"] / m["invokes"], 1)
+        return {"invoke_us": round(samples[len(samples) // 2], 1), "with_metrics_on": phases}
 
     out = {}
     c1 = wl.int8_fc()

@@ -45,6 +45,9 @@ typedef struct litert_amd_metrics {
   int64_t bytes_downloaded;  /* device -> host */
   double host_time_us;       /* wall time inside the partitions' invoke callbacks */
   double device_time_us;     /* per invoke: first enqueued copy to last finished one (HIP events) */
+  /* host_time_us by phase of an invoke: host tensors gathered into page-locked memory; copies and
+   * kernels enqueued; the wait for the device to finish; outputs scattered back to the tensors. */
+  double host_gather_us, host_enqueue_us, host_wait_us, host_scatter_us;
 } litert_amd_metrics;
 /* Both return 0, or 1 when `delegate` is not one of this library's (or, for stop, when no
  * collection is running). start clears the totals. */

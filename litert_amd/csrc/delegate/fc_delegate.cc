@@ -47,6 +47,9 @@ struct Options {
   bool claim_int4_per_channel = true;
   bool claim_embedding_lookup = true;
   bool claim_batch_matmul = true;
+  // Decode-sized host inputs are read by the kernels straight from page-locked host memory
+  // instead of being copied to the device first ("direct_inputs": "0" turns that off).
+  bool direct_inputs = true;
 };
 
 // Device memory the application registered for a tensor (litert_amd_register_device_buffer);
@@ -68,6 +71,7 @@ struct MetricsState {
   int64_t downloaded = 0;     // bytes copied device -> host
   double host_us = 0.0;       // wall time inside the partitions' invoke callbacks
   double device_us = 0.0;     // first enqueued copy to last finished one, per invoke, by HIP events
+  double gather_us = 0.0, enqueue_us = 0.0, wait_us = 0.0, scatter_us = 0.0;  // host_us by phase
 };
 
 struct DelegateState {
@@ -518,6 +522,11 @@ constexpr int kInt4PerChannelNibbleMaxBatches = 32;
 // node kinds below launch today; a new kind, or a kernel form that breaks it, must stay out of
 // the list and take the copy-out path.
 constexpr size_t kDirectOutputMaxBytes = 16 << 20;
+// Up to this many bytes of host inputs per partition are read by the kernels straight from
+// page-locked host memory, when every node that reads them is decode-shaped (a row is then
+// fetched a handful of times, not once per tile of a GEMM).
+constexpr size_t kDirectInputMaxBytes = 64 << 10;
+constexpr int kDirectInputMaxBatches = 16;
 
 bool WritesOutputOnce(FcKind kind) {
   switch (kind) {
@@ -555,11 +564,19 @@ struct PartitionKernel {
   // any of the downloaded tensors back.
   bool direct_outputs = false;
   uint8_t* download_stage_device = nullptr;  // the staging area as the device addresses it
+  // The mirror image for small sets of host inputs (decode rows): the kernels read them straight
+  // from the page-locked upload staging area, which saves the copy command ahead of the first
+  // kernel. A row is read once per workgroup and the device's L2 serves all but the first read;
+  // what it costs is one round trip over PCIe inside the kernel's prologue instead of a copy
+  // command and its launch gap in front of the kernel.
+  bool direct_inputs = false;
+  uint8_t* upload_stage_device = nullptr;
   void* Activation(int tensor) const {
     auto bound = alias.find(tensor);
     if (bound != alias.end()) return bound->second;
     auto it = arena_offset.find(tensor);
     if (it == arena_offset.end()) return nullptr;
+    if (direct_inputs && it->second < upload_bytes) return upload_stage_device + it->second;
     if (direct_outputs && it->second >= download_offset &&
         it->second < download_offset + download_bytes) {
       return download_stage_device + (it->second - download_offset);
@@ -1141,6 +1158,26 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
       }
     }
   }
+  {
+    k->direct_inputs = false;
+    k->upload_stage_device = nullptr;
+    if (k->state->options.direct_inputs && k->upload_bytes > 0 &&
+        k->upload_bytes <= kDirectInputMaxBytes) {
+      bool decode_shaped = true;
+      for (const FcNode& n : k->nodes) {
+        if (std::find(k->uploads.begin(), k->uploads.end(), n.input) == k->uploads.end()) continue;
+        const bool kind_ok = n.kind == FcKind::kInt8 || n.kind == FcKind::kHybrid ||
+                             n.kind == FcKind::kInt4Blockwise || n.kind == FcKind::kHybridInt4;
+        decode_shaped = decode_shaped && kind_ok && n.batches <= kDirectInputMaxBatches;
+      }
+      void* device_view = nullptr;
+      if (decode_shaped &&
+          hipHostGetDevicePointer(&device_view, k->upload_stage.get(), 0) == hipSuccess) {
+        k->direct_inputs = true;
+        k->upload_stage_device = static_cast<uint8_t*>(device_view);
+      }
+    }
+  }
   // Levels: a node without a producer inside the partition is at level 0, a consumer one
   // above its producer (an FC node has one activation input, so one producer at most).
   std::vector<int> level(count, 0);
@@ -1411,7 +1448,8 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     std::memcpy(k->upload_stage.get() + k->arena_offset[t], tensor.data.raw, tensor.bytes);
     host_inputs = true;
   }
-  if (host_inputs) {
+  const auto gathered = std::chrono::steady_clock::now();
+  if (host_inputs && !k->direct_inputs) {
     RETURN_IF_HIP(ctx, hipMemcpyAsync(k->arena.get(), k->upload_stage.get(), k->upload_bytes,
                                       hipMemcpyHostToDevice, k->stream));
   }
@@ -1626,9 +1664,11 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                       k->download_bytes, hipMemcpyDeviceToHost, s));
   }
   if (measure) RETURN_IF_HIP(ctx, hipEventRecord(k->metrics_end, s));
+  const auto enqueued = std::chrono::steady_clock::now();
   // The runtime reads the outputs as soon as invoke returns; a consumer of a registered
   // buffer (another partition, the application's own kernels) may start right away too.
   RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+  const auto waited = std::chrono::steady_clock::now();
   if (measure) {
     float ms = 0.0f;
     RETURN_IF_HIP(ctx, hipEventElapsedTime(&ms, k->metrics_begin, k->metrics_end));
@@ -1657,8 +1697,15 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                 k->download_stage.get() + (k->arena_offset[t] - k->download_offset), tensor.bytes);
   }
   if (measure) {
-    metrics.host_us += std::chrono::duration<double, std::micro>(
-                           std::chrono::steady_clock::now() - host_begin).count();
+    const auto host_end = std::chrono::steady_clock::now();
+    auto us = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) {
+      return std::chrono::duration<double, std::micro>(b - a).count();
+    };
+    metrics.host_us += us(host_begin, host_end);
+    metrics.gather_us += us(host_begin, gathered);
+    metrics.enqueue_us += us(gathered, enqueued);
+    metrics.wait_us += us(enqueued, waited);
+    metrics.scatter_us += us(waited, host_end);
   }
   return kTfLiteOk;
 }
@@ -1782,6 +1829,12 @@ bool ParseOptions(const char* const* keys, const char* const* values, size_t n, 
         *error = "quant_variant must be portable, neon_v8 or neon_legacy, got '" + val + "'";
         return false;
       }
+    } else if (key == "direct_inputs") {
+      if (val != "0" && val != "1") {
+        *error = "direct_inputs must be 0 or 1, got '" + val + "'";
+        return false;
+      }
+      opt->direct_inputs = val == "1";
     } else if (key == "claim") {
       opt->claim_int8 = opt->claim_hybrid = opt->claim_int4_blockwise = false;
       opt->claim_int4_per_channel = opt->claim_embedding_lookup = false;
@@ -1895,7 +1948,8 @@ int litert_amd_stop_metrics(TfLiteDelegate* delegate, litert_amd_metrics* out) {
   auto* state = static_cast<DelegateState*>(delegate->data_);
   if (&state->delegate != delegate || !state->metrics.on) return 1;
   const MetricsState& m = state->metrics;
-  *out = litert_amd_metrics{m.invokes, m.nodes, m.uploaded, m.downloaded, m.host_us, m.device_us};
+  *out = litert_amd_metrics{m.invokes,   m.nodes,     m.uploaded,   m.downloaded, m.host_us,
+                            m.device_us, m.gather_us, m.enqueue_us, m.wait_us,    m.scatter_us};
   state->metrics.on = false;
   return 0;
 }

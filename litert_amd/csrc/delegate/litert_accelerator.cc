@@ -131,6 +131,10 @@ LiteRtStatus StopMetricsCollection(LiteRtRuntimeContext* runtime_context,
       {"litert_amd.bytes_downloaded", integer(m.bytes_downloaded)},
       {"litert_amd.host_time_us", real(m.host_time_us)},
       {"litert_amd.device_time_us", real(m.device_time_us)},
+      {"litert_amd.host_gather_us", real(m.host_gather_us)},
+      {"litert_amd.host_enqueue_us", real(m.host_enqueue_us)},
+      {"litert_amd.host_wait_us", real(m.host_wait_us)},
+      {"litert_amd.host_scatter_us", real(m.host_scatter_us)},
   };
   return kLiteRtStatusOk;
 }

@@ -237,6 +237,29 @@ class FakeHost:
     def invoke(self):
         return self.L.fh_invoke(self.h)
 
+    METRIC_FIELDS = ("invokes", "nodes_run", "bytes_uploaded", "bytes_downloaded", "host_time_us",
+                     "device_time_us", "host_gather_us", "host_enqueue_us", "host_wait_us",
+                     "host_scatter_us")
+
+    def start_metrics(self, path=DELEGATE_LIB):
+        """litert_amd_start_metrics on the loaded delegate (0 on success)."""
+        d = C.CDLL(path)
+        d.litert_amd_start_metrics.argtypes = [C.c_void_p, C.c_int]
+        return d.litert_amd_start_metrics(self.L.fh_delegate(self.h), 0)
+
+    def stop_metrics(self, path=DELEGATE_LIB):
+        """litert_amd_stop_metrics: the totals since start_metrics, as a dict keyed by the fields
+        of struct litert_amd_metrics."""
+        class Metrics(C.Structure):
+            _fields_ = ([(n, C.c_int64) for n in self.METRIC_FIELDS[:4]] +
+                        [(n, C.c_double) for n in self.METRIC_FIELDS[4:]])
+        d = C.CDLL(path)
+        d.litert_amd_stop_metrics.argtypes = [C.c_void_p, C.POINTER(Metrics)]
+        m = Metrics()
+        if d.litert_amd_stop_metrics(self.L.fh_delegate(self.h), C.byref(m)) != 0:
+            raise RuntimeError("litert_amd_stop_metrics: no collection was running")
+        return {n: getattr(m, n) for n in self.METRIC_FIELDS}
+
     def classify(self, node, path=DELEGATE_LIB):
         buf = C.create_string_buffer(256)
         kind = self.L.fh_classify(self.h, path.encode(), node, buf, 256)

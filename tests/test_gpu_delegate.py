@@ -44,11 +44,12 @@ def _oracle_int8(c, x, activation=0, bias=True, in_scale=None, in_zp=None):
                                       c["out_zp"], lo, hi)
 
 
-def test_int8_node_config1_through_delegate():
+@pytest.mark.parametrize("direct_inputs", ["1", "0"])  # kernels read the host's rows / a copy
+def test_int8_node_config1_through_delegate(direct_inputs):
     c = wl.int8_fc()
     with FakeHost() as h:
         node, x, y = _add_int8_fc(h, c)
-        assert h.load_delegate() == 0, h.errors()
+        assert h.load_delegate({"direct_inputs": direct_inputs}) == 0, h.errors()
         assert h.modify_graph_with_delegate() == OK, h.errors()
         assert h.plan()[0][:2] == ("delegate", [node])
         assert h.allocate_tensors() == OK, h.errors()
@@ -62,8 +63,9 @@ def test_int8_node_config1_through_delegate():
         assert np.array_equal(h.read(y), _oracle_int8(c, np.roll(c["x"], 7, axis=1)))
 
 
-@pytest.mark.parametrize("B", [1, 4, 8, 19])  # up to 4 rows fuse the quantizer, more split it off
-def test_hybrid_node_through_delegate(B):
+@pytest.mark.parametrize("direct_inputs", ["1", "0"])
+@pytest.mark.parametrize("B", [1, 4, 8, 19])  # up to 8 rows fuse the quantizer, more split it off
+def test_hybrid_node_through_delegate(B, direct_inputs):
     c = wl.hybrid_fc(B, 4096, 1024)
     bias = np.random.default_rng(1).standard_normal(1024).astype(np.float32)
     with FakeHost() as h:
@@ -73,10 +75,15 @@ def test_hybrid_node_through_delegate(B):
         b = h.tensor(FLOAT32, (1024,), data=bias, const=True)
         y = h.tensor(FLOAT32, (B, 1024))
         h.fc(x, w, b, y, activation=1, asymmetric=True)
-        assert h.load_delegate() == 0, h.errors()
+        assert h.load_delegate({"direct_inputs": direct_inputs}) == 0, h.errors()
         assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
         assert h.invoke() == OK, h.errors()
         want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"], 1.0, bias, True, oracle.ACT_RELU)
+        assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+        x2 = np.roll(c["x"], 3, axis=1)  # a second invoke sees the new rows, not the first ones
+        h.write(x, x2)
+        assert h.invoke() == OK, h.errors()
+        want = oracle.fc_hybrid(x2, c["w"], c["pcs"], 1.0, bias, True, oracle.ACT_RELU)
         assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
 
 

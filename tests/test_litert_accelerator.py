@@ -199,4 +199,7 @@ def test_metrics_collection_reports_what_the_partitions_did():
         assert got["litert_amd.bytes_uploaded"] == 3 * c["x"].nbytes
         assert got["litert_amd.bytes_downloaded"] == 3 * 2 * 64 * 4
         assert 0 < got["litert_amd.device_time_us"] <= got["litert_amd.host_time_us"]
+        phases = [got["litert_amd.host_%s_us" % p] for p in ("gather", "enqueue", "wait", "scatter")]
+        assert all(v > 0 for v in phases)
+        assert abs(sum(phases) - got["litert_amd.host_time_us"]) < 1e-6 * got["litert_amd.host_time_us"] + 1e-3
         assert h.invoke() == OK  # collection is off again
