@@ -482,6 +482,17 @@ int lrtfc_embedding_lookup_hybrid(const int32_t* lookup, int count, const void* 
                                   const float* row_scales, int out_type, void* output,
                                   int32_t* status, void* stream);
 
+/* ---- completion mark ------------------------------------------------------------------------
+ * No counterpart in the reference, whose kernels return when their work is done. Enqueues on
+ * `stream` a one-wavefront kernel that stores `value` to *flag once everything enqueued on the
+ * stream before it has finished and its results are visible to the host. `flag` is the device
+ * address of 4 bytes of page-locked host memory (hipHostMalloc + hipHostGetDevicePointer). For
+ * callers that wait for a short chain of kernels by polling that word from the CPU: on an idle
+ * stream the store is seen about 3.5 us earlier than hipStreamSynchronize returns. The caller
+ * bounds its polling and falls back to hipStreamSynchronize, which also reports a failed
+ * kernel. */
+int lrtfc_mark_completion(uint32_t* flag, uint32_t value, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -84,6 +84,7 @@ SYMBOLS = [
                                                   _vp]),
     ("lrtfc_embedding_lookup_blockwise_int4", _i, [_vp, _i, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_embedding_lookup_hybrid", _i, [_vp, _i, _vp, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp]),
+    ("lrtfc_mark_completion", _i, [_vp, C.c_uint32, _vp]),
     ("lrtfc_int4_group_table_bytes", _sz, []),
     ("lrtfc_int4_group_prepare", _i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_fc_blockwise_int4_packed_grouped", _i, [_vp, _vp, _i, _vp]),

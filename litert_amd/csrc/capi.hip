@@ -1092,6 +1092,26 @@ int lrtfc_embedding_lookup_hybrid(const int32_t* lookup, int count, const void* 
                  "hybrid embedding lookup");
 }
 
+namespace {
+// Stream order puts this kernel after everything enqueued before it, and a kernel's end makes
+// its stores visible system-wide, so the host that reads `value` here may read those results.
+__global__ void MarkCompletionKernel(volatile uint32_t* flag, uint32_t value) {
+  if (threadIdx.x == 0) {
+    __threadfence_system();
+    *flag = value;
+  }
+}
+}  // namespace
+
+int lrtfc_mark_completion(uint32_t* flag, uint32_t value, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(flag, "null pointer");
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(flag) & 3) == 0, "flag must be 4-byte aligned");
+  hipLaunchKernelGGL(MarkCompletionKernel, dim3(1), dim3(lrtfc::kWaveSize), 0, AsStream(stream),
+                     flag, value);
+  return FromHip(hipGetLastError(), "completion mark");
+}
+
 size_t lrtfc_int4_group_table_bytes(void) { return lrtfc::Int4GroupTableBytes(); }
 
 int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,

@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
@@ -50,6 +51,10 @@ struct Options {
   // Decode-sized host inputs are read by the kernels straight from page-locked host memory
   // instead of being copied to the device first ("direct_inputs": "0" turns that off).
   bool direct_inputs = true;
+  // How an invoke waits for the device: by polling a word of page-locked memory that a
+  // one-wavefront kernel behind the partition's last command stores to ("completion": "poll"),
+  // or in hipStreamSynchronize ("sync"). Polling sees the end about 3.5 us earlier.
+  bool poll_completion = true;
 };
 
 // Device memory the application registered for a tensor (litert_amd_register_device_buffer);
@@ -583,6 +588,10 @@ struct PartitionKernel {
     }
     return arena.as<uint8_t>() + it->second;
   }
+  // The word an invoke polls for its own serial number (Options::poll_completion).
+  PinnedBuffer completion;
+  uint32_t* completion_dev = nullptr;
+  uint32_t completion_serial = 0;
   // Three int32 per EMBEDDING_LOOKUP node, in page-locked host memory the lookup kernels write
   // straight into: {0 or 1, first offending position, the index found there}.
   PinnedBuffer lookup_status;
@@ -1263,6 +1272,13 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
   for (FcNode& n : k->nodes) {
     if (n.kind == FcKind::kEmbeddingLookup) n.status_slot = k->lookup_nodes++;
   }
+  if (k->state->options.poll_completion && !k->completion_dev) {
+    RETURN_IF_HIP(ctx, k->completion.Ensure(64));
+    std::memset(k->completion.get(), 0, 64);
+    void* dev = nullptr;
+    RETURN_IF_HIP(ctx, hipHostGetDevicePointer(&dev, k->completion.get(), 0));
+    k->completion_dev = static_cast<uint32_t*>(dev);
+  }
   if (k->lookup_nodes > 0) {
     RETURN_IF_HIP(ctx, k->lookup_status.Ensure(static_cast<size_t>(k->lookup_nodes) * 12));
     void* dev = nullptr;
@@ -1664,12 +1680,32 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                       k->download_bytes, hipMemcpyDeviceToHost, s));
   }
   if (measure) RETURN_IF_HIP(ctx, hipEventRecord(k->metrics_end, s));
+  if (k->completion_dev) {
+    if (++k->completion_serial == 0) k->completion_serial = 1;  // the word starts out as 0
+    RETURN_IF_FC(ctx, lrtfc_mark_completion(k->completion_dev, k->completion_serial, s));
+  }
   const auto enqueued = std::chrono::steady_clock::now();
   // The runtime reads the outputs as soon as invoke returns; a consumer of a registered
   // buffer (another partition, the application's own kernels) may start right away too.
-  RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+  bool finished = false;
+  if (k->completion_dev) {
+    // Poll for a bounded time: short partitions end inside it; a long one, or one whose kernel
+    // failed and never reaches the mark, goes on to hipStreamSynchronize, which reports errors.
+    const volatile uint32_t* word = reinterpret_cast<const volatile uint32_t*>(k->completion.get());
+    constexpr auto kPollFor = std::chrono::microseconds(150);
+    for (;;) {
+      for (int spin = 0; spin < 64 && !finished; ++spin) {
+        finished = *word == k->completion_serial;
+        if (!finished) __builtin_ia32_pause();
+      }
+      if (finished || std::chrono::steady_clock::now() - enqueued > kPollFor) break;
+    }
+    if (finished) std::atomic_thread_fence(std::memory_order_acquire);
+  }
+  if (!finished) RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
   const auto waited = std::chrono::steady_clock::now();
   if (measure) {
+    if (finished) RETURN_IF_HIP(ctx, hipEventSynchronize(k->metrics_end));
     float ms = 0.0f;
     RETURN_IF_HIP(ctx, hipEventElapsedTime(&ms, k->metrics_begin, k->metrics_end));
     metrics.device_us += 1e3 * ms;
@@ -1835,6 +1871,12 @@ bool ParseOptions(const char* const* keys, const char* const* values, size_t n, 
         return false;
       }
       opt->direct_inputs = val == "1";
+    } else if (key == "completion") {
+      if (val != "poll" && val != "sync") {
+        *error = "completion must be poll or sync, got '" + val + "'";
+        return false;
+      }
+      opt->poll_completion = val == "poll";
     } else if (key == "claim") {
       opt->claim_int8 = opt->claim_hybrid = opt->claim_int4_blockwise = false;
       opt->claim_int4_per_channel = opt->claim_embedding_lookup = false;

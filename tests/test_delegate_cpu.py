@@ -151,6 +151,9 @@ def test_bad_options_are_rejected_before_touching_the_device():
     with FakeHost() as h:
         assert h.load_delegate({"direct_inputs": "yes"}) == 1
         assert "direct_inputs must be 0 or 1" in h.errors()
+    with FakeHost() as h:
+        assert h.load_delegate({"completion": "spin"}) == 1
+        assert "completion must be poll or sync" in h.errors()
 
 
 def test_no_gpu_means_no_delegate():

@@ -44,12 +44,17 @@ def _oracle_int8(c, x, activation=0, bias=True, in_scale=None, in_zp=None):
                                       c["out_zp"], lo, hi)
 
 
-@pytest.mark.parametrize("direct_inputs", ["1", "0"])  # kernels read the host's rows / a copy
-def test_int8_node_config1_through_delegate(direct_inputs):
+# kernels read the host's rows / a copy of them; the invoke polls for its end / synchronizes
+BOUNDARY_OPTIONS = [{}, {"direct_inputs": "0"}, {"completion": "sync"},
+                    {"direct_inputs": "0", "completion": "sync"}]
+
+
+@pytest.mark.parametrize("options", BOUNDARY_OPTIONS, ids=lambda o: ",".join(o.values()) or "default")
+def test_int8_node_config1_through_delegate(options):
     c = wl.int8_fc()
     with FakeHost() as h:
         node, x, y = _add_int8_fc(h, c)
-        assert h.load_delegate({"direct_inputs": direct_inputs}) == 0, h.errors()
+        assert h.load_delegate(options) == 0, h.errors()
         assert h.modify_graph_with_delegate() == OK, h.errors()
         assert h.plan()[0][:2] == ("delegate", [node])
         assert h.allocate_tensors() == OK, h.errors()
@@ -63,9 +68,9 @@ def test_int8_node_config1_through_delegate(direct_inputs):
         assert np.array_equal(h.read(y), _oracle_int8(c, np.roll(c["x"], 7, axis=1)))
 
 
-@pytest.mark.parametrize("direct_inputs", ["1", "0"])
+@pytest.mark.parametrize("options", BOUNDARY_OPTIONS, ids=lambda o: ",".join(o.values()) or "default")
 @pytest.mark.parametrize("B", [1, 4, 8, 19])  # up to 8 rows fuse the quantizer, more split it off
-def test_hybrid_node_through_delegate(B, direct_inputs):
+def test_hybrid_node_through_delegate(B, options):
     c = wl.hybrid_fc(B, 4096, 1024)
     bias = np.random.default_rng(1).standard_normal(1024).astype(np.float32)
     with FakeHost() as h:
@@ -75,7 +80,7 @@ def test_hybrid_node_through_delegate(B, direct_inputs):
         b = h.tensor(FLOAT32, (1024,), data=bias, const=True)
         y = h.tensor(FLOAT32, (B, 1024))
         h.fc(x, w, b, y, activation=1, asymmetric=True)
-        assert h.load_delegate({"direct_inputs": direct_inputs}) == 0, h.errors()
+        assert h.load_delegate(options) == 0, h.errors()
         assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
         assert h.invoke() == OK, h.errors()
         want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"], 1.0, bias, True, oracle.ACT_RELU)
@@ -796,3 +801,38 @@ def test_blockwise_int4_resize_between_decode_and_prefill():
                 want = oracle.fc_blockwise_int4(c["x"][:rows], c["packed"], n,
                                                 c["scales"].view(np.uint16), 32)
                 assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32)), (rows, n)
+
+
+def test_completion_mark_follows_the_work_enqueued_before_it():
+    """lrtfc_mark_completion: the word turns into the value only after the kernel in front of it
+    on the stream has written its output, so a host that has seen the value reads the output."""
+    import time
+    from litert_amd import capi
+    lib = capi.load()
+    capi.init(0)
+    c = wl.hybrid_fc(1, 4096, 1024)
+    x = torch.from_numpy(c["x"]).cuda()
+    w = torch.from_numpy(c["w"]).cuda()
+    pcs = torch.from_numpy(c["pcs"]).cuda()
+    sums = torch.from_numpy(c["w"].astype(np.int32).sum(1).astype(np.int32)).cuda()
+    y = torch.zeros((1, 1024), dtype=torch.float32).pin_memory()
+    word = torch.zeros(16, dtype=torch.int32).pin_memory()
+    ws = torch.empty(lib.lrtfc_activation_workspace_bytes(1, 4096), dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream().cuda_stream
+    want = oracle.fc_hybrid(c["x"], c["w"], c["pcs"])
+    for serial in (7, 8, 0x7FFFFFFF):
+        y.zero_()
+        rc = lib.lrtfc_fc_hybrid(x.data_ptr(), w.data_ptr(), pcs.data_ptr(), 1.0, sums.data_ptr(), None,
+                                 y.data_ptr(), 1, 4096, 1024, 1, 0, capi.QUANT_PORTABLE,
+                                 ws.data_ptr(), ws.numel(), stream)
+        capi.check(rc)
+        capi.check(lib.lrtfc_mark_completion(word.data_ptr(), serial, stream))
+        deadline = time.perf_counter() + 5.0
+        while int(word[0]) != serial and time.perf_counter() < deadline:
+            pass
+        assert int(word[0]) == serial
+        assert np.array_equal(y.numpy().view(np.uint32), want.view(np.uint32))
+    torch.cuda.synchronize()
+    assert lib.lrtfc_mark_completion(None, 1, stream) != 0
+    assert lib.lrtfc_mark_completion(word.data_ptr() + 2, 1, stream) != 0
