@@ -69,6 +69,9 @@ def main():
                     help="with --gemm-probe: afterwards keep launching the GEMM for this many seconds "
                          "on the seeded operands, then as long on the constant ones, printing a "
                          "time-stamped line at each switch (for power / clock sampling from outside)")
+    ap.add_argument("--roofline-probe", action="store_true",
+                    help="only the cold B=1 launches of config 2 that roofline.avg_launch_us is "
+                         "taken over (for a rocprofv3 --kernel-trace --stats run)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch only the dominant kernel (cold, 12 times) and a 64 MiB device "
                          "copy (3 times), for a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run")
@@ -125,6 +128,10 @@ def main():
             fn()
         return g
 
+    if args.roofline_probe:
+        roofline_probe(torch, fc, wl, capture, timed_replays)
+        return
+
     # ---- headline workload: config 2 -------------------------------------------------
     c = wl.hybrid_fc(max(BATCHES))
     ops = []
@@ -169,7 +176,7 @@ def main():
     value = step_bytes / (ms_cold * 1e-3) / 1e9
 
     # ---- per-kernel durations for the roofline -----------------------------------------
-    # The op is ONE kernel (FcInt8PackedGemvKernel, hybrid epilogue, quantization fused into
+    # The op is ONE kernel (FcInt8ResidentGemvKernel, hybrid epilogue, quantization fused into
     # its prologue), so op time and dominant-kernel time coincide.
     ROUNDS = 4  # launches per graph = ROUNDS x weight copies
 
@@ -314,6 +321,26 @@ def mfma_rate(torch, seconds, random_operands):
         launch(20)   # 20 launches of about 0.8 ms
         launches += 20
     return ops.value * launches / (time.time() - t0) / 1e12
+
+
+def roofline_probe(torch, fc, wl, capture, timed_replays):
+    """Only the launches behind roofline.avg_launch_us: config 2 at B = 1, one fused kernel per
+    op, the filter copies rotated so that every launch streams from HBM, 24 launches per graph
+    replayed 25 times (after one warm call per copy and one capture pass). Under
+    `rocprofv3 --kernel-trace --stats` the kernel's average duration is over the same launches
+    as the figure printed here, which is taken with events around the replays and so also holds
+    the gaps between launches."""
+    c = wl.hybrid_fc(1)
+    ops = [fc.FullyConnectedHybrid(np.roll(c["w"], i, axis=0) if i else c["w"],
+                                   np.roll(c["pcs"], i) if i else c["pcs"])
+           for i in range(WEIGHT_COPIES)]
+    x = torch.from_numpy(c["x"]).cuda()
+    y = torch.empty((1, N_OUT), dtype=torch.float32, device="cuda")
+    g = capture(lambda: [op(x, out=y) for _ in range(4) for op in ops])
+    us = timed_replays([g], 25) * 1e3 / (4 * len(ops))
+    print(json.dumps({"probe": "roofline", "launches_per_replay": 4 * len(ops), "replays": 25,
+                      "avg_launch_us_by_events": round(us, 3),
+                      "algorithmic_bytes": hybrid_bytes(1)}))
 
 
 def traffic_probe(torch, fc, wl):
@@ -482,6 +509,10 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
                 1, 4096, 14336, stream()))
         return run
 
+    def decode_rows(op, xin, yout):
+        capi.check(lib.lrtfc_fc_blockwise_int4_packed(p(xin), p(op.retiled), p(op.kfsum), None, p(yout),
+                                                       xin.shape[0], 4096, 14336, op.variant, stream()))
+
     # op = one kernel (quantizer fused into the prologue); "prequantized" = the same kernel
     # handed rows that were quantized beforehand, i.e. without the prologue's work.
     o_cold = per_launch_us([(lambda o: lambda: o(x3, out=y3))(op) for op in ops3])
@@ -516,6 +547,28 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
     entry["kernel"] = "FcInt4BlockwiseGemmKernel (v_mfma_i32_16x16x32_i8 per block, float32 accumulators in block order)"
     out["next_int4_blockwise_prefill_14336x4096"] = entry
     del op3
+
+    # Between decode and prefill on the blockwise int4 path (not a BASELINE configuration): the
+    # op as dispatched (lrtfc_fc_blockwise_int4_preferred_form picks the form per shape), filter
+    # copies rotated (cold), and the forms it chose against at 8 and 16 rows.
+    forms = {capi.INT4_FORM_DECODE: "decode kernel", capi.INT4_FORM_GEMM_NIBBLES: "4-bit-resident GEMM",
+             capi.INT4_FORM_GEMM_INT8: "int8-expanded GEMM"}
+    entry = {}
+    for rows in (2, 4, 8, 16, 32):
+        xg = torch.randn((rows, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(rows))
+        yg = torch.empty((rows, 14336), dtype=torch.float32, device="cuda")
+        us = per_launch_us([(lambda o: lambda: o(xg, out=yg))(o) for o in ops3])
+        entry["us_%d_rows" % rows] = round(us, 2)
+        entry["form_%d_rows" % rows] = forms[lib.lrtfc_fc_blockwise_int4_preferred_form(rows, 4096, 14336)]
+        if rows in (8, 16):
+            entry["us_%d_rows_decode_kernel_passes" % rows] = round(per_launch_us(
+                [(lambda o: lambda: [decode_rows(o, xg[i:i + 4], yg[i:i + 4]) for i in range(0, rows, 4)])(o)
+                 for o in ops3]), 2)
+            entry["us_%d_rows_int8_expanded_gemm" % rows] = round(per_launch_us(
+                [(lambda o: lambda: o.call_gemm(xg, out=yg))(o) for o in ops3]), 2)
+    entry["kernel"] = ("FcInt4NibbleGemmKernel (filter stays 4 bits per weight; nibbles expanded in registers "
+                       "into the v_mfma_i32_16x16x32_i8 operand; row quantizer launch + GEMM launch)")
+    out["next_int4_blockwise_between_decode_and_prefill_14336x4096"] = entry
 
     del ops3
 
