@@ -320,6 +320,24 @@ int lrtfc_batch_matmul_hybrid_packed(const float* lhs, int lhs_batches, int rows
                                      int asymmetric_quantize_inputs, int quant_variant,
                                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same op with everything its shapes allow (tflite/kernels/batch_matmul.cc:745-813 in front
+ * of EvalHybrid): up to three batch dimensions per side (the op extends both shapes to rank 5,
+ * reference/batch_matmul.h:120-146), each pair equal or 1 on either side -- also 1 on different
+ * sides in different dimensions --, and adj_x. lhs_batch_dims / weight_batch_dims: three ints
+ * each, leading 1s for shapes of lower rank. adj_x: lhs is [.., depth, rows] and is transposed
+ * into the workspace first, as the op transposes it into a temporary (:811-813). Output:
+ * [d0, d1, d2, rows, units] with d_i the broadcast of the two sides' dimension i. workspace:
+ * lrtfc_batch_matmul_workspace_bytes(product of lhs_batch_dims, rows, depth, adj_x) bytes,
+ * 256-byte aligned. Everything else as above. */
+size_t lrtfc_batch_matmul_workspace_bytes(int lhs_matrices, int rows, int depth, int adj_x);
+int lrtfc_batch_matmul_hybrid_packed_nd(const float* lhs, const int* lhs_batch_dims, int rows,
+                                        int depth, int adj_x, const int8_t* packed_weights,
+                                        const int* weight_batch_dims, int units,
+                                        const float* per_channel_scales, float filter_scale,
+                                        const int32_t* row_sums, float* output,
+                                        int asymmetric_quantize_inputs, int quant_variant,
+                                        void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- Per-channel int4 hybrid FULLY_CONNECTED ------------------------------------------
  * Replaces EvalHybridDense4Bit (tflite/kernels/fully_connected.cc:1088-1178) in the
  * arithmetic of its reference kernels

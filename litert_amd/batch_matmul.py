@@ -13,11 +13,12 @@ from .fully_connected import _dev, _ensure_init, _ptr, _stream
 
 class BatchMatMulHybrid:
     """rhs: int8 [..., K, N] (adj_y: [..., N, K]), constant. per_channel_scales: [N] or None
-    (then filter_scale). Left operands are float32 [..., M, K]; adj_x is not offered. Batch
-    dimensions must be equal, or all 1 on one side."""
+    (then filter_scale). Left operands are float32 [..., M, K] (adj_x: [..., K, M]). Batch
+    dimensions broadcast as the op's do: each pair equal, or 1 on either side."""
 
     def __init__(self, rhs, per_channel_scales=None, filter_scale=1.0,
-                 asymmetric_quantize_inputs=True, adj_y=False, quant_variant=capi.QUANT_PORTABLE):
+                 asymmetric_quantize_inputs=True, adj_y=False, quant_variant=capi.QUANT_PORTABLE,
+                 adj_x=False):
         _ensure_init()
         lib = capi.load()
         rhs = np.ascontiguousarray(rhs, dtype=np.int8)
@@ -42,28 +43,32 @@ class BatchMatMulHybrid:
         self.filter_scale = float(filter_scale)
         self.asymmetric = bool(asymmetric_quantize_inputs)
         self.variant = quant_variant
+        self.adj_x = bool(adj_x)
         self._ws = None
 
     def __call__(self, lhs):
         lhs = lhs.contiguous()
-        if lhs.shape[-1] != self.depth:
+        if lhs.dim() < 2 or lhs.dim() > 5:
+            raise ValueError("BATCH_MATMUL operands have 2 to 5 dimensions")
+        rows, depth = (lhs.shape[-1], lhs.shape[-2]) if self.adj_x else (lhs.shape[-2], lhs.shape[-1])
+        if depth != self.depth:
             raise ValueError("accumulation depths differ")
-        rows = lhs.shape[-2]
         lhs_batch_shape = tuple(lhs.shape[:-2])
         lhs_batches = int(np.prod(lhs_batch_shape, dtype=np.int64))
+        lb = (1,) * (3 - len(lhs_batch_shape)) + lhs_batch_shape
+        rb = (1,) * (3 - len(self.rhs_batch_shape)) + self.rhs_batch_shape
+        if any(a != b and a != 1 and b != 1 for a, b in zip(lb, rb)):
+            raise ValueError("batch dimensions must be equal or 1, pair by pair")
         rank = max(len(lhs_batch_shape), len(self.rhs_batch_shape))
-        lb = (1,) * (rank - len(lhs_batch_shape)) + lhs_batch_shape
-        rb = (1,) * (rank - len(self.rhs_batch_shape)) + self.rhs_batch_shape
-        if not (lb == rb or lhs_batches == 1 or self.matrices == 1):
-            raise ValueError("batch dimensions must be equal, or all 1 on one side")
-        out_batch = tuple(max(a, b) for a, b in zip(lb, rb))
+        out_batch = tuple(b if a == 1 else a for a, b in zip(lb, rb))[3 - rank:]
         out = torch.empty(out_batch + (rows, self.units), dtype=torch.float32, device=lhs.device)
         lib = capi.load()
-        need = lib.lrtfc_activation_workspace_bytes(lhs_batches * rows, self.depth)
+        need = lib.lrtfc_batch_matmul_workspace_bytes(lhs_batches, rows, self.depth, int(self.adj_x))
         if self._ws is None or self._ws.numel() < need:
             self._ws = torch.empty(need, dtype=torch.uint8, device="cuda")
-        capi.check(lib.lrtfc_batch_matmul_hybrid_packed(
-            _ptr(lhs), lhs_batches, rows, self.depth, _ptr(self.packed), self.matrices, self.units,
-            _ptr(self.pcs), self.filter_scale, _ptr(self.row_sums), _ptr(out), int(self.asymmetric),
-            self.variant, _ptr(self._ws), self._ws.numel(), _stream()))
+        capi.check(lib.lrtfc_batch_matmul_hybrid_packed_nd(
+            _ptr(lhs), (C.c_int * 3)(*lb), rows, self.depth, int(self.adj_x), _ptr(self.packed),
+            (C.c_int * 3)(*rb), self.units, _ptr(self.pcs), self.filter_scale, _ptr(self.row_sums),
+            _ptr(out), int(self.asymmetric), self.variant, _ptr(self._ws), self._ws.numel(),
+            _stream()))
         return out

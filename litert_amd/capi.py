@@ -56,6 +56,9 @@ SYMBOLS = [
                                               _i, _i, _vp, _sz, _vp]),
     ("lrtfc_batch_matmul_hybrid_packed", _i, [_vp, _i, _i, _i, _vp, _i, _i, _vp, _f, _vp, _vp, _i,
                                               _i, _vp, _sz, _vp]),
+    ("lrtfc_batch_matmul_workspace_bytes", _sz, [_i, _i, _i, _i]),
+    ("lrtfc_batch_matmul_hybrid_packed_nd", _i, [_vp, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _f, _vp,
+                                                 _vp, _i, _i, _vp, _sz, _vp]),
     ("lrtfc_static_scratch_bytes", _sz, []),
     ("lrtfc_fc_hybrid_static_scratch", _i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i,
                                             _i, _vp]),

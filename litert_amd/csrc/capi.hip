@@ -519,6 +519,109 @@ int lrtfc_fc_hybrid_packed_workspace(const float* input, const int8_t* packed_fi
                             batches, depth, out_depth, activation, /*zero_input_exit=*/1, stream);
 }
 
+namespace {
+size_t TransposedBytes(int64_t lhs_matrices, int rows, int depth) {
+  const size_t bytes = static_cast<size_t>(lhs_matrices) * rows * depth * sizeof(float);
+  return (bytes + 255) & ~static_cast<size_t>(255);
+}
+}  // namespace
+
+size_t lrtfc_batch_matmul_workspace_bytes(int lhs_matrices, int rows, int depth, int adj_x) {
+  if (lhs_matrices <= 0 || rows <= 0 || depth <= 0) return 0;
+  const int64_t quant_rows = static_cast<int64_t>(lhs_matrices) * rows;
+  if (quant_rows > 0x7fffffff) return 0;
+  return WorkspaceBytes(static_cast<int>(quant_rows), depth) +
+         (adj_x ? TransposedBytes(lhs_matrices, rows, depth) : 0);
+}
+
+int lrtfc_batch_matmul_hybrid_packed_nd(const float* lhs, const int* lhs_batch_dims, int rows,
+                                        int depth, int adj_x, const int8_t* packed_weights,
+                                        const int* weight_batch_dims, int units,
+                                        const float* per_channel_scales, float filter_scale,
+                                        const int32_t* row_sums, float* output,
+                                        int asymmetric_quantize_inputs, int quant_variant,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(lhs_batch_dims && weight_batch_dims, "null pointer");
+  LRTFC_REQUIRE(rows >= 0 && depth > 0 && units >= 0, "bad dimension");
+  int64_t lhs_matrices = 1, weight_matrices = 1, out_matrices = 1;
+  int out_dims[3];
+  for (int i = 0; i < 3; ++i) {
+    const int l = lhs_batch_dims[i], w = weight_batch_dims[i];
+    LRTFC_REQUIRE(l >= 0 && w >= 0, "bad dimension");
+    LRTFC_REQUIRE(l == w || l == 1 || w == 1,
+                  "batch dimension %d: %d against %d can not be broadcast", i, l, w);
+    out_dims[i] = l == 1 ? w : l;  // batch_matmul.h:33-38
+    lhs_matrices *= l;
+    weight_matrices *= w;
+    out_matrices *= out_dims[i];
+    LRTFC_REQUIRE(out_matrices <= 0x7fffffff, "too many matrices");
+  }
+  if (out_matrices == 0 || rows == 0 || units == 0) return LRTFC_OK;
+  const int64_t quant_rows = lhs_matrices * rows;
+  LRTFC_REQUIRE(quant_rows <= 0x7fffffff, "too many rows");
+  LRTFC_REQUIRE(lhs && packed_weights && row_sums && output && workspace, "null pointer");
+  const size_t need =
+      lrtfc_batch_matmul_workspace_bytes(static_cast<int>(lhs_matrices), rows, depth, adj_x);
+  LRTFC_REQUIRE(workspace_bytes >= need, "workspace too small: %zu < %zu bytes", workspace_bytes,
+                need);
+  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
+                "workspace must be 256-byte aligned");
+  void* quant_space = workspace;
+  if (adj_x) {
+    // The op's own first step (batch_matmul.cc:811-813): [.., depth, rows] -> [.., rows, depth].
+    float* transposed = static_cast<float*>(workspace);
+    quant_space = static_cast<char*>(workspace) + TransposedBytes(lhs_matrices, rows, depth);
+    int rc = FromHip(lrtfc::LaunchTransposeLastTwoF32(lhs, static_cast<int>(lhs_matrices), depth,
+                                                      rows, transposed, AsStream(stream)),
+                     "left operand transposition");
+    if (rc != LRTFC_OK) return rc;
+    lhs = transposed;
+  }
+  // BatchQuantizeFloats over every row of the float operand (batch_matmul.cc:472-497); symmetric
+  // quantization leaves the offsets at zero (:487-489).
+  const Workspace w = SplitWorkspace(quant_space, static_cast<int>(quant_rows), depth);
+  int rc = lrtfc_batch_quantize_floats(lhs, static_cast<int>(quant_rows), depth, w.q, w.sf, w.zp,
+                                       asymmetric_quantize_inputs, quant_variant, stream);
+  if (rc != LRTFC_OK) return rc;
+  const int32_t* zp = asymmetric_quantize_inputs ? w.zp : nullptr;
+  // Output matrix (b0, b1, b2) pairs the left matrix and the weight matrix whose indices keep
+  // b_i where that side's dimension is not 1 (the extents of batch_matmul.h:42-52, :139-146).
+  // Consecutive output matrices that share a weight matrix and take consecutive left matrices
+  // are one product over all their rows.
+  const size_t matrix_bytes = lrtfc::PackedInt8FilterBytes(units, depth);
+  auto side_index = [&](const int* dims, int64_t o) {
+    int64_t index = 0;
+    int b[3];
+    b[2] = static_cast<int>(o % out_dims[2]);
+    b[1] = static_cast<int>((o / out_dims[2]) % out_dims[1]);
+    b[0] = static_cast<int>(o / (static_cast<int64_t>(out_dims[2]) * out_dims[1]));
+    for (int i = 0; i < 3; ++i) index = index * dims[i] + (dims[i] == 1 ? 0 : b[i]);
+    return index;
+  };
+  int64_t o = 0;
+  while (o < out_matrices) {
+    const int64_t l0 = side_index(lhs_batch_dims, o), w0 = side_index(weight_batch_dims, o);
+    int64_t run = 1;
+    while (o + run < out_matrices && side_index(weight_batch_dims, o + run) == w0 &&
+           side_index(lhs_batch_dims, o + run) == l0 + run &&
+           (run + 1) * static_cast<int64_t>(rows) <= 0x7fffffff) {
+      ++run;
+    }
+    const size_t row0 = static_cast<size_t>(l0) * rows;
+    rc = FcHybridInt8Packed(w.q + row0 * depth, w.sf + row0, zp ? zp + row0 : nullptr,
+                            packed_weights + static_cast<size_t>(w0) * matrix_bytes,
+                            per_channel_scales, filter_scale,
+                            row_sums + static_cast<size_t>(w0) * units, nullptr,
+                            output + static_cast<size_t>(o) * rows * units,
+                            static_cast<int>(run * rows), depth, units, LRTFC_ACT_NONE, 0, stream,
+                            /*batch_matmul=*/1);
+    if (rc != LRTFC_OK) return rc;
+    o += run;
+  }
+  return LRTFC_OK;
+}
+
 int lrtfc_batch_matmul_hybrid_packed(const float* lhs, int lhs_batches, int rows, int depth,
                                      const int8_t* packed_weights, int weight_matrices, int units,
                                      const float* per_channel_scales, float filter_scale,
@@ -526,47 +629,16 @@ int lrtfc_batch_matmul_hybrid_packed(const float* lhs, int lhs_batches, int rows
                                      int asymmetric_quantize_inputs, int quant_variant,
                                      void* workspace, size_t workspace_bytes, void* stream) {
   if (int rc = RequireInit()) return rc;
-  LRTFC_REQUIRE(lhs_batches >= 0 && rows >= 0 && depth > 0 && weight_matrices >= 0 && units >= 0,
-                "bad dimension");
+  LRTFC_REQUIRE(lhs_batches >= 0 && weight_matrices >= 0, "bad dimension");
   LRTFC_REQUIRE(lhs_batches == weight_matrices || lhs_batches == 1 || weight_matrices == 1,
                 "%d input batches against %d weight matrices: only equal counts, or one side "
                 "broadcast, are supported", lhs_batches, weight_matrices);
-  const int out_batches = lhs_batches > weight_matrices ? lhs_batches : weight_matrices;
-  if (out_batches == 0 || lhs_batches == 0 || weight_matrices == 0 || rows == 0 || units == 0) {
-    return LRTFC_OK;
-  }
-  const int64_t quant_rows = static_cast<int64_t>(lhs_batches) * rows;
-  LRTFC_REQUIRE(quant_rows <= 0x7fffffff, "too many rows");
-  LRTFC_REQUIRE(lhs && packed_weights && row_sums && output && workspace, "null pointer");
-  LRTFC_REQUIRE(workspace_bytes >= WorkspaceBytes(static_cast<int>(quant_rows), depth),
-                "workspace too small: %zu < %zu bytes", workspace_bytes,
-                WorkspaceBytes(static_cast<int>(quant_rows), depth));
-  LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0,
-                "workspace must be 256-byte aligned");
-  // BatchQuantizeFloats over every row of the float operand (batch_matmul.cc:472-497); symmetric
-  // quantization leaves the offsets at zero (:487-489).
-  const Workspace w = SplitWorkspace(workspace, static_cast<int>(quant_rows), depth);
-  int rc = lrtfc_batch_quantize_floats(lhs, static_cast<int>(quant_rows), depth, w.q, w.sf, w.zp,
-                                       asymmetric_quantize_inputs, quant_variant, stream);
-  if (rc != LRTFC_OK) return rc;
-  const int32_t* zp = asymmetric_quantize_inputs ? w.zp : nullptr;
-  if (weight_matrices == 1) {  // one weight matrix for every row: a single product
-    return FcHybridInt8Packed(w.q, w.sf, zp, packed_weights, per_channel_scales, filter_scale,
-                              row_sums, nullptr, output, static_cast<int>(quant_rows), depth, units,
-                              LRTFC_ACT_NONE, 0, stream, /*batch_matmul=*/1);
-  }
-  const size_t matrix_bytes = lrtfc::PackedInt8FilterBytes(units, depth);
-  for (int b = 0; b < out_batches; ++b) {
-    const size_t row0 = lhs_batches == 1 ? 0 : static_cast<size_t>(b) * rows;
-    rc = FcHybridInt8Packed(w.q + row0 * depth, w.sf + row0, zp ? zp + row0 : nullptr,
-                            packed_weights + static_cast<size_t>(b) * matrix_bytes,
-                            per_channel_scales, filter_scale,
-                            row_sums + static_cast<size_t>(b) * units, nullptr,
-                            output + static_cast<size_t>(b) * rows * units, rows, depth, units,
-                            LRTFC_ACT_NONE, 0, stream, /*batch_matmul=*/1);
-    if (rc != LRTFC_OK) return rc;
-  }
-  return LRTFC_OK;
+  const int lhs_dims[3] = {1, 1, lhs_batches}, weight_dims[3] = {1, 1, weight_matrices};
+  return lrtfc_batch_matmul_hybrid_packed_nd(lhs, lhs_dims, rows, depth, /*adj_x=*/0,
+                                             packed_weights, weight_dims, units,
+                                             per_channel_scales, filter_scale, row_sums, output,
+                                             asymmetric_quantize_inputs, quant_variant, workspace,
+                                             workspace_bytes, stream);
 }
 
 int lrtfc_batch_quantize_floats(const float* values, int n_batch, int n_data, int8_t* quantized,

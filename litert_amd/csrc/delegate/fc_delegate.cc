@@ -188,34 +188,40 @@ FcKind ClassifyEmbeddingLookup(const TfLiteContext* ctx, const TfLiteNode* node,
 }
 
 // Shape facts of a BATCH_MATMUL node with a float left operand and a constant int8 right one:
-// the op extends both shapes to a common rank and broadcasts the batch dimensions
-// (tflite/kernels/batch_matmul.cc:356-391); this delegate takes the forms in which the batch
-// dimensions are equal or all 1 on one side.
+// the op extends both shapes to rank 5 and broadcasts the three batch dimensions pair by pair
+// (tflite/kernels/batch_matmul.cc:356-391, reference/batch_matmul.h:120-146); adj_x / adj_y say
+// which of an operand's last two dimensions is the accumulation depth.
 struct BatchMatMulShape {
   int lhs_batches = 1, matrices = 1, rows = 0, depth = 0, units = 0;
+  int64_t out_batches = 1;
+  int lhs_dims[3] = {1, 1, 1}, weight_dims[3] = {1, 1, 1};
 };
-bool BatchMatMulGeometry(const TfLiteTensor& lhs, const TfLiteTensor& rhs, bool adj_y,
+bool BatchMatMulGeometry(const TfLiteTensor& lhs, const TfLiteTensor& rhs, bool adj_x, bool adj_y,
                          BatchMatMulShape* out, const char** why) {
   const int lr = lhs.dims->size, rr = rhs.dims->size;
   if (lr < 2 || lr > 5 || rr < 2 || rr > 5) return *why = "operand rank outside 2..5", false;
   BatchMatMulShape g;
-  g.rows = lhs.dims->data[lr - 2];
-  g.depth = lhs.dims->data[lr - 1];
+  g.rows = lhs.dims->data[adj_x ? lr - 1 : lr - 2];
+  g.depth = lhs.dims->data[adj_x ? lr - 2 : lr - 1];
   g.units = adj_y ? rhs.dims->data[rr - 2] : rhs.dims->data[rr - 1];
   if ((adj_y ? rhs.dims->data[rr - 1] : rhs.dims->data[rr - 2]) != g.depth) {
     return *why = "accumulation depths differ", false;
   }
-  const int rank = std::max(lr, rr);
-  bool equal = true;
-  for (int i = 0; i < rank - 2; ++i) {
-    const int l = i - (rank - lr) >= 0 ? lhs.dims->data[i - (rank - lr)] : 1;
-    const int r = i - (rank - rr) >= 0 ? rhs.dims->data[i - (rank - rr)] : 1;
-    g.lhs_batches *= l;
-    g.matrices *= r;
-    equal = equal && l == r;
-  }
-  if (!equal && g.lhs_batches != 1 && g.matrices != 1) {
-    return *why = "batch dimensions broadcast on both sides", false;
+  for (int i = 0; i < 3; ++i) {
+    const int l = i - (5 - lr) >= 0 ? lhs.dims->data[i - (5 - lr)] : 1;
+    const int r = i - (5 - rr) >= 0 ? rhs.dims->data[i - (5 - rr)] : 1;
+    if (l != r && l != 1 && r != 1) return *why = "batch dimensions do not broadcast", false;
+    if (l < 0 || r < 0) return *why = "negative dimension", false;
+    g.lhs_dims[i] = l;
+    g.weight_dims[i] = r;
+    g.out_batches *= l == 1 ? r : l;
+    const int64_t lhs_batches = static_cast<int64_t>(g.lhs_batches) * l;
+    const int64_t matrices = static_cast<int64_t>(g.matrices) * r;
+    if (lhs_batches > 0x7fffffff || matrices > 0x7fffffff || g.out_batches > 0x7fffffff) {
+      return *why = "too many matrices", false;
+    }
+    g.lhs_batches = static_cast<int>(lhs_batches);
+    g.matrices = static_cast<int>(matrices);
   }
   if (g.depth <= 0) return *why = "empty depth", false;
   *out = g;
@@ -242,13 +248,12 @@ FcKind ClassifyBatchMatMul(const TfLiteContext* ctx, const TfLiteNode* node,
   if (lhs.type != kTfLiteFloat32 || rhs.type != kTfLiteInt8 || output.type != kTfLiteFloat32) {
     return no("not the float32 x int8 form");
   }
-  if (params->adj_x) return no("adj_x is left to the CPU kernels");
   if (!lhs.dims || !rhs.dims) return no("operand has no shape");
   if (!IsConstant(rhs)) return no("right operand is not a constant tensor");
   if (rhs.quantization.type != kTfLiteAffineQuantization) return no("right operand not affine");
   BatchMatMulShape g;
   const char* why = "";
-  if (!BatchMatMulGeometry(lhs, rhs, params->adj_y, &g, &why)) return no(why);
+  if (!BatchMatMulGeometry(lhs, rhs, params->adj_x, params->adj_y, &g, &why)) return no(why);
   const auto* q = static_cast<const TfLiteAffineQuantization*>(rhs.quantization.params);
   if (!q || !q->scale || q->scale->size < 1) return no("right operand has no scales");
   if (q->scale->size > 1) {
@@ -498,7 +503,8 @@ struct FcNode {
   // matrix product, out_depth = output units; retiled_dev holds `matrices` re-tiled weight
   // matrices one after another, row_sums_dev their row sums.
   int lhs_batches = 1, matrices = 1;
-  bool adj_y = false;
+  bool adj_x = false, adj_y = false;
+  int lhs_dims[3] = {1, 1, 1}, weight_dims[3] = {1, 1, 1};
   // Scheduling inside the partition: the stream the node runs on, the node that produces its
   // input (-1: the input is uploaded from the host), and whether a node on another stream
   // waits for this one.
@@ -709,6 +715,7 @@ void* KernelInit(TfLiteContext* ctx, const char* buffer, size_t /*length*/) {
     n.output = node->outputs->data[0];
     if (kind == FcKind::kBatchMatMul) {
       const auto* bp = static_cast<const TfLiteBatchMatMulParams*>(node->builtin_data);
+      n.adj_x = bp->adj_x;
       n.adj_y = bp->adj_y;
       n.params.asymmetric_quantize_inputs = bp->asymmetric_quantize_inputs;
     } else if (kind != FcKind::kEmbeddingLookup) {
@@ -838,16 +845,18 @@ TfLiteStatus PrepareBatchMatMulNode(TfLiteContext* ctx, PartitionKernel* k, FcNo
   const TfLiteTensor& output = ctx->tensors[n->output];
   BatchMatMulShape g;
   const char* why = "";
-  if (!BatchMatMulGeometry(lhs, rhs, n->adj_y, &g, &why)) {
+  if (!BatchMatMulGeometry(lhs, rhs, n->adj_x, n->adj_y, &g, &why)) {
     ctx->ReportError(ctx, "litert_amd delegate: node %d: %s", n->node_index, why);
     return kTfLiteError;
   }
   n->lhs_batches = g.lhs_batches;
   n->matrices = g.matrices;
+  std::copy(g.lhs_dims, g.lhs_dims + 3, n->lhs_dims);
+  std::copy(g.weight_dims, g.weight_dims + 3, n->weight_dims);
   n->batches = g.rows;
   n->depth = g.depth;
   n->out_depth = g.units;
-  const int64_t out_batches = std::max(g.lhs_batches, g.matrices);
+  const int64_t out_batches = g.out_batches;
   if (NumElements(output.dims) != out_batches * g.rows * g.units) {
     ctx->ReportError(ctx, "litert_amd delegate: node %d output shape does not hold %lld x %d x %d values",
                      n->node_index, static_cast<long long>(out_batches), g.rows, g.units);
@@ -1293,8 +1302,8 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
       continue;
     }
     if (n.kind == FcKind::kBatchMatMul) {
-      RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(lrtfc_activation_workspace_bytes(
-                             n.lhs_batches * n.batches, n.depth)));
+      RETURN_IF_HIP(ctx, k->workspace[n.lane].Ensure(lrtfc_batch_matmul_workspace_bytes(
+                             n.lhs_batches, n.batches, n.depth, n.adj_x)));
       continue;
     }
     if (n.kind == FcKind::kHybridInt4 ||
@@ -1625,9 +1634,9 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
         }
         break;
       case FcKind::kBatchMatMul:
-        RETURN_IF_FC(ctx, lrtfc_batch_matmul_hybrid_packed(
-                              static_cast<const float*>(in_dev), n.lhs_batches, n.batches, n.depth,
-                              n.retiled_dev.as<int8_t>(), n.matrices, n.out_depth,
+        RETURN_IF_FC(ctx, lrtfc_batch_matmul_hybrid_packed_nd(
+                              static_cast<const float*>(in_dev), n.lhs_dims, n.batches, n.depth,
+                              n.adj_x, n.retiled_dev.as<int8_t>(), n.weight_dims, n.out_depth,
                               n.per_channel ? n.pcs_dev.as<float>() : nullptr, n.filter_scale,
                               n.row_sums_dev.as<int32_t>(), static_cast<float*>(out_dev),
                               n.params.asymmetric_quantize_inputs, variant, scratch.get(),

@@ -80,6 +80,9 @@ hipError_t LaunchBatchQuantize(const float* values, int n_batch, int n_data, int
 hipError_t LaunchBatchQuantize4Bit(const float* values, int n_batch, int n_data, int8_t* quantized,
                                    float* scaling_factors, int32_t* input_offsets,
                                    hipStream_t stream);
+// `matrices` row-major [in_rows, in_cols] float32 matrices -> [in_cols, in_rows] each.
+hipError_t LaunchTransposeLastTwoF32(const float* src, int matrices, int in_rows, int in_cols,
+                                     float* dst, hipStream_t stream);
 hipError_t LaunchZeroFill(void* dst, size_t bytes, hipStream_t stream);
 hipError_t LaunchRowSumsInt8(const int8_t* filter, int out_depth, int depth, int32_t* row_sums,
                              hipStream_t stream);

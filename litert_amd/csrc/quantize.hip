@@ -59,7 +59,42 @@ __global__ __launch_bounds__(kThreads) void BatchQuantize4BitKernel(
   }
 }
 
+// BATCH_MATMUL with adj_x: the op transposes the last two dimensions of its left operand into a
+// temporary before anything else (TransposeRowsColumns, tflite/kernels/batch_matmul.cc:811-813).
+// Per matrix, src [in_rows, in_cols] -> dst [in_cols, in_rows], through a 32 x 32 tile in LDS so
+// that reads and writes both run along rows (one padding column keeps the transposed reads off
+// a single bank).
+constexpr int kTransposeTile = 32;
+__global__ __launch_bounds__(kTransposeTile * 8) void TransposeLastTwoF32Kernel(
+    const float* __restrict__ src, int in_rows, int in_cols, float* __restrict__ dst) {
+  __shared__ float tile[kTransposeTile][kTransposeTile + 1];
+  const size_t matrix = static_cast<size_t>(blockIdx.z) * in_rows * in_cols;
+  const int c0 = blockIdx.x * kTransposeTile, r0 = blockIdx.y * kTransposeTile;
+  const int tx = threadIdx.x & (kTransposeTile - 1), ty = threadIdx.x / kTransposeTile;
+  for (int j = ty; j < kTransposeTile; j += 8) {
+    const int r = r0 + j, c = c0 + tx;
+    if (r < in_rows && c < in_cols) tile[j][tx] = src[matrix + static_cast<size_t>(r) * in_cols + c];
+  }
+  __syncthreads();
+  for (int j = ty; j < kTransposeTile; j += 8) {
+    const int c = c0 + j, r = r0 + tx;  // dst row = source column
+    if (r < in_rows && c < in_cols) dst[matrix + static_cast<size_t>(c) * in_rows + r] = tile[tx][j];
+  }
+}
+
 }  // namespace
+
+hipError_t LaunchTransposeLastTwoF32(const float* src, int matrices, int in_rows, int in_cols,
+                                     float* dst, hipStream_t stream) {
+  if (matrices == 0 || in_rows == 0 || in_cols == 0) return hipSuccess;
+  if (matrices > 65535) return hipErrorInvalidValue;
+  const dim3 grid((in_cols + kTransposeTile - 1) / kTransposeTile,
+                  (in_rows + kTransposeTile - 1) / kTransposeTile, matrices);
+  if (grid.y > 65535) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(TransposeLastTwoF32Kernel, grid, dim3(kTransposeTile * 8), 0, stream, src,
+                     in_rows, in_cols, dst);
+  return hipGetLastError();
+}
 
 hipError_t LaunchBatchQuantize4Bit(const float* values, int n_batch, int n_data, int8_t* quantized,
                                    float* scaling_factors, int32_t* input_offsets,

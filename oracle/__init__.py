@@ -342,7 +342,8 @@ def fc_hybrid(x, w, per_channel_scales=None, filter_scale=1.0, bias=None, asymme
 def batch_matmul_broadcast(lhs_shape, rhs_shape, adj_y=False):
     """Shapes and batch pairing of BATCH_MATMUL (tflite/kernels/batch_matmul.cc:356-391 and
     reference/batch_matmul.h:120-146): returns (rows, depth, units, output shape, lhs batch
-    index per output batch, rhs batch index per output batch). adj_x is not supported."""
+    index per output batch, rhs batch index per output batch). lhs_shape is the left operand's
+    shape after the op's adj_x transposition, [..., rows, depth]."""
     rank = max(len(lhs_shape), len(rhs_shape))
     le = (1,) * (rank - len(lhs_shape)) + tuple(lhs_shape)
     re = (1,) * (rank - len(rhs_shape)) + tuple(rhs_shape)
@@ -362,9 +363,14 @@ def batch_matmul_broadcast(lhs_shape, rhs_shape, adj_y=False):
 
 
 def batch_matmul_hybrid(lhs, rhs, per_channel_scales=None, filter_scale=1.0, asymmetric=True,
-                        adj_y=False, variant=QUANT_PORTABLE):
-    """lhs float32 [..., M, K]; rhs int8 [..., K, N] (adj_y: [..., N, K]); float32 [..., M, N]."""
+                        adj_y=False, variant=QUANT_PORTABLE, adj_x=False):
+    """lhs float32 [..., M, K] (adj_x: [..., K, M]); rhs int8 [..., K, N] (adj_y: [..., N, K]);
+    float32 [..., M, N]. adj_x is the op's own first step: the left operand's last two dimensions
+    are transposed into a temporary (TransposeRowsColumns, batch_matmul.cc:811-813), and nothing
+    after that knows of it."""
     lhs = _c(lhs, np.float32)
+    if adj_x:
+        lhs = np.ascontiguousarray(np.swapaxes(lhs, -1, -2))
     rhs = _c(rhs, np.int8)
     rows, depth, units, out_shape, li, ri = batch_matmul_broadcast(lhs.shape, rhs.shape, adj_y)
     w = rhs if adj_y else np.ascontiguousarray(np.swapaxes(rhs, -1, -2))  # the op's transposition

@@ -127,20 +127,25 @@ def batch_matmul_hybrid_cases():
                 247, 247, 247, 1511, 1511, 1511, 2222, 2222, 2222]
     cases = []
 
-    def add(source, lhs_shape, rhs_shape, weights, x, want, tol, asym=True, adj_y=False):
+    def add(source, lhs_shape, rhs_shape, weights, x, want, tol, asym=True, adj_y=False,
+            adj_x=False):
         q, scale = kh.symmetric_quantize_tensor(weights)
         cases.append(dict(source=source, lhs_shape=lhs_shape, rhs_shape=rhs_shape,
                           rhs=q.reshape(rhs_shape).tolist(), filter_scale=float(scale),
                           lhs=np.asarray(x, np.float32).reshape(lhs_shape).tolist(),
-                          asymmetric_quantize_inputs=asym, adj_y=adj_y, expected=want,
-                          max_abs_err=tol))
+                          asymmetric_quantize_inputs=asym, adj_y=adj_y, adj_x=adj_x,
+                          expected=want, max_abs_err=tol))
 
     add(b + ":504-533", [2, 10], [10, 3], w3, x_big, [193] * 3 + [247] * 3, 3.0)
     add(b + ":535-565", [1, 2, 2, 3], [3, 10], w10, [11, 12, 13] * 4, [73] * 40, 0.64)
     add(b + ":567-592", [2, 3], [3, 10], w10, [11, 12, 13] * 2, [73] * 20, 0.64)
     add(b + ":600-631", [6, 3], [3, 8], [1] * 8 + [2] * 8 + [3] * 8, [11, 12, 13] * 6, [74] * 48, 0.15)
+    add(b + ":633-661", [3, 6], [3, 8], [1] * 8 + [2] * 8 + [3] * 8, [11] * 6 + [12] * 6 + [13] * 6,
+        [74] * 48, 0.15, adj_x=True)
     add(b + ":663-698", [6, 3], [8, 3], [1, 2, 3] * 8, [11, 12, 13] * 6, [74] * 48, 0.15,
         adj_y=True)
+    add(b + ":700-727", [3, 6], [8, 3], [1, 2, 3] * 8, [11] * 6 + [12] * 6 + [13] * 6, [74] * 48,
+        0.15, adj_x=True, adj_y=True)
     add(b + ":729-758", [2, 2, 10], [10, 3], w3, x_small + x_big,
         [23] * 3 + [57] * 3 + [193] * 3 + [247] * 3, 3.0)
     add(b + ":760-798", [2, 2, 10], [10, 9], w9, x_small + x_big, big_want, 10.0)

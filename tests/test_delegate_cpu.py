@@ -119,7 +119,8 @@ def _bmm_node(h, lhs_shape=(2, 5, 64), rhs_shape=(64, 8), lhs_type=FLOAT32, cons
 
 def test_claim_predicate_batch_matmul():
     """The hybrid form of BATCH_MATMUL (tflite/kernels/batch_matmul.cc:363-374): float32 left
-    operand, constant int8 right operand; adj_x and two-sided broadcasting stay on the CPU."""
+    operand, constant int8 right operand, adj_x / adj_y and the op's broadcasting of up to three
+    batch dimensions included."""
     with FakeHost() as h:
         assert h.classify(_bmm_node(h))[0] == "batch_matmul"
         assert h.classify(_bmm_node(h, rhs_shape=(8, 64), adj_y=True))[0] == "batch_matmul"
@@ -127,15 +128,17 @@ def test_claim_predicate_batch_matmul():
         assert h.classify(_bmm_node(h, scales=np.full(8, 0.01), qdim=1))[0] == "batch_matmul"
         assert h.classify(_bmm_node(h, scales=np.full(8, 0.01), qdim=0)) == (
             None, "per-channel scales do not run along the output units")
-        assert h.classify(_bmm_node(h, adj_x=True)) == (None, "adj_x is left to the CPU kernels")
+        assert h.classify(_bmm_node(h, lhs_shape=(2, 64, 5), adj_x=True))[0] == "batch_matmul"
+        assert h.classify(_bmm_node(h, adj_x=True)) == (None, "accumulation depths differ")
         # register.cc:327-329 registers versions 1..4; a newer one may mean other arithmetic
         assert h.classify(_bmm_node(h, version=4))[0] == "batch_matmul"
         assert h.classify(_bmm_node(h, version=5)) == (None, "op version newer than 4")
         assert h.classify(_bmm_node(h, const=False)) == (None, "right operand is not a constant tensor")
         assert h.classify(_bmm_node(h, lhs_type=INT8)) == (None, "not the float32 x int8 form")
         assert h.classify(_bmm_node(h, rhs_shape=(32, 8))) == (None, "accumulation depths differ")
-        assert h.classify(_bmm_node(h, lhs_shape=(2, 1, 5, 64), rhs_shape=(1, 3, 64, 8))) == (
-            None, "batch dimensions broadcast on both sides")
+        assert h.classify(_bmm_node(h, lhs_shape=(2, 1, 5, 64), rhs_shape=(1, 3, 64, 8)))[0] == "batch_matmul"
+        assert h.classify(_bmm_node(h, lhs_shape=(2, 5, 64), rhs_shape=(3, 64, 8))) == (
+            None, "batch dimensions do not broadcast")
 
 
 def test_bad_options_are_rejected_before_touching_the_device():

@@ -49,6 +49,28 @@ def test_matches_oracle(bmm, lhs_shape, rhs_shape, adj_y, asym, per_channel):
     assert _bits_equal(got, want)
 
 
+@pytest.mark.parametrize("lhs_shape,rhs_shape,adj_x,adj_y", [
+    ((40, 3), (40, 7), True, False),                       # adj_x, rank 2
+    ((2, 3, 64, 5), (2, 1, 9, 64), True, True),            # adj_x and adj_y, weights broadcast inside
+    ((2, 1, 4, 48), (1, 3, 48, 6), False, False),          # 1 on different sides
+    ((2, 1, 48, 4), (1, 3, 48, 6), True, False),           # the same under adj_x
+    ((3, 1, 2, 5, 16), (1, 4, 1, 16, 6), False, False),    # rank 5, both sides broadcast
+    ((1, 2, 3, 16), (4, 1, 16, 6), False, False),          # runs of left matrices per weight matrix
+    ((2, 512, 37), (2, 512, 130), True, False),            # tile edges of the transposition
+    ((1040, 20), (1040, 24), True, False)])
+@pytest.mark.parametrize("asym", [True, False])
+def test_adj_x_and_two_sided_broadcasting_match_oracle(bmm, lhs_shape, rhs_shape, adj_x, adj_y, asym):
+    rng = np.random.default_rng([len(lhs_shape), lhs_shape[-1], rhs_shape[-1], int(asym)])
+    lhs = rng.standard_normal(lhs_shape).astype(np.float32)
+    rhs = rng.integers(-127, 128, rhs_shape).astype(np.int8)
+    units = rhs_shape[-2] if adj_y else rhs_shape[-1]
+    pcs = rng.uniform(2e-3, 8e-3, units).astype(np.float32)
+    op = bmm.BatchMatMulHybrid(rhs, pcs, 1.0, asym, adj_y, adj_x=adj_x)
+    got = op(torch.from_numpy(lhs).cuda()).cpu().numpy()
+    want = oracle.batch_matmul_hybrid(lhs, rhs, pcs, 1.0, asym, adj_y, adj_x=adj_x)
+    assert _bits_equal(got, want)
+
+
 @pytest.mark.parametrize("rows", [3, 40])  # matrix-core GEMV / GEMM
 def test_float_zero_point_correction_on_deep_rows(bmm, rows):
     """Dot products beyond 2^24: the reference kernel's `total -= row_sum * batch_offset` in
@@ -72,26 +94,28 @@ def test_reference_vectors_through_hip(bmm):
         lhs = np.asarray(case["lhs"], np.float32)
         rhs = np.asarray(case["rhs"], np.int8)
         op = bmm.BatchMatMulHybrid(rhs, None, case["filter_scale"],
-                                   case["asymmetric_quantize_inputs"], case["adj_y"])
+                                   case["asymmetric_quantize_inputs"], case["adj_y"],
+                                   adj_x=case["adj_x"])
         got = op(torch.from_numpy(lhs).cuda()).cpu().numpy()
         want = np.asarray(case["expected"], np.float32)
         assert np.max(np.abs(got.ravel() - want)) <= case["max_abs_err"], case["source"]
         assert _bits_equal(got, oracle.batch_matmul_hybrid(
-            lhs, rhs, None, case["filter_scale"], case["asymmetric_quantize_inputs"], case["adj_y"]))
+            lhs, rhs, None, case["filter_scale"], case["asymmetric_quantize_inputs"], case["adj_y"],
+            adj_x=case["adj_x"]))
 
 
-def test_rejects_partial_broadcasting(bmm):
-    from litert_amd import capi
+def test_rejects_shapes_that_do_not_broadcast(bmm):
     rhs = np.zeros((2, 1, 16, 4), np.int8)
     op = bmm.BatchMatMulHybrid(rhs)
     with pytest.raises(ValueError):
-        op(torch.zeros((1, 3, 2, 16), device="cuda"))
+        op(torch.zeros((3, 3, 2, 16), device="cuda"))
 
 
-@pytest.mark.parametrize("lhs_shape,rhs_shape,adj_y,asym", [
-    ((3, 40), (40, 7), False, True), ((2, 3, 5, 64), (2, 3, 9, 64), True, False),
-    ((4, 48), (5, 48, 6), False, True), ((2, 20, 512), (512, 130), False, True)])
-def test_node_through_the_delegate(lhs_shape, rhs_shape, adj_y, asym):
+@pytest.mark.parametrize("lhs_shape,rhs_shape,adj_y,asym,adj_x", [
+    ((3, 40), (40, 7), False, True, False), ((2, 3, 5, 64), (2, 3, 9, 64), True, False, False),
+    ((4, 48), (5, 48, 6), False, True, False), ((2, 20, 512), (512, 130), False, True, False),
+    ((2, 1, 48, 4), (1, 3, 48, 6), False, True, True), ((3, 1, 5, 64), (1, 2, 9, 64), True, True, False)])
+def test_node_through_the_delegate(lhs_shape, rhs_shape, adj_y, asym, adj_x):
     """A BATCH_MATMUL node claimed by the plugin, then a FULLY_CONNECTED node fed by it in the
     same partition."""
     if not torch.cuda.is_available():
@@ -102,7 +126,7 @@ def test_node_through_the_delegate(lhs_shape, rhs_shape, adj_y, asym):
     rhs = rng.integers(-127, 128, rhs_shape).astype(np.int8)
     units = rhs_shape[-2] if adj_y else rhs_shape[-1]
     pcs = rng.uniform(2e-3, 8e-3, units).astype(np.float32)
-    want = oracle.batch_matmul_hybrid(lhs, rhs, pcs, 1.0, asym, adj_y)
+    want = oracle.batch_matmul_hybrid(lhs, rhs, pcs, 1.0, asym, adj_y, adj_x=adj_x)
     w2 = rng.integers(-127, 128, (12, units)).astype(np.int8)
     pcs2 = rng.uniform(2e-3, 8e-3, 12).astype(np.float32)
     with FakeHost() as h:
@@ -110,7 +134,7 @@ def test_node_through_the_delegate(lhs_shape, rhs_shape, adj_y, asym):
         w = h.tensor(INT8, rhs_shape, data=rhs, const=True)
         h.affine(w, pcs, quantized_dimension=len(rhs_shape) - (2 if adj_y else 1))
         y = h.tensor(FLOAT32, want.shape)
-        node = h.batch_matmul(x, w, y, adj_y=adj_y, asymmetric=asym)
+        node = h.batch_matmul(x, w, y, adj_x=adj_x, adj_y=adj_y, asymmetric=asym)
         f = h.tensor(INT8, w2.shape, data=w2, const=True)
         h.affine(f, pcs2)
         z = h.tensor(FLOAT32, (want.size // units, 12))

@@ -29,7 +29,8 @@ def test_reference_vectors(case):
     lhs = np.asarray(case["lhs"], np.float32)
     rhs = np.asarray(case["rhs"], np.int8)
     got = oracle.batch_matmul_hybrid(lhs, rhs, None, case["filter_scale"],
-                                     case["asymmetric_quantize_inputs"], case["adj_y"])
+                                     case["asymmetric_quantize_inputs"], case["adj_y"],
+                                     adj_x=case["adj_x"])
     want = np.asarray(case["expected"], np.float32)
     assert got.size == want.size
     assert np.max(np.abs(got.ravel() - want)) <= case["max_abs_err"]
@@ -56,6 +57,37 @@ def test_equals_hybrid_fully_connected_where_the_float_detour_is_exact(lhs_shape
     for b in range(li.size):
         want = oracle.fc_hybrid(x[li[b]], w[ri[b]], pcs, 0.005, None, asym)
         assert np.array_equal(got[b].view(np.uint32), want.view(np.uint32)), b
+
+
+@pytest.mark.parametrize("lhs_shape,rhs_shape,adj_y", [
+    ((40, 3), (40, 7), False), ((2, 3, 64, 5), (2, 1, 9, 64), True),
+    ((2, 1, 48, 4), (1, 3, 48, 6), False), ((3, 1, 2, 16, 5), (1, 4, 1, 16, 6), False)])
+def test_adj_x_is_the_transposed_left_operand(lhs_shape, rhs_shape, adj_y):
+    """adj_x against the same oracle on the left operand transposed beforehand -- and against the
+    hybrid FULLY_CONNECTED per output matrix, with the pairing worked out here by numpy
+    broadcasting of index arrays (one-sided, two-sided and rank-5 batch shapes)."""
+    rng = np.random.default_rng([len(lhs_shape), lhs_shape[-1], int(adj_y)])
+    lhs = rng.standard_normal(lhs_shape).astype(np.float32)
+    rhs = rng.integers(-127, 128, rhs_shape).astype(np.int8)
+    units = rhs_shape[-2] if adj_y else rhs_shape[-1]
+    pcs = rng.uniform(2e-3, 8e-3, units).astype(np.float32)
+    got = oracle.batch_matmul_hybrid(lhs, rhs, pcs, 1.0, True, adj_y, adj_x=True)
+    lhs_t = np.ascontiguousarray(np.swapaxes(lhs, -1, -2))
+    same = oracle.batch_matmul_hybrid(lhs_t, rhs, pcs, 1.0, True, adj_y)
+    assert np.array_equal(got.view(np.uint32), same.view(np.uint32))
+    rows, depth = lhs_t.shape[-2:]
+    w = (rhs if adj_y else np.swapaxes(rhs, -1, -2))
+    rank = max(lhs.ndim, rhs.ndim) - 2
+    lb = (1,) * (rank - (lhs.ndim - 2)) + lhs_t.shape[:-2]
+    rb = (1,) * (rank - (rhs.ndim - 2)) + w.shape[:-2]
+    ob = np.broadcast_shapes(lb, rb)
+    assert got.shape == ob + (rows, units)
+    x = np.broadcast_to(lhs_t.reshape(lb + (rows, depth)), ob + (rows, depth))
+    wb = np.broadcast_to(w.reshape(rb + (units, depth)), ob + (units, depth))
+    for idx in np.ndindex(*ob):
+        want = oracle.fc_hybrid(np.ascontiguousarray(x[idx]), np.ascontiguousarray(wb[idx]), pcs,
+                                1.0, None, True)
+        assert np.array_equal(got[idx].view(np.uint32), want.view(np.uint32)), idx
 
 
 def test_float_detour_of_the_zero_point_correction_on_deep_rows():
