@@ -68,7 +68,8 @@ def main():
     ap.add_argument("--sustain", type=float, default=0.0,
                     help="with --gemm-probe: afterwards keep launching the GEMM for this many seconds "
                          "on the seeded operands, then as long on the constant ones, printing a "
-                         "time-stamped line at each switch (for power / clock sampling from outside)")
+                         "time-stamped line at each switch; socket power (hwmon) and `rocm-smi --showclocks` are "
+                         "sampled beside it by a child process and the medians per phase are printed")
     ap.add_argument("--roofline-probe", action="store_true",
                     help="only the cold B=1 launches of config 2 that roofline.avg_launch_us is "
                          "taken over (for a rocprofv3 --kernel-trace --stats run)")
@@ -81,6 +82,10 @@ def main():
               "by output channel with no collective). Run with --gpus 1.",
               file=sys.stderr)
         sys.exit(2)
+
+    sampler = None
+    if args.gemm_probe and args.sustain > 0:
+        sampler = start_smi_sampler()  # a child process, started before this one touches the GPU
 
     import torch
     from litert_amd import capi
@@ -103,7 +108,9 @@ def main():
         traffic_probe_int4(torch, fc, wl)
         return
     if args.gemm_probe:
-        gemm_probe(torch, fc, wl, args.sustain)
+        phases = gemm_probe(torch, fc, wl, args.sustain)
+        if sampler is not None:
+            report_smi_samples(sampler, phases)
         return
     if args.traffic_probe_int4_single:
         traffic_probe_int4_single(torch, fc, wl)
@@ -323,6 +330,63 @@ def mfma_rate(torch, seconds, random_operands):
     return ops.value * launches / (time.time() - t0) / 1e12
 
 
+def start_smi_sampler():
+    """Starts a sampling loop (a time stamp, the socket power from the amdgpu hwmon node
+    power1_input -- `rocm-smi --showpower` prints nothing for an ordinary user here --, then
+    `rocm-smi --showclocks`, about three times a second) as a child process group of its own,
+    writing to a temporary file. Returns (process, path)."""
+    import subprocess
+    import tempfile
+    fd, path = tempfile.mkstemp(prefix="lrtfc_smi_", suffix=".log")
+    loop = ("while true; do echo t=$(date +%s.%N); "
+            "echo power_uw=$(cat /sys/class/drm/card*/device/hwmon/hwmon*/power1_input 2>/dev/null | head -1); "
+            "rocm-smi --showclocks 2>&1; sleep 0.2; done")
+    proc = subprocess.Popen(["bash", "-c", loop], stdout=fd, stderr=subprocess.STDOUT,
+                            start_new_session=True)
+    os.close(fd)
+    return proc, path
+
+
+def report_smi_samples(sampler, phases):
+    """Stops the sampler and prints, per phase of the sustained run, the median shader clock and
+    socket power of the samples taken from one second into the phase on."""
+    import re
+    import signal
+    proc, path = sampler
+    try:
+        os.killpg(proc.pid, signal.SIGTERM)
+    except ProcessLookupError:
+        pass
+    proc.wait()
+    samples, now = [], None
+    for ln in open(path, errors="replace"):
+        m = re.match(r"t=([0-9.]+)", ln)
+        if m:
+            now = [float(m.group(1)), None, None]
+            samples.append(now)
+            continue
+        if now is None:
+            continue
+        m = re.search(r"sclk clock level:\s*\d+:?\s*\((\d+)Mhz\)", ln)
+        if m and now[1] is None:
+            now[1] = float(m.group(1))
+        m = re.match(r"power_uw=(\d+)", ln)
+        if m and now[2] is None:
+            now[2] = float(m.group(1)) / 1e6
+    os.unlink(path)
+
+    def median(v):
+        v = sorted(v)
+        return v[len(v) // 2] if v else None
+
+    for name, begin, end in phases:
+        inside = [s for s in samples if begin + 1.0 <= s[0] <= end]
+        print(json.dumps({"sustain": name, "smi_samples": len(inside),
+                          "sclk_mhz_median": median([s[1] for s in inside if s[1] is not None]),
+                          "power_w_median": median([s[2] for s in inside if s[2] is not None])}),
+              flush=True)
+
+
 def roofline_probe(torch, fc, wl, capture, timed_replays):
     """Only the launches behind roofline.avg_launch_us: config 2 at B = 1, one fused kernel per
     op, the filter copies rotated so that every launch streams from HBM, 24 launches per graph
@@ -386,11 +450,13 @@ def gemm_probe(torch, fc, wl, sustain=0.0):
         sets.append((name, op, x))
     print(json.dumps({"probe": "gemm", "launches_seeded": 10, "launches_constant": 10,
                       "ops_per_launch": 2 * 2048 * 4096 * 4096}), flush=True)
+    phases = []  # (name, begin, end) in unix seconds, for the power / clock samples
     if sustain > 0:
         for name, rnd in (("random", 1), ("constant", 0)):
             t0 = time.time()
             print(json.dumps({"sustain": "mfma_only_" + name, "begin_unix": round(t0, 3)}), flush=True)
             tops = mfma_rate(torch, sustain, rnd)
+            phases.append(("mfma_only_" + name, t0, time.time()))
             print(json.dumps({"sustain": "mfma_only_" + name, "end_unix": round(time.time(), 3),
                               "tops": round(tops, 1)}), flush=True)
     for name, op, x in sets if sustain > 0 else []:
@@ -407,8 +473,10 @@ def gemm_probe(torch, fc, wl, sustain=0.0):
             torch.cuda.synchronize()
             launches += 1000
         t1 = time.time()
+        phases.append((name, t0, t1))
         print(json.dumps({"sustain": name, "end_unix": round(t1, 3), "launches": launches,
                           "us_per_launch": round((t1 - t0) / launches * 1e6, 2)}), flush=True)
+    return phases
 
 
 def traffic_probe_int4_single(torch, fc, wl):
