@@ -66,9 +66,9 @@ bool FloatActivationOk(int activation) {
 
 // Batches from this size on go to the MFMA GEMM when its tiling fits.
 constexpr int kGemmMinBatches = 128;
-// On the re-tiled filter: up to this many rows the GEMV (16 rows per pass over the filter)
-// wins; beyond it the GEMM, which streams the filter once (14336 x 4096 hybrid: 16 rows
-// 19 us on the GEMV; 24 and 32 rows 27 us on the GEMM against 32 and 34 us in two passes).
+// On the re-tiled filter: up to this many rows the GEMV wins always (16 rows per pass over the
+// filter), and up to 32 rows where it can take them in one pass; beyond that the GEMM, which
+// streams the filter once.
 constexpr int kPackedGemmMinBatches = 16;
 
 // Workspace layout for the hybrid paths (kernels.h).
@@ -395,7 +395,8 @@ int lrtfc_fc_int8_packed(const int8_t* input, const int8_t* packed_filter, const
   a.act_min = act_min;
   a.act_max = act_max;
   a.output_i8 = output;
-  if (batches > kPackedGemmMinBatches && lrtfc::FcInt8PackedGemmSupports(a)) {
+  if (batches > kPackedGemmMinBatches && !lrtfc::FcInt8PackedGemvTakesRowsInOnePass(a) &&
+      lrtfc::FcInt8PackedGemmSupports(a)) {
     return FromHip(lrtfc::LaunchFcInt8PackedGemm(a, lrtfc::Int8Epilogue::kRequantize,
                                                  AsStream(stream)),
                    "packed int8 GEMM");
@@ -472,7 +473,8 @@ int FcHybridInt8Packed(const int8_t* quantized_input, const float* scaling_facto
   a.output_f32 = output;
   a.zero_input_exit = zero_input_exit;
   a.batch_matmul = batch_matmul;
-  if (batches > kPackedGemmMinBatches && lrtfc::FcInt8PackedGemmSupports(a)) {
+  if (batches > kPackedGemmMinBatches && !lrtfc::FcInt8PackedGemvTakesRowsInOnePass(a) &&
+      lrtfc::FcInt8PackedGemmSupports(a)) {
     return FromHip(lrtfc::LaunchFcInt8PackedGemm(a, lrtfc::Int8Epilogue::kHybrid,
                                                  AsStream(stream)),
                    "packed hybrid GEMM");
@@ -544,7 +546,7 @@ int lrtfc_batch_matmul_hybrid_packed_nd(const float* lhs, const int* lhs_batch_d
   if (int rc = RequireInit()) return rc;
   LRTFC_REQUIRE(lhs_batch_dims && weight_batch_dims, "null pointer");
   LRTFC_REQUIRE(rows >= 0 && depth > 0 && units >= 0, "bad dimension");
-  int64_t lhs_matrices = 1, weight_matrices = 1, out_matrices = 1;
+  int64_t lhs_matrices = 1, out_matrices = 1;
   int out_dims[3];
   for (int i = 0; i < 3; ++i) {
     const int l = lhs_batch_dims[i], w = weight_batch_dims[i];
@@ -553,7 +555,6 @@ int lrtfc_batch_matmul_hybrid_packed_nd(const float* lhs, const int* lhs_batch_d
                   "batch dimension %d: %d against %d can not be broadcast", i, l, w);
     out_dims[i] = l == 1 ? w : l;  // batch_matmul.h:33-38
     lhs_matrices *= l;
-    weight_matrices *= w;
     out_matrices *= out_dims[i];
     LRTFC_REQUIRE(out_matrices <= 0x7fffffff, "too many matrices");
   }
@@ -920,7 +921,8 @@ int lrtfc_fc_hybrid_int4_per_channel_packed(const float* input, const int8_t* pa
   a.bias_f32 = bias;
   a.activation = activation;
   a.output_f32 = output;
-  if (batches > kPackedGemmMinBatches && lrtfc::FcInt8PackedGemmSupports(a)) {
+  if (batches > kPackedGemmMinBatches && !lrtfc::FcInt8PackedGemvTakesRowsInOnePass(a) &&
+      lrtfc::FcInt8PackedGemmSupports(a)) {
     return FromHip(lrtfc::LaunchFcInt8PackedGemm(a, lrtfc::Int8Epilogue::kHybrid4Bit,
                                                  AsStream(stream)),
                    "packed int4 per-channel hybrid GEMM");

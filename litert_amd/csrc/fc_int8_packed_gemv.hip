@@ -511,9 +511,9 @@ constexpr size_t kResidentPackedArgsOffset =
     (sizeof(ResidentLeadingArgs) + alignof(PackedArgs) - 1) / alignof(PackedArgs) * alignof(PackedArgs);
 static_assert(kResidentPackedArgsOffset == 56, "argument layout of FcInt8ResidentGemvKernel");
 
-template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY, int WAVES>
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY, int WAVES, int RT = 1>
 __global__ __launch_bounds__(WAVES * kWaveSize)
-__attribute__((amdgpu_waves_per_eu(WAVES / 2, WAVES / 2)))
+__attribute__((amdgpu_waves_per_eu(WAVES / 2 / RT, WAVES / 2 / RT)))
 void FcInt8ResidentGemvKernel(
     const int8_t* early_filter, const float* early_input_f32, const int8_t* early_input_i8,
     int early_depth, int early_slabs, int early_out_depth, int batch0, int bt, int ksplit_log2,
@@ -535,7 +535,11 @@ void FcInt8ResidentGemvKernel(
   // multiplies its (clamped, re-read) tiles by zeros instead of branching.
   const int staged = ksplit * per_part * kSlabDepth;
   const int qstride = staged + kQPad;
-  const Shared sh = CarveShared(smem, bt, qstride, WAVES);
+  // RT: tiles of 16 batch rows a wavefront multiplies each weight tile with (2: 17 to 32 rows
+  // that arrive quantized; every row of a workgroup's LDS image is then read by eight
+  // wavefronts instead of four, and the workgroup has its compute unit to itself).
+  static_assert(RT == 1 || (RT == 2 && !FUSED), "two row tiles: rows that arrive quantized");
+  const Shared sh = CarveShared(smem, bt, qstride, WAVES * RT);
   const int tiles = (early_out_depth + kTileRows - 1) / kTileRows;
   const int tile = ((blockIdx.x * WAVES) >> ksplit_log2) + (wave >> ksplit_log2);
   const int part = wave & (ksplit - 1);
@@ -565,8 +569,9 @@ void FcInt8ResidentGemvKernel(
 
   // The row parameters of this lane's batch column: read from LDS behind the barrier (fused) or
   // requested with the per-channel parameters (rows that arrive quantized).
-  float lds_scale = 0.0f;
-  int32_t lds_zp = 0, lds_zero = 0;
+  float lds_scale[RT] = {};
+  int32_t lds_zp[RT] = {};
+  int32_t lds_zero = 0;
   bool ep_has_row_zero_points = false;
   // Per-channel epilogue parameters, requested behind the first tiles (they are needed last).
   // Unconditional loads: an absent array reads a valid dummy address.
@@ -601,9 +606,12 @@ void FcInt8ResidentGemvKernel(
         // whole weight stream.
         const float* row_scales = late->a.scaling_factors;
         const int32_t* row_zero_points = late->a.zero_points;
-        const int row = batch0 + min(col, bt - 1);
-        lds_scale = row_scales[row];
-        lds_zp = *(row_zero_points ? row_zero_points + row : dummy_i);
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+          const int row = batch0 + min(col + 16 * r, bt - 1);
+          lds_scale[r] = row_scales[row];
+          lds_zp[r] = *(row_zero_points ? row_zero_points + row : dummy_i);
+        }
         ep_has_row_zero_points = row_zero_points != nullptr;
       }
 #pragma unroll
@@ -639,25 +647,39 @@ void FcInt8ResidentGemvKernel(
     ep_offsets3 = late->a.act_max;
     ep_batches = late->a.batches;
   };
-  const int8_t* qbase = sh.q + (col < bt ? col : 0) * qstride + kgroup * 16 + s0 * kSlabDepth;
+  const int8_t* qbase[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    qbase[r] = sh.q + (col + 16 * r < bt ? col + 16 * r : 0) * qstride + kgroup * 16 +
+               s0 * kSlabDepth;
+  }
   const int8_t* pad_zero = sh.q + staged;  // the kQPad bytes behind row 0, cleared below
   constexpr int kAccs = 4;
-  i32x4 acc4[kAccs];
+  i32x4 acc4[RT][kAccs];
 #pragma unroll
-  for (int i = 0; i < kAccs; ++i) acc4[i] = i32x4{0, 0, 0, 0};
-  // Products of tiles g .. g + 3: four activation operands per LDS wait.
+  for (int r = 0; r < RT; ++r)
+#pragma unroll
+    for (int i = 0; i < kAccs; ++i) acc4[r][i] = i32x4{0, 0, 0, 0};
+  // Products of tiles g .. g + 3: four activation operands (per row tile) per LDS wait.
   auto multiply4 = [&](int g) {
-    i32x4 bq[4];
+    i32x4 bq[RT][4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      // Past the share (which only happens when TILES is larger than the share) the operand
-      // is the 16 bytes of zeros behind row 0.
-      const int8_t* at = g + u < per_part ? qbase + (g + u) * kSlabDepth : pad_zero;
-      bq[u] = *reinterpret_cast<const i32x4*>(at);
+    for (int r = 0; r < RT; ++r) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        // Past the share (which only happens when TILES is larger than the share) the operand
+        // is the 16 bytes of zeros behind row 0.
+        const int8_t* at = g + u < per_part ? qbase[r] + (g + u) * kSlabDepth : pad_zero;
+        bq[r][u] = *reinterpret_cast<const i32x4*>(at);
+      }
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      acc4[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ring[g + u], bq[u], acc4[u], 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < RT; ++r) {
+        acc4[r][u] =
+            __builtin_amdgcn_mfma_i32_16x16x64_i8(ring[g + u], bq[r][u], acc4[r][u], 0, 0, 0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -678,8 +700,8 @@ void FcInt8ResidentGemvKernel(
     fetch_epilogue_scalars();
     __syncthreads();
     if (FUSED) {  // the row's parameters for the epilogue, while nothing waits for them
-      lds_scale = sh.sf[col < bt ? col : 0];
-      lds_zp = sh.zp[col < bt ? col : 0];
+      lds_scale[0] = sh.sf[col < bt ? col : 0];
+      lds_zp[0] = sh.zp[col < bt ? col : 0];
       lds_zero = sh.zero[col < bt ? col : 0];
     }
 #pragma unroll
@@ -759,7 +781,7 @@ void FcInt8ResidentGemvKernel(
     // requested ahead of the weights and written to LDS when they are there.
     // 16-byte pieces of quantized rows per thread: 4 rows of depth 4096, or 16 (EARLY, which
     // has no other meaning for rows that arrive quantized).
-    constexpr int kQRegs = (EARLY ? 64 : 16) / WAVES;
+    constexpr int kQRegs = (EARLY ? 64 : 16) * RT / WAVES;
     constexpr int kFirst = TILES < 8 ? TILES : 8;
     i32x4 qr[kQRegs];
     const int chunks_per_row = staged / 16;
@@ -786,17 +808,26 @@ void FcInt8ResidentGemvKernel(
     __builtin_amdgcn_sched_barrier(0);
     stream(integral_constant<int, kFirst>{}, integral_constant<int, kStreamAhead>{});
   }
-  i32x4 acc = (acc4[0] + acc4[1]) + (acc4[2] + acc4[3]);
+  i32x4 acc_of[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc_of[r] = (acc4[r][0] + acc4[r][1]) + (acc4[r][2] + acc4[r][3]);
 
   if (ksplit > 1) {
-    sh.partial[wave * 64 + lane] = acc;
+#pragma unroll
+    for (int r = 0; r < RT; ++r) sh.partial[(r * WAVES + wave) * 64 + lane] = acc_of[r];
     __syncthreads();
     if (part != 0) return;
-    for (int w = 1; w < ksplit; ++w) acc += sh.partial[(wave + w) * 64 + lane];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      for (int w = 1; w < ksplit; ++w) acc_of[r] += sh.partial[(r * WAVES + wave + w) * 64 + lane];
+    }
   }
 
-  if (col >= bt || tile >= tiles) return;
-  const int b = batch0 + col;
+  if (tile >= tiles) return;
+  // The epilogue of one row tile: this lane's row is col + 16 * r.
+  auto finish = [&](int r, const i32x4 acc) {
+  if (col + 16 * r >= bt) return;
+  const int b = batch0 + col + 16 * r;
   const int out_depth = early_out_depth;
   const int n0 = tile * kTileRows + 4 * kgroup;  // this lane's four channels: n0 .. n0 + 3
   if (EPI == Int8Epilogue::kRequantize) {
@@ -822,8 +853,8 @@ void FcInt8ResidentGemvKernel(
   // Float epilogues. The four values of a lane are computed side by side without branches (the
   // tail of the slowest wavefront is the tail of the launch); the one rare case that needs a
   // scan of the input, a whole-zero input meeting a -0.0f bias, takes a branch of its own.
-  const float batch_scale = lds_scale;
-  const int32_t batch_zp = (FUSED || ep_has_row_zero_points) ? lds_zp : 0;
+  const float batch_scale = lds_scale[r];
+  const int32_t batch_zp = (FUSED || ep_has_row_zero_points) ? lds_zp[r] : 0;
   const bool row_zero = FUSED ? lds_zero != 0 : true;
   float value[4];
   bool rare = false;
@@ -886,6 +917,9 @@ void FcInt8ResidentGemvKernel(
       if (n0 + i < out_depth) out[i] = value[i];
     }
   }
+  };
+#pragma unroll
+  for (int r = 0; r < RT; ++r) finish(r, acc_of[r]);
 }
 
 // How many wavefronts share one channel group's depth (see LaunchSized below).
@@ -896,13 +930,14 @@ int ChooseKsplit(int slabs, int tiles, int waves = kWaves) {
   return ksplit;
 }
 
-template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY, int WAVES = kWaves>
+template <Int8Epilogue EPI, bool FUSED, int VARIANT, int TILES, bool EARLY, int WAVES = kWaves,
+          int RT = 1>
 hipError_t LaunchResidentSized(const PackedArgs& p, int batch0, int bt, int ksplit,
                               hipStream_t stream) {
   const int per_part = (p.slabs + ksplit - 1) / ksplit;
   const int qstride = ksplit * per_part * kSlabDepth + kQPad;
-  const size_t lds = SharedBytes(bt, qstride, WAVES);
-  auto kernel = FcInt8ResidentGemvKernel<EPI, FUSED, VARIANT, TILES, EARLY, WAVES>;
+  const size_t lds = SharedBytes(bt, qstride, WAVES * RT);
+  auto kernel = FcInt8ResidentGemvKernel<EPI, FUSED, VARIANT, TILES, EARLY, WAVES, RT>;
   if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
   const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
   const int tiles_per_wg = WAVES / ksplit;
@@ -922,12 +957,40 @@ hipError_t LaunchResidentSized(const PackedArgs& p, int batch0, int bt, int kspl
 // tiles each, so that the wavefronts that quantize (one per row) leave as many that only
 // stream (measured at 14336 x 4096, one launch, cold: 1 row 11.0 us narrow / 11.4 wide; 2 rows
 // 11.4 / 11.3; 4 rows 12.6 / 12.0; 8 rows 13.1 wide against 14.7 as row quantizer + product).
+// 17 to 32 rows that arrive quantized: one pass over the filter with two row tiles per weight
+// tile, on workgroups of eight wavefronts with at most 16 tiles each, as long as the rows' LDS
+// image (32 x depth) fits one compute unit. *ksplit receives the depth split.
+bool ResidentTwoRowTilesFit(const PackedArgs& p, int bt, int* ksplit_out) {
+  if (bt <= 16 || bt > 32) return false;
+  if (p.a.depth % 16 != 0 || (reinterpret_cast<uintptr_t>(p.a.input) & 15) != 0) return false;
+  int ksplit = 1;
+  while (ksplit < 8 && (p.slabs + ksplit - 1) / ksplit > 16) ksplit *= 2;
+  const int per_part = (p.slabs + ksplit - 1) / ksplit;
+  if (per_part > 16) return false;
+  const int staged = ksplit * per_part * kSlabDepth;
+  if (static_cast<int64_t>(bt) * (staged / 16) > 16 * 8 * kWaveSize) return false;
+  if (SharedBytes(bt, staged + kQPad, 16) > 150 * 1024) return false;
+  if (ksplit_out) *ksplit_out = ksplit;
+  return true;
+}
+
 template <Int8Epilogue EPI, bool FUSED, int VARIANT>
 hipError_t TryLaunchResident(const PackedArgs& p, int batch0, int bt, hipStream_t stream,
                             bool* launched) {
   *launched = false;
   const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
   const int depth = p.a.depth;
+  if constexpr (!FUSED) {
+    if (bt > 16) {
+      int ksplit = 1;
+      if (!ResidentTwoRowTilesFit(p, bt, &ksplit)) return hipSuccess;
+      *launched = true;
+      if ((p.slabs + ksplit - 1) / ksplit <= 8) {
+        return LaunchResidentSized<EPI, false, VARIANT, 8, true, 8, 2>(p, batch0, bt, ksplit, stream);
+      }
+      return LaunchResidentSized<EPI, false, VARIANT, 16, true, 8, 2>(p, batch0, bt, ksplit, stream);
+    }
+  }
   if (FUSED) {
     const bool vec_ok =
         (depth % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.input_f32) & 15) == 0);
@@ -1063,6 +1126,15 @@ int FcInt8PackedGemvFusedMaxRows(int depth) {
   return (depth % 4 == 0 && depth <= kFusedRowMaxDepth) ? kFusedMaxRows : 4;
 }
 
+bool FcInt8PackedGemvTakesRowsInOnePass(const FcInt8Args& a) {
+  if (a.batches <= 16) return FcInt8PackedGemvSupports(a);
+  if (!FcInt8PackedGemvSupports(a)) return false;
+  PackedArgs p;
+  p.a = a;
+  p.slabs = (a.depth + kSlabDepth - 1) / kSlabDepth;
+  return ResidentTwoRowTilesFit(p, a.batches, nullptr);
+}
+
 bool FcInt8PackedGemvSupports(const FcInt8Args& a) {
   // The per-tensor form with a non-zero filter zero point needs sum(x), which this
   // kernel does not carry; the row-major GEMV handles it.
@@ -1085,7 +1157,10 @@ hipError_t LaunchFcInt8PackedGemv(const FcInt8Args& a, Int8Epilogue epilogue,
   int batch0 = 0;
   while (batch0 < a.batches) {
     int bt = min(16, a.batches - batch0);
-    while (bt > 1 && SharedBytes(bt, qstride) > 150 * 1024) --bt;
+    if (!input_f32 && ResidentTwoRowTilesFit(p, a.batches - batch0, nullptr)) {
+      bt = a.batches - batch0;  // 17 to 32 rows in one pass
+    }
+    while (bt > 1 && bt <= 16 && SharedBytes(bt, qstride) > 150 * 1024) --bt;
     hipError_t err;
     if (epilogue == Int8Epilogue::kRequantize) {
       err = LaunchVariant<Int8Epilogue::kRequantize, false>(p, variant, batch0, bt, stream);

@@ -128,6 +128,9 @@ hipError_t LaunchFcInt4PerChannelGemv(const uint8_t* packed, const float* input_
 // Prefill batches on the same re-tiled filter: int8 MFMA GEMM (a.filter = packed, a.input =
 // int8 rows; the hybrid epilogue reads a.scaling_factors / a.zero_points). Any batch count,
 // any out_depth; depth a multiple of 16.
+// Whether the GEMV streams the filter once for all of a.batches rows (up to 16 always; 17 to 32
+// rows that arrive quantized when their LDS image fits a compute unit).
+bool FcInt8PackedGemvTakesRowsInOnePass(const FcInt8Args& a);
 bool FcInt8PackedGemmSupports(const FcInt8Args& a);
 hipError_t LaunchFcInt8PackedGemm(const FcInt8Args& a, Int8Epilogue epilogue, hipStream_t stream);
 

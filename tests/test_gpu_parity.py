@@ -224,6 +224,38 @@ def test_hybrid_packed_gemm_matches_oracle(fc, B, K, N, asym, per_channel):
     assert _bits_equal(y, want)
 
 
+@pytest.mark.parametrize("B,K,N", [(17, 64, 20), (24, 4096, 1024), (32, 4096, 520), (31, 1040, 301),
+                                   (32, 512, 14336), (20, 2064, 48), (29, 16, 4), (32, 272, 100),
+                                   (17, 8192, 64), (30, 4100, 40)])
+@pytest.mark.parametrize("asym", [True, False])
+def test_hybrid_17_to_32_rows_in_one_pass_matches_oracle(fc, B, K, N, asym):
+    """17 to 32 rows whose LDS image fits a compute unit take the register-resident GEMV with two
+    row tiles per weight tile (depth shares of 8 and 16 tiles, depths that end inside a slab, one
+    or several channel tiles per workgroup, ragged channel counts); the last two shapes -- too
+    deep, and a depth that is no multiple of 16 -- go to the GEMM instead. Same bits either way."""
+    c = wl.hybrid_fc(B, K, N, seed=29 + B + K)
+    bias = np.random.default_rng(5).standard_normal(N).astype(np.float32)
+    bias[::5] = -0.0
+    pcs = c["pcs"] if (B + N) % 2 else None
+    for activation, code in (("relu6", oracle.ACT_RELU6), ("none", oracle.ACT_NONE)):
+        op = fc.FullyConnectedHybrid(c["w"], pcs, filter_scale=0.005, bias=bias,
+                                     asymmetric_quantize_inputs=asym, activation=activation)
+        y = op(_cuda(c["x"])).cpu().numpy()
+        want = oracle.fc_hybrid(c["x"], c["w"], pcs, 0.005, bias, asym, code)
+        assert _bits_equal(y, want)
+    zeros = np.zeros_like(c["x"])  # the whole-zero input exit keeps the bias bits
+    y = op(_cuda(zeros)).cpu().numpy()
+    assert _bits_equal(y, oracle.fc_hybrid(zeros, c["w"], pcs, 0.005, bias, asym, oracle.ACT_NONE))
+
+
+@pytest.mark.parametrize("B,K,N", [(17, 64, 20), (32, 4096, 520), (31, 1040, 301), (24, 2048, 2048)])
+@pytest.mark.parametrize("activation", ["none", "relu6"])
+def test_int8_17_to_32_rows_in_one_pass_bit_exact(fc, B, K, N, activation):
+    c = wl.int8_fc(B, K, N, in_zp=(-3 if N % 2 else 0), seed=310 + B + K + N)
+    y, want = _run_int8(fc, c, activation, bias=(N % 3 != 0))
+    assert np.array_equal(y, want)
+
+
 def test_int8_prefill_full_size_properties(fc):
     """Config 4 at full size (2048 x 4096 x 4096), RELU6 on and off, checked through
     size-independent properties: a random sample of outputs against an int64 numpy
