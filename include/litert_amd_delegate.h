@@ -44,13 +44,16 @@ typedef struct litert_amd_metrics {
   int64_t bytes_uploaded;    /* host -> device */
   int64_t bytes_downloaded;  /* device -> host */
   double host_time_us;       /* wall time inside the partitions' invoke callbacks */
-  double device_time_us;     /* per invoke: first enqueued copy to last finished one (HIP events) */
+  double device_time_us;     /* per invoke: first enqueued command to last finished one (HIP
+                              * events; collected from detail_level 1 on, 0 below) */
   /* host_time_us by phase of an invoke: host tensors gathered into page-locked memory; copies and
    * kernels enqueued; the wait for the device to finish; outputs scattered back to the tensors. */
   double host_gather_us, host_enqueue_us, host_wait_us, host_scatter_us;
 } litert_amd_metrics;
 /* Both return 0, or 1 when `delegate` is not one of this library's (or, for stop, when no
- * collection is running). start clears the totals. */
+ * collection is running). start clears the totals. detail_level 0: counts, bytes and host times
+ * (a few clock reads per invoke); 1 and above: device_time_us as well (two event records per
+ * invoke, which lengthen the enqueue phase by a few microseconds). */
 int litert_amd_start_metrics(TfLiteDelegate* delegate, int detail_level);
 int litert_amd_stop_metrics(TfLiteDelegate* delegate, litert_amd_metrics* out);
 

@@ -1452,8 +1452,11 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   RETURN_IF_HIP(ctx, hipSetDevice(k->state->options.device));
   MetricsState& metrics = k->state->metrics;
   const bool measure = metrics.on;
+  // Device time costs two event records per invoke and their read-back; it is taken from
+  // detail level 1 on, so that level 0 times the invoke as it runs without a collection.
+  const bool measure_device = measure && metrics.detail_level >= 1;
   const auto host_begin = std::chrono::steady_clock::now();
-  if (measure) {
+  if (measure_device) {
     if (!k->metrics_begin) {
       RETURN_IF_HIP(ctx, hipEventCreate(&k->metrics_begin));
       RETURN_IF_HIP(ctx, hipEventCreate(&k->metrics_end));
@@ -1688,7 +1691,7 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
                                       k->arena.as<uint8_t>() + k->download_offset,
                                       k->download_bytes, hipMemcpyDeviceToHost, s));
   }
-  if (measure) RETURN_IF_HIP(ctx, hipEventRecord(k->metrics_end, s));
+  if (measure_device) RETURN_IF_HIP(ctx, hipEventRecord(k->metrics_end, s));
   if (k->completion_dev) {
     if (++k->completion_serial == 0) k->completion_serial = 1;  // the word starts out as 0
     RETURN_IF_FC(ctx, lrtfc_mark_completion(k->completion_dev, k->completion_serial, s));
@@ -1713,11 +1716,13 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   }
   if (!finished) RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
   const auto waited = std::chrono::steady_clock::now();
-  if (measure) {
+  if (measure_device) {
     if (finished) RETURN_IF_HIP(ctx, hipEventSynchronize(k->metrics_end));
     float ms = 0.0f;
     RETURN_IF_HIP(ctx, hipEventElapsedTime(&ms, k->metrics_begin, k->metrics_end));
     metrics.device_us += 1e3 * ms;
+  }
+  if (measure) {
     metrics.invokes += 1;
     metrics.nodes += static_cast<int64_t>(k->nodes.size());
     if (host_inputs) metrics.uploaded += static_cast<int64_t>(k->upload_bytes);

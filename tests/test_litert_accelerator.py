@@ -188,13 +188,22 @@ def test_metrics_collection_reports_what_the_partitions_did():
         m = lib.litert_amd_metrics_object_new()
         assert d.stop_metrics_collection(C.byref(ctx), 0xABC0, m) == 1  # nothing was started
         assert h.invoke() == OK  # before the collection: not counted
-        assert d.start_metrics_collection(C.byref(ctx), 0xABC0, 0) == 0
+        assert d.start_metrics_collection(C.byref(ctx), 0xABC0, 1) == 0  # level 1: device time too
         for _ in range(3):
             assert h.invoke() == OK, h.errors()
         assert d.stop_metrics_collection(C.byref(ctx), 0xABC0, m) == 0
         got = {lib.litert_amd_metrics_object_name(m, i).decode(): lib.litert_amd_metrics_object_value(m, i)
                for i in range(lib.litert_amd_metrics_object_size(m))}
         lib.litert_amd_metrics_object_free(m)
+        m0 = lib.litert_amd_metrics_object_new()
+        assert d.start_metrics_collection(C.byref(ctx), 0xABC0, 0) == 0  # level 0: host side only
+        assert h.invoke() == OK, h.errors()
+        assert d.stop_metrics_collection(C.byref(ctx), 0xABC0, m0) == 0
+        got0 = {lib.litert_amd_metrics_object_name(m0, i).decode(): lib.litert_amd_metrics_object_value(m0, i)
+                for i in range(lib.litert_amd_metrics_object_size(m0))}
+        lib.litert_amd_metrics_object_free(m0)
+        assert got0["litert_amd.partition_invokes"] == 1 and got0["litert_amd.device_time_us"] == 0
+        assert got0["litert_amd.host_time_us"] > 0
         assert got["litert_amd.partition_invokes"] == 3 and got["litert_amd.nodes_run"] == 3
         assert got["litert_amd.bytes_uploaded"] == 3 * c["x"].nbytes
         assert got["litert_amd.bytes_downloaded"] == 3 * 2 * 64 * 4
