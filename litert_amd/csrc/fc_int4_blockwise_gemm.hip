@@ -530,6 +530,173 @@ __global__ __launch_bounds__(kThreads) void FcInt4NibbleGemmKernel(NibbleGemmArg
   }
 }
 
+
+// ---- the same filter for one to four rows: four blocks per matrix-core tile ----------------
+//
+// With at most four batch rows a 16 x 16 result tile per block is three quarters padding, and
+// what bounds the kernel above is the vector work per tile (conversion, scale, add: per block
+// whatever the row count). Here the sixteen columns of a result tile are (block j of the quad,
+// row r), column 4 j + r: the quad's four MFMAs accumulate into ONE tile, MFMA j with a B operand
+// that holds the rows' values of block j in columns 4 j .. 4 j + 3 and zeros elsewhere (a lane
+// loads the eight activation bytes of its own column's block once per quad; a move that writes
+// only lane group j of every row of 16 (DPP bank mask) over zeros makes the four operands). One
+// conversion and one scale per tile instead of four; the products of blocks 1..3 then reach the
+// lanes of block 0 by row shifts and are added there in block order, which is the reference's
+// order of float additions, so the results are bit-identical to every other form. Rows are read
+// from the standard row quantizer's row-major output; there is no LDS image and no barrier.
+struct NibbleQuadArgs {
+  const i32x4* filter;   // tile16x128n
+  const uint2* scales;   // fp16 [tiles][ng][64 lanes][4]
+  const int8_t* rows;    // [batches][depth] int8
+  const float* scaling_factors;
+  const int32_t* zero_points;
+  const float* kfsum;
+  const float* bias;
+  float* output;
+  int batches, depth, out_depth, nb, channel_tiles, vector_store;
+};
+
+template <int J>
+__device__ __forceinline__ i64 OnlyLaneGroup(i64 x) {
+  // quad_perm identity, every row, bank J only; the other lanes keep the zero.
+  const int lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0xE4, 0xF, 1 << J, false);
+  const int hi = __builtin_amdgcn_update_dpp(0, static_cast<int>(x >> 32), 0xE4, 0xF, 1 << J, false);
+  return static_cast<i64>(static_cast<uint64_t>(static_cast<uint32_t>(lo)) |
+                          (static_cast<uint64_t>(static_cast<uint32_t>(hi)) << 32));
+}
+
+// The value of the lane N places up in the same row of 16 (row_shl:N); lanes past the row read 0.
+template <int N>
+__device__ __forceinline__ float FromLaneAbove(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x100 + N, 0xF, 0xF, true));
+}
+
+template <int WQ, int XQ>
+__device__ __forceinline__ void FcInt4NibbleQuadBody(const NibbleQuadArgs& a, int ct0) {
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 15;
+  const int jl = col >> 2;                     // the block of a quad this lane's column belongs to
+  const int r = min(col & 3, a.batches - 1);   // its batch row (clamped: the copy is not stored)
+  const int nb = a.nb;
+  const int nq = (nb + 3) / 4;
+  const int ng = (nb + 15) / 16;
+  const i32x4* wp = a.filter + static_cast<size_t>(ct0) * nq * 64 + lane;
+  const uint2* sp = a.scales + static_cast<size_t>(ct0) * ng * 64 + lane;
+  const int8_t* xrow = a.rows + static_cast<size_t>(r) * a.depth + 8 * (lane >> 4);
+  auto fetch_w = [&](int q) {
+    return __builtin_nontemporal_load(wp + static_cast<size_t>(min(q, nq - 1)) * 64);
+  };
+  // Past the depth: the last block again (its weights there are zeros).
+  auto fetch_x = [&](int q) {
+    const int b = min(4 * min(q, nq - 1) + jl, nb - 1);
+    return *reinterpret_cast<const i64*>(xrow + b * kBlock);
+  };
+  constexpr int kGroups = WQ / 4 + 1 <= 2 ? 2 : (WQ / 4 + 1 <= 4 ? 4 : 8);
+  static_assert((kGroups - 1) * 4 >= WQ, "scale groups must lead the weight ring");
+  uint2 sg[kGroups];
+  auto fetch_scales = [&](int g) { return sp[static_cast<size_t>(min(g, ng - 1)) * 64]; };
+#pragma unroll
+  for (int g = 0; g + 1 < kGroups; ++g) sg[g] = fetch_scales(g);
+  i32x4 wring[WQ];
+  i64 xring[XQ];
+#pragma unroll
+  for (int s = 0; s < WQ; ++s) wring[s] = fetch_w(s);
+#pragma unroll
+  for (int s = 0; s < XQ; ++s) xring[s] = fetch_x(s);
+  // Where quad t of a group of 16 blocks keeps this lane's scales: the lane of this row of 16
+  // whose block is 4 t + jl (byte index for ds_bpermute).
+  int from[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) from[t] = 4 * ((lane & 48) + 4 * t + jl);
+
+  // out[i]: channel 16 ct0 + 4 (lane / 16) + i, batch row col (lanes with col < 4), times 16.
+  float out[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  const i32x4 zero = {0, 0, 0, 0};
+  constexpr int kTrip = WQ > 4 * kGroups ? WQ : 4 * kGroups;
+  static_assert(kTrip % WQ == 0 && kTrip % XQ == 0 && kTrip % (4 * kGroups) == 0, "trip");
+  float4 cur_scales = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  for (int base = 0; base < nq; base += kTrip) {
+    StaticFor<kTrip>([&](auto u_const) {
+      constexpr int u = decltype(u_const)::value;
+      constexpr int cur = (u / 4) % kGroups;
+      if constexpr (u % 4 == 0) {
+        const uint2 raw = sg[cur];
+        cur_scales = make_float4(HalfBitsToFloatFast(static_cast<uint16_t>(raw.x & 0xFFFF)),
+                                 HalfBitsToFloatFast(static_cast<uint16_t>(raw.x >> 16)),
+                                 HalfBitsToFloatFast(static_cast<uint16_t>(raw.y & 0xFFFF)),
+                                 HalfBitsToFloatFast(static_cast<uint16_t>(raw.y >> 16)));
+        sg[(cur + kGroups - 1) % kGroups] = fetch_scales((base + u) / 4 + kGroups - 1);
+      }
+      const i32x4 w = wring[u % WQ];
+      wring[u % WQ] = fetch_w(base + u + WQ);
+      const i64 x = xring[u % XQ];
+      xring[u % XQ] = fetch_x(base + u + XQ);
+      if (base + u < nq) {
+        i32x4 acc = zero;
+        StaticFor<4>([&](auto h_const) {
+          constexpr int h = decltype(h_const)::value;
+          const uint32_t d = static_cast<uint32_t>(w[h]);
+          const uint32_t lo = (d << 4) & 0xF0F0F0F0u;
+          const uint32_t hi = d & 0xF0F0F0F0u;
+          const i64 wa = static_cast<i64>(static_cast<uint64_t>(lo) |
+                                          (static_cast<uint64_t>(hi) << 32));
+          acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(wa, OnlyLaneGroup<h>(x), acc, 0, 0, 0);
+        });
+        constexpr int t = u % 4;
+        const float sc[4] = {
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from[t], __float_as_int(cur_scales.x))),
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from[t], __float_as_int(cur_scales.y))),
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from[t], __float_as_int(cur_scales.z))),
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from[t], __float_as_int(cur_scales.w)))};
+        // Blocks past the depth have zero weights and zero scales: they add +0.0f, which cannot
+        // change a sum that has already taken its first block.
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = __fmul_rn(static_cast<float>(acc[i]), sc[i]);
+          float o = __fadd_rn(out[i], p);
+          o = __fadd_rn(o, FromLaneAbove<4>(p));
+          o = __fadd_rn(o, FromLaneAbove<8>(p));
+          o = __fadd_rn(o, FromLaneAbove<12>(p));
+          out[i] = o;
+        }
+      }
+    });
+  }
+
+  // fully_connected.cc:1078-1082, after taking the factor 16 back out (exact).
+  const int m = col;
+  if (m >= a.batches || m >= 4) return;
+  const float zp = static_cast<float>(a.zero_points[m]);
+  const float row_scale = a.scaling_factors[m];
+  const int n0 = ct0 * kTile + 4 * (lane >> 4);
+  float o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = min(n0 + i, a.out_depth - 1);
+    float v = __fsub_rn(__fmul_rn(out[i], 0.0625f), __fmul_rn(zp, a.kfsum[n]));
+    v = __fmul_rn(v, row_scale);
+    if (a.bias) v = __fadd_rn(v, a.bias[n]);
+    o[i] = v;
+  }
+  float* dst = a.output + static_cast<size_t>(m) * a.out_depth + n0;
+  if (n0 + 3 < a.out_depth && a.vector_store) {
+    *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (n0 + i < a.out_depth) dst[i] = o[i];
+    }
+  }
+}
+
+template <int WQ, int XQ>
+__global__ __launch_bounds__(kThreads) void FcInt4NibbleQuadKernel(NibbleQuadArgs a) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int ct0 = blockIdx.x * 4 + wave;
+  if (ct0 >= a.channel_tiles) return;
+  FcInt4NibbleQuadBody<WQ, XQ>(a, ct0);
+}
+
 }  // namespace
 
 size_t GemmInt4BlockwiseBytes(int out_depth, int depth) {
@@ -682,6 +849,33 @@ hipError_t LaunchFcInt4BlockwiseNibbleGemm(const float* input, int variant,
   const int nb = depth / kBlock;
   const int row_tiles = (batches + kTile - 1) / kTile;
   const int channel_tiles = (out_depth + kTile - 1) / kTile;
+  if (batches <= 4) {
+    // Row-major quantized rows (they fit where the tiled rows of a 16-row tile would lie).
+    if (hipError_t err = LaunchBatchQuantize(input, batches, depth, static_cast<int8_t*>(tiled_rows),
+                                             scaling_factors, zero_points, /*do_asymmetric=*/1,
+                                             variant, stream)) {
+      return err;
+    }
+    NibbleQuadArgs q;
+    q.filter = reinterpret_cast<const i32x4*>(nibble_filter);
+    q.scales = reinterpret_cast<const uint2*>(
+        nibble_filter + static_cast<size_t>(channel_tiles) * ((nb + 3) / 4) * 1024);
+    q.rows = static_cast<const int8_t*>(tiled_rows);
+    q.scaling_factors = scaling_factors;
+    q.zero_points = zero_points;
+    q.kfsum = kfsum;
+    q.bias = bias;
+    q.output = output;
+    q.batches = batches;
+    q.depth = depth;
+    q.out_depth = out_depth;
+    q.nb = nb;
+    q.channel_tiles = channel_tiles;
+    q.vector_store = (out_depth % 4 == 0) && (reinterpret_cast<uintptr_t>(output) % 16 == 0);
+    hipLaunchKernelGGL((FcInt4NibbleQuadKernel<8, 4>), dim3((channel_tiles + 3) / 4), dim3(kThreads),
+                       0, stream, q);
+    return hipGetLastError();
+  }
   switch (variant) {
     case LRTFC_QUANT_NEON_V8:
       LaunchTiledQuantizer<LRTFC_QUANT_NEON_V8>(input, batches, depth, row_tiles, tiled_rows,

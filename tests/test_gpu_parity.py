@@ -604,6 +604,26 @@ def test_blockwise_int4_gemm_matches_oracle(fc, B, K, N, bias):
     assert _bits_equal(op.call_gemm_nibbles(_cuda(c["x"])).cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("B,K,N,bias", [(1, 32, 16, True), (2, 64, 5, False), (3, 96, 40, True),
+                                        (4, 2048, 72, False), (4, 16384, 24, True),
+                                        (3, 4128, 33, False), (4, 160, 100, True), (1, 4096, 520, False),
+                                        (2, 544, 17, True)])
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_blockwise_int4_nibble_gemm_up_to_four_rows_matches_oracle(fc, B, K, N, bias, variant):
+    """One to four rows on the filter kept at 4 bits per weight: the four blocks of a quad share
+    one matrix-core tile (columns = block x row), the products of blocks 1..3 reach block 0's
+    lanes by row shifts and are added there in block order. Depths that end inside a quad and
+    inside a group of 16 scales, fewer than four rows (the clamped copies are not stored),
+    ragged channel counts, every quantizer variant."""
+    c = wl.blockwise_int4_fc(B, K, N, seed=21 + B + K + N, lo=-8, hi=7)
+    b = np.random.default_rng(B).standard_normal(N).astype(np.float32) if bias else None
+    op = fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], K, 32, b, quant_variant=variant)
+    y = op.call_gemm_nibbles(_cuda(c["x"])).cpu().numpy()
+    want = oracle.fc_blockwise_int4(c["x"], c["packed"], N, c["scales"].view(np.uint16), 32, b,
+                                    variant=variant)
+    assert _bits_equal(y, want)
+
+
 def test_blockwise_int4_nibble_gemm_full_width_and_dispatch(fc):
     """The nibble-resident GEMM on config 3's filter at 5, 8 and 24 rows: what the op picks by
     itself for this shape (lrtfc_fc_blockwise_int4_preferred_form), bit-identical to the decode
