@@ -23,7 +23,8 @@
 extern "C" {
 #endif
 
-#define LRTFC_ABI_VERSION 1
+/* 2: lrtfc_int4_group_node gained nibble_filter, lrtfc_int4_group_launch gained form. */
+#define LRTFC_ABI_VERSION 2
 
 typedef enum LrtFcStatus {
   LRTFC_OK = 0,
@@ -392,6 +393,7 @@ int lrtfc_fc_hybrid_int4_per_channel_nibbles(const float* input, const uint8_t* 
  *     one kernel per 4 rows on them, so that every filter is streamed once); allocates and
  *     copies nothing. */
 #define LRTFC_INT4_GROUP_MAX 128
+enum { LRTFC_INT4_FORM_DECODE = 0, LRTFC_INT4_FORM_GEMM_NIBBLES = 1, LRTFC_INT4_FORM_GEMM_INT8 = 2 };
 typedef struct lrtfc_int4_group_node {
   const float* input;            /* [batches, depth] */
   const uint8_t* retiled_filter; /* from lrtfc_pack_int4_blockwise */
@@ -401,12 +403,25 @@ typedef struct lrtfc_int4_group_node {
   int out_depth;
   void* workspace;               /* NULL, or lrtfc_activation_workspace_bytes(batches, depth)
                                     bytes of this node's own, 256-byte aligned */
+  const uint8_t* nibble_filter;  /* NULL, or from lrtfc_pack_int4_blockwise_gemm_nibbles. When
+                                    every node of a group brings one (and a workspace) and the
+                                    group's shape is one the 4-bit-resident form is faster on
+                                    (three or four rows deeper than 8192), the group runs on it;
+                                    retiled_filter may then be NULL. Otherwise it is ignored and
+                                    retiled_filter is required. */
 } lrtfc_int4_group_node;
 typedef struct lrtfc_int4_group_launch {
   int count, grid_blocks, ksplit, groups_per_wave, batches, depth;
   int split_quantize;            /* rows are quantized by a launch of their own */
+  int form;                      /* LRTFC_INT4_FORM_DECODE or LRTFC_INT4_FORM_GEMM_NIBBLES */
 } lrtfc_int4_group_launch;
 size_t lrtfc_int4_group_table_bytes(void);
+/* Which filter form a group of `count` nodes with these output depths runs fastest on at this
+ * batch count and depth: LRTFC_INT4_FORM_DECODE (retiled_filter), or
+ * LRTFC_INT4_FORM_GEMM_NIBBLES (nibble_filter and a workspace per node: three or four rows of
+ * filters deeper than 8192 with at least a wavefront's worth of channels per SIMD in all).
+ * lrtfc_int4_group_prepare applies the same rule to what the nodes bring. */
+int lrtfc_int4_group_preferred_form(const int* out_depths, int count, int batches, int depth);
 int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,
                              int depth, void* device_table, lrtfc_int4_group_launch* launch,
                              void* stream);
@@ -452,7 +467,7 @@ int lrtfc_fc_blockwise_int4_gemm(const float* input, const uint8_t* gemm_filter,
  * (16-byte aligned), and lrtfc_fc_blockwise_int4_gemm_nibbles takes that filter with the
  * arguments, the workspace and the results -- bit for bit -- of lrtfc_fc_blockwise_int4_gemm.
  * A wavefront expands each block's nibbles to the matrix cores' int8 operand itself. */
-enum { LRTFC_INT4_FORM_DECODE = 0, LRTFC_INT4_FORM_GEMM_NIBBLES = 1, LRTFC_INT4_FORM_GEMM_INT8 = 2 };
+/* (the LRTFC_INT4_FORM_* values are declared with the grouped launch above) */
 /* Which of the three forms of the blockwise-int4 op runs a shape fastest (block size 32): the
  * streaming kernel of lrtfc_fc_blockwise_int4_packed (up to four rows per pass over the filter),
  * this nibble-resident GEMM, or the int8-expanded GEMM. All three give the same bits; a caller

@@ -89,6 +89,7 @@ SYMBOLS = [
     ("lrtfc_embedding_lookup_hybrid", _i, [_vp, _i, _vp, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp]),
     ("lrtfc_mark_completion", _i, [_vp, C.c_uint32, _vp]),
     ("lrtfc_int4_group_table_bytes", _sz, []),
+    ("lrtfc_int4_group_preferred_form", _i, [_vp, _i, _i, _i]),
     ("lrtfc_int4_group_prepare", _i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     ("lrtfc_fc_blockwise_int4_packed_grouped", _i, [_vp, _vp, _i, _vp]),
     ("lrtfc_fc_blockwise_int4_quantized", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
@@ -133,11 +134,11 @@ class Int4GroupNode(C.Structure):
     """lrtfc_int4_group_node."""
     _fields_ = [("input", C.c_void_p), ("retiled_filter", C.c_void_p), ("kfsum", C.c_void_p),
                 ("bias", C.c_void_p), ("output", C.c_void_p), ("out_depth", C.c_int),
-                ("workspace", C.c_void_p)]
+                ("workspace", C.c_void_p), ("nibble_filter", C.c_void_p)]
 
 
 class Int4GroupLaunch(C.Structure):
     """lrtfc_int4_group_launch."""
     _fields_ = [("count", C.c_int), ("grid_blocks", C.c_int), ("ksplit", C.c_int),
                 ("groups_per_wave", C.c_int), ("batches", C.c_int), ("depth", C.c_int),
-                ("split_quantize", C.c_int)]
+                ("split_quantize", C.c_int), ("form", C.c_int)]

@@ -1188,6 +1188,15 @@ int lrtfc_mark_completion(uint32_t* flag, uint32_t value, void* stream) {
 
 size_t lrtfc_int4_group_table_bytes(void) { return lrtfc::Int4GroupTableBytes(); }
 
+int lrtfc_int4_group_preferred_form(const int* out_depths, int count, int batches, int depth) {
+  if (!out_depths || count < 1) return LRTFC_INT4_FORM_DECODE;
+  int64_t tiles = 0;
+  for (int i = 0; i < count; ++i) tiles += (static_cast<int64_t>(out_depths[i]) + 15) / 16;
+  return lrtfc::Int4NibbleGroupWins(batches, depth, tiles > 0x7fffffff ? 0x7fffffff : static_cast<int>(tiles))
+             ? LRTFC_INT4_FORM_GEMM_NIBBLES
+             : LRTFC_INT4_FORM_DECODE;
+}
+
 int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int batches,
                              int depth, void* device_table, lrtfc_int4_group_launch* launch,
                              void* stream) {
@@ -1198,16 +1207,21 @@ int lrtfc_int4_group_prepare(const lrtfc_int4_group_node* nodes, int count, int 
   LRTFC_REQUIRE(lrtfc::FcInt4PackedSupports(depth, 32), "depth %d is not a multiple of 32", depth);
   LRTFC_REQUIRE(batches >= 1, "a grouped launch needs at least one batch row");
   for (int i = 0; i < count; ++i) {
-    LRTFC_REQUIRE(nodes[i].input && nodes[i].retiled_filter && nodes[i].kfsum && nodes[i].output,
+    LRTFC_REQUIRE(nodes[i].input && (nodes[i].retiled_filter || nodes[i].nibble_filter) &&
+                      nodes[i].kfsum && nodes[i].output,
                   "null pointer in node %d", i);
     LRTFC_REQUIRE(nodes[i].out_depth >= 1, "node %d has no output channels", i);
-    LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(nodes[i].retiled_filter) & 15) == 0,
-                  "retiled filter of node %d must be 16-byte aligned", i);
+    LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(nodes[i].retiled_filter) & 15) == 0 &&
+                      (reinterpret_cast<uintptr_t>(nodes[i].nibble_filter) & 15) == 0,
+                  "re-tiled filter of node %d must be 16-byte aligned", i);
     LRTFC_REQUIRE((reinterpret_cast<uintptr_t>(nodes[i].workspace) & 255) == 0,
                   "workspace of node %d must be 256-byte aligned", i);
   }
   const hipError_t err = lrtfc::PrepareInt4Group(nodes, count, batches, depth, device_table,
                                                  launch, AsStream(stream));
+  LRTFC_REQUIRE(err != hipErrorInvalidValue,
+                "a node of the group brings neither the filter form this shape runs on nor the "
+                "decode tiling (and, for the 4-bit-resident form, a workspace)");
   return FromHip(err, "int4 group table upload");
 }
 
@@ -1220,7 +1234,9 @@ int lrtfc_fc_blockwise_int4_packed_grouped(const void* device_table,
                     launch->grid_blocks >= 1 && launch->ksplit >= 1 && launch->ksplit <= 4 &&
                     launch->groups_per_wave >= 1 && launch->groups_per_wave <= 8 &&
                     (launch->ksplit == 1 || launch->groups_per_wave == 1) &&
-                    (launch->split_quantize == 0 || launch->split_quantize == 1),
+                    (launch->split_quantize == 0 || launch->split_quantize == 1) &&
+                    (launch->form == LRTFC_INT4_FORM_DECODE ||
+                     launch->form == LRTFC_INT4_FORM_GEMM_NIBBLES),
                 "launch record was not filled by lrtfc_int4_group_prepare");
   LRTFC_REQUIRE(quant_variant >= 0 && quant_variant <= LRTFC_QUANT_NEON_LEGACY,
                 "unknown quantizer variant");

@@ -493,6 +493,11 @@ struct FcNode {
   // ... and batches in between on the GEMM that keeps the filter at 4 bits per weight
   // (gemm_layout is set too; retiled_dev then holds that form).
   bool gemm_nibbles = false;
+  // A member of a grouped launch whose shape runs faster on the 4-bit-resident matrix-core form
+  // (lrtfc_int4_group_preferred_form) keeps that form of its filter here, beside the decode
+  // tiling that the same node needs when a resize changes the group's batch count.
+  DeviceBuffer group_nibbles_dev;
+  const void* group_nibbles_from = nullptr;  // host filter the copy was made from
   bool split_quantize = false;  // quantize rows in a launch of their own, not in the prologue
   // EMBEDDING_LOOKUP nodes: input = the lookup vector, filter = the table (filter_dev), batches =
   // lookups, depth = out_depth = columns of a row; block scales in scales_dev or per-row scales
@@ -1231,6 +1236,46 @@ TfLiteStatus PlanSchedule(TfLiteContext* ctx, PartitionKernel* k) {
       }
     }
   }
+  // Groups whose shape the library runs faster on the filters kept at 4 bits per weight for the
+  // matrix cores: their members get that form of their filters as well.
+  for (const PartitionKernel::Group& g : k->groups) {
+    std::vector<int> out_depths;
+    for (int m : g.members) out_depths.push_back(k->nodes[m].out_depth);
+    const FcNode& head = k->nodes[g.members.front()];
+    const bool nibbles = lrtfc_int4_group_preferred_form(
+                             out_depths.data(), static_cast<int>(out_depths.size()), head.batches,
+                             head.depth) == LRTFC_INT4_FORM_GEMM_NIBBLES;
+    for (int m : g.members) {
+      FcNode& n = k->nodes[m];
+      const TfLiteTensor& filter = ctx->tensors[n.filter];
+      if (!nibbles) {
+        n.group_nibbles_dev.Release();
+        n.group_nibbles_from = nullptr;
+        continue;
+      }
+      if (n.group_nibbles_from == filter.data.raw) continue;
+      const TfLiteTensor& scales = ctx->tensors[n.scales];
+      const size_t weights = static_cast<size_t>(n.out_depth) * n.depth;
+      DeviceBuffer model_nibbles, block_scales;
+      hipStream_t s = k->stream;
+      RETURN_IF_HIP(ctx, model_nibbles.Upload(filter.data.raw, weights / 2, s));
+      RETURN_IF_HIP(ctx, block_scales.Upload(
+                             scales.data.raw, static_cast<size_t>(NumElements(scales.dims)) * 2, s));
+      RETURN_IF_HIP(ctx, n.group_nibbles_dev.Ensure(
+                             lrtfc_gemm_int4_blockwise_nibble_bytes(n.out_depth, n.depth)));
+      RETURN_IF_FC(ctx, lrtfc_pack_int4_blockwise_gemm_nibbles(
+                            model_nibbles.as<uint8_t>(), block_scales.as<uint16_t>(), n.out_depth,
+                            n.depth, n.blocksize, n.group_nibbles_dev.as<uint8_t>(), s));
+      RETURN_IF_HIP(ctx, hipStreamSynchronize(s));  // the two uploads are locals
+      n.group_nibbles_from = filter.data.raw;
+    }
+  }
+  for (FcNode& n : k->nodes) {  // a node that left its group keeps no such copy
+    if (n.group < 0) {
+      n.group_nibbles_dev.Release();
+      n.group_nibbles_from = nullptr;
+    }
+  }
   // Launch order: units (a group, or a node on its own) by level, then by first node. A unit
   // only reads what lower levels wrote, so this is a topological order of the partition.
   k->order.clear();
@@ -1337,6 +1382,8 @@ TfLiteStatus BuildGroupTables(TfLiteContext* ctx, PartitionKernel* k) {
       nodes[m].output = static_cast<float*>(k->Activation(n.output));
       nodes[m].out_depth = n.out_depth;
       nodes[m].workspace = per_node ? g.workspace.as<uint8_t>() + per_node * m : nullptr;
+      nodes[m].nibble_filter =
+          n.group_nibbles_from ? n.group_nibbles_dev.as<uint8_t>() : nullptr;
     }
     const FcNode& first = k->nodes[g.members.front()];
     RETURN_IF_HIP(ctx, g.table.Ensure(lrtfc_int4_group_table_bytes()));
@@ -2035,7 +2082,10 @@ int litert_amd_describe_partition(const void* user_data, char* out, size_t out_s
     const FcNode& n = k->nodes[i];
     text += (i ? " " : "") + std::to_string(n.node_index) + ":" +
             std::to_string(static_cast<int>(n.kind)) + "/s" + std::to_string(n.lane);
-    if (n.group >= 0) text += "/g" + std::to_string(n.group);
+    if (n.group >= 0) {
+      // "n" behind the group: the member runs on the 4-bit-resident matrix-core form
+      text += "/g" + std::to_string(n.group) + (n.group_nibbles_from ? "n" : "");
+    }
   }
   std::snprintf(out, out_size, "%s", text.c_str());
   return static_cast<int>(k->groups.size());

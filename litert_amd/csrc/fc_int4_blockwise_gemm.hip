@@ -23,6 +23,8 @@
 // No LDS: a wavefront owns CT x RT tiles (16 to 32 channels x 16 to 64 rows, by batch size)
 // and requests the operands of the next blocks while it works on the current ones (a ring of
 // pairs of blocks in registers); both operands are re-read by other wavefronts from L2.
+#include <mutex>
+
 #include "kernels.h"
 #include "quantize_device.h"
 
@@ -697,6 +699,52 @@ __global__ __launch_bounds__(kThreads) void FcInt4NibbleQuadKernel(NibbleQuadArg
   FcInt4NibbleQuadBody<WQ, XQ>(a, ct0);
 }
 
+
+// Several filters of one depth in one launch (independent nodes of a graph, as in the decode
+// kernel's grouped form): per node its arguments and the index of its first workgroup, in a
+// table in device memory; every node's rows are quantized into its own workspace by one launch.
+struct NibbleQuadGroupTable {
+  int first_block[LRTFC_INT4_GROUP_MAX + 1];
+  int reserved[3];
+  NibbleQuadArgs node[LRTFC_INT4_GROUP_MAX];
+  const float* input_f32[LRTFC_INT4_GROUP_MAX];
+};
+
+template <int WQ, int XQ>
+__global__ __launch_bounds__(kThreads) void FcInt4NibbleQuadGroupedKernel(
+    const NibbleQuadGroupTable* __restrict__ table, int count) {
+  // first_block is ascending: this workgroup's node is the number of later nodes whose first
+  // workgroup is not beyond it (vector loads and ballots, 64 nodes per turn).
+  const int lane = threadIdx.x & 63;
+  int node = 0;
+  for (int base = 0; base + 1 < count; base += 64) {
+    const int probe = base + lane + 1;
+    const bool not_beyond =
+        probe < count && static_cast<int>(blockIdx.x) >= table->first_block[min(probe, count)];
+    node += __popcll(__ballot(not_beyond));
+  }
+  node = __builtin_amdgcn_readfirstlane(node);
+  const NibbleQuadArgs a = table->node[node];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int ct0 = (static_cast<int>(blockIdx.x) - table->first_block[node]) * 4 + wave;
+  if (ct0 >= a.channel_tiles) return;
+  FcInt4NibbleQuadBody<WQ, XQ>(a, ct0);
+}
+
+// Workgroup r quantizes row r % batches of node r / batches into that node's workspace
+// (EvalBlockwise4Bit always quantizes asymmetrically, fully_connected.cc:1044-1047).
+template <int VARIANT>
+__global__ __launch_bounds__(kQuantizeThreads) void QuantizeNibbleGroupRowsKernel(
+    const NibbleQuadGroupTable* __restrict__ table, int batches) {
+  const int node = blockIdx.x / batches;
+  const int row = blockIdx.x - node * batches;
+  const NibbleQuadArgs& a = table->node[node];
+  QuantizeRow<VARIANT>(table->input_f32[node] + static_cast<size_t>(row) * a.depth, a.depth,
+                       const_cast<int8_t*>(a.rows) + static_cast<size_t>(row) * a.depth,
+                       const_cast<float*>(a.scaling_factors) + row,
+                       const_cast<int32_t*>(a.zero_points) + row, /*do_asymmetric=*/1);
+}
+
 }  // namespace
 
 size_t GemmInt4BlockwiseBytes(int out_depth, int depth) {
@@ -914,6 +962,105 @@ hipError_t LaunchFcInt4BlockwiseNibbleGemm(const float* input, int variant,
     hipLaunchKernelGGL((FcInt4NibbleGemmKernel<1, 8, 4>), grid, dim3(kThreads), 0, stream, a);
   } else {
     hipLaunchKernelGGL((FcInt4NibbleGemmKernel<2, 8, 2>), grid, dim3(kThreads), 0, stream, a);
+  }
+  return hipGetLastError();
+}
+
+
+size_t Int4NibbleGroupTableBytes() { return sizeof(NibbleQuadGroupTable); }
+
+// With fewer than about one wavefront per SIMD the decode kernel, which splits a channel
+// group's depth among wavefronts, is the faster one.
+constexpr int kNibbleGroupMinTiles = 1024;
+
+// The grouped launch takes the 4-bit-resident form where it is the faster one: three or four
+// rows of filters deeper than 8192, whose rows the decode kernel parks in 64 KB of LDS per
+// workgroup (28672 x 16384 at four rows: 64 us here against 82 us there).
+bool Int4NibbleGroupWins(int batches, int depth, int total_channel_tiles) {
+  return (batches == 3 || batches == 4) && depth > 8192 && depth % kBlock == 0 &&
+         total_channel_tiles >= kNibbleGroupMinTiles;
+}
+
+hipError_t PrepareInt4NibbleGroup(const lrtfc_int4_group_node* nodes, int count, int batches,
+                                  int depth, void* device_table, lrtfc_int4_group_launch* launch,
+                                  hipStream_t stream) {
+  if (count < 1 || count > LRTFC_INT4_GROUP_MAX || batches < 1 || batches > 4 ||
+      depth % kBlock != 0) {
+    return hipErrorInvalidValue;
+  }
+  static NibbleQuadGroupTable host;  // 20 KB: not on the stack
+  static std::mutex host_mutex;
+  std::lock_guard<std::mutex> lock(host_mutex);
+  host = NibbleQuadGroupTable{};
+  const int nb = depth / kBlock;
+  int next = 0;
+  for (int i = 0; i < count; ++i) {
+    if (!nodes[i].nibble_filter || !nodes[i].workspace) return hipErrorInvalidValue;
+    host.first_block[i] = next;
+    NibbleQuadArgs& q = host.node[i];
+    const int channel_tiles = (nodes[i].out_depth + kTile - 1) / kTile;
+    const ActivationWorkspace w = SplitActivationWorkspace(nodes[i].workspace, batches, depth);
+    q.filter = reinterpret_cast<const i32x4*>(nodes[i].nibble_filter);
+    q.scales = reinterpret_cast<const uint2*>(
+        nodes[i].nibble_filter + static_cast<size_t>(channel_tiles) * ((nb + 3) / 4) * 1024);
+    q.rows = w.q;
+    q.scaling_factors = w.sf;
+    q.zero_points = w.zp;
+    q.kfsum = nodes[i].kfsum;
+    q.bias = nodes[i].bias;
+    q.output = nodes[i].output;
+    q.batches = batches;
+    q.depth = depth;
+    q.out_depth = nodes[i].out_depth;
+    q.nb = nb;
+    q.channel_tiles = channel_tiles;
+    q.vector_store = (nodes[i].out_depth % 4 == 0) &&
+                     (reinterpret_cast<uintptr_t>(nodes[i].output) % 16 == 0);
+    host.input_f32[i] = nodes[i].input;
+    next += (channel_tiles + 3) / 4;
+  }
+  host.first_block[count] = next;
+  hipError_t err = hipMemcpyAsync(device_table, &host, sizeof(host), hipMemcpyHostToDevice, stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(stream);  // `host` is reused by the next call
+  if (err != hipSuccess) return err;
+  launch->count = count;
+  launch->grid_blocks = next;
+  launch->ksplit = 1;
+  launch->groups_per_wave = 1;
+  launch->batches = batches;
+  launch->depth = depth;
+  launch->split_quantize = 1;
+  launch->form = LRTFC_INT4_FORM_GEMM_NIBBLES;
+  return hipSuccess;
+}
+
+hipError_t LaunchFcInt4NibbleGrouped(const void* table, const lrtfc_int4_group_launch& l,
+                                     int variant, hipStream_t stream) {
+  if (l.count < 1 || l.grid_blocks < 1) return hipSuccess;
+  const auto* t = static_cast<const NibbleQuadGroupTable*>(table);
+  const dim3 qgrid(static_cast<unsigned>(l.count) * l.batches), qblock(kQuantizeThreads);
+  switch (variant) {
+    case LRTFC_QUANT_NEON_V8:
+      hipLaunchKernelGGL(QuantizeNibbleGroupRowsKernel<LRTFC_QUANT_NEON_V8>, qgrid, qblock, 0,
+                         stream, t, l.batches);
+      break;
+    case LRTFC_QUANT_NEON_LEGACY:
+      hipLaunchKernelGGL(QuantizeNibbleGroupRowsKernel<LRTFC_QUANT_NEON_LEGACY>, qgrid, qblock, 0,
+                         stream, t, l.batches);
+      break;
+    default:
+      hipLaunchKernelGGL(QuantizeNibbleGroupRowsKernel<LRTFC_QUANT_PORTABLE>, qgrid, qblock, 0,
+                         stream, t, l.batches);
+      break;
+  }
+  if (hipError_t err = hipGetLastError()) return err;
+  // Few wavefronts per SIMD (narrow, deep filters): each keeps twice the loads in flight.
+  if (l.grid_blocks * 4 <= 4096) {
+    hipLaunchKernelGGL((FcInt4NibbleQuadGroupedKernel<16, 8>), dim3(l.grid_blocks), dim3(kThreads),
+                       0, stream, t, l.count);
+  } else {
+    hipLaunchKernelGGL((FcInt4NibbleQuadGroupedKernel<8, 4>), dim3(l.grid_blocks), dim3(kThreads),
+                       0, stream, t, l.count);
   }
   return hipGetLastError();
 }

@@ -843,6 +843,20 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
     return hipErrorInvalidValue;
   }
   if (batches < 1) return hipErrorInvalidValue;
+  {
+    int total_tiles = 0;
+    for (int i = 0; i < count; ++i) total_tiles += (nodes[i].out_depth + 15) / 16;
+    bool nibbles = Int4NibbleGroupWins(batches, depth, total_tiles);
+    bool decode = true;
+    for (int i = 0; i < count; ++i) {
+      nibbles = nibbles && nodes[i].nibble_filter != nullptr && nodes[i].workspace != nullptr;
+      decode = decode && nodes[i].retiled_filter != nullptr;
+    }
+    if (nibbles) {
+      return PrepareInt4NibbleGroup(nodes, count, batches, depth, device_table, launch, stream);
+    }
+    if (!decode) return hipErrorInvalidValue;
+  }
   const int chunks = (depth / kBlock + kTileBlocks - 1) / kTileBlocks;
   int total_out = 0;
   for (int i = 0; i < count; ++i) total_out += nodes[i].out_depth;
@@ -900,10 +914,14 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
   launch->batches = batches;
   launch->depth = depth;
   launch->split_quantize = split ? 1 : 0;
+  launch->form = LRTFC_INT4_FORM_DECODE;
   return hipSuccess;
 }
 
-size_t Int4GroupTableBytes() { return sizeof(Int4GroupTable); }
+size_t Int4GroupTableBytes() {
+  return sizeof(Int4GroupTable) > Int4NibbleGroupTableBytes() ? sizeof(Int4GroupTable)
+                                                              : Int4NibbleGroupTableBytes();
+}
 
 namespace {
 template <int BT, bool FUSED, int VARIANT, int GPT>
@@ -958,6 +976,9 @@ hipError_t LaunchGroupQuantizer(const void* table, const lrtfc_int4_group_launch
 hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_launch& l,
                                      int variant, hipStream_t stream) {
   if (l.count < 1 || l.grid_blocks < 1) return hipSuccess;
+  if (l.form == LRTFC_INT4_FORM_GEMM_NIBBLES) {
+    return LaunchFcInt4NibbleGrouped(table, l, variant, stream);
+  }
   const int chunks = (l.depth / kBlock + kTileBlocks - 1) / kTileBlocks;
   const int padded = chunks * kTileBlocks * kBlock;
   if (l.split_quantize) {

@@ -165,6 +165,16 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
                             hipStream_t stream);
 hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_launch& launch,
                                      int variant, hipStream_t stream);
+// The grouped launch on the 4-bit-resident filters (one to four rows; every node brings its
+// nibble filter and a workspace). Int4NibbleGroupWins: the shapes for which PrepareInt4Group
+// chooses it when it can.
+size_t Int4NibbleGroupTableBytes();
+bool Int4NibbleGroupWins(int batches, int depth, int total_channel_tiles);
+hipError_t PrepareInt4NibbleGroup(const lrtfc_int4_group_node* nodes, int count, int batches,
+                                  int depth, void* device_table, lrtfc_int4_group_launch* launch,
+                                  hipStream_t stream);
+hipError_t LaunchFcInt4NibbleGrouped(const void* table, const lrtfc_int4_group_launch& launch,
+                                     int variant, hipStream_t stream);
 hipError_t LaunchFcInt4Packed(const FcInt4Args& q, const uint8_t* packed, const float* input_f32,
                               int variant, hipStream_t stream);
 

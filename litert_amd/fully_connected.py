@@ -322,6 +322,20 @@ class FullyConnectedBlockwiseInt4:
             _stream()))
         return out
 
+    def _nibble_filter_tensor(self):
+        """The filter re-tiled at 4 bits per weight for the matrix cores (made once)."""
+        if self.blocksize != 32 or self.depth % 32:
+            raise RuntimeError("the 4-bit-resident matrix-core form needs block size 32")
+        if self._nibble_filter is None:
+            lib = capi.load()
+            self._nibble_filter = torch.empty(
+                lib.lrtfc_gemm_int4_blockwise_nibble_bytes(self.out_depth, self.depth),
+                dtype=torch.uint8, device="cuda")
+            capi.check(lib.lrtfc_pack_int4_blockwise_gemm_nibbles(
+                _ptr(self.filter), _ptr(self.scales), self.out_depth, self.depth, 32,
+                _ptr(self._nibble_filter), _stream()))
+        return self._nibble_filter
+
     def call_gemm_nibbles(self, x, out=None):
         """The same GEMM on the filter kept at 4 bits per weight (made on first use and kept):
         the form for batches between decode and prefill. Same results as the other forms."""
@@ -332,13 +346,7 @@ class FullyConnectedBlockwiseInt4:
         batches = x.numel() // self.depth
         if out is None:
             out = torch.empty((batches, self.out_depth), dtype=torch.float32, device=x.device)
-        if self._nibble_filter is None:
-            self._nibble_filter = torch.empty(
-                lib.lrtfc_gemm_int4_blockwise_nibble_bytes(self.out_depth, self.depth),
-                dtype=torch.uint8, device="cuda")
-            capi.check(lib.lrtfc_pack_int4_blockwise_gemm_nibbles(
-                _ptr(self.filter), _ptr(self.scales), self.out_depth, self.depth, 32,
-                _ptr(self._nibble_filter), _stream()))
+        self._nibble_filter_tensor()
         need = lib.lrtfc_fc_blockwise_int4_gemm_workspace_bytes(batches, self.depth)
         if self._gemm_ws is None or self._gemm_ws.numel() < need:
             self._gemm_ws = torch.empty(need, dtype=torch.uint8, device="cuda")
@@ -501,6 +509,9 @@ class GroupedBlockwiseInt4:
             need = capi.load().lrtfc_activation_workspace_bytes(batches, self.depth)
             workspaces = torch.empty((len(self.ops), (need + 255) // 256 * 256), dtype=torch.uint8,
                                      device="cuda")
+        out_depths = (C.c_int * len(self.ops))(*[op.out_depth for op in self.ops])
+        nibbles = capi.load().lrtfc_int4_group_preferred_form(
+            out_depths, len(self.ops), batches, self.depth) == capi.INT4_FORM_GEMM_NIBBLES
         for i, (op, x, y) in enumerate(zip(self.ops, inputs, outputs)):
             if not (x.is_contiguous() and y.is_contiguous()):
                 raise ValueError("grouped inputs and outputs must be contiguous")
@@ -513,6 +524,9 @@ class GroupedBlockwiseInt4:
             nodes[i].output = y.data_ptr()
             nodes[i].out_depth = op.out_depth
             nodes[i].workspace = workspaces[i].data_ptr() if workspaces is not None else None
+            # Some shapes run faster on the filters kept at 4 bits per weight for the matrix
+            # cores (three or four rows of wide groups deeper than 8192).
+            nodes[i].nibble_filter = op._nibble_filter_tensor().data_ptr() if nibbles else None
         launch = capi.Int4GroupLaunch()
         capi.check(capi.load().lrtfc_int4_group_prepare(
             C.byref(nodes), len(self.ops), batches, self.depth, _ptr(self.table),

@@ -56,7 +56,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     assert sorted(n for n, _, _ in capi.SYMBOLS) == declared
-    assert lib.lrtfc_abi_version() == 1
+    assert lib.lrtfc_abi_version() == 2
 
 
 def test_host_prepare_math_matches_oracle():

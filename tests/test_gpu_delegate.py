@@ -769,6 +769,42 @@ def test_int4_grouped_nodes_with_more_than_two_rows(B, K):
                 assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32)), (trial, n)
 
 
+def test_int4_wide_deep_group_runs_on_the_4bit_resident_form_and_leaves_it_on_resize():
+    """Two independent nodes of 8200 channels and depth 8224 at four rows: a group wide and deep
+    enough for the library to prefer the filters kept at 4 bits per weight for the matrix cores
+    (lrtfc_int4_group_preferred_form); the partition packs that form for the group's members
+    ("n" behind the group in the description). At two rows the same group runs on the decode
+    tiling. Bit-identical to the oracle both ways."""
+    K, Ns = 8224, (8200, 8200)
+    cs = [wl.blockwise_int4_fc(4, K, n, seed=700 + i, lo=-8, hi=7) for i, n in enumerate(Ns)]
+    with FakeHost() as h:
+        xs, ys = [], []
+        for c, n in zip(cs, Ns):
+            x = h.tensor(FLOAT32, (4, K), data=c["x"])
+            w = h.tensor(INT4, (n, K), data=c["packed"], const=True)
+            s_ = h.tensor(FLOAT16, (n, K // 32), data=c["scales"], const=True)
+            h.blockwise(w, s_, 32)
+            y = h.tensor(FLOAT32, (4, n))
+            h.fc(x, w, None, y)
+            xs.append(x)
+            ys.append(y)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        for rows in (4, 2, 3):
+            for c, n, x, y in zip(cs, Ns, xs, ys):
+                h.resize(x, (rows, K))
+                h.resize(y, (rows, n))
+                h.write(x, c["x"][:rows])
+            assert h.allocate_tensors() == OK, h.errors()
+            groups, text = h.describe_partition(h.plan()[0][2])
+            assert groups == 1 and text.count("/g0n") == (2 if rows >= 3 else 0), (rows, text)
+            assert h.invoke() == OK, h.errors()
+            for c, n, y in zip(cs, Ns, ys):
+                want = oracle.fc_blockwise_int4(c["x"][:rows], c["packed"], n,
+                                                c["scales"].view(np.uint16), 32)
+                assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32)), (rows, n)
+
+
 def test_blockwise_int4_resize_between_decode_and_prefill():
     """Two rows run the streaming kernel, 40 rows the matrix-core GEMM (the filter is re-tiled
     for it at that prepare), 3 rows the streaming kernel again. Every step bit-identical to the

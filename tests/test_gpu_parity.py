@@ -532,6 +532,9 @@ def test_blockwise_int4_split_launch_matches_oracle(fc, B, K, N):
                                     # group's depth and four deep rows no longer fit the LDS, so
                                     # the launch falls back to two rows at a time
                                     (4, 16384, (2048, 2056)), (3, 16384, (4100,)),
+                                    # wide and deep: the 4-bit-resident matrix-core form
+                                    (4, 16384, (2048,) * 8), (3, 16384, (8200, 8200)),
+                                    (4, 8224, (9000, 7400, 33)),
                                     # deeper than the register forms: rows re-read, LDS-bound tile
                                     (3, 32768, (16, 24)), (4, 32768, (8,))])
 def test_blockwise_int4_grouped_launch_matches_oracle(fc, B, K, Ns):
@@ -550,6 +553,12 @@ def test_blockwise_int4_grouped_launch_matches_oracle(fc, B, K, Ns):
         ys = [torch.full((B, n), float("nan"), dtype=torch.float32, device="cuda") for n in Ns]
         group.bind(xs, ys)()
         torch.cuda.synchronize()
+        # three or four rows deeper than 8192 run on the filters kept at 4 bits per weight for
+        # the matrix cores (four blocks per tile); everything else on the decode tiling
+        from litert_amd import capi
+        wide = sum((n + 15) // 16 for n in Ns) >= 1024  # a wavefront per SIMD at least
+        assert group.launch.form == (capi.INT4_FORM_GEMM_NIBBLES
+                                     if B in (3, 4) and K > 8192 and wide else capi.INT4_FORM_DECODE)
         for c, b, x, y, n in zip(cs, biases, xs_np, ys, Ns):
             want = oracle.fc_blockwise_int4(x, c["packed"], n, c["scales"].view(np.uint16), 32, b)
             assert _bits_equal(y.cpu().numpy(), want), (trial, n)
