@@ -540,8 +540,8 @@ __global__ __launch_bounds__(kThreads) void FcInt4NibbleGemmKernel(NibbleGemmArg
 // whatever the row count). Here the sixteen columns of a result tile are (block j of the quad,
 // row r), column 4 j + r: the quad's four MFMAs accumulate into ONE tile, MFMA j with a B operand
 // that holds the rows' values of block j in columns 4 j .. 4 j + 3 and zeros elsewhere (a lane
-// loads the eight activation bytes of its own column's block once per quad; a move that writes
-// only lane group j of every row of 16 (DPP bank mask) over zeros makes the four operands). One
+// loads the eight activation bytes of its own column's block once per quad; a select under the
+// mask "this lane's column belongs to block j" makes the four operands). One
 // conversion and one scale per tile instead of four; the products of blocks 1..3 then reach the
 // lanes of block 0 by row shifts and are added there in block order, which is the reference's
 // order of float additions, so the results are bit-identical to every other form. Rows are read
@@ -557,15 +557,6 @@ struct NibbleQuadArgs {
   float* output;
   int batches, depth, out_depth, nb, channel_tiles, vector_store;
 };
-
-template <int J>
-__device__ __forceinline__ i64 OnlyLaneGroup(i64 x) {
-  // quad_perm identity, every row, bank J only; the other lanes keep the zero.
-  const int lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0xE4, 0xF, 1 << J, false);
-  const int hi = __builtin_amdgcn_update_dpp(0, static_cast<int>(x >> 32), 0xE4, 0xF, 1 << J, false);
-  return static_cast<i64>(static_cast<uint64_t>(static_cast<uint32_t>(lo)) |
-                          (static_cast<uint64_t>(static_cast<uint32_t>(hi)) << 32));
-}
 
 // The value of the lane N places up in the same row of 16 (row_shl:N); lanes past the row read 0.
 template <int N>
@@ -584,14 +575,18 @@ __device__ __forceinline__ void FcInt4NibbleQuadBody(const NibbleQuadArgs& a, in
   const int ng = (nb + 15) / 16;
   const i32x4* wp = a.filter + static_cast<size_t>(ct0) * nq * 64 + lane;
   const uint2* sp = a.scales + static_cast<size_t>(ct0) * ng * 64 + lane;
-  const int8_t* xrow = a.rows + static_cast<size_t>(r) * a.depth + 8 * (lane >> 4);
+  // This lane's eight activation bytes of quad q lie at rows + x_first + 128 q (clamped to the
+  // row's last block: past the depth the weights are zeros).
+  const uint32_t x_lane = static_cast<uint32_t>(r) * a.depth + 8 * (lane >> 4);
+  const uint32_t x_first = x_lane + jl * kBlock;
+  const uint32_t x_last = x_lane + (nb - 1) * kBlock;
   auto fetch_w = [&](int q) {
     return __builtin_nontemporal_load(wp + static_cast<size_t>(min(q, nq - 1)) * 64);
   };
   // Past the depth: the last block again (its weights there are zeros).
   auto fetch_x = [&](int q) {
-    const int b = min(4 * min(q, nq - 1) + jl, nb - 1);
-    return *reinterpret_cast<const i64*>(xrow + b * kBlock);
+    const uint32_t at = min(x_first + static_cast<uint32_t>(min(q, nq - 1)) * (4 * kBlock), x_last);
+    return *reinterpret_cast<const i64*>(a.rows + at);
   };
   constexpr int kGroups = WQ / 4 + 1 <= 2 ? 2 : (WQ / 4 + 1 <= 4 ? 4 : 8);
   static_assert((kGroups - 1) * 4 >= WQ, "scale groups must lead the weight ring");
@@ -634,7 +629,7 @@ __device__ __forceinline__ void FcInt4NibbleQuadBody(const NibbleQuadArgs& a, in
       const i64 x = xring[u % XQ];
       xring[u % XQ] = fetch_x(base + u + XQ);
       if (base + u < nq) {
-        i32x4 acc = zero;
+        i32x4 acc;
         StaticFor<4>([&](auto h_const) {
           constexpr int h = decltype(h_const)::value;
           const uint32_t d = static_cast<uint32_t>(w[h]);
@@ -642,7 +637,11 @@ __device__ __forceinline__ void FcInt4NibbleQuadBody(const NibbleQuadArgs& a, in
           const uint32_t hi = d & 0xF0F0F0F0u;
           const i64 wa = static_cast<i64>(static_cast<uint64_t>(lo) |
                                           (static_cast<uint64_t>(hi) << 32));
-          acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(wa, OnlyLaneGroup<h>(x), acc, 0, 0, 0);
+          if constexpr (h == 0) {
+            acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(wa, jl == h ? x : i64{0}, zero, 0, 0, 0);
+          } else {
+            acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(wa, jl == h ? x : i64{0}, acc, 0, 0, 0);
+          }
         });
         constexpr int t = u % 4;
         const float sc[4] = {
