@@ -108,9 +108,12 @@ def main():
         traffic_probe_int4(torch, fc, wl)
         return
     if args.gemm_probe:
-        phases = gemm_probe(torch, fc, wl, args.sustain)
-        if sampler is not None:
-            report_smi_samples(sampler, phases)
+        phases = []
+        try:
+            phases = gemm_probe(torch, fc, wl, args.sustain)
+        finally:  # the sampler is a child process of its own: never leave it behind
+            if sampler is not None:
+                report_smi_samples(sampler, phases)
         return
     if args.traffic_probe_int4_single:
         traffic_probe_int4_single(torch, fc, wl)
@@ -338,12 +341,22 @@ def start_smi_sampler():
     import subprocess
     import tempfile
     fd, path = tempfile.mkstemp(prefix="lrtfc_smi_", suffix=".log")
-    loop = ("while true; do echo t=$(date +%s.%N); "
+    # The loop ends by itself after five minutes, whatever becomes of this process.
+    loop = ("end=$((SECONDS+300)); while [ $SECONDS -lt $end ]; do echo t=$(date +%s.%N); "
             "echo power_uw=$(cat /sys/class/drm/card*/device/hwmon/hwmon*/power1_input 2>/dev/null | head -1); "
             "rocm-smi --showclocks 2>&1; sleep 0.2; done")
     proc = subprocess.Popen(["bash", "-c", loop], stdout=fd, stderr=subprocess.STDOUT,
                             start_new_session=True)
     os.close(fd)
+
+    def stop():  # also on an early exit of bench.py (no GPU, an import that fails)
+        import signal
+        try:
+            os.killpg(proc.pid, signal.SIGTERM)
+        except (ProcessLookupError, PermissionError):
+            pass
+    import atexit
+    atexit.register(stop)
     return proc, path
 
 

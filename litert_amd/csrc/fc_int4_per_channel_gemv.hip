@@ -306,7 +306,7 @@ __global__ __launch_bounds__(kThreads) void FcInt4PerChannelGemvKernel(NibbleArg
     }
   }
 #pragma unroll
-  for (int u = 0; u < kRing; ++u) {  // last round
+  for (int u = 0; u < kRing; ++u) {  // last turn of the ring
     if (base + u < s1) consume(ring[u], base + u, u);
   }
   i32x4 acc = (acc4[0] + acc4[1]) + (acc4[2] + acc4[3]);

@@ -410,7 +410,7 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(
     }
   }
 #pragma unroll
-  for (int u = 0; u < kRing; ++u) {  // last round
+  for (int u = 0; u < kRing; ++u) {  // last turn of the ring
     if (base + u < s1) {
       const i32x4 bq = *reinterpret_cast<const i32x4*>(qbase + (base + u) * kSlabDepth);
       acc4[u % kAccs] =

@@ -786,7 +786,9 @@ def test_empty_and_zero_depth(fc):
 # ---- per-channel int4 hybrid (EvalHybridDense4Bit) ----------------------------------------
 
 @pytest.mark.parametrize("B,K,N", [(1, 32, 4), (4, 40, 5), (3, 46, 7), (2, 256, 17), (1, 4096, 512),
-                                   (8, 2048, 130), (16, 1000, 33), (40, 512, 72), (130, 272, 48)])
+                                   (8, 2048, 130), (16, 1000, 33), (40, 512, 72), (130, 272, 48),
+                                   # 17..32 rows: on the int8 expansion they take the one-pass GEMV
+                                   (20, 2048, 130), (32, 4096, 40), (17, 1008, 33)])
 @pytest.mark.parametrize("activation", ["none", "relu", "relu6"])
 def test_hybrid_int4_per_channel_matches_oracle(fc, B, K, N, activation):
     """Bit-identical floats against the oracle (itself bit-identical to the reference's 4-bit
