@@ -355,6 +355,10 @@ def start_smi_sampler():
             os.killpg(proc.pid, signal.SIGTERM)
         except (ProcessLookupError, PermissionError):
             pass
+        try:
+            os.unlink(path)
+        except OSError:
+            pass
     import atexit
     atexit.register(stop)
     return proc, path
