@@ -480,9 +480,10 @@ __global__ __launch_bounds__(kThreads) void FcInt8PackedGemvKernel(
 // loads that could have been in flight were not is added to that. A ring that is refilled as
 // it is consumed ties the stream to the consumer: a slot is requested again only after the
 // product that empties it, and nothing beyond the ring is requested until the activation rows
-// are quantized and staged. This form unties them. A wavefront's whole share of the depth (at
-// most TILES tiles of 1 KiB; the vector register file of the chip holds 128 MB, a filter of
-// this class fits) has a register of its own, so a request never waits for a product:
+// are quantized and staged. This form unties them. Every tile of a wavefront's share of the
+// depth (at most TILES tiles of 1 KiB) has a variable of its own in straight-line code, so in
+// program order a request never waits for a product (the tiles between request and product
+// are what stays live in registers: kStreamAhead at the barrier, about kStreamLag afterwards):
 //   * kAhead tiles are requested before anything waits for anything; the one barrier of the
 //     kernel (rows staged) follows, and from there on the wavefront alternates "request tile
 //     u" with "multiply tile u - kLag", in straight-line code whose waits the compiler counts
