@@ -1494,6 +1494,15 @@ TfLiteStatus RefreshBindings(TfLiteContext* ctx, PartitionKernel* k) {
   return kTfLiteOk;
 }
 
+// One turn of a polling loop: tell the core that this is a spin-wait.
+inline void SpinPause() {
+#if defined(__x86_64__) || defined(__i386__)
+  __builtin_ia32_pause();
+#elif defined(__aarch64__)
+  asm volatile("yield" ::: "memory");
+#endif
+}
+
 TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
   auto* k = static_cast<PartitionKernel*>(node->user_data);
   RETURN_IF_HIP(ctx, hipSetDevice(k->state->options.device));
@@ -1755,7 +1764,7 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     for (;;) {
       for (int spin = 0; spin < 64 && !finished; ++spin) {
         finished = *word == k->completion_serial;
-        if (!finished) __builtin_ia32_pause();
+        if (!finished) SpinPause();
       }
       if (finished || std::chrono::steady_clock::now() - enqueued > kPollFor) break;
     }
