@@ -959,15 +959,27 @@ hipError_t LaunchResidentSized(const PackedArgs& p, int batch0, int bt, int kspl
 // stream (measured at 14336 x 4096, one launch, cold: 1 row 11.0 us narrow / 11.4 wide; 2 rows
 // 11.4 / 11.3; 4 rows 12.6 / 12.0; 8 rows 13.1 wide against 14.7 as row quantizer + product).
 // 17 to 32 rows that arrive quantized: one pass over the filter with two row tiles per weight
-// tile, on workgroups of eight wavefronts with at most 16 tiles each, as long as the rows' LDS
+// tile, on workgroups of eight wavefronts with at most 32 tiles each, as long as the rows' LDS
 // image (32 x depth) fits one compute unit. *ksplit receives the depth split.
 bool ResidentTwoRowTilesFit(const PackedArgs& p, int bt, int* ksplit_out) {
   if (bt <= 16 || bt > 32) return false;
   if (p.a.depth % 16 != 0 || (reinterpret_cast<uintptr_t>(p.a.input) & 15) != 0) return false;
-  int ksplit = 1;
-  while (ksplit < 8 && (p.slabs + ksplit - 1) / ksplit > 16) ksplit *= 2;
+  // The rows' image leaves room for one workgroup per compute unit, and every workgroup stages
+  // the whole image: the fewest workgroups that still cover the chip in one round win (measured
+  // at 14336 x 4096, 32 rows: shares of 32 tiles, 224 workgroups, 17.6 us for quantizer +
+  // product; shares of 16 tiles, 448 workgroups in two rounds, 21.5 us). So: the largest share
+  // (at most 32 tiles) that still gives about one workgroup per compute unit, else the split
+  // with the most workgroups.
+  const int tiles = (p.a.out_depth + kTileRows - 1) / kTileRows;
+  int ksplit = 0;
+  for (int k = 1; k <= 8; k *= 2) {
+    if ((p.slabs + k - 1) / k > 32) continue;
+    ksplit = k;  // candidates come with growing workgroup counts
+    const int tiles_per_wg = 8 / k;
+    if ((tiles + tiles_per_wg - 1) / tiles_per_wg >= 192) break;
+  }
+  if (ksplit == 0) return false;
   const int per_part = (p.slabs + ksplit - 1) / ksplit;
-  if (per_part > 16) return false;
   const int staged = ksplit * per_part * kSlabDepth;
   if (static_cast<int64_t>(bt) * (staged / 16) > 16 * 8 * kWaveSize) return false;
   if (SharedBytes(bt, staged + kQPad, 16) > 150 * 1024) return false;
@@ -988,6 +1000,9 @@ hipError_t TryLaunchResident(const PackedArgs& p, int batch0, int bt, hipStream_
       *launched = true;
       if ((p.slabs + ksplit - 1) / ksplit <= 8) {
         return LaunchResidentSized<EPI, false, VARIANT, 8, true, 8, 2>(p, batch0, bt, ksplit, stream);
+      }
+      if ((p.slabs + ksplit - 1) / ksplit > 16) {
+        return LaunchResidentSized<EPI, false, VARIANT, 32, true, 8, 2>(p, batch0, bt, ksplit, stream);
       }
       return LaunchResidentSized<EPI, false, VARIANT, 16, true, 8, 2>(p, batch0, bt, ksplit, stream);
     }
