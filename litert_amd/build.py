@@ -26,7 +26,7 @@ COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=
 COMMON += ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
 COMMON += os.environ.get("LITERT_AMD_EXTRA_HIPCC_FLAGS", "").split()
 
-FC_SOURCES = ["capi.hip", "quantize.hip", "fc_int8_gemv.hip", "fc_int8_packed_gemv.hip", "fc_int8_packed_gemm.hip",
+FC_SOURCES = ["capi.hip", "quantize.hip", "fc_int8_gemv.hip", "fc_int8_packed_gemv.hip", "fc_int8_rows_gemv.hip", "fc_int8_packed_gemm.hip",
               "fc_int8_gemm_mfma.hip", "fc_int4_blockwise.hip", "fc_int4_packed.hip", "fc_int4_per_channel_gemv.hip",
               "embedding_lookup.hip", "fc_int4_blockwise_gemm.hip"]
 

@@ -1145,6 +1145,7 @@ int FcInt8PackedGemvFusedMaxRows(int depth) {
 bool FcInt8PackedGemvTakesRowsInOnePass(const FcInt8Args& a) {
   if (a.batches <= 16) return FcInt8PackedGemvSupports(a);
   if (!FcInt8PackedGemvSupports(a)) return false;
+  if (a.batches > 32) return FcInt8RowsGemvTakes(a);
   PackedArgs p;
   p.a = a;
   p.slabs = (a.depth + kSlabDepth - 1) / kSlabDepth;
@@ -1164,6 +1165,9 @@ hipError_t LaunchFcInt8PackedGemv(const FcInt8Args& a, Int8Epilogue epilogue,
                                   hipStream_t stream) {
   if (a.batches == 0 || a.out_depth == 0) return hipSuccess;
   if (!FcInt8PackedGemvSupports(a)) return hipErrorNotSupported;
+  if (!input_f32 && a.batches > 32 && FcInt8RowsGemvTakes(a)) {
+    return LaunchFcInt8RowsGemv(a, epilogue, stream);
+  }
   PackedArgs p;
   p.a = a;
   p.input_f32 = input_f32;

@@ -131,6 +131,10 @@ hipError_t LaunchFcInt4PerChannelGemv(const uint8_t* packed, const float* input_
 // Whether the GEMV streams the filter once for all of a.batches rows (up to 16 always; 17 to 32
 // rows that arrive quantized when their LDS image fits a compute unit).
 bool FcInt8PackedGemvTakesRowsInOnePass(const FcInt8Args& a);
+// 33 to 128 quantized rows on wide re-tiled filters: the filter streamed once, the rows through
+// LDS in depth chunks (fc_int8_rows_gemv.hip). FcInt8RowsGemvTakes: the shapes it is meant for.
+bool FcInt8RowsGemvTakes(const FcInt8Args& a);
+hipError_t LaunchFcInt8RowsGemv(const FcInt8Args& a, Int8Epilogue epilogue, hipStream_t stream);
 bool FcInt8PackedGemmSupports(const FcInt8Args& a);
 hipError_t LaunchFcInt8PackedGemm(const FcInt8Args& a, Int8Epilogue epilogue, hipStream_t stream);
 

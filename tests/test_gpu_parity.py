@@ -256,6 +256,42 @@ def test_int8_17_to_32_rows_in_one_pass_bit_exact(fc, B, K, N, activation):
     assert np.array_equal(y, want)
 
 
+ROWS_33_TO_128 = [(33, 1024, 10225), (40, 4096, 14336), (64, 1040, 10256), (100, 2064, 10240),
+                  (128, 1536, 12000), (65, 1024, 10240), (130, 1024, 10240)]
+
+
+@pytest.mark.parametrize("B,K,N", ROWS_33_TO_128)
+@pytest.mark.parametrize("asym", [True, False])
+def test_hybrid_33_to_128_rows_on_wide_filters_matches_oracle(fc, B, K, N, asym):
+    """33 to 128 rows against a filter of 640 or more channel tiles take the kernel that streams
+    the filter once and walks the rows through LDS in depth chunks: four and eight row tiles per
+    weight tile, odd and even chunk counts, depths that end 16 into a chunk, a ragged last channel
+    tile, a ragged last row tile; 130 rows stay on the GEMM. Same bits either way."""
+    c = wl.hybrid_fc(B, K, N, seed=41 + B + K)
+    bias = np.random.default_rng(6).standard_normal(N).astype(np.float32)
+    bias[::5] = -0.0
+    pcs = c["pcs"] if (B + N) % 2 else None
+    for activation, code in (("relu6", oracle.ACT_RELU6), ("none", oracle.ACT_NONE)):
+        op = fc.FullyConnectedHybrid(c["w"], pcs, filter_scale=0.005, bias=bias,
+                                     asymmetric_quantize_inputs=asym, activation=activation)
+        y = op(_cuda(c["x"])).cpu().numpy()
+        want = oracle.fc_hybrid(c["x"], c["w"], pcs, 0.005, bias, asym, code)
+        assert _bits_equal(y, want)
+    zeros = np.zeros_like(c["x"])
+    zeros[B // 2] = c["x"][B // 2]  # one live row among whole-zero ones
+    y = op(_cuda(zeros)).cpu().numpy()
+    assert _bits_equal(y, oracle.fc_hybrid(zeros, c["w"], pcs, 0.005, bias, asym, oracle.ACT_NONE))
+
+
+@pytest.mark.parametrize("B,K,N", [(33, 1024, 10225), (64, 1040, 10256), (100, 2064, 10240),
+                                   (128, 1536, 12000)])
+@pytest.mark.parametrize("activation", ["none", "relu6"])
+def test_int8_33_to_128_rows_on_wide_filters_bit_exact(fc, B, K, N, activation):
+    c = wl.int8_fc(B, K, N, in_zp=(-3 if N % 2 else 0), seed=510 + B + K + N)
+    y, want = _run_int8(fc, c, activation, bias=(N % 3 != 0))
+    assert np.array_equal(y, want)
+
+
 def test_int8_prefill_full_size_properties(fc):
     """Config 4 at full size (2048 x 4096 x 4096), RELU6 on and off, checked through
     size-independent properties: a random sample of outputs against an int64 numpy
@@ -788,7 +824,9 @@ def test_empty_and_zero_depth(fc):
 @pytest.mark.parametrize("B,K,N", [(1, 32, 4), (4, 40, 5), (3, 46, 7), (2, 256, 17), (1, 4096, 512),
                                    (8, 2048, 130), (16, 1000, 33), (40, 512, 72), (130, 272, 48),
                                    # 17..32 rows: on the int8 expansion they take the one-pass GEMV
-                                   (20, 2048, 130), (32, 4096, 40), (17, 1008, 33)])
+                                   (20, 2048, 130), (32, 4096, 40), (17, 1008, 33),
+                                   # 33..128 rows on a wide filter: the chunked one-pass kernel
+                                   (48, 1040, 10240), (100, 1536, 10255)])
 @pytest.mark.parametrize("activation", ["none", "relu", "relu6"])
 def test_hybrid_int4_per_channel_matches_oracle(fc, B, K, N, activation):
     """Bit-identical floats against the oracle (itself bit-identical to the reference's 4-bit
