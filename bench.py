@@ -268,8 +268,9 @@ def main():
                                                                   HBM_PEAK_GBPS * 100))
 
     # Between decode and prefill (not a BASELINE configuration): config 2's filters against 16
-    # rows (row quantizer + GEMV) and 32 to 512 rows (row quantizer + MFMA GEMM, 64 x 128 tiles
-    # up to 256 rows).
+    # and 32 rows (row quantizer + register-resident GEMV), 64 and 128 rows (row quantizer + the
+    # GEMV that walks the rows through LDS in depth chunks) and 512 rows (row quantizer + MFMA
+    # GEMM).
     between = {}
     gen = torch.Generator(device="cuda").manual_seed(99)
     for rows in (16, 32, 64, 128, 512):
