@@ -22,6 +22,9 @@
 // (batches of a few dozen to a few hundred rows) run the same kernel with 64 rows x 128
 // channels per workgroup (32 channels per wavefront).
 //
+// The int8 outputs of an interior tile are put together in LDS (the row buffers, free by then)
+// and stored in 16-byte pieces, whole cache lines per row.
+//
 // int32 accumulation is exact, so tiling cannot change the accumulator; bit-exactness rests
 // on the epilogues, which are the ones of the GEMV kernels (fc_epilogues.h).
 #include <type_traits>
@@ -282,9 +285,17 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
   int32_t act_lo = a.act_min, act_hi = a.act_max;
   asm volatile("" : "+v"(act_lo), "+v"(act_hi));
   // Interior tiles (the common case) store whole dwords without any bounds test.
-  auto epilogue = [&](auto full_tag, auto short_tag) {
+  // kStaged (int8 outputs of an interior tile): the tile is put together in LDS and leaves in
+  // 16-byte pieces, sixteen lanes to a row, i.e. in whole cache lines. Stored from the
+  // accumulator layout a store instruction touches 32 rows with 8 bytes each, and the 8 MB of
+  // config 4's output reach L2 as a million partial-line writes behind the last MFMA.
+  constexpr int kOutStride = BN + 16;
+  static_assert(BM * kOutStride <= 2 * kStageBytes, "output tile does not fit the row buffers");
+  auto epilogue = [&](auto full_tag, auto short_tag, auto staged_tag) {
   constexpr bool kFull = decltype(full_tag)::value;
   constexpr bool kShort = decltype(short_tag)::value;
+  constexpr bool kStaged = decltype(staged_tag)::value;
+  if (kStaged) __syncthreads();  // every wavefront has read its last row operands
 #pragma unroll
   for (int i = 0; i < kWaveTiles; ++i) {
 #pragma unroll
@@ -312,7 +323,10 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
                           : RequantizeCore(acc[i][j][4 * g + r] + addend[r], mult[r], shift[r],
                                            a.output_offset, a.act_min, a.act_max);
           }
-          if (kFull || m < M) {
+          if (kStaged) {
+            *reinterpret_cast<int32_t*>(smem + (j * 32 + row_in_tile) * kOutStride + local) =
+                PackLowBytes(q[0], q[1], q[2], q[3]);
+          } else if (kFull || m < M) {
             int8_t* dst = a.output_i8 + static_cast<size_t>(m) * N + c0;
             if (kFull || (vec_ok && c0 + 3 < N)) {
               *reinterpret_cast<int32_t*>(dst) = PackLowBytes(q[0], q[1], q[2], q[3]);
@@ -364,18 +378,82 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
       }
     }
   }
+  if (kStaged) {
+    __syncthreads();
+    constexpr int kPiecesPerRow = BN / 16;
+#pragma unroll
+    for (int k = 0; k < BM * kPiecesPerRow / kThreads; ++k) {
+      const int piece = k * kThreads + tid;
+      const int row = piece / kPiecesPerRow, at = (piece % kPiecesPerRow) * 16;
+      *reinterpret_cast<i32x4*>(a.output_i8 + static_cast<size_t>(m0 + row) * N + n0 + at) =
+          *reinterpret_cast<const i32x4*>(smem + row * kOutStride + at);
+    }
+  }
+  };
+  // The float outputs of an interior tile take the same way, 32 rows (one batch tile) at a time:
+  // a wavefront then stores one row's whole kilobyte per instruction instead of 32 bytes in each
+  // of 32 rows.
+  auto epilogue_float_staged = [&]() {
+    constexpr int kRowBytes = BN * 4 + 16;
+    static_assert(32 * kRowBytes <= 2 * kStageBytes, "a batch tile of floats does not fit");
+    constexpr int kPiecesPerRow = BN / 4;
+#pragma unroll
+    for (int j = 0; j < kBatchTiles; ++j) {
+      const int m = m0 + j * 32 + row_in_tile;
+      const float bscale = a.scaling_factors[m];
+      const int32_t bzp = a.zero_points ? a.zero_points[m] : 0;
+      __syncthreads();  // the buffer's last readers (main loop, previous batch tile) are through
+#pragma unroll
+      for (int i = 0; i < kWaveTiles; ++i) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int local = (wave * kWaveTiles + i) * 32 + 8 * g + 4 * (lane >> 5);
+          float v[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const i32x4 p = chan_params[local + r];
+            v[r] = EPI == Int8Epilogue::kHybrid4Bit
+                       ? Hybrid4BitCore(acc[i][j][4 * g + r], bscale, __int_as_float(p[0]), bzp,
+                                        __int_as_float(p[1]), a.bias_f32 != nullptr, a.activation)
+                       : HybridCoreSelect(acc[i][j][4 * g + r], bscale, __int_as_float(p[0]), bzp,
+                                          p[2], __int_as_float(p[1]), a.activation,
+                                          a.batch_matmul != 0, zero_input);
+          }
+          *reinterpret_cast<float4*>(smem + row_in_tile * kRowBytes + local * 4) =
+              make_float4(v[0], v[1], v[2], v[3]);
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < 32 * kPiecesPerRow / kThreads; ++k) {
+        const int piece = k * kThreads + tid;
+        const int row = piece / kPiecesPerRow, at = (piece % kPiecesPerRow) * 16;
+        *reinterpret_cast<i32x4*>(reinterpret_cast<int8_t*>(a.output_f32) +
+                                  (static_cast<size_t>(m0 + j * 32 + row) * N + n0) * 4 + at) =
+            *reinterpret_cast<const i32x4*>(smem + row * kRowBytes + at);
+      }
+    }
   };
   const bool interior = vec_ok && m0 + BM <= M && n0 + BN <= N;
+  if (EPI != Int8Epilogue::kRequantize && interior &&
+      (reinterpret_cast<uintptr_t>(a.output_f32) & 15) == 0) {
+    epilogue_float_staged();
+    return;
+  }
   if (EPI == Int8Epilogue::kRequantize && !general_requantize) {
-    if (interior) {
-      epilogue(std::true_type{}, std::true_type{});
+    const bool staged =
+        interior && (N & 15) == 0 && (reinterpret_cast<uintptr_t>(a.output_i8) & 15) == 0;
+    if (staged) {
+      epilogue(std::true_type{}, std::true_type{}, std::true_type{});
+    } else if (interior) {
+      epilogue(std::true_type{}, std::true_type{}, std::false_type{});
     } else {
-      epilogue(std::false_type{}, std::true_type{});
+      epilogue(std::false_type{}, std::true_type{}, std::false_type{});
     }
   } else if (interior) {
-    epilogue(std::true_type{}, std::false_type{});
+    epilogue(std::true_type{}, std::false_type{}, std::false_type{});
   } else {
-    epilogue(std::false_type{}, std::false_type{});
+    epilogue(std::false_type{}, std::false_type{}, std::false_type{});
   }
 }
 

@@ -153,13 +153,14 @@ def test_int8_prefill_gemm_bit_exact(fc, activation):
 @pytest.mark.parametrize("B,K,N", [(33, 64, 20), (128, 256, 256), (130, 272, 48), (200, 1040, 300),
                                    (64, 16, 4), (257, 192, 513), (40, 4096, 70), (300, 80, 257),
                                    (129, 128, 30), (96, 2048, 64), (1030, 48, 4100),
-                                   (2050, 80, 2049)])
+                                   (2050, 80, 2049), (1152, 96, 4096), (1100, 208, 4112)])
 @pytest.mark.parametrize("activation", ["none", "relu6"])
 def test_int8_packed_gemm_ragged_shapes_bit_exact(fc, B, K, N, activation):
     """More than 16 rows on the re-tiled filter take the MFMA GEMM: batch and channel counts
-    off the tile (64 x 128 for the small launches, 128 x 256 for the last two), depths that
-    end inside a 64-deep slab or give an odd slab count, channel counts that rule out vector
-    stores."""
+    off the tile (64 x 128 for the small launches, 128 x 256 from (1030, 48, 4100) on), depths
+    that end inside a 64-deep slab or give an odd slab count, channel counts that rule out vector
+    stores; the last two have interior tiles whose int8 outputs leave through LDS in whole
+    cache lines (all of them, and beside ragged last rows and columns)."""
     c = wl.int8_fc(B, K, N, in_zp=(-3 if N % 2 else 0), seed=300 + B + K + N)
     y, want = _run_int8(fc, c, activation, bias=(N % 3 != 0))
     assert np.array_equal(y, want)
@@ -826,7 +827,9 @@ def test_empty_and_zero_depth(fc):
                                    # 17..32 rows: on the int8 expansion they take the one-pass GEMV
                                    (20, 2048, 130), (32, 4096, 40), (17, 1008, 33),
                                    # 33..128 rows on a wide filter: the chunked one-pass kernel
-                                   (48, 1040, 10240), (100, 1536, 10255)])
+                                   (48, 1040, 10240), (100, 1536, 10255),
+                                   # GEMM tiles whose outputs leave through LDS, beside ragged ones
+                                   (200, 512, 384)])
 @pytest.mark.parametrize("activation", ["none", "relu", "relu6"])
 def test_hybrid_int4_per_channel_matches_oracle(fc, B, K, N, activation):
     """Bit-identical floats against the oracle (itself bit-identical to the reference's 4-bit
