@@ -229,13 +229,16 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
   //   * after the last use of fa[j][h] (i = last tile): its LDS read for step s + 1;
   //   * after the last use of weight piece (i, h) (j = last batch tile): its load for step s + 2;
   //   * spread over the step: the loads of the rows of step s + 3;
-  //   * after the last MFMAs: the LDS writes of the rows of step s + 2, into the buffer whose
-  //     readers all passed this step's barrier.
+  //   * from the middle of the step on, one every few MFMAs: the LDS writes of the rows of step
+  //     s + 2, into the buffer whose readers all passed this step's barrier (behind the last
+  //     MFMAs instead they are still in the LDS queue when the next step's barrier waits for
+  //     them: 1.6 us per launch of config 4 at the nominal clock).
   // The scheduling fences keep exactly this order. Vector memory returns in issue order, which
   // the waits the compiler derives from the registers respect.
   constexpr int kHalf = kBatchTiles * kWaveTiles;
   constexpr int kMfmas = kSub * kHalf;
   constexpr int kFirstFree = (kWaveTiles - 1) * kBatchTiles;
+  constexpr int kStoreAt = kMfmas / 4, kStoreEvery = (kMfmas / 2) / kXChunks;
   auto step_body = [&](int s, auto slot) {
     constexpr int kSlot = decltype(slot)::value;
     using Slot = std::integral_constant<int, kSlot>;
@@ -261,8 +264,10 @@ __global__ __launch_bounds__(kThreads, 1) void FcInt8PackedGemmKernel(FcInt8Args
         load_x_piece(s + 3, Other{}, std::integral_constant<int, m / (kMfmas / kXChunks)>{});
         __builtin_amdgcn_sched_barrier(0);
       }
-      if constexpr (m >= kMfmas - kXChunks) {
-        store_x_piece(s + 2, Slot{}, std::integral_constant<int, m - (kMfmas - kXChunks)>{});
+      if constexpr (m >= kStoreAt && (m - kStoreAt) % kStoreEvery == 0 &&
+                    (m - kStoreAt) / kStoreEvery < kXChunks) {
+        store_x_piece(s + 2, Slot{},
+                      std::integral_constant<int, (m - kStoreAt) / kStoreEvery>{});
         __builtin_amdgcn_sched_barrier(0);
       }
     });
