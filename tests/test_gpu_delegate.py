@@ -603,6 +603,33 @@ def test_int8_resize_between_decode_and_prefill():
             assert np.array_equal(h.read(y), _oracle_int8(c, c["x"][:rows])), rows
 
 
+def test_wide_hybrid_node_resized_through_every_row_regime():
+    """A hybrid node wide enough for every kernel the row count can select (10240 channels): the
+    fused GEMV (1, 8 rows), quantizer + register-resident GEMV (16, 24 rows), the GEMV that walks
+    the rows through LDS in depth chunks (40, 100 rows), the MFMA GEMM (150 rows), then back to one
+    row; all on one re-tiled filter, each against the oracle bit for bit."""
+    K, N = 1040, 10240
+    c = wl.hybrid_fc(150, K, N, seed=77)
+    bias = np.random.default_rng(2).standard_normal(N).astype(np.float32)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (1, K), data=c["x"][:1])
+        w = h.tensor(INT8, (N, K), data=c["w"], const=True)
+        h.affine(w, c["pcs"])
+        b = h.tensor(FLOAT32, (N,), data=bias, const=True)
+        y = h.tensor(FLOAT32, (1, N))
+        h.fc(x, w, b, y, activation=1, asymmetric=True)
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        for rows in (1, 8, 16, 24, 40, 100, 150, 1):
+            h.resize(x, (rows, K))
+            h.resize(y, (rows, N))
+            h.write(x, c["x"][:rows])
+            assert h.allocate_tensors() == OK, h.errors()
+            assert h.invoke() == OK, h.errors()
+            want = oracle.fc_hybrid(c["x"][:rows], c["w"], c["pcs"], 1.0, bias, True, oracle.ACT_RELU)
+            assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32)), rows
+
+
 def test_prepare_failure_is_reported_not_hidden():
     """An output tensor whose shape cannot hold batches x channels makes the delegate
     kernel's prepare fail with a message, like a builtin kernel's Prepare would."""
