@@ -258,7 +258,9 @@ def test_int8_17_to_32_rows_in_one_pass_bit_exact(fc, B, K, N, activation):
 
 
 ROWS_33_TO_128 = [(33, 1024, 10225), (40, 4096, 14336), (64, 1040, 10256), (100, 2064, 10240),
-                  (128, 1536, 12000), (65, 1024, 10240), (130, 1024, 10240)]
+                  (128, 1536, 12000), (65, 1024, 10240), (130, 1024, 10240),
+                  # 641 and 642 channel tiles: the last workgroup owns one / two real tiles of four
+                  (50, 1024, 10250), (100, 1024, 10270)]
 
 
 @pytest.mark.parametrize("B,K,N", ROWS_33_TO_128)
@@ -267,7 +269,8 @@ def test_hybrid_33_to_128_rows_on_wide_filters_matches_oracle(fc, B, K, N, asym)
     """33 to 128 rows against a filter of 640 or more channel tiles take the kernel that streams
     the filter once and walks the rows through LDS in depth chunks: four and eight row tiles per
     weight tile, odd and even chunk counts, depths that end 16 into a chunk, a ragged last channel
-    tile, a ragged last row tile; 130 rows stay on the GEMM. Same bits either way."""
+    tile, a ragged last row tile, workgroups whose last tiles lie past the filter; 130 rows stay on
+    the GEMM. Same bits either way."""
     c = wl.hybrid_fc(B, K, N, seed=41 + B + K)
     bias = np.random.default_rng(6).standard_normal(N).astype(np.float32)
     bias[::5] = -0.0
@@ -285,7 +288,7 @@ def test_hybrid_33_to_128_rows_on_wide_filters_matches_oracle(fc, B, K, N, asym)
 
 
 @pytest.mark.parametrize("B,K,N", [(33, 1024, 10225), (64, 1040, 10256), (100, 2064, 10240),
-                                   (128, 1536, 12000)])
+                                   (128, 1536, 12000), (70, 1024, 10250)])
 @pytest.mark.parametrize("activation", ["none", "relu6"])
 def test_int8_33_to_128_rows_on_wide_filters_bit_exact(fc, B, K, N, activation):
     c = wl.int8_fc(B, K, N, in_zp=(-3 if N % 2 else 0), seed=510 + B + K + N)
