@@ -101,6 +101,13 @@ int lrtfc_row_sums_int8(const int8_t* filter, int out_depth, int depth, int32_t*
 int lrtfc_unpack_int4(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
                       void* stream);
 
+/* The same routine with bit_width 2 (tflite/kernels/internal/portable_tensor_utils.cc:128-163):
+ * four signed values per byte, the first in bits 0-1. What FULLY_CONNECTED does with an Int2
+ * filter before its int8 kernels, hybrid (tflite/kernels/fully_connected.cc:812-818) and
+ * full-integer (:1678-1685) alike. */
+int lrtfc_unpack_int2(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
+                      void* stream);
+
 /* kfsum[n] = sum over blocks, in block order and float32, of
  * scale[n,b] * float(sum_k filter[n, b*blocksize + k]): the weight-only part of
  * EvalBlockwise4Bit's zero-point correction

@@ -266,6 +266,17 @@ int lrtfc_unpack_int4(const uint8_t* packed, int64_t num_elements, int8_t* unpac
                  "int4 unpack");
 }
 
+int lrtfc_unpack_int2(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
+                      void* stream) {
+  if (int rc = RequireInit()) return rc;
+  LRTFC_REQUIRE(num_elements >= 0, "negative element count");
+  if (num_elements == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(packed && unpacked, "null pointer");
+  LRTFC_REQUIRE((num_elements + 3) / 4 <= 0x7fffffffll * 256, "tensor too large");
+  return FromHip(lrtfc::LaunchUnpackInt2(packed, num_elements, unpacked, AsStream(stream)),
+                 "int2 unpack");
+}
+
 int lrtfc_blockwise_int4_kfsum(const uint8_t* packed_filter, const uint16_t* scales_f16,
                                int out_depth, int depth, int blocksize, float* kfsum,
                                void* stream) {

@@ -308,7 +308,7 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
   if (bias && NumElements(bias->dims) != out_depth) return no("bias size != output channels");
 
   if (input.type == kTfLiteInt8 && output.type == kTfLiteInt8 &&
-      (filter.type == kTfLiteInt8 || filter.type == kTfLiteInt4)) {
+      (filter.type == kTfLiteInt8 || filter.type == kTfLiteInt4 || filter.type == kTfLiteInt2)) {
     if (!opt.claim_int8) return no("int8 path disabled by option");
     if (!ClippingActivation(params->activation)) return no("activation not a clamp");
     if (bias && bias->type != kTfLiteInt32) return no("bias is not int32");
@@ -325,7 +325,9 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
     if (fq->zero_point) {
       const bool per_channel = fq->scale->size > 1;
       for (int i = 0; i < fq->zero_point->size; ++i) {
-        if ((per_channel || filter.type == kTfLiteInt4) && fq->zero_point->data[i] != 0) {
+        // Int4 and Int2 filters: Prepare insists on zero points of 0 (fully_connected.cc:754-759).
+        if ((per_channel || filter.type == kTfLiteInt4 || filter.type == kTfLiteInt2) &&
+            fq->zero_point->data[i] != 0) {
           return no("non-zero filter zero point");
         }
       }
@@ -349,6 +351,27 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
       if (!fq || !fq->scale || fq->scale->size < 1) return no("filter has no scales");
       if (fq->scale->size > 1 && (fq->quantized_dimension != 0 || fq->scale->size != out_depth)) {
         return no("per-channel scales do not match output channels");
+      }
+      if (depth == 0) return no("empty depth");
+      return FcKind::kHybrid;
+    }
+    if (filter.type == kTfLiteInt2 && filter.quantization.type == kTfLiteAffineQuantization) {
+      // An Int2 filter under float activations: the builtin unpacks it to int8 on every Eval and
+      // runs EvalHybridDense on the result (fully_connected.cc:812-818). Here: unpacked once at
+      // prepare, then the int8 hybrid path.
+      if (!opt.claim_hybrid) return no("hybrid path disabled by option");
+      if (!ClippingActivation(params->activation) && params->activation != kTfLiteActSignBit) {
+        return no("activation is tanh or sigmoid");
+      }
+      const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
+      if (!fq || !fq->scale || fq->scale->size < 1) return no("filter has no scales");
+      if (fq->scale->size > 1 && (fq->quantized_dimension != 0 || fq->scale->size != out_depth)) {
+        return no("per-channel scales do not match output channels");
+      }
+      if (fq->zero_point) {
+        for (int i = 0; i < fq->zero_point->size; ++i) {
+          if (fq->zero_point->data[i] != 0) return no("non-zero filter zero point");
+        }
       }
       if (depth == 0) return no("empty depth");
       return FcKind::kHybrid;
@@ -976,6 +999,14 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
           RETURN_IF_FC(ctx, lrtfc_unpack_int4(packed.as<uint8_t>(), static_cast<int64_t>(weights),
                                               n->filter_dev.as<int8_t>(), s));
           RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+        } else if (filter.type == kTfLiteInt2) {
+          // Four values per byte over the flat tensor (fully_connected.cc:812-818, 1678-1685).
+          DeviceBuffer packed;
+          RETURN_IF_HIP(ctx, packed.Upload(filter.data.raw, (weights + 3) / 4, s));
+          RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
+          RETURN_IF_FC(ctx, lrtfc_unpack_int2(packed.as<uint8_t>(), static_cast<int64_t>(weights),
+                                              n->filter_dev.as<int8_t>(), s));
+          RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
         } else {
           RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
         }
@@ -1003,6 +1034,14 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
           RETURN_IF_HIP(ctx, packed.Upload(filter.data.raw, (weights + 1) / 2, s));
           RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
           RETURN_IF_FC(ctx, lrtfc_unpack_int4(packed.as<uint8_t>(), static_cast<int64_t>(weights),
+                                              n->filter_dev.as<int8_t>(), s));
+          RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
+        } else if (filter.type == kTfLiteInt2) {
+          // Four values per byte over the flat tensor (fully_connected.cc:812-818, 1678-1685).
+          DeviceBuffer packed;
+          RETURN_IF_HIP(ctx, packed.Upload(filter.data.raw, (weights + 3) / 4, s));
+          RETURN_IF_HIP(ctx, n->filter_dev.Ensure(weights));
+          RETURN_IF_FC(ctx, lrtfc_unpack_int2(packed.as<uint8_t>(), static_cast<int64_t>(weights),
                                               n->filter_dev.as<int8_t>(), s));
           RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
         } else {

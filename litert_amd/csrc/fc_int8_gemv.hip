@@ -179,6 +179,23 @@ __global__ __launch_bounds__(kThreads) void UnpackInt4Kernel(const uint8_t* __re
   if (2 * i + 1 < num_elements) unpacked[2 * i + 1] = static_cast<int8_t>(byte >> 4);
 }
 
+__global__ __launch_bounds__(kThreads) void UnpackInt2Kernel(const uint8_t* __restrict__ packed,
+                                                             int64_t num_elements,
+                                                             int8_t* __restrict__ unpacked) {
+  // tflite/kernels/internal/portable_tensor_utils.cc:128-163: element 4i + k is field k of byte
+  // i (bits 2k, 2k + 1), sign-extended; a last partial byte gives num_elements % 4 elements.
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t num_bytes = (num_elements + 3) / 4;
+  if (i >= num_bytes) return;
+  const uint32_t byte = packed[i];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int8_t value =
+        static_cast<int8_t>(static_cast<int8_t>((byte << (6 - 2 * k)) & 0xFF) >> 6);
+    if (4 * i + k < num_elements) unpacked[4 * i + k] = value;
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void ZeroFillKernel(uint8_t* __restrict__ dst, size_t bytes) {
   const size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i < bytes) dst[i] = 0;
@@ -248,6 +265,16 @@ hipError_t LaunchUnpackInt4(const uint8_t* packed, int64_t num_elements, int8_t*
   const int64_t num_bytes = (num_elements + 1) / 2;
   const int grid = static_cast<int>((num_bytes + kThreads - 1) / kThreads);
   hipLaunchKernelGGL(UnpackInt4Kernel, dim3(grid), dim3(kThreads), 0, stream, packed, num_elements,
+                     unpacked);
+  return hipGetLastError();
+}
+
+hipError_t LaunchUnpackInt2(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
+                            hipStream_t stream) {
+  if (num_elements == 0) return hipSuccess;
+  const int64_t num_bytes = (num_elements + 3) / 4;
+  const int grid = static_cast<int>((num_bytes + kThreads - 1) / kThreads);
+  hipLaunchKernelGGL(UnpackInt2Kernel, dim3(grid), dim3(kThreads), 0, stream, packed, num_elements,
                      unpacked);
   return hipGetLastError();
 }

@@ -88,6 +88,8 @@ hipError_t LaunchRowSumsInt8(const int8_t* filter, int out_depth, int depth, int
                              hipStream_t stream);
 hipError_t LaunchUnpackInt4(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
                             hipStream_t stream);
+hipError_t LaunchUnpackInt2(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
+                            hipStream_t stream);
 
 // Small-batch path: bandwidth-bound GEMV (any shape; fast path needs depth % 16 == 0).
 hipError_t LaunchFcInt8Gemv(const FcInt8Args& a, Int8Epilogue epilogue, hipStream_t stream);

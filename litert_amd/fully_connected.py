@@ -99,13 +99,14 @@ class FullyConnectedInt8:
     """Full-integer int8 FC: Prepare = fully_connected.cc:526-581, Eval = :1383-1421 / :1254-1284.
 
     filter: int8 [N,K], or packed int4 (pass int4=True: [N, ceil(K/2)] bytes, unpacked once here
-    as fully_connected.cc:1670-1677 does on every call). filter_scales of size N > 1 selects
+    as fully_connected.cc:1670-1677 does on every call), or packed int2 (int2=True: the flat
+    tensor, four values per byte, fully_connected.cc:1678-1685). filter_scales of size N > 1 selects
     the per-channel form, otherwise per-tensor (filter_zero_point then applies).
     """
 
     def __init__(self, filter, bias, input_scale, input_zero_point, filter_scales,
                  output_scale, output_zero_point, activation="none", filter_zero_point=0,
-                 bias_scale=None, int4=False, depth=None, packed=True):
+                 bias_scale=None, int4=False, depth=None, packed=True, int2=False, out_depth=None):
         _ensure_init()
         lib = capi.load()
         fs = np.atleast_1d(np.asarray(filter_scales, dtype=np.float32))
@@ -117,6 +118,13 @@ class FullyConnectedInt8:
                 raise ValueError("depth is required for packed int4 filters")
             self.filter = torch.empty((n, depth), dtype=torch.int8, device="cuda")
             capi.check(lib.lrtfc_unpack_int4(_ptr(nibbles), n * depth, _ptr(self.filter), _stream()))
+        elif int2:
+            fields = _dev(filter, torch.uint8).reshape(-1)
+            if depth is None or out_depth is None:
+                raise ValueError("depth and out_depth are required for packed int2 filters")
+            self.filter = torch.empty((out_depth, depth), dtype=torch.int8, device="cuda")
+            capi.check(lib.lrtfc_unpack_int2(_ptr(fields), out_depth * depth, _ptr(self.filter),
+                                             _stream()))
         else:
             self.filter = _dev(filter, torch.int8)
         self.out_depth, self.depth = self.filter.shape

@@ -18,14 +18,14 @@ if os.environ.get("LITERT_AMD_SANITIZED") == "1":  # the builds of `make san` be
     DELEGATE_LIB = os.path.join(os.path.dirname(HERE), "lib", "liblitert_amd_delegate_san.so")
 
 # TfLiteType / TfLiteAllocationType values (include/tflite_abi.h)
-FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, INT16 = 1, 2, 3, 9, 10, 18, 7
+FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, INT16, INT2 = 1, 2, 3, 9, 10, 18, 7, 20
 MMAP_RO, ARENA_RW = 1, 2
 OK, ERROR, DELEGATE_ERROR = 0, 1, 2
 KIND = {0: None, 1: "int8", 2: "hybrid", 3: "int4_blockwise", 4: "int4_per_channel",
         5: "embedding_lookup", 6: "batch_matmul"}
 
 _NP = {FLOAT32: np.float32, INT32: np.int32, UINT8: np.uint8, INT8: np.int8, FLOAT16: np.float16,
-       INT16: np.int16, INT4: np.uint8}
+       INT16: np.int16, INT4: np.uint8, INT2: np.uint8}
 _lib = None
 CPU_CB = C.CFUNCTYPE(C.c_int, C.c_int)
 

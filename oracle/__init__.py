@@ -59,6 +59,7 @@ def lib():
         L.orc_half_to_float.argtypes = [C.c_uint16]
         L.orc_half_to_float.restype = C.c_float
         L.orc_unpack_int4.argtypes = [_i8p, C.c_int, _i8p]
+        L.orc_unpack_int2.argtypes = [_i8p, C.c_int, _i8p]
         L.orc_fc_prepare_per_channel.argtypes = [C.c_float, _f32p, C.c_int, C.c_float, _i32p, _i32p]
         L.orc_fc_prepare_per_tensor.argtypes = [C.c_float, C.c_float, C.c_int, C.c_float,
                                                 C.c_float, _i32p, _i32p]
@@ -109,6 +110,8 @@ def ref_lib():
         R = C.CDLL(path)
         R.ref_quantize_multiplier.argtypes = [C.c_double, _i32p, _intp]
         R.ref_unpack_int4.argtypes = [_i8p, C.c_int, _i8p]
+        if hasattr(R, "ref_unpack_int2"):
+            R.ref_unpack_int2.argtypes = [_i8p, C.c_int, _i8p]
         for name in ("ref_apply_relu", "ref_apply_relu1", "ref_apply_relu6"):
             getattr(R, name).argtypes = [_f32p, C.c_int, _f32p]
         if hasattr(R, "ref_fc_hybrid_int4"):
@@ -164,6 +167,13 @@ def unpack_int4(packed, num_elements):
     src = _c(packed, np.int8).ravel()
     dst = np.empty(num_elements, dtype=np.int8)
     lib().orc_unpack_int4(_p(src, _i8p), num_elements, _p(dst, _i8p))
+    return dst
+
+
+def unpack_int2(packed, num_elements):
+    src = _c(packed, np.int8).ravel()
+    dst = np.empty(num_elements, dtype=np.int8)
+    lib().orc_unpack_int2(_p(src, _i8p), num_elements, _p(dst, _i8p))
     return dst
 
 

@@ -289,6 +289,23 @@ void orc_unpack_int4(const int8_t* src, int num_elements, int8_t* dst) {
   if (num_elements % 2 != 0) dst[num_elements - 1] = low(src[num_elements / 2]);
 }
 
+void orc_unpack_int2(const int8_t* src, int num_elements, int8_t* dst) {
+  // Field k of a byte (bits 2k, 2k + 1) is moved to the top of the byte and shifted back down
+  // arithmetically, as the reference does; formed from the unsigned byte for the reason given
+  // in orc_unpack_int4.
+  auto field = [](int8_t byte, int k) {
+    return static_cast<int8_t>(
+        static_cast<int8_t>((static_cast<uint8_t>(byte) << (6 - 2 * k)) & 0xFF) >> 6);
+  };
+  for (int i = 0; i < num_elements / 4; ++i) {
+    for (int k = 0; k < 4; ++k) dst[4 * i + k] = field(src[i], k);
+  }
+  const int remaining = num_elements % 4;
+  for (int k = 0; k < remaining; ++k) {
+    dst[num_elements - remaining + k] = field(src[num_elements / 4], k);
+  }
+}
+
 int orc_fc_prepare_per_channel(float input_scale, const float* filter_scales, int num_channels,
                                float output_scale, int32_t* multipliers, int32_t* shifts) {
   for (int i = 0; i < num_channels; ++i) {

@@ -72,6 +72,10 @@ float orc_half_to_float(uint16_t h);
 /* tflite/kernels/internal/portable_tensor_utils.cc:96-127, bit_width 4, signed. */
 void orc_unpack_int4(const int8_t* src, int num_elements, int8_t* dst);
 
+/* tflite/kernels/internal/portable_tensor_utils.cc:128-163, bit_width 2, signed: four values
+ * per byte, the first in bits 0-1; a last partial byte gives num_elements % 4 values. */
+void orc_unpack_int2(const int8_t* src, int num_elements, int8_t* dst);
+
 /* ---- Prepare-time derivations ------------------------------------------ */
 
 /* tflite/kernels/fully_connected.cc:552-564. Returns 0. */

@@ -26,6 +26,11 @@ void ref_unpack_int4(const int8_t* src, int num_elements, int8_t* dst) {
                                               /*unpack_unsigned=*/false);
 }
 
+void ref_unpack_int2(const int8_t* src, int num_elements, int8_t* dst) {
+  tflite::tensor_utils::UnpackPackedIntToInt8(src, num_elements, /*bit_width=*/2, dst,
+                                              /*unpack_unsigned=*/false);
+}
+
 void ref_apply_relu(const float* in, int n, float* out) {
   tflite::tensor_utils::ApplyReluToVector(in, n, out);
 }

@@ -21,13 +21,21 @@ from tests import kat_harness as kh  # noqa: E402
 W10 = [1, 2, 3, 4, 5, 6, 7, 8, 9, 10]
 X2 = [1, 2, 3, 4, 5, 6, 7, 8, -9, -10, 1, 2, 3, 4, 5, 6, 7, -8, 9, -10]
 W4 = [1, 2, 3, 4, 5, 6, 7, 6, 5, 4] * 3
+W2 = [1, 0, 1, 0, 1, 0, 1, 0, -1, 0] * 3
 ACT = {"none": 0, "relu": 1}
 
 
-def per_tensor(source, in_range, out_range, weights, bias, x, units, act="none", int4=False):
+def per_tensor(source, in_range, out_range, weights, bias, x, units, act="none", int4=False,
+               int2=False):
     in_s, in_zp = kh.quantization_params(*in_range)
     out_s, out_zp = kh.quantization_params(*out_range)
-    if int4:
+    if int2:
+        # An Int2 filter takes the range [-1, 1] (fully_connected_test.cc:189-192), its scale is
+        # derived for quantized values -1 .. 1 (test_util.h:1133-1135) and the values are
+        # clamped to -2 .. 1 (test_util.h:209-211).
+        w_s, w_zp = kh.quantization_params(-1.0, 1.0, -1, 1)
+        wq = kh.quantize(weights, w_s, w_zp, -2, 1).reshape(units, -1)
+    elif int4:
         w_s, w_zp = kh.quantization_params(-7.0, 7.0, -7, 7)
         wq = kh.quantize(weights, w_s, w_zp, -7, 7).reshape(units, -1)
     else:
@@ -36,7 +44,7 @@ def per_tensor(source, in_range, out_range, weights, bias, x, units, act="none",
     xq = kh.quantize(x, in_s, in_zp).reshape(-1, wq.shape[1])
     bias_scale = np.float32(in_s * w_s)
     bq = None if bias is None else kh.quantize_bias(bias, bias_scale)
-    return dict(source=source, per_channel=False, int4=int4, activation=ACT[act],
+    return dict(source=source, per_channel=False, int4=int4, int2=int2, activation=ACT[act],
                 input=xq.tolist(), filter=wq.tolist(), bias=None if bq is None else bq.tolist(),
                 input_scale=float(in_s), input_zero_point=int(in_zp),
                 filter_scales=[float(w_s)], filter_zero_point=int(w_zp),
@@ -44,18 +52,20 @@ def per_tensor(source, in_range, out_range, weights, bias, x, units, act="none",
                 output_scale=float(out_s), output_zero_point=int(out_zp))
 
 
-def per_channel(source, scales, weights, bias, x, units, depth, act="none", int4=False):
+def per_channel(source, scales, weights, bias, x, units, depth, act="none", int4=False,
+                int2=False):
     in_s, in_zp = kh.quantization_params(-63.5, 64)
     out_s, out_zp = kh.quantization_params(-127, 128)
     scales = np.asarray(scales, np.float32)
     w = np.asarray(weights, np.float32).reshape(units, depth)
     inv = (np.float32(1.0) / scales).astype(np.float32)
     lim = 7 if int4 else 127
-    wq = np.clip(kh._round_half_away(w * inv[:, None]), -lim, lim).astype(np.int8)
+    lo, hi = (-2, 1) if int2 else (-lim, lim)  # quantization_utils.cc:428-431 for Int2
+    wq = np.clip(kh._round_half_away(w * inv[:, None]), lo, hi).astype(np.int8)
     xq = kh.quantize(x, in_s, in_zp).reshape(-1, depth)
     bscale = (scales * in_s).astype(np.float32)
     bq = kh._round_half_away(np.asarray(bias, np.float32) / bscale).astype(np.int32)
-    return dict(source=source, per_channel=True, int4=int4, activation=ACT[act],
+    return dict(source=source, per_channel=True, int4=int4, int2=int2, activation=ACT[act],
                 input=xq.tolist(), filter=wq.tolist(), bias=bq.tolist(),
                 input_scale=float(in_s), input_zero_point=int(in_zp),
                 filter_scales=[float(s) for s in scales], filter_zero_point=0, bias_scale=None,
@@ -180,7 +190,13 @@ def main():
                          [1, 2, 3, 4, -5, 1, 2, 3, -4, 5, 1, 2, -3, 4, 5, 1, -2, 3, 4, 5], 3, 5, "relu"),
              [5, 6, 7, 23, 24, 25, 37, 38, 39, 47, 48, 49]),
             (per_channel(t + ":950-976", [1.0, 1.0, 1.0], W4, [1, 2, 3], X2, 3, 10, "relu", True),
-             [103, 104, 105, 97, 98, 99])):
+             [103, 104, 105, 97, 98, 99]),
+            (per_tensor(t + ":784-814", (-63.5, 64), (-127, 128), W2, [1, 2, 3], X2, 3, "relu",
+                        int2=True),
+             [25, 26, 27, 7, 8, 9]),
+            (per_channel(t + ":978-1004", [1.0, 1.0, 1.0], W2, [1, 2, 3], X2, 3, 10, "relu",
+                         int2=True),
+             [25, 26, 27, 7, 8, 9])):
         case["expected_output"] = want
         fc.append(case)
 
@@ -242,6 +258,10 @@ def main():
                quantize_multiplier=multiplier, multiply_by_quantized_multiplier=mbqm,
                hybrid_dot_per_channel=hybrid_dot,
                batch_matmul_hybrid=batch_matmul_hybrid_cases(),
+               unpack_int2=[dict(source=u + ":2131-2140", packed=[0x6C], count=4,
+                                 expected=[0, -1, -2, 1]),
+                            dict(source=u + ":2142-2150", packed=[0xD8], count=3,
+                                 expected=[0, -2, 1])],
                unpack_int4=[dict(source=u + ":2110-2119", packed=[0x38, 0xBE], count=4,
                                  expected=[-8, 3, -2, -5]),
                             dict(source=u + ":2121-2130", packed=[0x21, 0x43], count=3,

@@ -56,6 +56,16 @@ def pack_int4(values_i8):
     return (lo | (hi << 4)).astype(np.uint8)
 
 
+def pack_int2(values_i8):
+    """Four signed 2-bit values per byte, the first in bits 0-1 (PopulateTensor2bit; the inverse of
+    portable_tensor_utils.cc:128-163)."""
+    v = np.asarray(values_i8, dtype=np.int8).ravel()
+    if v.size % 4:
+        v = np.concatenate([v, np.zeros(4 - v.size % 4, np.int8)])
+    u = v.astype(np.uint8) & 0x3
+    return (u[0::4] | (u[1::4] << 2) | (u[2::4] << 4) | (u[3::4] << 6)).astype(np.uint8)
+
+
 def symmetric_quantize_tensor(values):
     """SingleOpModel::QuantizeTensor (tflite/kernels/test_util.h:1407-1430): the whole tensor
     through SymmetricQuantizeFloats (reference/portable_tensor_utils.cc:41-71). Returns

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from tests import fake_host as fhm
-from tests.fake_host import FakeHost, FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, INT16
+from tests.fake_host import FakeHost, FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, INT16, INT2
 
 
 def test_plugin_exports_entry_points():
@@ -25,7 +25,7 @@ def _int8_node(h, B=2, K=32, N=8, per_channel=True, filter_type=INT8, in_type=IN
                const_filter=True, w_zp=0, bias=True, **kw):
     x = h.tensor(in_type, (B, K), scale=0.02, zero_point=-3)
     h.affine(x, [0.02], [-3])
-    wbytes = N * K if filter_type != INT4 else N * K // 2
+    wbytes = {INT4: N * K // 2, INT2: N * K // 4}.get(filter_type, N * K)
     w = h.tensor(filter_type, (N, K), data=np.zeros(wbytes, np.int8), const=const_filter)
     if per_channel:
         h.affine(w, np.full(N, 0.005), np.full(N, w_zp))
@@ -42,6 +42,11 @@ def test_claim_predicate_int8():
         assert h.classify(_int8_node(h))[0] == "int8"
         assert h.classify(_int8_node(h, per_channel=False, w_zp=-1))[0] == "int8"
         assert h.classify(_int8_node(h, filter_type=INT4))[0] == "int8"
+        # Int2 filters are unpacked to int8 like Int4 ones (fully_connected.cc:1678-1685)
+        assert h.classify(_int8_node(h, filter_type=INT2))[0] == "int8"
+        assert h.classify(_int8_node(h, filter_type=INT2, per_channel=False))[0] == "int8"
+        assert h.classify(_int8_node(h, per_channel=False, filter_type=INT2, w_zp=1)) == (
+            None, "non-zero filter zero point")
         assert h.classify(_int8_node(h, bias=False))[0] == "int8"
         assert h.classify(_int8_node(h, bias=False, optional_bias_slot=True))[0] == "int8"
         for act in (0, 1, 2, 3):
@@ -68,7 +73,7 @@ def _float_node(h, B=2, K=64, N=8, filter_type=INT8, blockwise=False, bs=32, per
         s = h.tensor(scale_type, (N, K // bs), data=np.ones((N, K // bs), np.float16 if scale_type == FLOAT16 else np.float32), const=True)
         h.blockwise(w, s, bs)
     else:
-        nbytes = N * K if filter_type == INT8 else N * K // 2
+        nbytes = {INT8: N * K, INT2: N * K // 4}.get(filter_type, N * K // 2)
         w = h.tensor(filter_type, (N, K), data=np.zeros(nbytes, np.int8), const=True)
         h.affine(w, np.full(N if per_channel else 1, 0.004), quantized_dimension=quantized_dimension)
     y = h.tensor(FLOAT32, (B, N))
@@ -103,6 +108,12 @@ def test_claim_predicate_float_activations():
             None, "activation is tanh or sigmoid")
         assert h.classify(_float_node(h, filter_type=INT4, activation=4)) == (None, "activation is tanh or sigmoid")
         assert h.classify(_float_node(h, filter_type=INT4, activation=5))[0] == "int4_per_channel"
+        # an Int2 filter under float activations: unpacked, then EvalHybridDense
+        # (fully_connected.cc:812-818): claimed as a hybrid node, whatever the shape
+        assert h.classify(_float_node(h, filter_type=INT2))[0] == "hybrid"
+        assert h.classify(_float_node(h, filter_type=INT2, per_channel=False, N=2, K=16))[0] == "hybrid"
+        assert h.classify(_float_node(h, filter_type=INT2, activation=6)) == (
+            None, "activation is tanh or sigmoid")
         # scales along the depth are not per-output-channel scales
         assert h.classify(_float_node(h, filter_type=INT4, N=8, K=8 * 8, quantized_dimension=1)) == (
             None, "per-channel scales do not match output channels")

@@ -23,6 +23,9 @@ def _filter_int8(case):
     if case["int4"]:  # stored two per byte in the model; what the kernels see after unpacking
         from tests import kat_harness as kh
         w = oracle.unpack_int4(kh.pack_int4(w).view(np.int8), w.size).reshape(w.shape)
+    if case.get("int2"):  # four per byte
+        from tests import kat_harness as kh
+        w = oracle.unpack_int2(kh.pack_int2(w).view(np.int8), w.size).reshape(w.shape)
     return w
 
 
@@ -56,6 +59,12 @@ def test_oracle_batch_quantize_floats(case, variant):
 @pytest.mark.parametrize("case", KATS["unpack_int4"], ids=lambda c: str(c["count"]))
 def test_oracle_unpack_int4(case):
     got = oracle.unpack_int4(np.array(case["packed"], np.uint8).view(np.int8), case["count"])
+    assert got.tolist() == case["expected"]
+
+
+@pytest.mark.parametrize("case", KATS["unpack_int2"], ids=lambda c: str(c["count"]))
+def test_oracle_unpack_int2(case):
+    got = oracle.unpack_int2(np.array(case["packed"], np.uint8).view(np.int8), case["count"])
     assert got.tolist() == case["expected"]
 
 
@@ -122,6 +131,45 @@ def test_hip_fully_connected_int8(fc, case, packed):
         filter_zero_point=case["filter_zero_point"], bias_scale=case["bias_scale"], packed=packed)
     y = op(_cuda(np.array(case["input"], np.int8))).cpu().numpy()
     assert y.ravel().tolist() == case["expected_output"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", [c for c in KATS["fully_connected_int8"] if c.get("int2")],
+                         ids=lambda c: c["source"].split(":", 1)[1])
+def test_hip_fully_connected_int2_filter_unpacked_on_the_device(fc, case):
+    """The two Int2 cases with the filter handed over as the model holds it (four values per
+    byte) and unpacked by lrtfc_unpack_int2."""
+    from tests import kat_harness as kh
+    w = np.array(case["filter"], np.int8)
+    scales = case["filter_scales"] if case["per_channel"] else [case["filter_scales"][0]]
+    op = fc.FullyConnectedInt8(
+        kh.pack_int2(w), np.array(case["bias"], np.int32), case["input_scale"],
+        case["input_zero_point"], np.array(scales, np.float32), case["output_scale"],
+        case["output_zero_point"], activation=case["activation"],
+        filter_zero_point=case["filter_zero_point"], bias_scale=case["bias_scale"], int2=True,
+        depth=w.shape[1], out_depth=w.shape[0])
+    y = op(_cuda(np.array(case["input"], np.int8))).cpu().numpy()
+    assert y.ravel().tolist() == case["expected_output"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("count", [1, 2, 3, 4, 5, 7, 64, 1001, 1002, 1003, 70000])
+def test_hip_unpack_int2_matches_oracle(fc, count):
+    import torch
+    from litert_amd import capi
+    rng = np.random.default_rng(count)
+    packed = rng.integers(0, 256, (count + 3) // 4).astype(np.uint8)
+    src = _cuda(packed)
+    dst = torch.full((count + 8,), 99, dtype=torch.int8, device="cuda")
+    capi.check(capi.load().lrtfc_unpack_int2(src.data_ptr(), count, dst.data_ptr(), None))
+    got = dst.cpu().numpy()
+    assert np.array_equal(got[:count], oracle.unpack_int2(packed.view(np.int8), count))
+    assert (got[count:] == 99).all()  # nothing written past the last element
+    for case in KATS["unpack_int2"]:
+        src = _cuda(np.array(case["packed"], np.uint8))
+        dst = torch.empty(case["count"], dtype=torch.int8, device="cuda")
+        capi.check(capi.load().lrtfc_unpack_int2(src.data_ptr(), case["count"], dst.data_ptr(), None))
+        assert dst.cpu().numpy().tolist() == case["expected"]
 
 
 @pytest.mark.gpu

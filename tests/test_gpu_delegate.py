@@ -7,7 +7,7 @@ import pytest
 
 import oracle
 from litert_amd import workloads as wl
-from tests.fake_host import (FakeHost, FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, OK,
+from tests.fake_host import (FakeHost, FLOAT32, INT32, UINT8, INT8, FLOAT16, INT4, INT2, OK,
                              DELEGATE_ERROR)
 
 pytestmark = pytest.mark.gpu
@@ -447,6 +447,57 @@ def test_int4_affine_filter_outside_the_4bit_gate_runs_the_int8_hybrid_path(B, N
                                 1.0 if per_channel else float(fs[0]), bias, asymmetric,
                                 oracle.ACT_RELU6)
         assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("B,N,K,per_channel", [(1, 8, 64, True), (3, 5, 33, False), (20, 130, 272, True)])
+def test_int2_filter_runs_the_int8_paths_after_unpacking(B, N, K, per_channel):
+    """An Int2 filter (four values per byte over the flat tensor, rows not byte-aligned when the
+    depth is odd) under float activations and under int8 ones: unpacked once at prepare
+    (fully_connected.cc:812-818, 1678-1685), then the hybrid and the full-integer kernels. Oracle:
+    unpack_int2 followed by fc_hybrid / fc_int8, each pinned on its own."""
+    from tests import kat_harness as kh
+    rng = np.random.default_rng(60 + N + K)
+    w_np = rng.integers(-2, 2, (N, K)).astype(np.int8)
+    packed = kh.pack_int2(w_np.ravel())
+    unpacked = oracle.unpack_int2(packed.view(np.int8), N * K).reshape(N, K)
+    assert np.array_equal(unpacked, w_np)
+    fs = rng.uniform(0.01, 0.1, N).astype(np.float32) if per_channel else np.array([0.05], np.float32)
+    # float activations
+    x_np = rng.standard_normal((B, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    with FakeHost() as h:
+        x = h.tensor(FLOAT32, (B, K), data=x_np)
+        w = h.tensor(INT2, (N, K), data=packed, const=True)
+        h.affine(w, fs)
+        b = h.tensor(FLOAT32, (N,), data=bias, const=True)
+        y = h.tensor(FLOAT32, (B, N))
+        node = h.fc(x, w, b, y, activation=1, asymmetric=True)
+        assert h.classify(node)[0] == "hybrid"
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.plan()[0][:2] == ("delegate", [node])
+        assert h.invoke() == OK, h.errors()
+        want = oracle.fc_hybrid(x_np, unpacked, fs if per_channel else None,
+                                1.0 if per_channel else float(fs[0]), bias, True, oracle.ACT_RELU)
+        assert np.array_equal(h.read(y).view(np.uint32), want.view(np.uint32))
+    # int8 activations
+    c = wl.int8_fc(B, K, N, in_zp=-3, seed=61 + N)
+    w_scale = fs if per_channel else np.full(N, fs[0], np.float32)  # per-channel scales either way
+    with FakeHost() as h:
+        x = h.tensor(INT8, (B, K), data=c["x"])
+        h.affine(x, [c["in_scale"]], [c["in_zp"]])
+        w = h.tensor(INT2, (N, K), data=packed, const=True)
+        h.affine(w, w_scale)
+        b = h.tensor(INT32, (N,), data=c["bias"], const=True)
+        y = h.tensor(INT8, (B, N))
+        h.affine(y, [c["out_scale"]], [c["out_zp"]])
+        node = h.fc(x, w, b, y, activation=1)
+        assert h.classify(node)[0] == "int8"
+        assert h.load_delegate() == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.invoke() == OK, h.errors()
+        c2 = dict(c, w=unpacked, w_scale=w_scale)
+        assert np.array_equal(h.read(y), _oracle_int8(c2, c["x"], activation=1))
 
 
 def test_int4_per_channel_node_switches_layout_with_the_batch():

@@ -173,6 +173,29 @@ def test_unpack_int4_matches_reference_build():
         assert np.array_equal(oracle.unpack_int4(src, n), want)
 
 
+# ---- int2 unpack: tflite/kernels/internal/tensor_utils_test.cc:2131-2150 + reference build
+
+def test_unpack_int2_kat():
+    # UnpackInt2Basic: 0x6C = fields 0, 3, 2, 1 -> 0, -1, -2, 1; UnpackInt2OddLength: 0xD8, 3 values
+    assert oracle.unpack_int2(np.array([0x6C], np.uint8).view(np.int8), 4).tolist() == [0, -1, -2, 1]
+    assert oracle.unpack_int2(np.array([0xD8], np.uint8).view(np.int8), 3).tolist() == [0, -2, 1]
+    values = np.array([1, -2, 0, -1, 1, 1, -2, 0, -1], np.int8)
+    assert oracle.unpack_int2(kh.pack_int2(values).view(np.int8), 9).tolist() == values.tolist()
+
+
+def test_unpack_int2_matches_reference_build():
+    R = oracle.ref_lib()
+    if R is None or not hasattr(R, "ref_unpack_int2"):
+        pytest.skip("oracle/_ref not built (reference tree absent)")
+    rng = np.random.default_rng(4)
+    for n in (1, 2, 3, 4, 5, 7, 64, 1001, 1002, 1003):
+        src = rng.integers(-128, 128, (n + 3) // 4).astype(np.int8)
+        want = np.empty(n, np.int8)
+        R.ref_unpack_int2(src.ctypes.data_as(C.POINTER(C.c_int8)), n,
+                          want.ctypes.data_as(C.POINTER(C.c_int8)))
+        assert np.array_equal(oracle.unpack_int2(src, n), want)
+
+
 def test_relu_matches_reference_build():
     R = oracle.ref_lib()
     if R is None:
