@@ -108,6 +108,14 @@ int lrtfc_unpack_int4(const uint8_t* packed, int64_t num_elements, int8_t* unpac
 int lrtfc_unpack_int2(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
                       void* stream);
 
+/* dst[i] = src[i] ^ 0x80: a uint8 tensor as int8 (value - 128) and back; src == dst is allowed.
+ * With it the legacy uint8 FULLY_CONNECTED (tflite/kernels/internal/reference/fully_connected.h
+ * :118-166, reached from tflite/kernels/fully_connected.cc:1607-1626) runs on the int8 kernels:
+ *   sum (w_u8 + fo)(x_u8 + io) = sum (w_i8 + fo + 128)(x_i8 + io + 128),
+ *   y_u8 = clamp(M(acc) + oo, lo, hi)  <=>  y_i8 = clamp(M(acc) + oo - 128, lo - 128, hi - 128),
+ * i.e. lrtfc_fc_int8 with every zero point lowered by 128 and the same multiplier and shift. */
+int lrtfc_xor_sign_bit(const uint8_t* src, uint8_t* dst, size_t bytes, void* stream);
+
 /* kfsum[n] = sum over blocks, in block order and float32, of
  * scale[n,b] * float(sum_k filter[n, b*blocksize + k]): the weight-only part of
  * EvalBlockwise4Bit's zero-point correction

@@ -33,6 +33,7 @@ SYMBOLS = [
     ("lrtfc_row_sums_int8", _i, [_vp, _i, _i, _vp, _vp]),
     ("lrtfc_unpack_int4", _i, [_vp, _i64, _vp, _vp]),
     ("lrtfc_unpack_int2", _i, [_vp, _i64, _vp, _vp]),
+    ("lrtfc_xor_sign_bit", _i, [_vp, _vp, _sz, _vp]),
     ("lrtfc_blockwise_int4_kfsum", _i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     ("lrtfc_fc_int8_preferred_layout", _i, [_i, _i, _i, _i]),
     ("lrtfc_fc_blockwise_int4_preferred_layout", _i, [_i, _i]),

@@ -266,6 +266,13 @@ int lrtfc_unpack_int4(const uint8_t* packed, int64_t num_elements, int8_t* unpac
                  "int4 unpack");
 }
 
+int lrtfc_xor_sign_bit(const uint8_t* src, uint8_t* dst, size_t bytes, void* stream) {
+  if (int rc = RequireInit()) return rc;
+  if (bytes == 0) return LRTFC_OK;
+  LRTFC_REQUIRE(src && dst, "null pointer");
+  return FromHip(lrtfc::LaunchXorSignBit(src, dst, bytes, AsStream(stream)), "sign bit flip");
+}
+
 int lrtfc_unpack_int2(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
                       void* stream) {
   if (int rc = RequireInit()) return rc;

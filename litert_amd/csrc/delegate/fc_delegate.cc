@@ -307,6 +307,21 @@ FcKind Classify(const TfLiteContext* ctx, const TfLiteNode* node,
   const int depth = filter.dims->data[1];
   if (bias && NumElements(bias->dims) != out_depth) return no("bias size != output channels");
 
+  if (input.type == kTfLiteUInt8 && output.type == kTfLiteUInt8 && filter.type == kTfLiteUInt8) {
+    // The legacy uint8 op (fully_connected.cc:1607-1626): per-tensor only, any zero points. It runs
+    // on the int8 kernels with every tensor taken as value - 128 (PrepareNode, KernelInvoke).
+    if (!opt.claim_int8) return no("int8 path disabled by option");
+    if (!ClippingActivation(params->activation)) return no("activation not a clamp");
+    if (bias && bias->type != kTfLiteInt32) return no("bias is not int32");
+    if (input.quantization.type != kTfLiteAffineQuantization ||
+        filter.quantization.type != kTfLiteAffineQuantization) {
+      return no("input/filter lack affine quantization");
+    }
+    const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
+    if (!fq || !fq->scale || fq->scale->size != 1) return no("uint8 filter is not per-tensor");
+    if (output.params.scale <= 0.0f || input.params.scale <= 0.0f) return no("missing scales");
+    return FcKind::kInt8;
+  }
   if (input.type == kTfLiteInt8 && output.type == kTfLiteInt8 &&
       (filter.type == kTfLiteInt8 || filter.type == kTfLiteInt4 || filter.type == kTfLiteInt2)) {
     if (!opt.claim_int8) return no("int8 path disabled by option");
@@ -503,6 +518,9 @@ struct FcNode {
   bool per_channel = false;
   float filter_scale = 1.0f;
   int32_t input_offset = 0, filter_offset = 0, output_offset = 0, act_min = 0, act_max = 0;
+  // A uint8 node: its rows and its result pass through these as int8 (value - 128).
+  bool uint8_io = false;
+  DeviceBuffer u8_rows_dev, u8_result_dev;
   const void* uploaded_filter = nullptr;  // host pointer the device copies were made from
   // The filter lives on the device in the layout the node's shape runs fastest on: the
   // model's own (row-major / nibble-packed rows) or the re-tiled copy. Only one is kept.
@@ -966,9 +984,13 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
   if (n->kind == FcKind::kInt8) {
     const auto* fq = static_cast<const TfLiteAffineQuantization*>(filter.quantization.params);
     n->per_channel = fq->scale->size > 1;
-    n->input_offset = -input.params.zero_point;
-    n->filter_offset = n->per_channel ? 0 : -filter.params.zero_point;
-    n->output_offset = output.params.zero_point;
+    // uint8 tensors are handled as int8, value - 128: every zero point moves down with them, and
+    // each term (w - zw)(x - zx), the multiplier and the clamped result stay what they were.
+    n->uint8_io = input.type == kTfLiteUInt8;
+    const int32_t moved = n->uint8_io ? 128 : 0;
+    n->input_offset = -(input.params.zero_point - moved);
+    n->filter_offset = n->per_channel ? 0 : -(filter.params.zero_point - moved);
+    n->output_offset = output.params.zero_point - moved;
     std::vector<int32_t> mult(n->per_channel ? n->out_depth : 1), shift(mult.size());
     if (n->per_channel) {
       RETURN_IF_FC(ctx, lrtfc_prepare_per_channel(input.params.scale, fq->scale->data,
@@ -981,8 +1003,12 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
                                                  output.params.scale, &mult[0], &shift[0]));
     }
     RETURN_IF_FC(ctx, lrtfc_activation_range_int8(n->params.activation, output.params.scale,
-                                                  output.params.zero_point, &n->act_min,
+                                                  output.params.zero_point - moved, &n->act_min,
                                                   &n->act_max));
+    if (n->uint8_io) {
+      RETURN_IF_HIP(ctx, n->u8_rows_dev.Ensure(static_cast<size_t>(n->batches) * n->depth));
+      RETURN_IF_HIP(ctx, n->u8_result_dev.Ensure(static_cast<size_t>(n->batches) * n->out_depth));
+    }
     RETURN_IF_HIP(ctx, n->mult_dev.Upload(mult.data(), mult.size() * 4, s));
     RETURN_IF_HIP(ctx, n->shift_dev.Upload(shift.data(), shift.size() * 4, s));
     RETURN_IF_HIP(ctx, hipStreamSynchronize(s));  // mult/shift are stack-owned
@@ -1009,6 +1035,10 @@ TfLiteStatus PrepareNode(TfLiteContext* ctx, PartitionKernel* k, FcNode* n) {
           RETURN_IF_HIP(ctx, hipStreamSynchronize(s));
         } else {
           RETURN_IF_HIP(ctx, n->filter_dev.Upload(filter.data.raw, weights, s));
+          if (n->uint8_io) {
+            RETURN_IF_FC(ctx, lrtfc_xor_sign_bit(n->filter_dev.as<uint8_t>(),
+                                                 n->filter_dev.as<uint8_t>(), weights, s));
+          }
         }
         RETURN_IF_HIP(ctx, n->row_sums_dev.Ensure(static_cast<size_t>(n->out_depth) * 4));
         RETURN_IF_FC(ctx, lrtfc_row_sums_int8(n->filter_dev.as<int8_t>(), n->out_depth, n->depth,
@@ -1631,27 +1661,42 @@ TfLiteStatus KernelInvoke(TfLiteContext* ctx, TfLiteNode* node) {
     const int variant = k->state->options.quant_variant;
     const float* bias_f32 = has_bias ? n.bias_dev.as<float>() : nullptr;
     switch (n.kind) {
-      case FcKind::kInt8:
+      case FcKind::kInt8: {
+        const void* rows = in_dev;
+        void* result = out_dev;
+        if (n.uint8_io) {
+          RETURN_IF_FC(ctx, lrtfc_xor_sign_bit(static_cast<const uint8_t*>(in_dev),
+                                               n.u8_rows_dev.as<uint8_t>(),
+                                               static_cast<size_t>(n.batches) * n.depth, s));
+          rows = n.u8_rows_dev.as<uint8_t>();
+          result = n.u8_result_dev.as<uint8_t>();
+        }
         if (n.use_retiled) {
-          RETURN_IF_FC(ctx, lrtfc_fc_int8_packed(static_cast<const int8_t*>(in_dev),
+          RETURN_IF_FC(ctx, lrtfc_fc_int8_packed(static_cast<const int8_t*>(rows),
                                                  n.retiled_dev.as<int8_t>(),
                                                  has_bias ? n.bias_dev.as<int32_t>() : nullptr,
                                                  n.mult_dev.as<int32_t>(), n.shift_dev.as<int32_t>(),
                                                  n.per_channel, n.row_sums_dev.as<int32_t>(),
-                                                 static_cast<int8_t*>(out_dev), n.batches, n.depth,
+                                                 static_cast<int8_t*>(result), n.batches, n.depth,
                                                  n.out_depth, n.input_offset, n.output_offset,
                                                  n.act_min, n.act_max, s));
         } else {
-          RETURN_IF_FC(ctx, lrtfc_fc_int8(static_cast<const int8_t*>(in_dev),
+          RETURN_IF_FC(ctx, lrtfc_fc_int8(static_cast<const int8_t*>(rows),
                                           n.filter_dev.as<int8_t>(),
                                           has_bias ? n.bias_dev.as<int32_t>() : nullptr,
                                           n.mult_dev.as<int32_t>(), n.shift_dev.as<int32_t>(),
                                           n.per_channel, n.row_sums_dev.as<int32_t>(),
-                                          static_cast<int8_t*>(out_dev), n.batches, n.depth,
+                                          static_cast<int8_t*>(result), n.batches, n.depth,
                                           n.out_depth, n.input_offset, n.filter_offset,
                                           n.output_offset, n.act_min, n.act_max, s));
         }
+        if (n.uint8_io) {
+          RETURN_IF_FC(ctx, lrtfc_xor_sign_bit(static_cast<const uint8_t*>(result),
+                                               static_cast<uint8_t*>(out_dev),
+                                               static_cast<size_t>(n.batches) * n.out_depth, s));
+        }
         break;
+      }
       case FcKind::kHybrid: {
         const float* pcs = n.per_channel ? n.pcs_dev.as<float>() : nullptr;
         const int asym = n.params.asymmetric_quantize_inputs;

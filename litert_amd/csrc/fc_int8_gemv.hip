@@ -196,6 +196,27 @@ __global__ __launch_bounds__(kThreads) void UnpackInt2Kernel(const uint8_t* __re
   }
 }
 
+// uint8 <-> int8 as a change of representation: value - 128 one way, value + 128 the other, both
+// the same flip of the top bit. 16 bytes per thread where the pointers allow it.
+__global__ __launch_bounds__(kThreads) void XorSignBitKernel(const uint8_t* __restrict__ src,
+                                                             uint8_t* __restrict__ dst,
+                                                             size_t bytes, bool vectors) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (vectors) {
+    const size_t at = i * 16;
+    if (at + 16 <= bytes) {
+      i32x4 v = *reinterpret_cast<const i32x4*>(src + at);
+      const int32_t flip = static_cast<int32_t>(0x80808080u);
+      v = i32x4{v[0] ^ flip, v[1] ^ flip, v[2] ^ flip, v[3] ^ flip};
+      *reinterpret_cast<i32x4*>(dst + at) = v;
+    } else {
+      for (size_t j = at; j < bytes; ++j) dst[j] = src[j] ^ 0x80;
+    }
+  } else if (i < bytes) {
+    dst[i] = src[i] ^ 0x80;
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void ZeroFillKernel(uint8_t* __restrict__ dst, size_t bytes) {
   const size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i < bytes) dst[i] = 0;
@@ -266,6 +287,17 @@ hipError_t LaunchUnpackInt4(const uint8_t* packed, int64_t num_elements, int8_t*
   const int grid = static_cast<int>((num_bytes + kThreads - 1) / kThreads);
   hipLaunchKernelGGL(UnpackInt4Kernel, dim3(grid), dim3(kThreads), 0, stream, packed, num_elements,
                      unpacked);
+  return hipGetLastError();
+}
+
+hipError_t LaunchXorSignBit(const uint8_t* src, uint8_t* dst, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return hipSuccess;
+  const bool vectors = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
+  const size_t threads = vectors ? (bytes + 15) / 16 : bytes;
+  const size_t grid = (threads + kThreads - 1) / kThreads;
+  if (grid > 0x7fffffffull) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(XorSignBitKernel, dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, stream,
+                     src, dst, bytes, vectors);
   return hipGetLastError();
 }
 

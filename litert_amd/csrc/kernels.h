@@ -90,6 +90,8 @@ hipError_t LaunchUnpackInt4(const uint8_t* packed, int64_t num_elements, int8_t*
                             hipStream_t stream);
 hipError_t LaunchUnpackInt2(const uint8_t* packed, int64_t num_elements, int8_t* unpacked,
                             hipStream_t stream);
+// dst[i] = src[i] ^ 0x80 (uint8 value - 128 as int8, and back); src == dst allowed.
+hipError_t LaunchXorSignBit(const uint8_t* src, uint8_t* dst, size_t bytes, hipStream_t stream);
 
 // Small-batch path: bandwidth-bound GEMV (any shape; fast path needs depth % 16 == 0).
 hipError_t LaunchFcInt8Gemv(const FcInt8Args& a, Int8Epilogue epilogue, hipStream_t stream);

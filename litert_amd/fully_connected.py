@@ -175,6 +175,38 @@ class FullyConnectedInt8:
         return out
 
 
+class FullyConnectedUInt8:
+    """The legacy full-integer uint8 FC (per-tensor; fully_connected.cc:1607-1626 with
+    reference/fully_connected.h:118-166) on the int8 kernels: every uint8 tensor is taken as
+    int8 (value - 128, a flip of the top bit: the filter once here, the rows and the result on
+    every call) and every zero point lowered by 128, which leaves each term of the sum, the
+    multiplier and the clamped result what they were."""
+
+    def __init__(self, filter, bias, input_scale, input_zero_point, filter_scale,
+                 filter_zero_point, output_scale, output_zero_point, activation="none",
+                 bias_scale=None, packed=True):
+        _ensure_init()
+        lib = capi.load()
+        w = _dev(filter, torch.uint8).contiguous()
+        capi.check(lib.lrtfc_xor_sign_bit(_ptr(w), _ptr(w), w.numel(), _stream()))
+        self.int8 = FullyConnectedInt8(
+            w.view(torch.int8), bias, input_scale, int(input_zero_point) - 128, [filter_scale],
+            output_scale, int(output_zero_point) - 128, activation=activation,
+            filter_zero_point=int(filter_zero_point) - 128, bias_scale=bias_scale, packed=packed)
+        self.out_depth, self.depth = self.int8.out_depth, self.int8.depth
+
+    def __call__(self, x, out=None):
+        lib = capi.load()
+        x = x.contiguous()
+        rows = torch.empty_like(x)
+        capi.check(lib.lrtfc_xor_sign_bit(_ptr(x), _ptr(rows), x.numel(), _stream()))
+        y = self.int8(rows.view(torch.int8))
+        if out is None:
+            out = torch.empty(y.shape, dtype=torch.uint8, device=x.device)
+        capi.check(lib.lrtfc_xor_sign_bit(_ptr(y), _ptr(out), y.numel(), _stream()))
+        return out
+
+
 class FullyConnectedHybrid:
     """Hybrid FC (float activations, int8 filter): EvalHybridDense, fully_connected.cc:763-858."""
 

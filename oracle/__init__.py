@@ -73,6 +73,10 @@ def lib():
         L.orc_fc_int8_per_tensor.argtypes = [
             _i8p, _i8p, _i32p, C.c_int32, C.c_int, _i8p, C.c_int, C.c_int, C.c_int, C.c_int32,
             C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+        L.orc_fc_uint8_per_tensor.argtypes = [
+            _u8p, _u8p, _i32p, C.c_int32, C.c_int, _u8p, C.c_int, C.c_int, C.c_int, C.c_int32,
+            C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+        L.orc_activation_range_uint8.argtypes = [C.c_int, C.c_float, C.c_int32, _i32p, _i32p]
         L.orc_fc_int8_per_tensor_float_scale.argtypes = [
             _i8p, _i8p, _i32p, C.c_float, C.c_float, C.c_float, _i8p, C.c_int, C.c_int, C.c_int,
             C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]
@@ -148,6 +152,14 @@ def mbqm_single_rounding(x, m, shift):
 def activation_range_int8(activation, out_scale, out_zp):
     lo, hi = C.c_int32(), C.c_int32()
     rc = lib().orc_activation_range_int8(activation, out_scale, out_zp, C.byref(lo), C.byref(hi))
+    if rc:
+        raise ValueError("activation range overflows int32")
+    return lo.value, hi.value
+
+
+def activation_range_uint8(activation, out_scale, out_zp):
+    lo, hi = C.c_int32(), C.c_int32()
+    rc = lib().orc_activation_range_uint8(activation, out_scale, out_zp, C.byref(lo), C.byref(hi))
     if rc:
         raise ValueError("activation range overflows int32")
     return lo.value, hi.value
@@ -238,6 +250,21 @@ def fc_int8_per_tensor(x, w, bias, mult, shift, input_offset, filter_offset, out
     lib().orc_fc_int8_per_tensor(_p(x, _i8p), _p(w, _i8p), _p(bias, _i32p), int(mult), int(shift),
                                  _p(y, _i8p), B, K, N, input_offset, filter_offset, output_offset,
                                  act_min, act_max)
+    return y
+
+
+def fc_uint8_per_tensor(x, w, bias, mult, shift, input_offset, filter_offset, output_offset,
+                        act_min, act_max):
+    """x [B,K] and w [N,K] uint8; offsets are the negated uint8 zero points."""
+    x = _c(x, np.uint8)
+    w = _c(w, np.uint8)
+    x = x.reshape(-1, w.shape[1])
+    B, K, N = x.shape[0], w.shape[1], w.shape[0]
+    bias = _c(bias, np.int32)
+    y = np.empty((B, N), dtype=np.uint8)
+    lib().orc_fc_uint8_per_tensor(_p(x, _u8p), _p(w, _u8p), _p(bias, _i32p), int(mult), int(shift),
+                                  _p(y, _u8p), B, K, N, input_offset, filter_offset, output_offset,
+                                  act_min, act_max)
     return y
 
 

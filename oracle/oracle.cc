@@ -418,6 +418,53 @@ void orc_fc_int8_per_tensor(const int8_t* input, const int8_t* filter, const int
   }
 }
 
+void orc_fc_uint8_per_tensor(const uint8_t* input, const uint8_t* filter, const int32_t* bias,
+                             int32_t multiplier, int shift, uint8_t* output, int batches, int depth,
+                             int out_depth, int32_t input_offset, int32_t filter_offset,
+                             int32_t output_offset, int32_t act_min, int32_t act_max) {
+  for (int b = 0; b < batches; ++b) {
+    for (int c = 0; c < out_depth; ++c) {
+      int32_t acc = 0;
+      for (int d = 0; d < depth; ++d) {
+        const int32_t input_val = input[b * depth + d];
+        const int32_t filter_val = filter[c * depth + d];
+        acc += (filter_val + filter_offset) * (input_val + input_offset);
+      }
+      if (bias) acc += bias[c];
+      acc = Mbqm(acc, multiplier, shift);
+      acc += output_offset;
+      acc = std::max(acc, act_min);
+      acc = std::min(acc, act_max);
+      output[c + out_depth * b] = static_cast<uint8_t>(acc);
+    }
+  }
+}
+
+int orc_activation_range_uint8(int activation, float out_scale, int32_t out_zero_point,
+                               int32_t* act_min, int32_t* act_max) {
+  const int32_t qmin = 0, qmax = 255;
+  int32_t q;
+  if (activation == ORC_ACT_RELU) {
+    if (!QuantizeForRange(out_scale, out_zero_point, 0.0f, &q)) return 1;
+    *act_min = std::max(qmin, q);
+    *act_max = qmax;
+  } else if (activation == ORC_ACT_RELU6) {
+    if (!QuantizeForRange(out_scale, out_zero_point, 0.0f, &q)) return 1;
+    *act_min = std::max(qmin, q);
+    if (!QuantizeForRange(out_scale, out_zero_point, 6.0f, &q)) return 1;
+    *act_max = std::min(qmax, q);
+  } else if (activation == ORC_ACT_RELU_N1_TO_1) {
+    if (!QuantizeForRange(out_scale, out_zero_point, -1.0f, &q)) return 1;
+    *act_min = std::max(qmin, q);
+    if (!QuantizeForRange(out_scale, out_zero_point, 1.0f, &q)) return 1;
+    *act_max = std::min(qmax, q);
+  } else {
+    *act_min = qmin;
+    *act_max = qmax;
+  }
+  return 0;
+}
+
 void orc_fc_int8_per_tensor_float_scale(const int8_t* input, const int8_t* filter,
                                         const int32_t* bias, float input_scale,
                                         float filter_scale, float output_scale, int8_t* output,

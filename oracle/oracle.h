@@ -122,6 +122,20 @@ void orc_fc_int8_per_tensor(const int8_t* input, const int8_t* filter, const int
                             int out_depth, int32_t input_offset, int32_t filter_offset,
                             int32_t output_offset, int32_t act_min, int32_t act_max);
 
+/* The legacy uint8 kernel, tflite/kernels/internal/reference/fully_connected.h:118-166
+ * (multiplier form: what the op computes unless built with the reference kernel type, whose
+ * float-scale form :68-116 the reference's test vectors do not tell apart). Offsets are the
+ * negated zero points of the uint8 tensors. */
+void orc_fc_uint8_per_tensor(const uint8_t* input, const uint8_t* filter, const int32_t* bias,
+                             int32_t multiplier, int shift, uint8_t* output, int batches, int depth,
+                             int out_depth, int32_t input_offset, int32_t filter_offset,
+                             int32_t output_offset, int32_t act_min, int32_t act_max);
+
+/* CalculateActivationRangeQuantized for a uint8 output (kernel_util.cc:354-412 with the limits
+ * 0 and 255). Returns 1 where the quantized bound leaves int32. */
+int orc_activation_range_uint8(int activation, float out_scale, int32_t out_zero_point,
+                               int32_t* act_min, int32_t* act_max);
+
 /* reference/integer_ops/fully_connected.h:186-233 (per-tensor, float-scale form). */
 void orc_fc_int8_per_tensor_float_scale(const int8_t* input, const int8_t* filter,
                                         const int32_t* bias, float input_scale,

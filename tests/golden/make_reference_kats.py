@@ -52,6 +52,25 @@ def per_tensor(source, in_range, out_range, weights, bias, x, units, act="none",
                 output_scale=float(out_s), output_zero_point=int(out_zp))
 
 
+def per_tensor_uint8(source, in_range, out_range, weights, bias, x, units, act="none"):
+    """QuantizedFullyConnectedOpModel with uint8 tensors: a UINT8 filter takes the INPUT's range
+    (fully_connected_test.cc:182-203: no case of its own), every tensor is quantized to 0 .. 255
+    (test_util.h:1123-1190), the bias with input scale x filter scale."""
+    in_s, in_zp = kh.quantization_params(*in_range, 0, 255)
+    out_s, out_zp = kh.quantization_params(*out_range, 0, 255)
+    w_s, w_zp = in_s, in_zp
+    wq = kh.quantize(weights, w_s, w_zp, 0, 255, np.uint8).reshape(units, -1)
+    xq = kh.quantize(x, in_s, in_zp, 0, 255, np.uint8).reshape(-1, wq.shape[1])
+    bias_scale = np.float32(in_s * w_s)
+    bq = None if bias is None else kh.quantize_bias(bias, bias_scale)
+    return dict(source=source, activation=ACT[act], input=xq.tolist(), filter=wq.tolist(),
+                bias=None if bq is None else bq.tolist(),
+                input_scale=float(in_s), input_zero_point=int(in_zp),
+                filter_scale=float(w_s), filter_zero_point=int(w_zp),
+                bias_scale=None if bias is None else float(bias_scale),
+                output_scale=float(out_s), output_zero_point=int(out_zp))
+
+
 def per_channel(source, scales, weights, bias, x, units, depth, act="none", int4=False,
                 int2=False):
     in_s, in_zp = kh.quantization_params(-63.5, 64)
@@ -200,6 +219,22 @@ def main():
         case["expected_output"] = want
         fc.append(case)
 
+    # The legacy uint8 op. The 4-D inputs {4, 1, 5, 1} of :2079-2158 flatten to the same [2, 10].
+    fc_u8 = []
+    for case, want in (
+            (per_tensor_uint8(t + ":674-712", (-63.5, 64), (-127, 128), W10 * 3, [1, 2, 3], X2, 3, "relu"),
+             [151, 152, 153, 185, 186, 187]),
+            (per_tensor_uint8(t + ":714-752", (-63.5, 64), (-127, 128), W10 * 3, None, X2, 3, "relu"),
+             [150, 150, 150, 184, 184, 184]),
+            (per_tensor_uint8(t + ":1489-1528", (-127, 128), (-63.5, 64), W10 * 3, [1, 2, 3], X2, 3, "relu"),
+             [175, 177, 179, 243, 245, 247]),
+            (per_tensor_uint8(t + ":2079-2117", (-63.5, 64), (-127, 128), W10 * 3, [1, 2, 3], X2, 3, "relu"),
+             [151, 152, 153, 185, 186, 187]),
+            (per_tensor_uint8(t + ":2119-2158", (-127, 128), (-63.5, 64), W10 * 3, [1, 2, 3], X2, 3, "relu"),
+             [175, 177, 179, 243, 245, 247])):
+        case["expected_output"] = want
+        fc_u8.append(case)
+
     u = "tflite/kernels/internal/tensor_utils_test.cc"
     a = [-640, -635.0, -630, 10.0, 2.0, -5.0, -10.0, 0.0, 1000.0]
     small = [-1e-5, 3e-5, -7e-6, -9e-5, 1e-6, 4e-5, 9e-6, 2e-4, 0]
@@ -254,7 +289,8 @@ def main():
 
     lookups = embedding_lookup_cases()
 
-    out = dict(embedding_lookup=lookups, fully_connected_int8=fc, batch_quantize_floats=quantize,
+    out = dict(embedding_lookup=lookups, fully_connected_int8=fc, fully_connected_uint8=fc_u8,
+               batch_quantize_floats=quantize,
                quantize_multiplier=multiplier, multiply_by_quantized_multiplier=mbqm,
                hybrid_dot_per_channel=hybrid_dot,
                batch_matmul_hybrid=batch_matmul_hybrid_cases(),

@@ -52,8 +52,15 @@ def test_claim_predicate_int8():
         for act in (0, 1, 2, 3):
             assert h.classify(_int8_node(h, activation=act))[0] == "int8"
         # declined: left to the CPU kernels
+        # the legacy uint8 op: per-tensor only, claimed (it runs on the int8 kernels, value - 128)
+        assert h.classify(_int8_node(h, in_type=UINT8, out_type=UINT8, filter_type=UINT8,
+                                     per_channel=False, w_zp=131))[0] == "int8"
         assert h.classify(_int8_node(h, in_type=UINT8, out_type=UINT8, filter_type=UINT8)) == (
-            None, "tensor type combination not handled")
+            None, "uint8 filter is not per-tensor")
+        assert h.classify(_int8_node(h, in_type=UINT8, out_type=UINT8, filter_type=UINT8,
+                                     per_channel=False, activation=4)) == (None, "activation not a clamp")
+        assert h.classify(_int8_node(h, in_type=UINT8, out_type=INT8, filter_type=UINT8,
+                                     per_channel=False)) == (None, "tensor type combination not handled")
         assert h.classify(_int8_node(h, in_type=INT16, out_type=INT16))[0] is None
         assert h.classify(_int8_node(h, const_filter=False)) == (None, "filter is not a constant tensor")
         assert h.classify(_int8_node(h, weights_format=1)) == (None, "shuffled weights format")

@@ -102,6 +102,58 @@ def test_oracle_fully_connected_int8(case):
     assert _oracle_fc(case).ravel().tolist() == case["expected_output"]
 
 
+def _uint8_case(case):
+    x = np.array(case["input"], np.uint8)
+    w = np.array(case["filter"], np.uint8)
+    bias = None if case["bias"] is None else np.array(case["bias"], np.int32)
+    return x, w, bias
+
+
+@pytest.mark.parametrize("case", KATS["fully_connected_uint8"],
+                         ids=lambda c: c["source"].split(":", 1)[1])
+def test_oracle_fully_connected_uint8(case):
+    """The legacy uint8 op's vectors (the same for every kernel type the reference's test is
+    instantiated with), and the change of representation the HIP path rests on: the int8 oracle on
+    the tensors taken as value - 128, every zero point lowered by 128, gives the same bytes + 128."""
+    x, w, bias = _uint8_case(case)
+    m, s = oracle.fc_prepare_per_tensor(case["input_scale"], case["filter_scale"],
+                                        case["output_scale"], case["bias_scale"])
+    lo, hi = oracle.activation_range_uint8(case["activation"], case["output_scale"],
+                                           case["output_zero_point"])
+    got = oracle.fc_uint8_per_tensor(x, w, bias, m, s, -case["input_zero_point"],
+                                     -case["filter_zero_point"], case["output_zero_point"], lo, hi)
+    assert got.ravel().tolist() == case["expected_output"]
+    lo8, hi8 = oracle.activation_range_int8(case["activation"], case["output_scale"],
+                                            case["output_zero_point"] - 128)
+    assert (lo8, hi8) == (lo - 128, hi - 128)
+    moved = oracle.fc_int8_per_tensor((x ^ 0x80).view(np.int8), (w ^ 0x80).view(np.int8), bias, m, s,
+                                      -(case["input_zero_point"] - 128),
+                                      -(case["filter_zero_point"] - 128),
+                                      case["output_zero_point"] - 128, lo8, hi8)
+    assert np.array_equal(moved.view(np.uint8) ^ 0x80, got)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_oracle_uint8_equals_int8_on_moved_tensors(seed):
+    """The same identity on random tensors, zero points and activations (clamps that bite)."""
+    rng = np.random.default_rng(seed)
+    B, K, N = int(rng.integers(1, 5)), int(rng.integers(1, 70)), int(rng.integers(1, 9))
+    x = rng.integers(0, 256, (B, K)).astype(np.uint8)
+    w = rng.integers(0, 256, (N, K)).astype(np.uint8)
+    bias = rng.integers(-2000, 2000, N).astype(np.int32)
+    zx, zw, zy = (int(v) for v in rng.integers(0, 256, 3))
+    in_s, w_s, out_s = 0.02, 0.01, float(rng.uniform(0.05, 0.5))
+    m, s = oracle.fc_prepare_per_tensor(in_s, w_s, out_s, None)
+    act = int(rng.integers(0, 4))
+    lo, hi = oracle.activation_range_uint8(act, out_s, zy)
+    lo8, hi8 = oracle.activation_range_int8(act, out_s, zy - 128)
+    assert (lo8, hi8) == (lo - 128, hi - 128)
+    got = oracle.fc_uint8_per_tensor(x, w, bias, m, s, -zx, -zw, zy, lo, hi)
+    moved = oracle.fc_int8_per_tensor((x ^ 0x80).view(np.int8), (w ^ 0x80).view(np.int8), bias, m, s,
+                                      -(zx - 128), -(zw - 128), zy - 128, lo8, hi8)
+    assert np.array_equal(moved.view(np.uint8) ^ 0x80, got)
+
+
 # ---- HIP path through the C ABI (gpu) ----------------------------------------------------------
 
 @pytest.fixture(scope="module")
@@ -131,6 +183,47 @@ def test_hip_fully_connected_int8(fc, case, packed):
         filter_zero_point=case["filter_zero_point"], bias_scale=case["bias_scale"], packed=packed)
     y = op(_cuda(np.array(case["input"], np.int8))).cpu().numpy()
     assert y.ravel().tolist() == case["expected_output"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", KATS["fully_connected_uint8"],
+                         ids=lambda c: c["source"].split(":", 1)[1])
+@pytest.mark.parametrize("packed", [True, False])
+def test_hip_fully_connected_uint8(fc, case, packed):
+    x, w, bias = _uint8_case(case)
+    op = fc.FullyConnectedUInt8(w, bias, case["input_scale"], case["input_zero_point"],
+                                case["filter_scale"], case["filter_zero_point"],
+                                case["output_scale"], case["output_zero_point"],
+                                activation=case["activation"], bias_scale=case["bias_scale"],
+                                packed=packed)
+    y = op(_cuda(x)).cpu().numpy()
+    assert y.dtype == np.uint8 and y.ravel().tolist() == case["expected_output"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,K,N,zw", [(1, 64, 40, 128), (4, 1000, 33, 128), (3, 272, 130, 121),
+                                     (40, 512, 72, 128), (130, 96, 300, 7), (2, 17, 5, 255)])
+@pytest.mark.parametrize("activation", [0, 1, 3])
+def test_hip_uint8_shapes_match_oracle(fc, B, K, N, zw, activation):
+    """Filter zero point 128 (0 once moved: the re-tiled filter, GEMV and GEMM) and other values
+    (the row-major kernels), input and output zero points at both ends of the range where the
+    filter is centred."""
+    rng = np.random.default_rng(B + K + N + zw)
+    x = rng.integers(0, 256, (B, K)).astype(np.uint8)
+    w = rng.integers(0, 256, (N, K)).astype(np.uint8)
+    bias = rng.integers(-5000, 5000, N).astype(np.int32)
+    # one of the two factors stays centred, or every sum lands beyond a clamp
+    zx, zy = (127, 130) if zw != 128 else ((0, 255) if (B + N) % 2 else (250, 3))
+    in_s, w_s = 0.02, 0.01
+    out_s = float(0.02 * 0.01 * np.sqrt(K) * 60)
+    op = fc.FullyConnectedUInt8(w, bias, in_s, zx, w_s, zw, out_s, zy, activation=activation)
+    y = op(_cuda(x)).cpu().numpy()
+    m, s = oracle.fc_prepare_per_tensor(in_s, w_s, out_s, None)
+    lo, hi = oracle.activation_range_uint8(activation, out_s, zy)
+    want = oracle.fc_uint8_per_tensor(x, w, bias, m, s, -zx, -zw, zy, lo, hi)
+    assert np.array_equal(y, want)
+    if activation == 0:  # (a ReLU under an output zero point of 255 leaves one value: 255)
+        assert len(np.unique(want)) > 3
 
 
 @pytest.mark.gpu

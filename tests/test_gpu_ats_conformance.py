@@ -1,7 +1,9 @@
 """The full-integer FULLY_CONNECTED cases of the reference's accelerator test suite, restated:
 `litert/ats/register_fully_connected.cc:103-124` registers rank {2, 3} x keep_num_dims x
-{NONE, RELU} x bias x per-channel for int8 (the uint8 and shuffled-weights columns are nodes this
-delegate declines, see test_delegate_cpu.py), and `litert/test/generators/fully_connected.h`
+{NONE, RELU} x bias x per-channel for int8 and for uint8 (the shuffled-weights column and
+per-channel uint8 filters, which the builtin's Prepare refuses too (fully_connected.cc:528-531),
+are nodes this delegate declines, see test_delegate_cpu.py), and
+`litert/test/generators/fully_connected.h`
 builds each case: every dimension drawn from [2, 6] (:107-117), weights all 1 and bias all 0
 (:122-123), every scale 0.01 with zero point 0 (:344-395), inputs uniform over int8. The suite's
 own reference is a float FULLY_CONNECTED on the raw integers, times 0.01, cast to int8
@@ -17,7 +19,7 @@ import numpy as np
 import pytest
 
 import oracle
-from tests.fake_host import FakeHost, INT32, INT8, OK
+from tests.fake_host import FakeHost, INT32, INT8, UINT8, OK
 
 pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
@@ -33,8 +35,8 @@ def _need_gpu():
         pytest.fail("GPU tests need a gfx950 device; none visible")
 
 
-def _suite_reference(x, w, bias, activation):
-    """ReferenceFullyConnected on the integers as floats, scaled by 0.01, cast to int8."""
+def _suite_reference(x, w, bias, activation, dtype=np.int8):
+    """ReferenceFullyConnected on the integers as floats, scaled by 0.01, cast to the output type."""
     B = int(np.prod(x.shape[:-1]))
     xf = x.reshape(B, -1).astype(np.float32)
     wf = w.astype(np.float32)
@@ -47,7 +49,7 @@ def _suite_reference(x, w, bias, activation):
             out[b, o] = s
     if activation == RELU:
         out = np.maximum(out, np.float32(0))
-    return np.trunc(out * np.float32(SCALE)).astype(np.int8)
+    return np.trunc(out * np.float32(SCALE)).astype(dtype)
 
 
 CASES = list(itertools.product((2, 3), (False, True), (NONE, RELU), (False, True), (False, True)))
@@ -99,4 +101,50 @@ def test_int8_cases_of_the_accelerator_suite(rank, keep_num_dims, activation, ha
                                                        BIAS_SCALE if has_bias else None)
             lo, hi = oracle.activation_range_int8(activation, SCALE, 0)
             want = oracle.fc_int8_per_tensor(x.reshape(B, K), w, bias, mult, shift, 0, 0, 0, lo, hi)
+        assert np.array_equal(got, want), (in_shape, N)
+
+
+UINT8_CASES = list(itertools.product((2, 3), (False, True), (NONE, RELU), (False, True)))
+
+
+@pytest.mark.parametrize("rank,keep_num_dims,activation,has_bias", UINT8_CASES)
+def test_uint8_cases_of_the_accelerator_suite(rank, keep_num_dims, activation, has_bias):
+    """The suite's uint8 column with a per-tensor filter: inputs uniform over uint8, zero points 0."""
+    seed = 100 + sum(int(v) << i for i, v in enumerate((rank, keep_num_dims, activation, has_bias)))
+    rng = np.random.default_rng(seed)
+    for _ in range(3):
+        dims = rng.integers(2, 7, size=rank + 1)
+        in_shape = tuple(int(d) for d in dims[:rank])
+        K, N = in_shape[-1], int(dims[rank])
+        B = int(np.prod(in_shape[:-1]))
+        x = rng.integers(0, 256, in_shape).astype(np.uint8)
+        w = np.ones((N, K), np.uint8)
+        bias = np.zeros(N, np.int32) if has_bias else None
+        out_shape = in_shape[:-1] + (N,) if keep_num_dims else (B, N)
+        with FakeHost() as h:
+            xt = h.tensor(UINT8, in_shape, data=x)
+            h.affine(xt, [SCALE], [0])
+            wt = h.tensor(UINT8, (N, K), data=w, const=True)
+            h.affine(wt, [SCALE])
+            bt = None
+            if has_bias:
+                bt = h.tensor(INT32, (N,), data=bias, const=True)
+                h.affine(bt, [BIAS_SCALE])
+            yt = h.tensor(UINT8, out_shape)
+            h.affine(yt, [SCALE], [0])
+            node = h.fc(xt, wt, bt, yt, activation=activation, keep_num_dims=keep_num_dims)
+            assert h.classify(node)[0] == "int8"
+            assert h.load_delegate() == 0, h.errors()
+            assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+            assert h.plan()[0][:2] == ("delegate", [node])
+            assert h.invoke() == OK, h.errors()
+            got = h.read(yt)
+        assert got.shape == out_shape and got.dtype == np.uint8
+        got = got.reshape(B, N)
+        ref = _suite_reference(x, w, bias, activation, np.uint8)
+        assert np.abs(got.astype(np.int64) - ref.astype(np.int64)).max() <= 1, (in_shape, N)
+        mult, shift = oracle.fc_prepare_per_tensor(SCALE, SCALE, SCALE,
+                                                   BIAS_SCALE if has_bias else None)
+        lo, hi = oracle.activation_range_uint8(activation, SCALE, 0)
+        want = oracle.fc_uint8_per_tensor(x.reshape(B, K), w, bias, mult, shift, 0, 0, 0, lo, hi)
         assert np.array_equal(got, want), (in_shape, N)

@@ -500,6 +500,58 @@ def test_int2_filter_runs_the_int8_paths_after_unpacking(B, N, K, per_channel):
         assert np.array_equal(h.read(y), _oracle_int8(c2, c["x"], activation=1))
 
 
+def _uint8_fc(h, rng, x, B, K, N, in_s, zx, w_s, zw, out_s, zy, activation=0, bias=True):
+    """Adds a uint8 FULLY_CONNECTED node reading tensor `x`; returns (node, output tensor, weights,
+    bias values)."""
+    w_np = rng.integers(0, 256, (N, K)).astype(np.uint8)
+    b_np = rng.integers(-3000, 3000, N).astype(np.int32) if bias else None
+    w = h.tensor(UINT8, (N, K), data=w_np, const=True)
+    h.affine(w, [w_s], [zw])
+    b = None
+    if bias:
+        b = h.tensor(INT32, (N,), data=b_np, const=True)
+        h.affine(b, [np.float32(in_s) * np.float32(w_s)])
+    y = h.tensor(UINT8, (B, N))
+    h.affine(y, [out_s], [zy])
+    return h.fc(x, w, b, y, activation=activation), y, w_np, b_np
+
+
+def _oracle_uint8(x, w, bias, in_s, zx, w_s, zw, out_s, zy, activation=0):
+    m, s = oracle.fc_prepare_per_tensor(in_s, w_s, out_s, None)
+    lo, hi = oracle.activation_range_uint8(activation, out_s, zy)
+    return oracle.fc_uint8_per_tensor(x, w, bias, m, s, -zx, -zw, zy, lo, hi)
+
+
+@pytest.mark.parametrize("options", [{}, {"direct_inputs": "0", "completion": "sync"}],
+                         ids=["default", "copied,sync"])
+@pytest.mark.parametrize("B,K,N,zw", [(1, 4096, 2048, 128), (5, 272, 130, 119), (40, 512, 72, 128)])
+def test_uint8_nodes_through_delegate(B, K, N, zw, options):
+    """The legacy uint8 op, one node and a chain of two whose link stays on the device as uint8:
+    filter zero point 128 (the re-tiled filter once the tensors are taken as int8) and another
+    (the row-major kernels), decode and prefill batches, a second invoke on new rows."""
+    rng = np.random.default_rng(B + K + N)
+    x_np = rng.integers(0, 256, (B, K)).astype(np.uint8)
+    in_s, w_s, zx = 0.02, 0.01, 131
+    s1 = float(in_s * w_s * np.sqrt(K) * 60)
+    s2 = float(s1 * 0.01 * np.sqrt(N) * 60)
+    with FakeHost() as h:
+        x = h.tensor(UINT8, (B, K), data=x_np)
+        h.affine(x, [in_s], [zx])
+        n1, y1, w1, b1 = _uint8_fc(h, rng, x, B, K, N, in_s, zx, w_s, zw, s1, 7, activation=1)
+        n2, y2, w2, b2 = _uint8_fc(h, rng, y1, B, N, 24, s1, 7, 0.01, 128, s2, 200, bias=False)
+        assert h.classify(n1)[0] == "int8" and h.classify(n2)[0] == "int8"
+        assert h.load_delegate(options) == 0, h.errors()
+        assert h.modify_graph_with_delegate() == OK and h.allocate_tensors() == OK, h.errors()
+        assert h.plan()[0][:2] == ("delegate", [n1, n2])
+        for rows in (x_np, np.roll(x_np, 5, axis=1)):
+            h.write(x, rows)
+            assert h.invoke() == OK, h.errors()
+            t = _oracle_uint8(rows, w1, b1, in_s, zx, w_s, zw, s1, 7, activation=1)
+            want = _oracle_uint8(t, w2, None, s1, 7, 0.01, 128, s2, 200)
+            assert np.array_equal(h.read(y2), want)
+            assert len(np.unique(want)) > 3
+
+
 def test_int4_per_channel_node_switches_layout_with_the_batch():
     """Decode batches run on the filter kept as nibbles, prefill batches on its int8 expansion;
     a resize moves the node from one to the other and back (prepare runs after every resize)."""
