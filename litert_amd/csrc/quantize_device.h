@@ -232,15 +232,19 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   // Pass 1: range of the row. Starting from 0 gives min(0, min v) / max(0, max v),
   // which is also what max(|min|, |max|) needs for the symmetric case.
   float mn = 0.0f, mx = 0.0f;
-  // Rows of up to kRowRegs * kQuantizeThreads * 4 values stay in registers between the two
-  // passes instead of being read again.
-  constexpr int kRowRegs = 4;
+  // Rows of up to kRowRegs * kQuantizeThreads * 4 values (16384) stay in registers between the
+  // two passes instead of being read again, and all their loads are in flight at once: a deep
+  // row read in a loop, twice, is a chain of memory latencies on the one workgroup that has it
+  // (4 rows of depth 16384 for each of 18 filters: 10 us and more, where this form takes 3).
+  // Steps past the row's end are skipped as a whole (the test is uniform).
+  constexpr int kRowRegs = 16;
   const bool in_regs = vec_ok && n_data / 4 <= kRowRegs * kQuantizeThreads;
   float4 held[kRowRegs];
   if (in_regs) {
     const float4* v4 = reinterpret_cast<const float4*>(v);
 #pragma unroll
     for (int j = 0; j < kRowRegs; ++j) {
+      if (j * kQuantizeThreads >= n_data / 4) break;
       const int i = threadIdx.x + j * kQuantizeThreads;
       // Past the end: zeros, which the range (it always includes 0) does not notice.
       const float4 t = i < n_data / 4 ? v4[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -301,6 +305,7 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   if (in_regs) {
 #pragma unroll
     for (int j = 0; j < kRowRegs; ++j) {
+      if (j * kQuantizeThreads >= n_data / 4) break;
       const int i = threadIdx.x + j * kQuantizeThreads;
       if (i < n_data / 4) emit4(i, held[j]);
     }
