@@ -234,23 +234,38 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   float mn = 0.0f, mx = 0.0f;
   // Rows of up to kRowRegs * kQuantizeThreads * 4 values (16384) stay in registers between the
   // two passes instead of being read again, and all their loads are in flight at once: a deep
-  // row read in a loop, twice, is a chain of memory latencies on the one workgroup that has it
-  // (4 rows of depth 16384 for each of 18 filters: 10 us and more, where this form takes 3).
-  // Steps past the row's end are skipped as a whole (the test is uniform).
-  constexpr int kRowRegs = 16;
-  const bool in_regs = vec_ok && n_data / 4 <= kRowRegs * kQuantizeThreads;
+  // row read in a loop, twice, is a chain of memory latencies on the one workgroup that has it.
+  // The loads of a row stand in ONE basic block (no test between them, or the compiler waits for
+  // each before it issues the next); rows of up to 4096 values take a block of four.
+  constexpr int kRowRegs = 16, kShortRegs = 4;
+  const int n4 = n_data / 4;
+  const bool in_regs = vec_ok && n4 <= kRowRegs * kQuantizeThreads;
+  const bool short_row = n4 <= kShortRegs * kQuantizeThreads;
   float4 held[kRowRegs];
   if (in_regs) {
     const float4* v4 = reinterpret_cast<const float4*>(v);
-#pragma unroll
-    for (int j = 0; j < kRowRegs; ++j) {
-      if (j * kQuantizeThreads >= n_data / 4) break;
+    // Past the end: the row's last piece again (an unconditional load), then taken as zeros, which
+    // the range (it always includes 0) does not notice.
+    auto take = [&](int j) {
       const int i = threadIdx.x + j * kQuantizeThreads;
-      // Past the end: zeros, which the range (it always includes 0) does not notice.
-      const float4 t = i < n_data / 4 ? v4[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      held[j] = t;
+      held[j] = v4[min(i, n4 - 1)];
+    };
+    auto widen = [&](int j) {
+      const int i = threadIdx.x + j * kQuantizeThreads;
+      const float4 t = i < n4 ? held[j] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
       mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
       mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
+    };
+    if (short_row) {
+#pragma unroll
+      for (int j = 0; j < kShortRegs; ++j) take(j);
+#pragma unroll
+      for (int j = 0; j < kShortRegs; ++j) widen(j);
+    } else {
+#pragma unroll
+      for (int j = 0; j < kRowRegs; ++j) take(j);
+#pragma unroll
+      for (int j = 0; j < kRowRegs; ++j) widen(j);
     }
   } else if (vec_ok) {
     const float4* v4 = reinterpret_cast<const float4*>(v);
@@ -303,11 +318,18 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
     *reinterpret_cast<char4*>(q + place(4 * i)) = o;
   };
   if (in_regs) {
+    if (short_row) {
 #pragma unroll
-    for (int j = 0; j < kRowRegs; ++j) {
-      if (j * kQuantizeThreads >= n_data / 4) break;
-      const int i = threadIdx.x + j * kQuantizeThreads;
-      if (i < n_data / 4) emit4(i, held[j]);
+      for (int j = 0; j < kShortRegs; ++j) {
+        const int i = threadIdx.x + j * kQuantizeThreads;
+        if (i < n4) emit4(i, held[j]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kRowRegs; ++j) {
+        const int i = threadIdx.x + j * kQuantizeThreads;
+        if (i < n4) emit4(i, held[j]);
+      }
     }
   } else if (vec_ok) {
     const float4* v4 = reinterpret_cast<const float4*>(v);
