@@ -732,13 +732,14 @@ __global__ __launch_bounds__(kThreads) void FcInt4NibbleQuadGroupedKernel(
 
 // Workgroup r quantizes row r % batches of node r / batches into that node's workspace
 // (EvalBlockwise4Bit always quantizes asymmetrically, fully_connected.cc:1044-1047).
-template <int VARIANT>
-__global__ __launch_bounds__(kQuantizeThreads) void QuantizeNibbleGroupRowsKernel(
+template <int VARIANT, int THREADS = kQuantizeThreads>
+__global__ __launch_bounds__(THREADS) void QuantizeNibbleGroupRowsKernel(
     const NibbleQuadGroupTable* __restrict__ table, int batches) {
   const int node = blockIdx.x / batches;
   const int row = blockIdx.x - node * batches;
   const NibbleQuadArgs& a = table->node[node];
-  QuantizeRow<VARIANT>(table->input_f32[node] + static_cast<size_t>(row) * a.depth, a.depth,
+  QuantizeRow<VARIANT, RowMajorPlacement, THREADS>(
+                       table->input_f32[node] + static_cast<size_t>(row) * a.depth, a.depth,
                        const_cast<int8_t*>(a.rows) + static_cast<size_t>(row) * a.depth,
                        const_cast<float*>(a.scaling_factors) + row,
                        const_cast<int32_t*>(a.zero_points) + row, /*do_asymmetric=*/1);
@@ -1037,19 +1038,21 @@ hipError_t LaunchFcInt4NibbleGrouped(const void* table, const lrtfc_int4_group_l
                                      int variant, hipStream_t stream) {
   if (l.count < 1 || l.grid_blocks < 1) return hipSuccess;
   const auto* t = static_cast<const NibbleQuadGroupTable*>(table);
-  const dim3 qgrid(static_cast<unsigned>(l.count) * l.batches), qblock(kQuantizeThreads);
+  // This form serves groups deeper than 8192 only: the wide row quantizer.
+  const dim3 qgrid(static_cast<unsigned>(l.count) * l.batches), qblock(kQuantizeDeepThreads);
   switch (variant) {
     case LRTFC_QUANT_NEON_V8:
-      hipLaunchKernelGGL(QuantizeNibbleGroupRowsKernel<LRTFC_QUANT_NEON_V8>, qgrid, qblock, 0,
-                         stream, t, l.batches);
+      hipLaunchKernelGGL((QuantizeNibbleGroupRowsKernel<LRTFC_QUANT_NEON_V8, kQuantizeDeepThreads>),
+                         qgrid, qblock, 0, stream, t, l.batches);
       break;
     case LRTFC_QUANT_NEON_LEGACY:
-      hipLaunchKernelGGL(QuantizeNibbleGroupRowsKernel<LRTFC_QUANT_NEON_LEGACY>, qgrid, qblock, 0,
-                         stream, t, l.batches);
+      hipLaunchKernelGGL(
+          (QuantizeNibbleGroupRowsKernel<LRTFC_QUANT_NEON_LEGACY, kQuantizeDeepThreads>), qgrid,
+          qblock, 0, stream, t, l.batches);
       break;
     default:
-      hipLaunchKernelGGL(QuantizeNibbleGroupRowsKernel<LRTFC_QUANT_PORTABLE>, qgrid, qblock, 0,
-                         stream, t, l.batches);
+      hipLaunchKernelGGL((QuantizeNibbleGroupRowsKernel<LRTFC_QUANT_PORTABLE, kQuantizeDeepThreads>),
+                         qgrid, qblock, 0, stream, t, l.batches);
       break;
   }
   if (hipError_t err = hipGetLastError()) return err;

@@ -656,13 +656,14 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedGroupedKernel(
 // The row quantizer for a whole group: workgroup r quantizes row r % batches of node
 // r / batches into that node's workspace (EvalBlockwise4Bit always quantizes asymmetrically,
 // tflite/kernels/fully_connected.cc:1044-1047).
-template <int VARIANT>
-__global__ __launch_bounds__(kQuantizeThreads) void QuantizeGroupRowsKernel(
+template <int VARIANT, int THREADS = kQuantizeThreads>
+__global__ __launch_bounds__(THREADS) void QuantizeGroupRowsKernel(
     const Int4GroupTable* __restrict__ table, int batches) {
   const int node = blockIdx.x / batches;
   const int row = blockIdx.x - node * batches;
   const Int4PackedArgs& a = table->node[node];
-  QuantizeRow<VARIANT>(a.input_f32 + static_cast<size_t>(row) * a.depth, a.depth,
+  QuantizeRow<VARIANT, RowMajorPlacement, THREADS>(
+                       a.input_f32 + static_cast<size_t>(row) * a.depth, a.depth,
                        const_cast<int8_t*>(a.input_q) + static_cast<size_t>(row) * a.depth,
                        const_cast<float*>(a.scaling_factors) + row,
                        const_cast<int32_t*>(a.zero_points) + row, /*do_asymmetric=*/1);
@@ -954,19 +955,27 @@ hipError_t LaunchGroupedVariant(const void* table, const lrtfc_int4_group_launch
 hipError_t LaunchGroupQuantizer(const void* table, const lrtfc_int4_group_launch& l, int variant,
                                 hipStream_t stream) {
   const auto* t = static_cast<const Int4GroupTable*>(table);
-  const dim3 grid(static_cast<unsigned>(l.count) * l.batches), block(kQuantizeThreads);
+  const dim3 grid(static_cast<unsigned>(l.count) * l.batches);
+  const bool deep = l.depth > kQuantizeDeepRow;
+  auto launch = [&](auto narrow, auto wide) {
+    if (deep) {
+      hipLaunchKernelGGL(wide, grid, dim3(kQuantizeDeepThreads), 0, stream, t, l.batches);
+    } else {
+      hipLaunchKernelGGL(narrow, grid, dim3(kQuantizeThreads), 0, stream, t, l.batches);
+    }
+  };
   switch (variant) {
     case LRTFC_QUANT_NEON_V8:
-      hipLaunchKernelGGL(QuantizeGroupRowsKernel<LRTFC_QUANT_NEON_V8>, grid, block, 0, stream, t,
-                         l.batches);
+      launch(QuantizeGroupRowsKernel<LRTFC_QUANT_NEON_V8>,
+             QuantizeGroupRowsKernel<LRTFC_QUANT_NEON_V8, kQuantizeDeepThreads>);
       break;
     case LRTFC_QUANT_NEON_LEGACY:
-      hipLaunchKernelGGL(QuantizeGroupRowsKernel<LRTFC_QUANT_NEON_LEGACY>, grid, block, 0, stream,
-                         t, l.batches);
+      launch(QuantizeGroupRowsKernel<LRTFC_QUANT_NEON_LEGACY>,
+             QuantizeGroupRowsKernel<LRTFC_QUANT_NEON_LEGACY, kQuantizeDeepThreads>);
       break;
     default:
-      hipLaunchKernelGGL(QuantizeGroupRowsKernel<LRTFC_QUANT_PORTABLE>, grid, block, 0, stream, t,
-                         l.batches);
+      launch(QuantizeGroupRowsKernel<LRTFC_QUANT_PORTABLE>,
+             QuantizeGroupRowsKernel<LRTFC_QUANT_PORTABLE, kQuantizeDeepThreads>);
       break;
   }
   return hipGetLastError();

@@ -10,14 +10,15 @@ namespace {
 
 constexpr int kThreads = kQuantizeThreads;
 
-template <int VARIANT>
-__global__ __launch_bounds__(kThreads) void BatchQuantizeKernel(
+template <int VARIANT, int THREADS = kThreads>
+__global__ __launch_bounds__(THREADS) void BatchQuantizeKernel(
     const float* __restrict__ values, int n_data, int8_t* __restrict__ quantized,
     float* __restrict__ scaling_factors, int32_t* __restrict__ zero_points, int do_asymmetric) {
   const int row = blockIdx.x;
-  QuantizeRow<VARIANT>(values + static_cast<size_t>(row) * n_data, n_data,
-                       quantized + static_cast<size_t>(row) * n_data, scaling_factors + row,
-                       zero_points ? zero_points + row : nullptr, do_asymmetric);
+  QuantizeRow<VARIANT, RowMajorPlacement, THREADS>(
+      values + static_cast<size_t>(row) * n_data, n_data,
+      quantized + static_cast<size_t>(row) * n_data, scaling_factors + row,
+      zero_points ? zero_points + row : nullptr, do_asymmetric);
 }
 
 // The row quantizer of the per-channel int4 hybrid path (ReferenceBatchQuantizeFloats4Bit,
@@ -109,19 +110,29 @@ hipError_t LaunchBatchQuantize(const float* values, int n_batch, int n_data, int
                                float* scaling_factors, int32_t* zero_points, int do_asymmetric,
                                int variant, hipStream_t stream) {
   if (n_batch == 0 || n_data == 0) return hipSuccess;
-  const dim3 grid(n_batch), block(kThreads);
+  const dim3 grid(n_batch);
+  const bool deep = n_data > kQuantizeDeepRow;
+  auto launch = [&](auto narrow, auto wide) {
+    if (deep) {
+      hipLaunchKernelGGL(wide, grid, dim3(kQuantizeDeepThreads), 0, stream, values, n_data, quantized,
+                         scaling_factors, zero_points, do_asymmetric);
+    } else {
+      hipLaunchKernelGGL(narrow, grid, dim3(kThreads), 0, stream, values, n_data, quantized,
+                         scaling_factors, zero_points, do_asymmetric);
+    }
+  };
   switch (variant) {
     case LRTFC_QUANT_NEON_V8:
-      hipLaunchKernelGGL(BatchQuantizeKernel<LRTFC_QUANT_NEON_V8>, grid, block, 0, stream, values,
-                         n_data, quantized, scaling_factors, zero_points, do_asymmetric);
+      launch(BatchQuantizeKernel<LRTFC_QUANT_NEON_V8>,
+             BatchQuantizeKernel<LRTFC_QUANT_NEON_V8, kQuantizeDeepThreads>);
       break;
     case LRTFC_QUANT_NEON_LEGACY:
-      hipLaunchKernelGGL(BatchQuantizeKernel<LRTFC_QUANT_NEON_LEGACY>, grid, block, 0, stream,
-                         values, n_data, quantized, scaling_factors, zero_points, do_asymmetric);
+      launch(BatchQuantizeKernel<LRTFC_QUANT_NEON_LEGACY>,
+             BatchQuantizeKernel<LRTFC_QUANT_NEON_LEGACY, kQuantizeDeepThreads>);
       break;
     default:
-      hipLaunchKernelGGL(BatchQuantizeKernel<LRTFC_QUANT_PORTABLE>, grid, block, 0, stream,
-                         values, n_data, quantized, scaling_factors, zero_points, do_asymmetric);
+      launch(BatchQuantizeKernel<LRTFC_QUANT_PORTABLE>,
+             BatchQuantizeKernel<LRTFC_QUANT_PORTABLE, kQuantizeDeepThreads>);
       break;
   }
   return hipGetLastError();

@@ -191,10 +191,17 @@ struct RowRange {
   float mx;
 };
 
+// Rows deeper than kQuantizeDeepRow are given a workgroup of kQuantizeDeepThreads threads by the
+// launchers: four loads, one row's worth of vector work per wavefront a quarter as long, where the
+// narrow workgroup spends 7 us on a row of 16384 (one latency chain on one compute unit).
+constexpr int kQuantizeDeepThreads = 1024;
+constexpr int kQuantizeDeepRow = 4096;
+
 // Block-wide min and max. Every thread returns the same pair.
+template <int THREADS = kQuantizeThreads>
 __device__ __forceinline__ RowRange BlockMinMax(float mn, float mx) {
-  __shared__ float s_min[kQuantizeThreads / kWaveSize];
-  __shared__ float s_max[kQuantizeThreads / kWaveSize];
+  __shared__ float s_min[THREADS / kWaveSize];
+  __shared__ float s_max[THREADS / kWaveSize];
   mn = WaveMinF32(mn);
   mx = WaveMaxF32(mx);
   const int wave = threadIdx.x / kWaveSize;
@@ -205,7 +212,7 @@ __device__ __forceinline__ RowRange BlockMinMax(float mn, float mx) {
   __syncthreads();
   RowRange r{s_min[0], s_max[0]};
 #pragma unroll
-  for (int w = 1; w < kQuantizeThreads / kWaveSize; ++w) {
+  for (int w = 1; w < THREADS / kWaveSize; ++w) {
     r.mn = fminf(r.mn, s_min[w]);
     r.mx = fmaxf(r.mx, s_max[w]);
   }
@@ -218,9 +225,9 @@ struct RowMajorPlacement {
   __device__ __forceinline__ size_t operator()(int i) const { return static_cast<size_t>(i); }
 };
 
-// One row through BatchQuantizeFloats by one workgroup of kQuantizeThreads threads: v[n_data]
+// One row through BatchQuantizeFloats by one workgroup of THREADS threads: v[n_data]
 // -> q[place(0 .. n_data-1)], *scaling_factor, *zero_point (may be null).
-template <int VARIANT, typename PLACEMENT = RowMajorPlacement>
+template <int VARIANT, typename PLACEMENT = RowMajorPlacement, int THREADS = kQuantizeThreads>
 __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_data,
                                             int8_t* __restrict__ q,
                                             float* __restrict__ scaling_factor,
@@ -232,26 +239,26 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   // Pass 1: range of the row. Starting from 0 gives min(0, min v) / max(0, max v),
   // which is also what max(|min|, |max|) needs for the symmetric case.
   float mn = 0.0f, mx = 0.0f;
-  // Rows of up to kRowRegs * kQuantizeThreads * 4 values (16384) stay in registers between the
+  // Rows of up to kRowRegs * THREADS * 4 values (16384) stay in registers between the
   // two passes instead of being read again, and all their loads are in flight at once: a deep
   // row read in a loop, twice, is a chain of memory latencies on the one workgroup that has it.
   // The loads of a row stand in ONE basic block (no test between them, or the compiler waits for
   // each before it issues the next); rows of up to 4096 values take a block of four.
-  constexpr int kRowRegs = 16, kShortRegs = 4;
+  constexpr int kRowRegs = THREADS > 256 ? 4 : 16, kShortRegs = 4;
   const int n4 = n_data / 4;
-  const bool in_regs = vec_ok && n4 <= kRowRegs * kQuantizeThreads;
-  const bool short_row = n4 <= kShortRegs * kQuantizeThreads;
+  const bool in_regs = vec_ok && n4 <= kRowRegs * THREADS;
+  const bool short_row = n4 <= kShortRegs * THREADS;
   float4 held[kRowRegs];
   if (in_regs) {
     const float4* v4 = reinterpret_cast<const float4*>(v);
     // Past the end: the row's last piece again (an unconditional load), then taken as zeros, which
     // the range (it always includes 0) does not notice.
     auto take = [&](int j) {
-      const int i = threadIdx.x + j * kQuantizeThreads;
+      const int i = threadIdx.x + j * THREADS;
       held[j] = v4[min(i, n4 - 1)];
     };
     auto widen = [&](int j) {
-      const int i = threadIdx.x + j * kQuantizeThreads;
+      const int i = threadIdx.x + j * THREADS;
       const float4 t = i < n4 ? held[j] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
       mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
       mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
@@ -269,18 +276,18 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
     }
   } else if (vec_ok) {
     const float4* v4 = reinterpret_cast<const float4*>(v);
-    for (int i = threadIdx.x; i < n_data / 4; i += kQuantizeThreads) {
+    for (int i = threadIdx.x; i < n_data / 4; i += THREADS) {
       const float4 t = v4[i];
       mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
       mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
     }
   } else {
-    for (int i = threadIdx.x; i < n_data; i += kQuantizeThreads) {
+    for (int i = threadIdx.x; i < n_data; i += THREADS) {
       mn = fminf(mn, v[i]);
       mx = fmaxf(mx, v[i]);
     }
   }
-  const RowRange range = BlockMinMax(mn, mx);
+  const RowRange range = BlockMinMax<THREADS>(mn, mx);
 
   // Scale and zero point, every thread redundantly (a few dozen flops).
   const RowQuantParams qp = do_asymmetric ? AsymmetricRowParams<VARIANT>(range.mn, range.mx)
@@ -321,21 +328,21 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
     if (short_row) {
 #pragma unroll
       for (int j = 0; j < kShortRegs; ++j) {
-        const int i = threadIdx.x + j * kQuantizeThreads;
+        const int i = threadIdx.x + j * THREADS;
         if (i < n4) emit4(i, held[j]);
       }
     } else {
 #pragma unroll
       for (int j = 0; j < kRowRegs; ++j) {
-        const int i = threadIdx.x + j * kQuantizeThreads;
+        const int i = threadIdx.x + j * THREADS;
         if (i < n4) emit4(i, held[j]);
       }
     }
   } else if (vec_ok) {
     const float4* v4 = reinterpret_cast<const float4*>(v);
-    for (int i = threadIdx.x; i < n_data / 4; i += kQuantizeThreads) emit4(i, v4[i]);
+    for (int i = threadIdx.x; i < n_data / 4; i += THREADS) emit4(i, v4[i]);
   } else {
-    for (int i = threadIdx.x; i < n_data; i += kQuantizeThreads) {
+    for (int i = threadIdx.x; i < n_data; i += THREADS) {
       int8_t o = 0;
       if (!all_zero) {
         const bool tail = i >= vector_end;
