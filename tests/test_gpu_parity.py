@@ -345,6 +345,27 @@ def test_batch_quantize_floats_bit_exact(fc, variant, asym):
         assert np.array_equal(zp.cpu().numpy(), wzp)
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("asym", [True, False])
+def test_batch_quantize_at_and_beside_every_tie(fc, variant, asym):
+    """Rows whose scale is exactly 1 (range [-128, 127], or |max| 127 for the symmetric form), so
+    every element reaches the rounding step unchanged: each k + 0.5, the floats just below and
+    above it, and the float just below 0.5, where adding one half and truncating goes wrong."""
+    ks = np.arange(-127, 127, dtype=np.float32) + np.float32(0.5)
+    near = np.concatenate([ks, np.nextafter(ks, np.float32(-1e9)), np.nextafter(ks, np.float32(1e9)),
+                           np.array([0.0, -0.0, 0.49999997, -0.49999997, 0.25, -0.25, 1e-30, -1e-30],
+                                    np.float32)]).astype(np.float32)
+    ends = np.array([-128.0 if asym else -127.0, 127.0], np.float32)
+    for pad in (0, 3, 5):   # rows of 772, 775, 777: with and without the NEON builds' scalar tail
+        row = np.concatenate([ends, near, np.zeros(pad, np.float32)])
+        x = np.stack([row, row[::-1]]).astype(np.float32)
+        q, sf, zp = fc.batch_quantize_floats(_cuda(x), asym, variant)
+        wq, wsf, wzp = oracle.batch_quantize_floats(x, asym, variant)
+        assert wsf.tolist() == [1.0, 1.0] and wzp.tolist() == [0, 0]
+        assert np.array_equal(q.cpu().numpy(), wq)
+        assert _bits_equal(sf.cpu().numpy(), wsf) and np.array_equal(zp.cpu().numpy(), wzp)
+
+
 def test_batch_quantize_reference_kats_through_hip(fc):
     """tflite/kernels/internal/tensor_utils_test.cc:220-345."""
     a = np.array([[-640, -635.0, -630, 10.0, 2.0, -5.0, -10.0, 0.0, 1000.0]], np.float32)
