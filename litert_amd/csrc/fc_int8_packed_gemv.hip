@@ -758,13 +758,24 @@ void FcInt8ResidentGemvKernel(
       qp.inv = ElementwiseInv(qp);
       const int vector_end = depth - (depth % 8);
       int8_t* qrow = sh.q + wave * qstride;
+      // A row of exactly 16 pieces per lane needs no test per piece (each test is a basic block
+      // of its own and keeps the pieces' arithmetic from overlapping).
+      auto quantize_pieces = [&](auto whole_c) {
+        constexpr bool kWhole = decltype(whole_c)::value;
 #pragma unroll
-      for (int j = 0; j < kPieces; ++j) {
-        const int i = (j * kWaveSize + lane) * 4;
-        const float4 t = xr[j];
-        int32_t packed = QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, i >= vector_end);
-        packed = i < depth ? packed : 0;
-        if (i < staged) *reinterpret_cast<int32_t*>(qrow + i) = packed;
+        for (int j = 0; j < kPieces; ++j) {
+          const int i = (j * kWaveSize + lane) * 4;
+          const float4 t = xr[j];
+          int32_t packed =
+              QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, kWhole ? false : i >= vector_end);
+          if (!kWhole) packed = i < depth ? packed : 0;
+          if (kWhole || i < staged) *reinterpret_cast<int32_t*>(qrow + i) = packed;
+        }
+      };
+      if (depth == kPieces * kWaveSize * 4) {
+        quantize_pieces(std::true_type{});
+      } else {
+        quantize_pieces(std::false_type{});
       }
       // Zeros between 16 pieces' worth and the end of the last share (a few slabs at most).
       for (int i = kPieces * kWaveSize * 4 + lane * 4; i < staged; i += kWaveSize * 4) {
