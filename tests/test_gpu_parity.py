@@ -895,6 +895,33 @@ def test_hybrid_int4_per_channel_nibble_layout_shapes(fc):
         assert _bits_equal(y, want), (B, K, N)
 
 
+@pytest.mark.parametrize("B,K,N", [
+    # fused rows (1..4) on the register-resident form: shares of 8 / 16 / 32 tiles, a depth that
+    # ends inside a lane's eight values, inside a slab, at one slab, at the form's limit
+    (1, 4096, 1040), (2, 4092, 520), (4, 4096, 300), (3, 2000, 700), (4, 1028, 100), (1, 100, 50),
+    (2, 4, 16), (4, 2048, 8200),
+    # few channel groups: the depth is split over the wavefronts of a workgroup
+    (1, 4096, 16), (3, 4096, 100), (2, 2048, 40),
+    # rows that arrive quantized: 4 and 16 chunks per thread, depth not a multiple of 128
+    (5, 1024, 300), (8, 4096, 520), (16, 4096, 1040), (16, 2000, 130), (12, 4080, 64), (9, 16, 20)])
+def test_hybrid_int4_per_channel_register_resident_form(fc, B, K, N):
+    from tests import kat_harness as kh
+    rng = np.random.default_rng(B * 7 + K + N)
+    x = (rng.standard_normal((B, K)) * rng.uniform(0.1, 30, (B, 1))).astype(np.float32)
+    if B > 2:
+        x[1] = 0
+    w = rng.integers(-7, 8, (N, K)).astype(np.int8)
+    packed = np.stack([kh.pack_int4(r) for r in w])
+    fs = rng.uniform(0.01, 0.1, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32) if N % 8 else None
+    op = fc.FullyConnectedHybridInt4PerChannel(packed, K, fs, bias, "relu" if K % 3 else "none")
+    flat = torch.empty(B * N + 1, device="cuda")
+    y = (flat[1:] if (B + N) % 2 else flat[:-1]).view(B, N)   # every other case: rows off 16 bytes
+    got = op(_cuda(x), out=y).cpu().numpy()
+    want = oracle.fc_hybrid_int4_per_channel(x, packed, N, fs, bias, op.activation)
+    assert _bits_equal(got, want), (B, K, N)
+
+
 def test_hybrid_int4_per_channel_reference_kat_and_scalar_scale(fc):
     """tflite/kernels/fully_connected_4bit_test.cc:102-190 through the HIP path (the test's own
     tolerance), with the single filter scale the test model uses."""
