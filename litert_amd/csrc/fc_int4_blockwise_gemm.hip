@@ -31,6 +31,8 @@
 namespace lrtfc {
 namespace {
 
+#define LRTFC_GLOBAL __attribute__((address_space(1)))
+
 constexpr int kThreads = 256;
 constexpr int kBlock = 32;    // depth positions per quantization block
 constexpr int kTile = 16;     // channels / rows per MFMA tile
@@ -394,11 +396,17 @@ struct NibbleGemmArgs {
 // 14336 x 4096, 16 rows: 8 and 4 quads 16.9 us for quantizer + product; 16 weight quads 18.1 us
 // -- a wavefront is alone on its SIMD here (896 wavefronts), and what bounds it is its own
 // chain of about 15 vector operations per block, not the loads.
+// The wavefronts of the 4-bit-resident kernels share nothing (no LDS image, no barrier), so each is
+// a workgroup of its own: the dispatcher then spreads them one by one over the compute units.
+// In workgroups of four, a launch of 2304 wavefronts leaves 64 compute units with three
+// workgroups and the rest with two, and takes as long as three everywhere (36864 x 16384 at four
+// rows: 84 us; as single wavefronts 71 us; 28672 x 16384: 59.6 -> 54.5 us).
+constexpr int kLoneWave = 64;
+
 template <int RT, int WQ, int XQ>
-__global__ __launch_bounds__(kThreads) void FcInt4NibbleGemmKernel(NibbleGemmArgs a) {
+__global__ __launch_bounds__(kLoneWave) void FcInt4NibbleGemmKernel(NibbleGemmArgs a) {
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int ct0 = blockIdx.x * 4 + wave;
+  const int ct0 = blockIdx.x;
   const int rt0 = blockIdx.y * RT;
   if (ct0 >= a.channel_tiles || rt0 >= a.row_tiles) return;
   int rt[RT];
@@ -573,8 +581,17 @@ __device__ __forceinline__ void FcInt4NibbleQuadBody(const NibbleQuadArgs& a, in
   const int nb = a.nb;
   const int nq = (nb + 3) / 4;
   const int ng = (nb + 15) / 16;
-  const i32x4* wp = a.filter + static_cast<size_t>(ct0) * nq * 64 + lane;
-  const uint2* sp = a.scales + static_cast<size_t>(ct0) * ng * 64 + lane;
+  // Every tensor is in global memory. The grouped kernel reads this struct from a table in
+  // memory, and pointers that come from memory carry no address space: accesses through them
+  // would go the flat path, whose waits also count LDS traffic (the scale broadcasts) and cannot
+  // leave the rings of loads in flight. So the address space is stated here.
+  const LRTFC_GLOBAL i32x4* wp =
+      (const LRTFC_GLOBAL i32x4*)a.filter + static_cast<size_t>(ct0) * nq * 64 + lane;
+  using U32x2 = unsigned __attribute__((ext_vector_type(2)));
+  using F32x4 = float __attribute__((ext_vector_type(4)));
+  const LRTFC_GLOBAL U32x2* sp =
+      (const LRTFC_GLOBAL U32x2*)a.scales + static_cast<size_t>(ct0) * ng * 64 + lane;
+  const LRTFC_GLOBAL int8_t* g_rows = (const LRTFC_GLOBAL int8_t*)a.rows;
   // This lane's eight activation bytes of quad q lie at rows + x_first + 128 q (clamped to the
   // row's last block: past the depth the weights are zeros).
   const uint32_t x_lane = static_cast<uint32_t>(r) * a.depth + 8 * (lane >> 4);
@@ -586,12 +603,15 @@ __device__ __forceinline__ void FcInt4NibbleQuadBody(const NibbleQuadArgs& a, in
   // Past the depth: the last block again (its weights there are zeros).
   auto fetch_x = [&](int q) {
     const uint32_t at = min(x_first + static_cast<uint32_t>(min(q, nq - 1)) * (4 * kBlock), x_last);
-    return *reinterpret_cast<const i64*>(a.rows + at);
+    return *reinterpret_cast<const LRTFC_GLOBAL i64*>(g_rows + at);
   };
   constexpr int kGroups = WQ / 4 + 1 <= 2 ? 2 : (WQ / 4 + 1 <= 4 ? 4 : 8);
   static_assert((kGroups - 1) * 4 >= WQ, "scale groups must lead the weight ring");
   uint2 sg[kGroups];
-  auto fetch_scales = [&](int g) { return sp[static_cast<size_t>(min(g, ng - 1)) * 64]; };
+  auto fetch_scales = [&](int g) {
+    const U32x2 raw = sp[static_cast<size_t>(min(g, ng - 1)) * 64];
+    return make_uint2(raw.x, raw.y);
+  };
 #pragma unroll
   for (int g = 0; g + 1 < kGroups; ++g) sg[g] = fetch_scales(g);
   i32x4 wring[WQ];
@@ -667,21 +687,23 @@ __device__ __forceinline__ void FcInt4NibbleQuadBody(const NibbleQuadArgs& a, in
   // fully_connected.cc:1078-1082, after taking the factor 16 back out (exact).
   const int m = col;
   if (m >= a.batches || m >= 4) return;
-  const float zp = static_cast<float>(a.zero_points[m]);
-  const float row_scale = a.scaling_factors[m];
+  const float zp = static_cast<float>(((const LRTFC_GLOBAL int32_t*)a.zero_points)[m]);
+  const float row_scale = ((const LRTFC_GLOBAL float*)a.scaling_factors)[m];
+  const LRTFC_GLOBAL float* g_kfsum = (const LRTFC_GLOBAL float*)a.kfsum;
+  const LRTFC_GLOBAL float* g_bias = (const LRTFC_GLOBAL float*)a.bias;
   const int n0 = ct0 * kTile + 4 * (lane >> 4);
   float o[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int n = min(n0 + i, a.out_depth - 1);
-    float v = __fsub_rn(__fmul_rn(out[i], 0.0625f), __fmul_rn(zp, a.kfsum[n]));
+    float v = __fsub_rn(__fmul_rn(out[i], 0.0625f), __fmul_rn(zp, g_kfsum[n]));
     v = __fmul_rn(v, row_scale);
-    if (a.bias) v = __fadd_rn(v, a.bias[n]);
+    if (a.bias) v = __fadd_rn(v, g_bias[n]);
     o[i] = v;
   }
-  float* dst = a.output + static_cast<size_t>(m) * a.out_depth + n0;
+  LRTFC_GLOBAL float* dst = (LRTFC_GLOBAL float*)a.output + static_cast<size_t>(m) * a.out_depth + n0;
   if (n0 + 3 < a.out_depth && a.vector_store) {
-    *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+    *reinterpret_cast<LRTFC_GLOBAL F32x4*>(dst) = F32x4{o[0], o[1], o[2], o[3]};
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -691,9 +713,8 @@ __device__ __forceinline__ void FcInt4NibbleQuadBody(const NibbleQuadArgs& a, in
 }
 
 template <int WQ, int XQ>
-__global__ __launch_bounds__(kThreads) void FcInt4NibbleQuadKernel(NibbleQuadArgs a) {
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int ct0 = blockIdx.x * 4 + wave;
+__global__ __launch_bounds__(kLoneWave) void FcInt4NibbleQuadKernel(NibbleQuadArgs a) {
+  const int ct0 = blockIdx.x;
   if (ct0 >= a.channel_tiles) return;
   FcInt4NibbleQuadBody<WQ, XQ>(a, ct0);
 }
@@ -710,22 +731,22 @@ struct NibbleQuadGroupTable {
 };
 
 template <int WQ, int XQ>
-__global__ __launch_bounds__(kThreads) void FcInt4NibbleQuadGroupedKernel(
+__global__ __launch_bounds__(kLoneWave) void FcInt4NibbleQuadGroupedKernel(
     const NibbleQuadGroupTable* __restrict__ table, int count) {
-  // first_block is ascending: this workgroup's node is the number of later nodes whose first
-  // workgroup is not beyond it (vector loads and ballots, 64 nodes per turn).
+  // The table counts in blocks of four channel tiles (first_block); a workgroup is one wavefront
+  // with one tile. first_block is ascending: this block's node is the number of later nodes whose
+  // first block is not beyond it (vector loads and ballots, 64 nodes per turn).
   const int lane = threadIdx.x & 63;
+  const int block = static_cast<int>(blockIdx.x >> 2);
   int node = 0;
   for (int base = 0; base + 1 < count; base += 64) {
     const int probe = base + lane + 1;
-    const bool not_beyond =
-        probe < count && static_cast<int>(blockIdx.x) >= table->first_block[min(probe, count)];
+    const bool not_beyond = probe < count && block >= table->first_block[min(probe, count)];
     node += __popcll(__ballot(not_beyond));
   }
   node = __builtin_amdgcn_readfirstlane(node);
   const NibbleQuadArgs a = table->node[node];
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int ct0 = (static_cast<int>(blockIdx.x) - table->first_block[node]) * 4 + wave;
+  const int ct0 = (block - table->first_block[node]) * 4 + static_cast<int>(blockIdx.x & 3);
   if (ct0 >= a.channel_tiles) return;
   FcInt4NibbleQuadBody<WQ, XQ>(a, ct0);
 }
@@ -920,8 +941,8 @@ hipError_t LaunchFcInt4BlockwiseNibbleGemm(const float* input, int variant,
     q.nb = nb;
     q.channel_tiles = channel_tiles;
     q.vector_store = (out_depth % 4 == 0) && (reinterpret_cast<uintptr_t>(output) % 16 == 0);
-    hipLaunchKernelGGL((FcInt4NibbleQuadKernel<8, 4>), dim3((channel_tiles + 3) / 4), dim3(kThreads),
-                       0, stream, q);
+    hipLaunchKernelGGL((FcInt4NibbleQuadKernel<8, 4>), dim3(channel_tiles), dim3(kLoneWave), 0,
+                       stream, q);
     return hipGetLastError();
   }
   switch (variant) {
@@ -956,12 +977,12 @@ hipError_t LaunchFcInt4BlockwiseNibbleGemm(const float* input, int variant,
   a.row_tiles = row_tiles;
   a.vector_store = (out_depth % 4 == 0) && (reinterpret_cast<uintptr_t>(output) % 16 == 0);
   const int RT = row_tiles <= 1 ? 1 : 2;
-  const dim3 grid((channel_tiles + 3) / 4, (row_tiles + RT - 1) / RT);
+  const dim3 grid(channel_tiles, (row_tiles + RT - 1) / RT);
   if (grid.y > 65535) return hipErrorInvalidValue;
   if (RT == 1) {
-    hipLaunchKernelGGL((FcInt4NibbleGemmKernel<1, 8, 4>), grid, dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((FcInt4NibbleGemmKernel<1, 8, 4>), grid, dim3(kLoneWave), 0, stream, a);
   } else {
-    hipLaunchKernelGGL((FcInt4NibbleGemmKernel<2, 8, 2>), grid, dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((FcInt4NibbleGemmKernel<2, 8, 2>), grid, dim3(kLoneWave), 0, stream, a);
   }
   return hipGetLastError();
 }
@@ -1058,11 +1079,11 @@ hipError_t LaunchFcInt4NibbleGrouped(const void* table, const lrtfc_int4_group_l
   if (hipError_t err = hipGetLastError()) return err;
   // Few wavefronts per SIMD (narrow, deep filters): each keeps twice the loads in flight.
   if (l.grid_blocks * 4 <= 4096) {
-    hipLaunchKernelGGL((FcInt4NibbleQuadGroupedKernel<16, 8>), dim3(l.grid_blocks), dim3(kThreads),
-                       0, stream, t, l.count);
+    hipLaunchKernelGGL((FcInt4NibbleQuadGroupedKernel<16, 8>), dim3(l.grid_blocks * 4),
+                       dim3(kLoneWave), 0, stream, t, l.count);
   } else {
-    hipLaunchKernelGGL((FcInt4NibbleQuadGroupedKernel<8, 4>), dim3(l.grid_blocks), dim3(kThreads),
-                       0, stream, t, l.count);
+    hipLaunchKernelGGL((FcInt4NibbleQuadGroupedKernel<8, 4>), dim3(l.grid_blocks * 4),
+                       dim3(kLoneWave), 0, stream, t, l.count);
   }
   return hipGetLastError();
 }

@@ -237,6 +237,21 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
                                             PLACEMENT place = PLACEMENT()) {
   const bool vec_ok = (n_data % 4 == 0) && ((reinterpret_cast<uintptr_t>(v) & 15) == 0) &&
                       ((reinterpret_cast<uintptr_t>(q) & 3) == 0);
+  // Rows and results are in global memory. Callers that read these pointers from a table in
+  // memory hand them over without an address space, and accesses through such pointers would go
+  // the flat path; so the address space is stated here.
+  using Float4 = float __attribute__((ext_vector_type(4)));
+  using GlobalF4 = const __attribute__((address_space(1))) Float4;
+  using GlobalF = const __attribute__((address_space(1))) float;
+  using GlobalI32 = __attribute__((address_space(1))) int32_t;
+  using GlobalC = __attribute__((address_space(1))) int8_t;
+  auto load4 = [](GlobalF4* at) {
+    const Float4 r = *at;
+    return make_float4(r.x, r.y, r.z, r.w);
+  };
+  GlobalF4* const gv4 = (GlobalF4*)v;
+  GlobalF* const gv = (GlobalF*)v;
+  GlobalC* const gq = (GlobalC*)q;
 
   // Pass 1: range of the row. Starting from 0 gives min(0, min v) / max(0, max v),
   // which is also what max(|min|, |max|) needs for the symmetric case.
@@ -252,12 +267,12 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   const bool short_row = n4 <= kShortRegs * THREADS;
   float4 held[kRowRegs];
   if (in_regs) {
-    const float4* v4 = reinterpret_cast<const float4*>(v);
+    GlobalF4* v4 = gv4;
     // Past the end: the row's last piece again (an unconditional load), then taken as zeros, which
     // the range (it always includes 0) does not notice.
     auto take = [&](int j) {
       const int i = threadIdx.x + j * THREADS;
-      held[j] = v4[min(i, n4 - 1)];
+      held[j] = load4(v4 + min(i, n4 - 1));
     };
     auto widen = [&](int j) {
       const int i = threadIdx.x + j * THREADS;
@@ -277,16 +292,16 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
       for (int j = 0; j < kRowRegs; ++j) widen(j);
     }
   } else if (vec_ok) {
-    const float4* v4 = reinterpret_cast<const float4*>(v);
+    GlobalF4* v4 = gv4;
     for (int i = threadIdx.x; i < n_data / 4; i += THREADS) {
-      const float4 t = v4[i];
+      const float4 t = load4(v4 + i);
       mn = fminf(fminf(mn, t.x), fminf(fminf(t.y, t.z), t.w));
       mx = fmaxf(fmaxf(mx, t.x), fmaxf(fmaxf(t.y, t.z), t.w));
     }
   } else {
     for (int i = threadIdx.x; i < n_data; i += THREADS) {
-      mn = fminf(mn, v[i]);
-      mx = fmaxf(mx, v[i]);
+      mn = fminf(mn, gv[i]);
+      mx = fmaxf(mx, gv[i]);
     }
   }
   const RowRange range = BlockMinMax<THREADS>(mn, mx);
@@ -299,8 +314,8 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   const int32_t zp = qp.zero_point;
   const bool all_zero = qp.all_zero;
   if (threadIdx.x == 0) {
-    *scaling_factor = sf;
-    if (zero_point) *zero_point = zp;
+    *(__attribute__((address_space(1))) float*)scaling_factor = sf;
+    if (zero_point) *(__attribute__((address_space(1))) int32_t*)zero_point = zp;
   }
 
   // Pass 2: elementwise. The NEON builds process 8 floats per step and finish
@@ -308,23 +323,17 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
   const int vector_end = n_data - (n_data % 8);
   // Elements 4 i .. 4 i + 3 of the row, given as t.
   auto emit4 = [&](int i, const float4& t) {
-    char4 o;
-    if (all_zero) {
-      o = make_char4(0, 0, 0, 0);
-    } else {
+    int32_t word = 0;
+    if (!all_zero) {
       const bool tail = 4 * i >= vector_end;
       if (do_asymmetric) {
-        const int32_t packed = QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, tail);
-        o = make_char4(static_cast<char>(packed), static_cast<char>(packed >> 8),
-                       static_cast<char>(packed >> 16), static_cast<char>(packed >> 24));
+        word = QuantizePack4<VARIANT>(t.x, t.y, t.z, t.w, qp, tail);
       } else {
-        o.x = static_cast<char>(QuantizeSym<VARIANT>(t.x, inv, tail));
-        o.y = static_cast<char>(QuantizeSym<VARIANT>(t.y, inv, tail));
-        o.z = static_cast<char>(QuantizeSym<VARIANT>(t.z, inv, tail));
-        o.w = static_cast<char>(QuantizeSym<VARIANT>(t.w, inv, tail));
+        word = PackBytes(QuantizeSym<VARIANT>(t.x, inv, tail), QuantizeSym<VARIANT>(t.y, inv, tail),
+                         QuantizeSym<VARIANT>(t.z, inv, tail), QuantizeSym<VARIANT>(t.w, inv, tail));
       }
     }
-    *reinterpret_cast<char4*>(q + place(4 * i)) = o;
+    *(GlobalI32*)(gq + place(4 * i)) = word;
   };
   if (in_regs) {
     if (short_row) {
@@ -341,17 +350,17 @@ __device__ __forceinline__ void QuantizeRow(const float* __restrict__ v, int n_d
       }
     }
   } else if (vec_ok) {
-    const float4* v4 = reinterpret_cast<const float4*>(v);
-    for (int i = threadIdx.x; i < n_data / 4; i += THREADS) emit4(i, v4[i]);
+    GlobalF4* v4 = gv4;
+    for (int i = threadIdx.x; i < n_data / 4; i += THREADS) emit4(i, load4(v4 + i));
   } else {
     for (int i = threadIdx.x; i < n_data; i += THREADS) {
       int8_t o = 0;
       if (!all_zero) {
         const bool tail = i >= vector_end;
-        o = static_cast<int8_t>(do_asymmetric ? QuantizeAsym<VARIANT>(v[i], inv, zp, tail)
-                                              : QuantizeSym<VARIANT>(v[i], inv, tail));
+        o = static_cast<int8_t>(do_asymmetric ? QuantizeAsym<VARIANT>(gv[i], inv, zp, tail)
+                                              : QuantizeSym<VARIANT>(gv[i], inv, tail));
       }
-      q[place(i)] = o;
+      gq[place(i)] = o;
     }
   }
 }
