@@ -1077,8 +1077,10 @@ hipError_t LaunchFcInt4NibbleGrouped(const void* table, const lrtfc_int4_group_l
       break;
   }
   if (hipError_t err = hipGetLastError()) return err;
-  // Few wavefronts per SIMD (narrow, deep filters): each keeps twice the loads in flight.
-  if (l.grid_blocks * 4 <= 4096) {
+  // At most one wavefront per SIMD (narrow, deep filters): each keeps twice the loads in flight
+  // (config 5's 18 down projections at four rows, 2304 wavefronts: 82.7 us on the small rings,
+  // 90.0 us on the large ones).
+  if (l.grid_blocks * 4 <= 1024) {
     hipLaunchKernelGGL((FcInt4NibbleQuadGroupedKernel<16, 8>), dim3(l.grid_blocks * 4),
                        dim3(kLoneWave), 0, stream, t, l.count);
   } else {
