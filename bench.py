@@ -267,7 +267,7 @@ def main():
                                      "this size, %.1f%% of peak" % (N_OUT * K_IN / floor2_us / 1e3 /
                                                                   HBM_PEAK_GBPS * 100))
 
-    # Between decode and prefill (not a BASELINE configuration): config 2's filters against 16
+    # Between decode and prefill (not one of the benchmark configurations): config 2's filters against 16
     # and 32 rows (row quantizer + register-resident GEMV), 64 and 128 rows (row quantizer + the
     # GEMV that walks the rows through LDS in depth chunks) and 512 rows (row quantizer + MFMA
     # GEMM).
@@ -616,7 +616,7 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         op_gbps_cold=round(b3 / o_cold / 1e3, 1), op_gbps_hot=round(b3 / o_hot / 1e3, 1),
         frac_of_hbm_peak_cold=round(b3 / o_cold / 1e3 / HBM_PEAK_GBPS, 4), algorithmic_bytes=b3,
         kernel="FcInt4PackedKernel<fused quantize> on the re-tiled filter")
-    # Prefill batches on the blockwise int4 path (not a BASELINE configuration): config 3's filter
+    # Prefill batches on the blockwise int4 path (not one of the benchmark configurations): config 3's filter
     # against 2048 and 128 rows through the matrix-core GEMM (row quantizer + GEMM launches),
     # and what the decode kernel needs for the same rows in passes of four.
     op3 = fc.FullyConnectedBlockwiseInt4(c3["packed"], c3["scales"], 4096, 32)
@@ -634,7 +634,7 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
     out["next_int4_blockwise_prefill_14336x4096"] = entry
     del op3
 
-    # Between decode and prefill on the blockwise int4 path (not a BASELINE configuration): the
+    # Between decode and prefill on the blockwise int4 path (not one of the benchmark configurations): the
     # op as dispatched (lrtfc_fc_blockwise_int4_preferred_form picks the form per shape), filter
     # copies rotated (cold), and the forms it chose against at 8 and 16 rows.
     forms = {capi.INT4_FORM_DECODE: "decode kernel", capi.INT4_FORM_GEMM_NIBBLES: "4-bit-resident GEMM",
@@ -658,7 +658,7 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
 
     del ops3
 
-    # Next-row op (not a BASELINE configuration): per-channel int4 hybrid FC (EvalHybridDense4Bit)
+    # Next-row op (not one of the benchmark configurations): per-channel int4 hybrid FC (EvalHybridDense4Bit)
     # at config 3's shape, B = 1, on the 4-bit-resident filter and on its int8 expansion.
     g4 = torch.Generator(device="cuda").manual_seed(11)
     nib = [torch.randint(0, 256, (14336, 2048), dtype=torch.uint8, device="cuda", generator=g4)

@@ -16,7 +16,7 @@
 //
 // Two kernels run on this layout. FcInt8ResidentGemvKernel (further down, with its own
 // account) takes the launches whose per-wavefront share of the depth fits the registers:
-// depth up to 8192 at decode widths, i.e. the BASELINE shapes. FcInt8PackedGemvKernel is the
+// depth up to 8192 at decode widths, i.e. the benchmark configurations. FcInt8PackedGemvKernel is the
 // general form for everything else: a wavefront streams a contiguous run of one 16-channel
 // group's tiles through a ring of 16 outstanding 1 KiB loads, refilling a slot as soon as the
 // matrix core has consumed it; four wavefronts form a workgroup and share the staged
