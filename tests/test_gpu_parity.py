@@ -922,6 +922,27 @@ def test_hybrid_int4_per_channel_register_resident_form(fc, B, K, N):
     assert _bits_equal(got, want), (B, K, N)
 
 
+def test_hybrid_int4_per_channel_seeded_random_shapes(fc):
+    """Forty seeded draws over row counts, even depths and channel counts that cross every launch
+    rule of the 4-bit-resident GEMV (fused rows or not, register-resident or ring, depth shares,
+    16-row passes), each bit-identical to the oracle."""
+    from tests import kat_harness as kh
+    rng = np.random.default_rng(20240607)
+    for case in range(40):
+        B = int(rng.integers(1, 21))
+        K = int(rng.choice([2, 4, 16]) * rng.integers(1, 300))
+        N = int(rng.integers(1, 600))
+        x = (rng.standard_normal((B, K)) * rng.uniform(0.05, 50)).astype(np.float32)
+        w = rng.integers(-7, 8, (N, K)).astype(np.int8)
+        packed = np.stack([kh.pack_int4(r) for r in w])
+        fs = rng.uniform(0.01, 0.1, N).astype(np.float32)
+        bias = rng.standard_normal(N).astype(np.float32) if case % 3 else None
+        op = fc.FullyConnectedHybridInt4PerChannel(packed, K, fs, bias, ("none", "relu", "relu6")[case % 3])
+        got = op(_cuda(x)).cpu().numpy()
+        want = oracle.fc_hybrid_int4_per_channel(x, packed, N, fs, bias, op.activation)
+        assert _bits_equal(got, want), (case, B, K, N)
+
+
 def test_hybrid_int4_per_channel_reference_kat_and_scalar_scale(fc):
     """tflite/kernels/fully_connected_4bit_test.cc:102-190 through the HIP path (the test's own
     tolerance), with the single filter scale the test model uses."""
