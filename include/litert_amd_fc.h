@@ -427,7 +427,9 @@ typedef struct lrtfc_int4_group_node {
 } lrtfc_int4_group_node;
 typedef struct lrtfc_int4_group_launch {
   int count, grid_blocks, ksplit, groups_per_wave, batches, depth;
-  int split_quantize;            /* rows are quantized by a launch of their own */
+  int split_quantize;            /* 0: rows quantized in the kernel's prologue; 1: by a launch of
+                                    their own; 2: in the prologue, three or four rows of a small
+                                    group as two pairs side by side in one launch */
   int form;                      /* LRTFC_INT4_FORM_DECODE or LRTFC_INT4_FORM_GEMM_NIBBLES */
 } lrtfc_int4_group_launch;
 size_t lrtfc_int4_group_table_bytes(void);

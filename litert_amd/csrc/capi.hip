@@ -1252,7 +1252,7 @@ int lrtfc_fc_blockwise_int4_packed_grouped(const void* device_table,
                     launch->grid_blocks >= 1 && launch->ksplit >= 1 && launch->ksplit <= 4 &&
                     launch->groups_per_wave >= 1 && launch->groups_per_wave <= 8 &&
                     (launch->ksplit == 1 || launch->groups_per_wave == 1) &&
-                    (launch->split_quantize == 0 || launch->split_quantize == 1) &&
+                    launch->split_quantize >= 0 && launch->split_quantize <= 2 &&
                     (launch->form == LRTFC_INT4_FORM_DECODE ||
                      launch->form == LRTFC_INT4_FORM_GEMM_NIBBLES),
                 "launch record was not filled by lrtfc_int4_group_prepare");

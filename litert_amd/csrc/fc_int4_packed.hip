@@ -43,6 +43,9 @@ constexpr int kPStride = kTileBlocks + 4;  // floats per (row, batch) line of pa
 constexpr int kMaxGroupNodes = LRTFC_INT4_GROUP_MAX;
 constexpr int kMaxGroupsPerWave = 8;  // 64 channels: one lane each when their kfsum is staged
 constexpr int kSplitShallowMinBlocks = 1024;  // grouped launches: see PrepareInt4Group
+constexpr int kRowPairsSideBySide = 2;        // lrtfc_int4_group_launch.split_quantize
+constexpr int kSideBySideMaxBlocks = 256;
+constexpr int64_t kSideBySideMaxFilterBytes = 24 << 20;
 
 __global__ __launch_bounds__(kThreads) void PackInt4BlockwiseKernel(
     const uint8_t* __restrict__ filter, const uint16_t* __restrict__ scales, int out_depth,
@@ -649,8 +652,11 @@ __global__ __launch_bounds__(kThreads) void FcInt4PackedGroupedKernel(
   }
   node = __builtin_amdgcn_readfirstlane(node);
   const Int4PackedArgs a = table->node[node];
-  FcInt4PackedBody<BT, FUSED, VARIANT, GPT>(a, blockIdx.x - table->first_block[node], batch0, bt,
-                                            ksplit, gpw, smem);
+  // Row tiles side by side (gridDim.y > 1): slice y of the grid takes rows batch0 + y * bt on.
+  const int first_row = batch0 + static_cast<int>(blockIdx.y) * bt;
+  const int rows = min(bt, a.batches - first_row);
+  FcInt4PackedBody<BT, FUSED, VARIANT, GPT>(a, blockIdx.x - table->first_block[node], first_row,
+                                            rows, ksplit, gpw, smem);
 }
 
 // The row quantizer for a whole group: workgroup r quantizes row r % batches of node
@@ -877,6 +883,18 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
   bool split = batches > 2 && depth <= kDeepDepth &&
                (depth > kShallowDepth || total_blocks >= kSplitShallowMinBlocks);
   for (int i = 0; i < count; ++i) split = split && nodes[i].workspace != nullptr;
+  // Three or four rows of a SMALL group (a stage of a decoder: one to three nodes that leave
+  // most of the chip without a workgroup, their filters a few megabytes that the second reader
+  // finds in the caches): the rows go as two pairs side by side in ONE launch, each workgroup
+  // quantizing and multiplying two rows (2048 x 2048 at four rows: 6.3 us as one tile of four,
+  // 4.7 us for two rows; 2048 x 16384: 16.5 us with the quantizer launch, 12.0 us for two fused
+  // rows). Two rows of depth up to kDeepDepth always fit the fused form's LDS.
+  const int64_t filter_bytes = static_cast<int64_t>(total_out) * depth / 2;
+  const bool side_by_side = (batches == 3 || batches == 4) && depth <= kDeepDepth &&
+                            total_blocks <= kSideBySideMaxBlocks &&
+                            filter_bytes <= kSideBySideMaxFilterBytes &&
+                            FitBatchTile(2, chunks * kTileBlocks * kBlock, ksplit) == 2;
+  if (side_by_side) split = false;
   Int4GroupTable host{};
   int next = 0;
   for (int i = 0; i < count; ++i) {
@@ -914,7 +932,7 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
   launch->groups_per_wave = gpw;
   launch->batches = batches;
   launch->depth = depth;
-  launch->split_quantize = split ? 1 : 0;
+  launch->split_quantize = side_by_side ? kRowPairsSideBySide : (split ? 1 : 0);
   launch->form = LRTFC_INT4_FORM_DECODE;
   return hipSuccess;
 }
@@ -927,13 +945,13 @@ size_t Int4GroupTableBytes() {
 namespace {
 template <int BT, bool FUSED, int VARIANT, int GPT>
 hipError_t LaunchGroupedOne(const void* table, const lrtfc_int4_group_launch& l, int batch0,
-                            int bt, hipStream_t stream) {
+                            int bt, hipStream_t stream, int row_tiles = 1) {
   const int chunks = (l.depth / kBlock + kTileBlocks - 1) / kTileBlocks;
   const int padded = chunks * kTileBlocks * kBlock;
   const size_t lds = Int4Shared<BT>::Bytes(padded, l.ksplit);
   auto kernel = FcInt4PackedGroupedKernel<BT, FUSED, VARIANT, GPT>;
   if (hipError_t err = EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds)) return err;
-  hipLaunchKernelGGL(kernel, dim3(l.grid_blocks), dim3(kThreads), lds, stream,
+  hipLaunchKernelGGL(kernel, dim3(l.grid_blocks, row_tiles), dim3(kThreads), lds, stream,
                      static_cast<const Int4GroupTable*>(table), l.count, batch0, bt, l.ksplit,
                      l.groups_per_wave);
   return hipGetLastError();
@@ -941,14 +959,17 @@ hipError_t LaunchGroupedOne(const void* table, const lrtfc_int4_group_launch& l,
 
 template <int BT, int GPT>
 hipError_t LaunchGroupedVariant(const void* table, const lrtfc_int4_group_launch& l, int variant,
-                                int batch0, int bt, hipStream_t stream) {
+                                int batch0, int bt, hipStream_t stream, int row_tiles = 1) {
   switch (variant) {
     case LRTFC_QUANT_NEON_V8:
-      return LaunchGroupedOne<BT, true, LRTFC_QUANT_NEON_V8, GPT>(table, l, batch0, bt, stream);
+      return LaunchGroupedOne<BT, true, LRTFC_QUANT_NEON_V8, GPT>(table, l, batch0, bt, stream,
+                                                                  row_tiles);
     case LRTFC_QUANT_NEON_LEGACY:
-      return LaunchGroupedOne<BT, true, LRTFC_QUANT_NEON_LEGACY, GPT>(table, l, batch0, bt, stream);
+      return LaunchGroupedOne<BT, true, LRTFC_QUANT_NEON_LEGACY, GPT>(table, l, batch0, bt, stream,
+                                                                      row_tiles);
     default:
-      return LaunchGroupedOne<BT, true, LRTFC_QUANT_PORTABLE, GPT>(table, l, batch0, bt, stream);
+      return LaunchGroupedOne<BT, true, LRTFC_QUANT_PORTABLE, GPT>(table, l, batch0, bt, stream,
+                                                                   row_tiles);
   }
 }
 
@@ -990,7 +1011,7 @@ hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_l
   }
   const int chunks = (l.depth / kBlock + kTileBlocks - 1) / kTileBlocks;
   const int padded = chunks * kTileBlocks * kBlock;
-  if (l.split_quantize) {
+  if (l.split_quantize == 1) {
     if (hipError_t err = LaunchGroupQuantizer(table, l, variant, stream)) return err;
     const bool deep_rows = l.depth > kShallowDepth;
     const int tile = FitBatchTile(4, padded, l.ksplit);
@@ -1011,6 +1032,11 @@ hipError_t LaunchFcInt4PackedGrouped(const void* table, const lrtfc_int4_group_l
     return hipSuccess;
   }
   const bool deep = l.depth > kShallowDepth && l.depth <= kDeepDepth;
+  if (l.split_quantize == kRowPairsSideBySide) {
+    // Three or four rows of a small group: two slices of the grid, two fused rows each.
+    return deep ? LaunchGroupedVariant<2, 8>(table, l, variant, 0, 2, stream, 2)
+                : LaunchGroupedVariant<2, 2>(table, l, variant, 0, 2, stream, 2);
+  }
   const int tile = FitBatchTile(MaxBatchTile<true>(l.depth), padded, l.ksplit);
   for (int batch0 = 0; batch0 < l.batches; batch0 += tile) {  // more rows: one launch per tile
     const int bt = min(tile, l.batches - batch0);

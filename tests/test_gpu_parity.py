@@ -746,9 +746,10 @@ def test_blockwise_int4_gemm_full_width_agrees_with_decode_kernel(fc):
 
 @pytest.mark.parametrize("variant", [1, 2])
 def test_blockwise_int4_grouped_deep_rows_quantizer_variants(fc, variant):
-    """The group's row quantizer launch (deep rows, more than two per node) in the two NEON
-    flavours, with elements on rounding ties."""
-    B, K, Ns = 4, 8200 - 8, (16, 24)
+    """The group's row quantizer launch (deep rows, more than two per node, filters too large in
+    all for the side-by-side form of small groups) in the two NEON flavours, with elements on
+    rounding ties."""
+    B, K, Ns = 4, 8200 - 8, (4104, 2056)
     cs = [wl.blockwise_int4_fc(B, K, n, seed=40 + n) for n in Ns]
     for c in cs:
         c["x"][0, :4] = [-125.0, 130.0, 2.5, -2.5]
@@ -757,6 +758,28 @@ def test_blockwise_int4_grouped_deep_rows_quantizer_variants(fc, variant):
     ys = [torch.empty((B, n), dtype=torch.float32, device="cuda") for n in Ns]
     group = fc.GroupedBlockwiseInt4(ops).bind([_cuda(c["x"]) for c in cs], ys)
     assert group.launch.split_quantize == 1
+    group()
+    torch.cuda.synchronize()
+    for c, y, n in zip(cs, ys, Ns):
+        want = oracle.fc_blockwise_int4(c["x"], c["packed"], n, c["scales"].view(np.uint16), 32,
+                                        variant=variant)
+        assert _bits_equal(y.cpu().numpy(), want), n
+
+
+@pytest.mark.parametrize("B,K,Ns,variant", [(4, 2048, (2048,), 0), (3, 2048, (2048, 256, 256), 1),
+                                            (4, 16384, (264,), 2), (3, 8192, (24, 40, 8), 0),
+                                            (4, 4096 + 64, (72,), 0)])
+def test_blockwise_int4_small_groups_run_row_pairs_side_by_side(fc, B, K, Ns, variant):
+    """Three or four rows of a small group (a decoder stage) go as two fused pairs in one launch:
+    rows 2 and 3 from the second slice of the grid, a third row alone in its slice."""
+    cs = [wl.blockwise_int4_fc(B, K, n, seed=90 + i + n, lo=-8, hi=7) for i, n in enumerate(Ns)]
+    for c in cs:
+        c["x"][B - 1, :4] = [-125.0, 130.0, 2.5, -2.5]
+    ops = [fc.FullyConnectedBlockwiseInt4(c["packed"], c["scales"], K, 32, quant_variant=variant)
+           for c in cs]
+    ys = [torch.full((B, n), float("nan"), dtype=torch.float32, device="cuda") for n in Ns]
+    group = fc.GroupedBlockwiseInt4(ops).bind([_cuda(c["x"]) for c in cs], ys)
+    assert group.launch.split_quantize == 2
     group()
     torch.cuda.synchronize()
     for c, y, n in zip(cs, ys, Ns):
