@@ -888,7 +888,8 @@ hipError_t PrepareInt4Group(const lrtfc_int4_group_node* nodes, int count, int b
   // finds in the caches): the rows go as two pairs side by side in ONE launch, each workgroup
   // quantizing and multiplying two rows (2048 x 2048 at four rows: 6.3 us as one tile of four,
   // 4.7 us for two rows; 2048 x 16384: 16.5 us with the quantizer launch, 12.0 us for two fused
-  // rows). Two rows of depth up to kDeepDepth always fit the fused form's LDS.
+  // rows). Larger filters lose: the two 2048 -> 16384 projections of a decoder layer, 33.5 MB,
+  // as pairs side by side take config 5's decoder-ordered token from 688 to 736 us.
   const int64_t filter_bytes = static_cast<int64_t>(total_out) * depth / 2;
   const bool side_by_side = (batches == 3 || batches == 4) && depth <= kDeepDepth &&
                             total_blocks <= kSideBySideMaxBlocks &&
