@@ -698,7 +698,7 @@ def extras(torch, fc, capi, lib, wl, p, stream, capture, timed_replays, per_laun
         if count == 2048:
             entry["frac_of_hbm_peak_2048_tokens"] = round(moved / us / 1e3 / HBM_PEAK_GBPS, 4)
             entry["algorithmic_bytes_2048_tokens"] = moved
-    entry["kernel"] = "EmbeddingLookupKernel<Int4, float32, 8 columns per thread>"
+    entry["kernel"] = "EmbeddingLookupKernel<Int4, float32, 8 columns per thread; from 32 rows on as two runs of 4>"
     out["next_embedding_lookup_blockwise_int4_256000x2048"] = entry
     del table, tscales, lookup_op
 
