@@ -389,6 +389,9 @@ void FcInt4PerChannelResidentKernel(const uint8_t* early_packed, const float* ea
                                     const int8_t* early_input, int early_depth, int early_slabs,
                                     int early_out_depth, int batch0, int bt, int ksplit_log2,
                                     int per_part, NibbleArgs unread) {
+  // `unread` is never named again: its fields are fetched from the argument segment through
+  // late_args() at the points where they are needed (naming it would let the compiler move all
+  // of those loads to the kernel's entry, in front of the first weight request).
   extern __shared__ __align__(16) int8_t smem[];
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
